@@ -1,0 +1,244 @@
+// Elementwise kernel engine: one N-ary kernel pair (contiguous / row-vectorised
+// strided) instantiated for every functor and element-type combination.
+//
+// Replaces the Unary/Binary{Contig,Strided,RowBroadcast}Functor kernels and
+// their launchers (libtensor/include/kernels/elementwise_functions/common.hpp:70-689,
+// common_inplace.hpp:69-273, libtensor/include/kernels/where.hpp:72-262).
+//
+// Layout choices for MI355X:
+//   * every thread moves 16 bytes of the widest operand per access
+//     (global_load_dwordx4 / global_store_dwordx4, non-temporal), 256 threads per
+//     block and exactly one access per operand per thread: many short-lived
+//     waves keep the HBM queues full and the hardware dispatcher walks the
+//     arrays front to back, which measured faster than grid-stride loops;
+//   * shape and strides of the collapsed iteration space travel in the kernel
+//     argument segment (no device-side metadata buffers to allocate or free);
+//   * strided kernels keep threads adjacent along the innermost output
+//     dimension and pay one div/mod chain per thread, not per element.
+#pragma once
+#include <tuple>
+#include <utility>
+#include "types.hpp"
+
+namespace dpx {
+
+constexpr int EW_BLOCK = 256;
+
+// operand access mode along the inner dimension (2 bits per operand)
+enum : uint32_t { MODE_STRIDED = 0, MODE_VEC = 1, MODE_BCAST = 2 };
+
+template <int NOPS> struct NdIndex {
+    int32_t nd; // >= 1; the last dim is the inner one
+    int32_t pad;
+    int64_t shape[DPX_MAX_ND];
+    int64_t strides[NOPS][DPX_MAX_ND];
+};
+
+template <int N> struct InPtrs {
+    const void *p[N];
+};
+
+template <class Out, class... Ins> struct ew_traits {
+    static constexpr int width = max_sizeof<Out, Ins...>();
+    static constexpr int E = 16 / width; // elements per thread
+};
+
+template <class T, int E> DPX_D pack<T, E> splat(T v)
+{
+    pack<T, E> p;
+#pragma unroll
+    for (int e = 0; e < E; ++e) p.v[e] = v;
+    return p;
+}
+
+// ---- contiguous ---------------------------------------------------------------
+// grid.x * 256 * E >= n.  bcast bit i set: input i is a single element.
+template <bool VEC, class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
+                          const InPtrs<sizeof...(Ins)> &in, std::index_sequence<I...>)
+{
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    const int64_t block_base = (int64_t)blockIdx.x * (EW_BLOCK * E);
+    if constexpr (VEC) {
+        const int64_t base = block_base + (int64_t)threadIdx.x * E;
+        if (base + E <= n) {
+            std::tuple<pack<Ins, E>...> v;
+            ((std::get<I>(v) = ((bcast >> I) & 1u)
+                                   ? splat<Ins, E>(load_one((const Ins *)in.p[I]))
+                                   : load_pack<Ins, E>((const Ins *)in.p[I] + base)),
+             ...);
+            pack<Out, E> r;
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+            store_pack<Out, E>(out + base, r);
+        }
+        else {
+            for (int64_t i = base; i < n; ++i)
+                out[i] = to_storage<Out>(fn(to_value(
+                    load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
+        }
+    }
+    else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int64_t i = block_base + e * EW_BLOCK + threadIdx.x;
+            if (i < n)
+                out[i] = to_storage<Out>(fn(to_value(
+                    load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
+        }
+    }
+}
+
+template <bool VEC, class Fn, class Out, class... Ins>
+__global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, uint32_t bcast,
+                                                            Out *out,
+                                                            InPtrs<sizeof...(Ins)> in)
+{
+    ew_contig_body<VEC, Fn, Out, Ins...>(fn, n, bcast, out, in,
+                                         std::index_sequence_for<Ins...>{});
+}
+
+// ---- strided, vectorised along the inner dimension -----------------------------
+// Block = TY rows x TX threads (TX = 1 << tx_log2, TX * TY = 256); a thread owns E
+// consecutive inner positions of one row.  ix.strides[k] for inputs k < N,
+// ix.strides[N] for the output.  modes: 2 bits per operand, output at bit 2*N.
+template <class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out *out,
+                        const InPtrs<sizeof...(Ins)> &in, uint32_t modes, int tx_log2,
+                        int64_t nrows, int64_t col_blocks, std::index_sequence<I...>)
+{
+    constexpr int N = sizeof...(Ins);
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    const int tx = threadIdx.x & ((1 << tx_log2) - 1);
+    const int ty = threadIdx.x >> tx_log2;
+    const int64_t rb = (int64_t)blockIdx.x / col_blocks;
+    const int64_t cb = (int64_t)blockIdx.x - rb * col_blocks;
+    const int64_t row = rb * (EW_BLOCK >> tx_log2) + ty;
+    const int inner = ix.nd - 1;
+    const int64_t ncols = ix.shape[inner];
+    const int64_t col0 = ((cb << tx_log2) + tx) * E;
+    if (row >= nrows || col0 >= ncols) return;
+
+    int64_t off[N + 1];
+#pragma unroll
+    for (int k = 0; k <= N; ++k) off[k] = col0 * ix.strides[k][inner];
+    {
+        int64_t r = row;
+        for (int d = inner - 1; d >= 0; --d) {
+            const int64_t q = (d == 0) ? 0 : r / ix.shape[d];
+            const int64_t i = r - q * ix.shape[d];
+#pragma unroll
+            for (int k = 0; k <= N; ++k) off[k] += i * ix.strides[k][d];
+            r = q;
+        }
+    }
+    const int cnt = (ncols - col0 < E) ? (int)(ncols - col0) : E;
+    std::tuple<pack<Ins, E>...> v;
+    auto load_operand = [&](auto *p, int64_t o, int64_t st, uint32_t mode) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        pack<T, E> r;
+        if (mode == MODE_VEC && cnt == E) {
+            r = load_pack<T, E>(p + o);
+        }
+        else if (mode == MODE_BCAST) {
+            r = splat<T, E>(load_one(p + o));
+        }
+        else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) r.v[e] = load_one(p + o + ((e < cnt) ? e : 0) * st);
+        }
+        return r;
+    };
+    ((std::get<I>(v) = load_operand((const Ins *)in.p[I], off[I], ix.strides[I][inner],
+                                    (modes >> (2 * I)) & 3u)),
+     ...);
+    pack<Out, E> r;
+#pragma unroll
+    for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+    if (((modes >> (2 * N)) & 3u) == MODE_VEC && cnt == E) {
+        store_pack<Out, E>(out + off[N], r);
+    }
+    else {
+        const int64_t st = ix.strides[N][inner];
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (e < cnt) out[off[N] + e * st] = r.v[e];
+    }
+}
+
+template <class Fn, class Out, class... Ins>
+__global__ __launch_bounds__(EW_BLOCK) void ew_rows_kernel(Fn fn,
+                                                          NdIndex<sizeof...(Ins) + 1> ix,
+                                                          Out *out, InPtrs<sizeof...(Ins)> in,
+                                                          uint32_t modes, int tx_log2,
+                                                          int64_t nrows, int64_t col_blocks)
+{
+    ew_rows_body<Fn, Out, Ins...>(fn, ix, out, in, modes, tx_log2, nrows, col_blocks,
+                                  std::index_sequence_for<Ins...>{});
+}
+
+// ---- host-side plan (element-type independent) ----------------------------------
+struct EwPlan {
+    int path; // dpx_path
+    int nops; // inputs + 1
+    int nd;
+    int64_t shape[DPX_MAX_ND];
+    int64_t strides[5][DPX_MAX_ND]; // inputs..., output (index nops-1)
+    int64_t offsets[5];             // element displacement per operand
+    int64_t n;                      // total elements
+    // launch parameters, filled by ew_finish_plan for a given E / item sizes
+    bool vec;
+    uint32_t bcast;
+    uint32_t modes;
+    int tx_log2;
+    int64_t nrows, col_blocks, grid;
+};
+
+// fills path/nd/shape/strides/offsets from (already validated) views
+void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views);
+// fills the launch parameters for E elements per thread and the operands' item sizes
+// and (displaced) base pointers
+void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs);
+
+// dry != 0: only fill the launch parameters of pl
+template <class Fn, class Out, class... Ins>
+inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *const *views,
+                            hipStream_t stream, bool dry = false)
+{
+    constexpr int N = sizeof...(Ins);
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    const int sizes[N + 1] = {(int)sizeof(Ins)..., (int)sizeof(Out)};
+    const void *ptrs[N + 1];
+    for (int k = 0; k <= N; ++k)
+        ptrs[k] = (const char *)views[k]->data + pl.offsets[k] * sizes[k];
+    ew_finish_plan(pl, E, sizes, ptrs);
+    if (pl.path == DPX_PATH_NOOP || dry) return hipSuccess;
+    InPtrs<N> in;
+    for (int k = 0; k < N; ++k) in.p[k] = ptrs[k];
+    Out *out = (Out *)ptrs[N];
+    if (pl.path == DPX_PATH_EW_CONTIG) {
+        if (pl.vec)
+            hipLaunchKernelGGL((ew_contig_kernel<true, Fn, Out, Ins...>), dim3((unsigned)pl.grid),
+                               dim3(EW_BLOCK), 0, stream, fn, pl.n, pl.bcast, out, in);
+        else
+            hipLaunchKernelGGL((ew_contig_kernel<false, Fn, Out, Ins...>),
+                               dim3((unsigned)pl.grid), dim3(EW_BLOCK), 0, stream, fn, pl.n,
+                               pl.bcast, out, in);
+    }
+    else {
+        NdIndex<N + 1> ix;
+        ix.nd = pl.nd;
+        ix.pad = 0;
+        for (int d = 0; d < DPX_MAX_ND; ++d) {
+            ix.shape[d] = d < pl.nd ? pl.shape[d] : 1;
+            for (int k = 0; k <= N; ++k) ix.strides[k][d] = d < pl.nd ? pl.strides[k][d] : 0;
+        }
+        hipLaunchKernelGGL((ew_rows_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid),
+                           dim3(EW_BLOCK), 0, stream, fn, ix, out, in, pl.modes, pl.tx_log2,
+                           pl.nrows, pl.col_blocks);
+    }
+    return hipGetLastError();
+}
+
+} // namespace dpx

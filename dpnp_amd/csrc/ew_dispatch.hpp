@@ -1,0 +1,35 @@
+// Glue between the C entry points and the templated elementwise launcher.
+#pragma once
+#include "ew.hpp"
+#include "host.hpp"
+#include "ops.hpp"
+
+namespace dpx {
+
+int ew_validate(int nops, const dpx_array_view *const *views, int64_t &n);
+void ew_export_plan(const EwPlan &pl, dpx_plan *out);
+
+// views = inputs..., dst (already validated).  plan_out != nullptr: report only.
+template <class Fn, class Out, class... Ins>
+inline int run_ew(const Fn &fn, const dpx_array_view *const *views, hipStream_t stream,
+                  dpx_plan *plan_out)
+{
+    EwPlan pl;
+    ew_make_plan(pl, (int)sizeof...(Ins) + 1, views);
+    hipError_t e = ew_launch<Fn, Out, Ins...>(fn, pl, views, stream, plan_out != nullptr);
+    if (plan_out) {
+        ew_export_plan(pl, plan_out);
+        plan_out->vec = pl.vec || (pl.path == DPX_PATH_EW_ROWS) ? ew_traits<Out, Ins...>::E : 1;
+        return DPX_OK;
+    }
+    return e == hipSuccess ? DPX_OK : fail_hip(e, "elementwise kernel launch");
+}
+
+template <class Op, class T> struct UnaryFn {
+    DPX_D auto operator()(V<T> x) const { return Op::template apply<T>(x); }
+};
+template <class Op, class T> struct BinaryFn {
+    DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
+};
+
+} // namespace dpx

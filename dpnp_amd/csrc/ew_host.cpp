@@ -1,0 +1,120 @@
+// Elementwise calls: validation and the choice of kernel, independent of element types.
+#include "ew.hpp"
+#include "host.hpp"
+
+namespace dpx {
+
+// Checks shared by unary / binary / where / copy calls, in the order of
+// py_binary_ufunc (libtensor/source/elementwise_functions/elementwise_functions.hpp:338-381).
+// views = inputs..., dst.  Returns DPX_OK with n == 0 for empty iteration spaces.
+int ew_validate(int nops, const dpx_array_view *const *views, int64_t &n)
+{
+    for (int k = 0; k < nops; ++k)
+        if (!view_ok(views[k])) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    const dpx_array_view *dst = views[nops - 1];
+    if (!(dst->flags & DPX_WRITABLE)) return fail(DPX_ERR_NOT_WRITABLE, "output array is read-only.");
+    for (int k = 0; k + 1 < nops; ++k)
+        if (views[k]->nd != dst->nd)
+            return fail(DPX_ERR_RANK_MISMATCH, "Array dimensions are not the same.");
+    for (int k = 0; k + 1 < nops; ++k)
+        if (!same_shape(views[k], dst)) return fail(DPX_ERR_SHAPE_MISMATCH, "Array shapes are not the same.");
+    n = view_size(dst);
+    if (n == 0) return DPX_OK;
+    for (int k = 0; k < nops; ++k)
+        if (views[k]->data == nullptr) return fail(DPX_ERR_BAD_ARGUMENT, "null data pointer");
+    int64_t lo, hi;
+    view_minmax(dst, lo, hi);
+    if (hi - lo + 1 < n)
+        return fail(DPX_ERR_NOT_AMPLE, "Memory addressed by the output array is not sufficiently ample.");
+    for (int k = 0; k + 1 < nops; ++k)
+        if (views_overlap(views[k], dst) && !views_same_logical(views[k], dst))
+            return fail(DPX_ERR_OVERLAP, "Arrays index overlapping segments of memory");
+    return DPX_OK;
+}
+
+void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
+{
+    const dpx_array_view *dst = views[nops - 1];
+    pl.nops = nops;
+    pl.n = view_size(dst);
+    pl.vec = false;
+    pl.bcast = pl.modes = 0;
+    pl.tx_log2 = 0;
+    pl.nrows = pl.col_blocks = pl.grid = 0;
+    for (int k = 0; k < 5; ++k) pl.offsets[k] = 0;
+    if (pl.n == 0) {
+        pl.path = DPX_PATH_NOOP;
+        pl.nd = 0;
+        return;
+    }
+    for (int d = 0; d < dst->nd; ++d) {
+        pl.shape[d] = dst->shape[d];
+        for (int k = 0; k < nops; ++k) pl.strides[k][d] = views[k]->strides[d];
+    }
+    pl.nd = collapse(dst->nd, nops, pl.shape, pl.strides, pl.offsets, false);
+    if (pl.nd == 0) { // a single element
+        pl.nd = 1;
+        pl.shape[0] = 1;
+        for (int k = 0; k < nops; ++k) pl.strides[k][0] = 1;
+    }
+    bool contig = pl.nd == 1 && pl.strides[nops - 1][0] == 1;
+    for (int k = 0; k + 1 < nops && contig; ++k)
+        contig = pl.strides[k][0] == 1 || pl.strides[k][0] == 0;
+    pl.path = contig ? DPX_PATH_EW_CONTIG : DPX_PATH_EW_ROWS;
+}
+
+void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs)
+{
+    if (pl.path == DPX_PATH_NOOP) return;
+    const int nops = pl.nops;
+    auto aligned = [&](int k) { return ((uintptr_t)ptrs[k] % (uintptr_t)(E * itemsize[k])) == 0; };
+    if (pl.path == DPX_PATH_EW_CONTIG) {
+        pl.vec = true;
+        pl.bcast = 0;
+        for (int k = 0; k < nops; ++k) {
+            if (k + 1 < nops && pl.strides[k][0] == 0 && pl.n > 1) pl.bcast |= 1u << k;
+            else pl.vec = pl.vec && aligned(k);
+        }
+        pl.grid = (pl.n + (int64_t)EW_BLOCK * E - 1) / ((int64_t)EW_BLOCK * E);
+        return;
+    }
+    const int inner = pl.nd - 1;
+    const int64_t ncols = pl.shape[inner];
+    pl.nrows = pl.n / ncols;
+    pl.modes = 0;
+    for (int k = 0; k < nops; ++k) {
+        uint32_t mode = MODE_STRIDED;
+        const int64_t s = pl.strides[k][inner];
+        if (s == 0 && k + 1 < nops) mode = MODE_BCAST;
+        else if (s == 1 && aligned(k)) {
+            mode = MODE_VEC;
+            for (int d = 0; d < inner; ++d)
+                if (pl.strides[k][d] % E != 0) mode = MODE_STRIDED;
+        }
+        pl.modes |= mode << (2 * k);
+    }
+    const int64_t per_row = (ncols + E - 1) / E; // threads wanted along a row
+    int lg = 0;
+    while (lg < 8 && ((int64_t)1 << lg) < per_row) ++lg;
+    pl.tx_log2 = lg;
+    const int64_t tx = (int64_t)1 << lg, ty = EW_BLOCK / tx;
+    pl.col_blocks = (per_row + tx - 1) / tx;
+    pl.grid = pl.col_blocks * ((pl.nrows + ty - 1) / ty);
+}
+
+void ew_export_plan(const EwPlan &pl, dpx_plan *out)
+{
+    *out = dpx_plan{};
+    out->path = pl.path;
+    out->nd = pl.nd;
+    for (int d = 0; d < pl.nd && pl.path != DPX_PATH_NOOP; ++d) {
+        out->shape[d] = pl.shape[d];
+        for (int k = 0; k < pl.nops && k < 4; ++k) out->strides[k][d] = pl.strides[k][d];
+    }
+    for (int k = 0; k < pl.nops && k < 4; ++k) out->offsets[k] = pl.offsets[k];
+    out->grid[0] = pl.grid;
+    out->grid[1] = out->grid[2] = 1;
+    out->block = EW_BLOCK;
+}
+
+} // namespace dpx

@@ -1,0 +1,249 @@
+// where, divide_by_scalar, fill and the fused chains.
+#include "ew_dispatch.hpp"
+
+namespace dpx {
+
+// ---- where: libtensor/include/kernels/where.hpp:72-262, host libtensor/source/where.cpp:74-247.
+// The select moves bit patterns, so x1/x2/dst are instantiated per element size;
+// the condition is any dtype, true when non-zero (type_utils.hpp:64-93).
+template <class C, class S> struct WhereFn {
+    DPX_D S operator()(V<C> c, S a, S b) const { return convert<bool_t, C>(to_storage<C>(c)).v ? a : b; }
+};
+
+template <class F> static bool for_size_class(int bytes, F &&f)
+{
+    switch (bytes) {
+    case 1: f(tag<uint8_t>{}); return true;
+    case 2: f(tag<uint16_t>{}); return true;
+    case 4: f(tag<uint32_t>{}); return true;
+    case 8: f(tag<uint64_t>{}); return true;
+    case 16: f(tag<c128>{}); return true;
+    default: return false;
+    }
+}
+
+static int where_call(const dpx_array_view *cond, const dpx_array_view *x1, const dpx_array_view *x2,
+                      const dpx_array_view *dst, void *stream, dpx_plan *plan_out)
+{
+    if (!view_ok(cond) || !view_ok(x1) || !view_ok(x2) || !view_ok(dst))
+        return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (x1->dtype != x2->dtype || x1->dtype != dst->dtype)
+        return fail(DPX_ERR_BAD_DTYPE, "Value arrays must have the same data type");
+    const dpx_array_view *views[4] = {cond, x1, x2, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(4, views, n)) return rc;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    for_dtype(cond->dtype, [&](auto ct) {
+        using C = typename decltype(ct)::type;
+        for_size_class(itemsize_of(dst->dtype), [&](auto st) {
+            using S = typename decltype(st)::type;
+            rc = run_ew<WhereFn<C, S>, S, C, S, S>({}, views, (hipStream_t)stream, plan_out);
+        });
+    });
+    return rc;
+}
+
+// ---- fused compare + select: dst = (lhs CMP rhs) ? x1 : x2 --------------------------------
+template <class Cmp, class T, class S> struct WhereCmpFn {
+    DPX_D S operator()(V<T> l, V<T> r, S a, S b) const { return Cmp::template apply<T>(l, r) ? a : b; }
+};
+
+static int where_compare_call(int cmp_op, const dpx_array_view *lhs, const dpx_array_view *rhs,
+                              const dpx_array_view *x1, const dpx_array_view *x2,
+                              const dpx_array_view *dst, void *stream)
+{
+    if (!view_ok(lhs) || !view_ok(rhs) || !view_ok(x1) || !view_ok(x2) || !view_ok(dst))
+        return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (cmp_op < DPX_B_EQUAL || cmp_op > DPX_B_GREATER_EQUAL)
+        return fail(DPX_ERR_BAD_ARGUMENT, "cmp_op is not a comparison");
+    if (lhs->dtype != rhs->dtype) return fail(DPX_ERR_BAD_DTYPE, "compared arrays must have the same data type");
+    if (x1->dtype != x2->dtype || x1->dtype != dst->dtype)
+        return fail(DPX_ERR_BAD_DTYPE, "Value arrays must have the same data type");
+    // only the 4- and 8-byte real types: the fused form exists for the hot cases
+    const int dt = lhs->dtype;
+    if (!(dt == DPX_FLOAT || dt == DPX_DOUBLE || dt == DPX_INT32 || dt == DPX_INT64))
+        return fail(DPX_ERR_NOT_IMPLEMENTED, "fused where-compare: unsupported comparison dtype");
+    const int vs = itemsize_of(dst->dtype);
+    if (vs != 4 && vs != 8) return fail(DPX_ERR_NOT_IMPLEMENTED, "fused where-compare: unsupported value dtype");
+    const dpx_array_view *views[5] = {lhs, rhs, x1, x2, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(5, views, n)) return rc;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    auto with_cmp = [&](auto cmptag) {
+        using Cmp = typename decltype(cmptag)::type;
+        auto with_t = [&](auto ttag) {
+            using T = typename decltype(ttag)::type;
+            if (vs == 4) rc = run_ew<WhereCmpFn<Cmp, T, uint32_t>, uint32_t, T, T, uint32_t, uint32_t>({}, views, (hipStream_t)stream, nullptr);
+            else rc = run_ew<WhereCmpFn<Cmp, T, uint64_t>, uint64_t, T, T, uint64_t, uint64_t>({}, views, (hipStream_t)stream, nullptr);
+        };
+        if (dt == DPX_FLOAT) with_t(tag<float>{});
+        else if (dt == DPX_DOUBLE) with_t(tag<double>{});
+        else if (dt == DPX_INT32) with_t(tag<int32_t>{});
+        else with_t(tag<int64_t>{});
+    };
+    switch (cmp_op) {
+    case DPX_B_EQUAL: with_cmp(tag<CmpOp<0>>{}); break;
+    case DPX_B_NOT_EQUAL: with_cmp(tag<CmpOp<1>>{}); break;
+    case DPX_B_LESS: with_cmp(tag<CmpOp<2>>{}); break;
+    case DPX_B_LESS_EQUAL: with_cmp(tag<CmpOp<3>>{}); break;
+    case DPX_B_GREATER: with_cmp(tag<CmpOp<4>>{}); break;
+    default: with_cmp(tag<CmpOp<5>>{}); break;
+    }
+    return rc;
+}
+
+// ---- divide by scalar: libtensor/source/elementwise_functions/true_divide.cpp:204-430 -------------
+template <class T> struct DivScalarFn {
+    real_of_t<T> s;
+    DPX_D T operator()(T x) const
+    {
+        if constexpr (is_cplx_v<T>) return T{x.re / s, x.im / s};
+        else return x / s;
+    }
+};
+
+static int divide_by_scalar_call(const dpx_array_view *src, double scalar, const dpx_array_view *dst,
+                                 void *stream)
+{
+    if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (src->dtype != dst->dtype)
+        return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    const dpx_array_view *views[2] = {src, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(2, views, n)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (src->dtype) {
+    case DPX_HALF: return run_ew<DivScalarFn<half_t>, half_t, half_t>({(half_t)scalar}, views, s, nullptr);
+    case DPX_FLOAT: return run_ew<DivScalarFn<float>, float, float>({(float)scalar}, views, s, nullptr);
+    case DPX_DOUBLE: return run_ew<DivScalarFn<double>, double, double>({scalar}, views, s, nullptr);
+    case DPX_CFLOAT: return run_ew<DivScalarFn<c64>, c64, c64>({(float)scalar}, views, s, nullptr);
+    case DPX_CDOUBLE: return run_ew<DivScalarFn<c128>, c128, c128>({scalar}, views, s, nullptr);
+    default: return fail(DPX_ERR_NOT_IMPLEMENTED, "divide_by_scalar: only floating and complex types");
+    }
+}
+
+// ---- fill ----------------------------------------------------------------------------------------------
+template <class T> struct FillFn {
+    T v;
+    DPX_D V<T> operator()() const { return to_value(v); }
+};
+
+static int fill_call(const dpx_array_view *dst, double re, double im, int64_t iv, int use_int, void *stream)
+{
+    if (!view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    const dpx_array_view *views[1] = {dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(1, views, n)) return rc;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    for_dtype(dst->dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        T v;
+        if constexpr (is_cplx_v<T>) v = T{(real_of_t<T>)(use_int ? (double)iv : re), (real_of_t<T>)(use_int ? 0.0 : im)};
+        else if constexpr (is_bool_v<T>) v = bool_t{(uint8_t)(use_int ? iv != 0 : (re != 0.0 || im != 0.0))};
+        else if constexpr (is_int_v<T>) v = use_int ? (T)iv : convert<T, double>(re);
+        else v = use_int ? (T)iv : (T)re;
+        rc = run_ew<FillFn<T>, T>(FillFn<T>{v}, views, (hipStream_t)stream, nullptr);
+    });
+    return rc;
+}
+
+// ---- Black-Scholes, formula of examples/example_bs.py:50-78 --------------------------------------------
+// One thread prices E options: 3 loads, 2 stores of 16 bytes.  Every product and sum is a
+// separate rounding (the library is built with -ffp-contract=off), matching the
+// reference's chain of one kernel per operation.
+template <class T> struct BlackScholesFn {
+    T mr, sig_sig_two, quarter, half_, one;
+    // returns call; put through the second output of the kernel below
+    DPX_D void price(T p, T s, T t, T &call, T &put) const
+    {
+        const T a = m_log(p / s);
+        const T b = t * mr;
+        const T z = t * sig_sig_two;
+        const T c = quarter * z;
+        const T y = one / m_sqrt(z);
+        const T w1 = (a - b + c) * y;
+        const T w2 = (a - b - c) * y;
+        const T d1 = half_ + half_ * m_erf(w1);
+        const T d2 = half_ + half_ * m_erf(w2);
+        const T se = m_exp(b) * s;
+        call = p * d1 - se * d2;
+        put = call - p + se;
+    }
+};
+
+template <class T>
+__global__ __launch_bounds__(256) void black_scholes_kernel(BlackScholesFn<T> fn, const T *price, const T *strike,
+                                                            const T *t, T *call, T *put, int64_t n)
+{
+    constexpr int E = 16 / sizeof(T);
+    const int64_t base = ((int64_t)blockIdx.x * 256 + threadIdx.x) * E;
+    if (base + E <= n) {
+        pack<T, E> p = load_pack<T, E>(price + base), s = load_pack<T, E>(strike + base),
+                   tt = load_pack<T, E>(t + base), c, q;
+#pragma unroll
+        for (int e = 0; e < E; ++e) fn.price(p.v[e], s.v[e], tt.v[e], c.v[e], q.v[e]);
+        store_pack<T, E>(call + base, c);
+        store_pack<T, E>(put + base, q);
+    }
+    else {
+        for (int64_t i = base; i < n; ++i) fn.price(price[i], strike[i], t[i], call[i], put[i]);
+    }
+}
+
+template <class T>
+static int black_scholes_call(const void *price, const void *strike, const void *t, double rate, double vol,
+                              void *call, void *put, int64_t n, hipStream_t stream)
+{
+    constexpr int E = 16 / sizeof(T);
+    const uintptr_t all = (uintptr_t)price | (uintptr_t)strike | (uintptr_t)t | (uintptr_t)call | (uintptr_t)put;
+    if (all % 16 != 0) return fail(DPX_ERR_BAD_ARGUMENT, "black_scholes: arrays must be 16-byte aligned");
+    BlackScholesFn<T> fn{(T)(-rate), (T)(vol * vol * 2), (T)0.25, (T)0.5, (T)1};
+    const int64_t grid = (n + 256 * E - 1) / (256 * E);
+    hipLaunchKernelGGL(black_scholes_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, fn, (const T *)price,
+                       (const T *)strike, (const T *)t, (T *)call, (T *)put, n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? DPX_OK : fail_hip(e, "black_scholes launch");
+}
+
+} // namespace dpx
+
+using namespace dpx;
+extern "C" {
+int dpx_where(const dpx_array_view *cond, const dpx_array_view *x1, const dpx_array_view *x2,
+              const dpx_array_view *dst, void *stream)
+{
+    return where_call(cond, x1, x2, dst, stream, nullptr);
+}
+int dpx_where_plan(const dpx_array_view *cond, const dpx_array_view *x1, const dpx_array_view *x2,
+                   const dpx_array_view *dst, dpx_plan *plan)
+{
+    if (!plan) return fail(DPX_ERR_BAD_ARGUMENT, "plan is null");
+    return where_call(cond, x1, x2, dst, nullptr, plan);
+}
+int dpx_where_compare(int cmp_op, const dpx_array_view *lhs, const dpx_array_view *rhs, const dpx_array_view *x1,
+                      const dpx_array_view *x2, const dpx_array_view *dst, void *stream)
+{
+    return where_compare_call(cmp_op, lhs, rhs, x1, x2, dst, stream);
+}
+int dpx_divide_by_scalar(const dpx_array_view *src, double scalar, const dpx_array_view *dst, void *stream)
+{
+    return divide_by_scalar_call(src, scalar, dst, stream);
+}
+int dpx_fill(const dpx_array_view *dst, double value_re, double value_im, int64_t value_int, int use_int,
+             void *stream)
+{
+    return fill_call(dst, value_re, value_im, value_int, use_int, stream);
+}
+int dpx_black_scholes(const void *price, const void *strike, const void *t, double rate, double vol, void *call,
+                      void *put, int64_t n, int dtype, void *stream)
+{
+    if (n < 0) return fail(DPX_ERR_BAD_ARGUMENT, "black_scholes: negative length");
+    if (n == 0) return DPX_OK;
+    if (!price || !strike || !t || !call || !put) return fail(DPX_ERR_BAD_ARGUMENT, "black_scholes: null pointer");
+    if (dtype == DPX_DOUBLE)
+        return black_scholes_call<double>(price, strike, t, rate, vol, call, put, n, (hipStream_t)stream);
+    if (dtype == DPX_FLOAT)
+        return black_scholes_call<float>(price, strike, t, rate, vol, call, put, n, (hipStream_t)stream);
+    return fail(DPX_ERR_NOT_IMPLEMENTED, "black_scholes: float32 or float64 only");
+}
+}

@@ -1,0 +1,539 @@
+// Per-op device functors and their dtype maps.
+//
+// Each op struct gives, for an input element type T (binary ops: both inputs
+// of type T): `ok<T>` whether a kernel exists, `out<T>` the result element
+// type, and `apply` on values.  The maps restate the *OutputType structs of
+// libtensor/include/kernels/elementwise_functions/<op>.hpp; everything not
+// listed there is reached through casts chosen by the Python layer.
+#pragma once
+#include "types.hpp"
+
+namespace dpx {
+
+// ---- complex arithmetic -------------------------------------------------------
+template <class R> DPX_HD cplx<R> operator+(cplx<R> a, cplx<R> b) { return {a.re + b.re, a.im + b.im}; }
+template <class R> DPX_HD cplx<R> operator-(cplx<R> a, cplx<R> b) { return {a.re - b.re, a.im - b.im}; }
+template <class R> DPX_HD cplx<R> operator-(cplx<R> a) { return {-a.re, -a.im}; }
+template <class R> DPX_HD cplx<R> operator*(cplx<R> a, cplx<R> b)
+{
+    return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+template <class R> DPX_HD cplx<R> operator/(cplx<R> a, cplx<R> b)
+{
+    // Smith's algorithm (what NumPy uses): no spurious overflow in |b|^2
+    R abr = b.re < 0 ? -b.re : b.re, abi = b.im < 0 ? -b.im : b.im;
+    if (abr >= abi) {
+        if (abr == 0 && abi == 0) return {a.re / abr, a.im / abr};
+        R rat = b.im / b.re, scl = R(1) / (b.re + b.im * rat);
+        return {(a.re + a.im * rat) * scl, (a.im - a.re * rat) * scl};
+    }
+    R rat = b.re / b.im, scl = R(1) / (b.re * rat + b.im);
+    return {(a.re * rat + a.im) * scl, (a.im * rat - a.re) * scl};
+}
+template <class R> DPX_HD bool operator==(cplx<R> a, cplx<R> b) { return a.re == b.re && a.im == b.im; }
+template <class R> DPX_HD bool operator!=(cplx<R> a, cplx<R> b) { return !(a == b); }
+
+template <class T> DPX_HD bool isnan_(T x)
+{
+    if constexpr (is_cplx_v<T>) return (x.re != x.re) || (x.im != x.im);
+    else if constexpr (is_fp_v<T>) return x != x;
+    else return false;
+}
+
+// ordering of complex numbers: libtensor/include/utils/math_utils.hpp:43-95
+template <class R> DPX_HD bool c_less(cplx<R> a, cplx<R> b)
+{
+    return (a.re == b.re) ? (a.im < b.im) : (a.re < b.re && !isnan_(a.im) && !isnan_(b.im));
+}
+template <class R> DPX_HD bool c_greater(cplx<R> a, cplx<R> b)
+{
+    return (a.re == b.re) ? (a.im > b.im) : (a.re > b.re && !isnan_(a.im) && !isnan_(b.im));
+}
+template <class R> DPX_HD bool c_less_eq(cplx<R> a, cplx<R> b)
+{
+    return (a.re == b.re) ? (a.im <= b.im) : (a.re < b.re && !isnan_(a.im) && !isnan_(b.im));
+}
+template <class R> DPX_HD bool c_greater_eq(cplx<R> a, cplx<R> b)
+{
+    return (a.re == b.re) ? (a.im >= b.im) : (a.re > b.re && !isnan_(a.im) && !isnan_(b.im));
+}
+
+// NaN-propagating extrema: Maximum / Minimum, libtensor/include/utils/sycl_utils.hpp:332-376
+// and max_complex / min_complex, math_utils.hpp:97-127
+template <class T> DPX_HD T max_nan(T x, T y)
+{
+    if constexpr (is_cplx_v<T>) return (isnan_(x.re) || isnan_(x.im) || c_greater(x, y)) ? x : y;
+    else if constexpr (is_fp_v<T>) return (x != x || x > y) ? x : y;
+    else if constexpr (std::is_same_v<T, bool>) return x || y;
+    else return (x > y) ? x : y;
+}
+template <class T> DPX_HD T min_nan(T x, T y)
+{
+    if constexpr (is_cplx_v<T>) return (isnan_(x.re) || isnan_(x.im) || c_less(x, y)) ? x : y;
+    else if constexpr (is_fp_v<T>) return (x != x || x < y) ? x : y;
+    else if constexpr (std::is_same_v<T, bool>) return x && y;
+    else return (x < y) ? x : y;
+}
+
+// ---- math on real fp types (half computes in float) -----------------------------
+#define DPX_FP_FN1(NAME, F32, F64)                                      \
+    template <class T> DPX_D T NAME(T x)                                \
+    {                                                                   \
+        if constexpr (std::is_same_v<T, double>) return F64(x);         \
+        else if constexpr (std::is_same_v<T, float>) return F32(x);     \
+        else return (T)F32((float)x);                                   \
+    }
+DPX_FP_FN1(m_sqrt, ::sqrtf, ::sqrt)
+DPX_FP_FN1(m_exp, ::expf, ::exp)
+DPX_FP_FN1(m_log, ::logf, ::log)
+DPX_FP_FN1(m_erf, ::erff, ::erf)
+DPX_FP_FN1(m_sin, ::sinf, ::sin)
+DPX_FP_FN1(m_cos, ::cosf, ::cos)
+DPX_FP_FN1(m_tan, ::tanf, ::tan)
+DPX_FP_FN1(m_tanh, ::tanhf, ::tanh)
+DPX_FP_FN1(m_exp2, ::exp2f, ::exp2)
+DPX_FP_FN1(m_expm1, ::expm1f, ::expm1)
+DPX_FP_FN1(m_log2, ::log2f, ::log2)
+DPX_FP_FN1(m_log10, ::log10f, ::log10)
+DPX_FP_FN1(m_log1p, ::log1pf, ::log1p)
+DPX_FP_FN1(m_cbrt, ::cbrtf, ::cbrt)
+DPX_FP_FN1(m_floor, ::floorf, ::floor)
+DPX_FP_FN1(m_ceil, ::ceilf, ::ceil)
+DPX_FP_FN1(m_trunc, ::truncf, ::trunc)
+#undef DPX_FP_FN1
+#define DPX_FP_FN2(NAME, F32, F64)                                          \
+    template <class T> DPX_D T NAME(T x, T y)                               \
+    {                                                                       \
+        if constexpr (std::is_same_v<T, double>) return F64(x, y);          \
+        else if constexpr (std::is_same_v<T, float>) return F32(x, y);      \
+        else return (T)F32((float)x, (float)y);                             \
+    }
+DPX_FP_FN2(m_pow, ::powf, ::pow)
+DPX_FP_FN2(m_atan2, ::atan2f, ::atan2)
+DPX_FP_FN2(m_hypot, ::hypotf, ::hypot)
+DPX_FP_FN2(m_copysign, ::copysignf, ::copysign)
+DPX_FP_FN2(m_fmod, ::fmodf, ::fmod)
+#undef DPX_FP_FN2
+
+template <class T> DPX_D bool m_signbit(T x)
+{
+    if constexpr (std::is_same_v<T, double>) return (__double_as_longlong(x) >> 63) != 0;
+    else if constexpr (std::is_same_v<T, float>) return (__float_as_int(x) >> 31) != 0;
+    else return (__float_as_int((float)x) >> 31) != 0;
+}
+template <class T> DPX_D bool m_isinf(T x)
+{
+    if constexpr (is_fp_v<T>) { T a = x < T(0) ? -x : x; return a == (T)__builtin_inff(); }
+    else return false;
+}
+
+template <class T> using V = value_of_t<T>;
+
+// =========================== binary ops =============================================
+// ok<T>: same-dtype pair (T, T) has a kernel.
+
+struct AddOp { // add.hpp:63-114,140-204; bool + bool is logical or
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b)
+    {
+        if constexpr (is_bool_v<T>) return a || b;
+        else return a + b;
+    }
+};
+struct SubOp { // subtract.hpp:62: every type but bool
+    template <class T> static constexpr bool ok = !is_bool_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b) { return a - b; }
+};
+struct MulOp { // multiply.hpp:64; bool * bool is logical and
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b)
+    {
+        if constexpr (is_bool_v<T>) return a && b;
+        else return a * b;
+    }
+};
+struct DivOp { // true_divide.hpp:63: floating and complex only
+    template <class T> static constexpr bool ok = is_fp_v<T> || is_cplx_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b) { return a / b; }
+};
+template <int WHICH> struct BitOp { // bitwise_and.hpp:59-118 (or/xor alike); bool: logical
+    template <class T> static constexpr bool ok = is_bool_v<T> || is_int_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b)
+    {
+        if constexpr (is_bool_v<T>) {
+            if constexpr (WHICH == 0) return a && b;
+            else if constexpr (WHICH == 1) return a || b;
+            else return a != b;
+        }
+        else {
+            if constexpr (WHICH == 0) return a & b;
+            else if constexpr (WHICH == 1) return a | b;
+            else return a ^ b;
+        }
+    }
+};
+// comparisons, greater.hpp:62-146 and siblings: all 14 same-dtype pairs -> bool;
+// CMP: 0 ==, 1 !=, 2 <, 3 <=, 4 >, 5 >=
+template <int CMP> struct CmpOp {
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = bool_t;
+    template <class T> DPX_D static bool apply(V<T> a, V<T> b)
+    {
+        if constexpr (CMP == 0) return a == b;
+        else if constexpr (CMP == 1) return a != b;
+        else if constexpr (is_cplx_v<T>) {
+            if constexpr (CMP == 2) return c_less(a, b);
+            else if constexpr (CMP == 3) return c_less_eq(a, b);
+            else if constexpr (CMP == 4) return c_greater(a, b);
+            else return c_greater_eq(a, b);
+        }
+        else {
+            if constexpr (CMP == 2) return a < b;
+            else if constexpr (CMP == 3) return a <= b;
+            else if constexpr (CMP == 4) return a > b;
+            else return a >= b;
+        }
+    }
+    // mixed int64/uint64 pairs compare exactly, without promotion to double
+    DPX_D static bool apply_iu(int64_t a, uint64_t b)
+    {
+        if constexpr (CMP == 0) return a >= 0 && (uint64_t)a == b;
+        else if constexpr (CMP == 1) return a < 0 || (uint64_t)a != b;
+        else if constexpr (CMP == 2) return a < 0 || (uint64_t)a < b;
+        else if constexpr (CMP == 3) return a < 0 || (uint64_t)a <= b;
+        else if constexpr (CMP == 4) return a >= 0 && (uint64_t)a > b;
+        else return a >= 0 && (uint64_t)a >= b;
+    }
+    DPX_D static bool apply_ui(uint64_t a, int64_t b)
+    {
+        if constexpr (CMP == 0) return b >= 0 && a == (uint64_t)b;
+        else if constexpr (CMP == 1) return b < 0 || a != (uint64_t)b;
+        else if constexpr (CMP == 2) return b >= 0 && a < (uint64_t)b;
+        else if constexpr (CMP == 3) return b >= 0 && a <= (uint64_t)b;
+        else if constexpr (CMP == 4) return b < 0 || a > (uint64_t)b;
+        else return b < 0 || a >= (uint64_t)b;
+    }
+};
+struct MaxOp { // maximum.hpp:63-90
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b) { return max_nan(a, b); }
+};
+struct MinOp { // minimum.hpp
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b) { return min_nan(a, b); }
+};
+template <int WHICH> struct LogicalOp { // logical_and.hpp / logical_or.hpp / logical_xor.hpp
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = bool_t;
+    template <class T> DPX_D static bool apply(V<T> a, V<T> b)
+    {
+        bool x = convert<bool_t, T>(to_storage<T>(a)).v, y = convert<bool_t, T>(to_storage<T>(b)).v;
+        if constexpr (WHICH == 0) return x && y;
+        else if constexpr (WHICH == 1) return x || y;
+        else return x != y;
+    }
+};
+struct FloorDivOp { // floor_divide.hpp:63-86: ints (x // 0 == 0) and real fp
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        if constexpr (is_int_v<T>) {
+            if (b == T(0)) return T(0);
+            if constexpr (std::is_signed_v<T>) {
+                if (b == T(-1)) return (T)(0 - (std::make_unsigned_t<T>)a); // INT_MIN // -1 wraps
+                T d = a / b, m = a % b;
+                return (T)(d - ((m != 0) && ((m < 0) != (b < 0))));
+            }
+            else return a / b;
+        }
+        else {
+            T d = a / b;
+            return (d == T(0)) ? d : m_floor(d);
+        }
+    }
+};
+struct RemainderOp { // remainder.hpp: Python-style modulo, x % 0 == 0 for ints
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        if constexpr (is_int_v<T>) {
+            if (b == T(0)) return T(0);
+            if constexpr (std::is_signed_v<T>) {
+                if (b == T(-1)) return T(0);
+                T m = a % b;
+                return (m != 0 && ((m < 0) != (b < 0))) ? (T)(m + b) : m;
+            }
+            else return a % b;
+        }
+        else {
+            T m = m_fmod(a, b);
+            if (m != T(0)) {
+                if ((b < T(0)) != (m < T(0))) m += b;
+            }
+            else m = m_copysign(T(0), b);
+            return m;
+        }
+    }
+};
+struct PowOp { // pow.hpp: ints by repeated squaring (negative exponent -> 0), fp via pow
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        if constexpr (is_int_v<T>) {
+            if constexpr (std::is_signed_v<T>) {
+                if (b < 0) return (a == 1) ? T(1) : ((a == -1) ? ((b & 1) ? T(-1) : T(1)) : T(0));
+            }
+            using U = std::make_unsigned_t<T>;
+            U r = 1, base = (U)a;
+            U e = (U)b;
+            while (e) {
+                if (e & 1) r = (U)(r * base);
+                base = (U)(base * base);
+                e >>= 1;
+            }
+            return (T)r;
+        }
+        else return m_pow(a, b);
+    }
+};
+struct Atan2Op {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b) { return m_atan2(a, b); }
+};
+struct HypotOp {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b) { return m_hypot(a, b); }
+};
+struct CopysignOp {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b) { return m_copysign(a, b); }
+};
+template <bool LEFT> struct ShiftOp { // bitwise_left_shift.hpp / bitwise_right_shift.hpp
+    template <class T> static constexpr bool ok = is_int_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        constexpr int bits = 8 * sizeof(T);
+        bool big;
+        if constexpr (std::is_signed_v<T>) big = (b < 0) || (b >= bits);
+        else big = b >= (T)bits;
+        if constexpr (LEFT) return big ? T(0) : (T)((std::make_unsigned_t<T>)a << b);
+        else {
+            if constexpr (std::is_signed_v<T>) return big ? (a < 0 ? T(-1) : T(0)) : (T)(a >> b);
+            else return big ? T(0) : (T)(a >> b);
+        }
+    }
+};
+
+// =========================== unary ops ==============================================
+
+struct AbsOp { // abs.hpp:61-90: complex -> real
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = real_of_t<T>;
+    template <class T> DPX_D static V<out<T>> apply(V<T> x)
+    {
+        if constexpr (is_bool_v<T> || is_uint_v<T>) return x;
+        else if constexpr (is_cplx_v<T>) return m_hypot(x.re, x.im);
+        else if constexpr (is_fp_v<T>) return m_signbit(x) ? -x : x;
+        else return (T)(x < 0 ? (T)(0 - (std::make_unsigned_t<T>)x) : x);
+    }
+};
+struct NegOp { // negative.hpp: all but bool
+    template <class T> static constexpr bool ok = !is_bool_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if constexpr (is_int_v<T>) return (T)(0 - (std::make_unsigned_t<T>)x);
+        else return -x;
+    }
+};
+struct PosOp {
+    template <class T> static constexpr bool ok = !is_bool_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x) { return x; }
+};
+struct SquareOp { // square.hpp:64-90; bool -> int8
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = std::conditional_t<is_bool_v<T>, int8_t, T>;
+    template <class T> DPX_D static V<out<T>> apply(V<T> x)
+    {
+        if constexpr (is_bool_v<T>) return (int8_t)(x ? 1 : 0);
+        else if constexpr (is_int_v<T>) return (T)((std::make_unsigned_t<T>)x * (std::make_unsigned_t<T>)x);
+        else return x * x;
+    }
+};
+// real floating-point functions; exp.hpp:153-163 and siblings list f2 f4 f8 (+ complex,
+// which this library does not implement for transcendentals)
+#define DPX_FP_UNARY(NAME, EXPR)                                   \
+    struct NAME {                                                  \
+        template <class T> static constexpr bool ok = is_fp_v<T>;  \
+        template <class T> using out = T;                          \
+        template <class T> DPX_D static T apply(T x) { return EXPR; } \
+    };
+DPX_FP_UNARY(SqrtOp, m_sqrt(x))
+DPX_FP_UNARY(ExpOp, m_exp(x))
+DPX_FP_UNARY(LogOp, m_log(x))
+DPX_FP_UNARY(SinOp, m_sin(x))
+DPX_FP_UNARY(CosOp, m_cos(x))
+DPX_FP_UNARY(TanOp, m_tan(x))
+DPX_FP_UNARY(TanhOp, m_tanh(x))
+DPX_FP_UNARY(Exp2Op, m_exp2(x))
+DPX_FP_UNARY(Expm1Op, m_expm1(x))
+DPX_FP_UNARY(Log2Op, m_log2(x))
+DPX_FP_UNARY(Log10Op, m_log10(x))
+DPX_FP_UNARY(Log1pOp, m_log1p(x))
+DPX_FP_UNARY(RsqrtOp, T(1) / m_sqrt(x))
+DPX_FP_UNARY(CbrtOp, m_cbrt(x))
+DPX_FP_UNARY(ReciprocalOp, T(1) / x)
+#undef DPX_FP_UNARY
+struct ErfOp { // dpnp/backend/kernels/elementwise_functions/erf.hpp:52-95; f2 -> f4
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = std::conditional_t<std::is_same_v<T, half_t>, float, T>;
+    template <class T> DPX_D static out<T> apply(T x) { return m_erf((out<T>)x); }
+};
+template <int WHICH> struct RoundOp { // floor.hpp / ceil.hpp / trunc.hpp: identity on ints and bool
+    template <class T> static constexpr bool ok = !is_cplx_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> x)
+    {
+        if constexpr (is_fp_v<T>) {
+            if constexpr (WHICH == 0) return m_floor(x);
+            else if constexpr (WHICH == 1) return m_ceil(x);
+            else return m_trunc(x);
+        }
+        else return x;
+    }
+};
+struct SignOp { // sign.hpp:63-110 (real types; NaN -> NaN)
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if constexpr (is_uint_v<T>) return (T)(x > 0);
+        else if constexpr (is_fp_v<T>) return (x != x) ? x : (T)((T(0) < x) - (x < T(0)));
+        else return (T)((T(0) < x) - (x < T(0)));
+    }
+};
+template <int WHICH> struct FpClassOp { // isnan.hpp / isinf.hpp / isfinite.hpp -> bool
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = bool_t;
+    template <class T> DPX_D static bool apply(V<T> x)
+    {
+        if constexpr (is_cplx_v<T>) {
+            bool n = isnan_(x), i = m_isinf(x.re) || m_isinf(x.im);
+            if constexpr (WHICH == 0) return n;
+            else if constexpr (WHICH == 1) return i;
+            else return !n && !i;
+        }
+        else if constexpr (is_fp_v<T>) {
+            if constexpr (WHICH == 0) return x != x;
+            else if constexpr (WHICH == 1) return m_isinf(x);
+            else return !(x != x) && !m_isinf(x);
+        }
+        else return WHICH == 2;
+    }
+};
+struct LogicalNotOp {
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = bool_t;
+    template <class T> DPX_D static bool apply(V<T> x) { return !convert<bool_t, T>(to_storage<T>(x)).v; }
+};
+struct InvertOp { // bitwise_invert.hpp: bool -> logical not, ints -> ~x
+    template <class T> static constexpr bool ok = is_bool_v<T> || is_int_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> x)
+    {
+        if constexpr (is_bool_v<T>) return !x;
+        else return (T)~x;
+    }
+};
+struct SignbitOp {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = bool_t;
+    template <class T> DPX_D static bool apply(T x) { return m_signbit(x); }
+};
+
+// op id -> op struct; f(tag<Op>{}) is called for a valid id
+template <class F> inline bool for_binary_op(int op, F &&f)
+{
+    switch (op) {
+    case DPX_B_ADD: f(tag<AddOp>{}); return true;
+    case DPX_B_SUBTRACT: f(tag<SubOp>{}); return true;
+    case DPX_B_MULTIPLY: f(tag<MulOp>{}); return true;
+    case DPX_B_DIVIDE: f(tag<DivOp>{}); return true;
+    case DPX_B_BITWISE_AND: f(tag<BitOp<0>>{}); return true;
+    case DPX_B_BITWISE_OR: f(tag<BitOp<1>>{}); return true;
+    case DPX_B_BITWISE_XOR: f(tag<BitOp<2>>{}); return true;
+    case DPX_B_EQUAL: f(tag<CmpOp<0>>{}); return true;
+    case DPX_B_NOT_EQUAL: f(tag<CmpOp<1>>{}); return true;
+    case DPX_B_LESS: f(tag<CmpOp<2>>{}); return true;
+    case DPX_B_LESS_EQUAL: f(tag<CmpOp<3>>{}); return true;
+    case DPX_B_GREATER: f(tag<CmpOp<4>>{}); return true;
+    case DPX_B_GREATER_EQUAL: f(tag<CmpOp<5>>{}); return true;
+    case DPX_B_MAXIMUM: f(tag<MaxOp>{}); return true;
+    case DPX_B_MINIMUM: f(tag<MinOp>{}); return true;
+    case DPX_B_LOGICAL_AND: f(tag<LogicalOp<0>>{}); return true;
+    case DPX_B_LOGICAL_OR: f(tag<LogicalOp<1>>{}); return true;
+    case DPX_B_LOGICAL_XOR: f(tag<LogicalOp<2>>{}); return true;
+    case DPX_B_POW: f(tag<PowOp>{}); return true;
+    case DPX_B_FLOOR_DIVIDE: f(tag<FloorDivOp>{}); return true;
+    case DPX_B_REMAINDER: f(tag<RemainderOp>{}); return true;
+    case DPX_B_ATAN2: f(tag<Atan2Op>{}); return true;
+    case DPX_B_HYPOT: f(tag<HypotOp>{}); return true;
+    case DPX_B_COPYSIGN: f(tag<CopysignOp>{}); return true;
+    case DPX_B_LEFT_SHIFT: f(tag<ShiftOp<true>>{}); return true;
+    case DPX_B_RIGHT_SHIFT: f(tag<ShiftOp<false>>{}); return true;
+    default: return false;
+    }
+}
+template <class F> inline bool for_unary_op(int op, F &&f)
+{
+    switch (op) {
+    case DPX_U_ABS: f(tag<AbsOp>{}); return true;
+    case DPX_U_NEGATIVE: f(tag<NegOp>{}); return true;
+    case DPX_U_POSITIVE: f(tag<PosOp>{}); return true;
+    case DPX_U_SQUARE: f(tag<SquareOp>{}); return true;
+    case DPX_U_SQRT: f(tag<SqrtOp>{}); return true;
+    case DPX_U_EXP: f(tag<ExpOp>{}); return true;
+    case DPX_U_LOG: f(tag<LogOp>{}); return true;
+    case DPX_U_ERF: f(tag<ErfOp>{}); return true;
+    case DPX_U_SIN: f(tag<SinOp>{}); return true;
+    case DPX_U_COS: f(tag<CosOp>{}); return true;
+    case DPX_U_TAN: f(tag<TanOp>{}); return true;
+    case DPX_U_TANH: f(tag<TanhOp>{}); return true;
+    case DPX_U_EXP2: f(tag<Exp2Op>{}); return true;
+    case DPX_U_EXPM1: f(tag<Expm1Op>{}); return true;
+    case DPX_U_LOG2: f(tag<Log2Op>{}); return true;
+    case DPX_U_LOG10: f(tag<Log10Op>{}); return true;
+    case DPX_U_LOG1P: f(tag<Log1pOp>{}); return true;
+    case DPX_U_RSQRT: f(tag<RsqrtOp>{}); return true;
+    case DPX_U_CBRT: f(tag<CbrtOp>{}); return true;
+    case DPX_U_RECIPROCAL: f(tag<ReciprocalOp>{}); return true;
+    case DPX_U_FLOOR: f(tag<RoundOp<0>>{}); return true;
+    case DPX_U_CEIL: f(tag<RoundOp<1>>{}); return true;
+    case DPX_U_TRUNC: f(tag<RoundOp<2>>{}); return true;
+    case DPX_U_SIGN: f(tag<SignOp>{}); return true;
+    case DPX_U_ISNAN: f(tag<FpClassOp<0>>{}); return true;
+    case DPX_U_ISINF: f(tag<FpClassOp<1>>{}); return true;
+    case DPX_U_ISFINITE: f(tag<FpClassOp<2>>{}); return true;
+    case DPX_U_LOGICAL_NOT: f(tag<LogicalNotOp>{}); return true;
+    case DPX_U_BITWISE_INVERT: f(tag<InvertOp>{}); return true;
+    case DPX_U_SIGNBIT: f(tag<SignbitOp>{}); return true;
+    default: return false;
+    }
+}
+
+} // namespace dpx

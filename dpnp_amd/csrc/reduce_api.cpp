@@ -1,0 +1,115 @@
+// extern "C" reduction entry points.
+#include "reduce_dispatch.hpp"
+
+namespace dpx {
+bool sum_pair_supported(int, int);
+bool prod_pair_supported(int, int);
+bool sqdev_pair_supported(int, int);
+int sum_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int prod_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int sqdev_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int sum_acc_size(int, int);
+int prod_acc_size(int, int);
+int minmax_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int arg_run_any(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+
+static bool reduce_supported(int op, int s, int d)
+{
+    if (s < 0 || s >= DPX_NUM_DTYPES || d < 0 || d >= DPX_NUM_DTYPES) return false;
+    switch (op) {
+    case DPX_R_SUM: return sum_pair_supported(s, d);
+    case DPX_R_PROD: return prod_pair_supported(s, d);
+    case DPX_R_MAX:
+    case DPX_R_MIN: return s == d;
+    case DPX_R_SUMSQDEV: return sqdev_pair_supported(s, d);
+    default: return false;
+    }
+}
+
+static int reduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
+                       const dpx_array_view *aux, void *stream, dpx_plan *plan_out)
+{
+    if (op < 0 || op >= DPX_R_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown reduction op id");
+    if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if ((op == DPX_R_SUMSQDEV) != (aux != nullptr))
+        return fail(DPX_ERR_BAD_ARGUMENT, "aux must be given for DPX_R_SUMSQDEV and only for it");
+    if (!reduce_supported(op, src->dtype, dst->dtype))
+        return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
+    const bool empty_ok = op == DPX_R_SUM || op == DPX_R_PROD || op == DPX_R_SUMSQDEV;
+    if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
+    RedPlan pl;
+    red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false);
+    if (plan_out) {
+        int acc = itemsize_of(dst->dtype);
+        if (op == DPX_R_SUM || op == DPX_R_SUMSQDEV) acc = sum_acc_size(src->dtype, dst->dtype) ? sum_acc_size(src->dtype, dst->dtype) : acc;
+        if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
+        if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
+        if (op == DPX_R_SUMSQDEV && dst->dtype == DPX_HALF) acc = 4;
+        red_finish_fold(pl, acc, false);
+        red_export_plan(pl, plan_out, acc);
+        return DPX_OK;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (op) {
+    case DPX_R_SUM: return sum_run(pl, src, dst, s);
+    case DPX_R_PROD: return prod_run(pl, src, dst, s);
+    case DPX_R_MAX: return minmax_run(true, pl, src, dst, s);
+    case DPX_R_MIN: return minmax_run(false, pl, src, dst, s);
+    default: return sqdev_run(pl, src, dst, aux, s);
+    }
+}
+
+static int argreduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
+                          void *stream, dpx_plan *plan_out)
+{
+    if (op != DPX_S_ARGMAX && op != DPX_S_ARGMIN) return fail(DPX_ERR_BAD_ARGUMENT, "unknown search op id");
+    if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (dst->dtype != DPX_INT64) return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
+    if (int rc = red_validate(src, trailing, dst, nullptr, false)) return rc;
+    RedPlan pl;
+    red_make_plan(pl, src, trailing, dst, nullptr, true, itemsize_of(src->dtype), true);
+    if (plan_out) {
+        red_finish_fold(pl, itemsize_of(src->dtype), true);
+        red_export_plan(pl, plan_out, itemsize_of(src->dtype) + 8);
+        return DPX_OK;
+    }
+    return arg_run_any(op == DPX_S_ARGMAX, pl, src, dst, (hipStream_t)stream);
+}
+
+} // namespace dpx
+
+using namespace dpx;
+extern "C" {
+int dpx_reduce_dtype_supported(int op, int src_dt, int dst_dt) { return reduce_supported(op, src_dt, dst_dt) ? 1 : 0; }
+int dpx_search_dtype_supported(int op, int src_dt, int dst_dt)
+{
+    return ((op == DPX_S_ARGMAX || op == DPX_S_ARGMIN) && src_dt >= 0 && src_dt < DPX_NUM_DTYPES &&
+            dst_dt == DPX_INT64)
+               ? 1
+               : 0;
+}
+int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
+               const dpx_array_view *aux, void *stream)
+{
+    return reduce_call(op, src, trailing_dims_to_reduce, dst, aux, stream, nullptr);
+}
+int dpx_reduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
+                    dpx_plan *plan)
+{
+    if (!plan) return fail(DPX_ERR_BAD_ARGUMENT, "plan is null");
+    // a plan for DPX_R_SUMSQDEV is that of DPX_R_SUM with the same dtypes
+    return reduce_call(op == DPX_R_SUMSQDEV ? DPX_R_SUM : op, src, trailing_dims_to_reduce, dst, nullptr, nullptr,
+                       plan);
+}
+int dpx_argreduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
+                  void *stream)
+{
+    return argreduce_call(op, src, trailing_dims_to_reduce, dst, stream, nullptr);
+}
+int dpx_argreduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
+                       const dpx_array_view *dst, dpx_plan *plan)
+{
+    if (!plan) return fail(DPX_ERR_BAD_ARGUMENT, "plan is null");
+    return argreduce_call(op, src, trailing_dims_to_reduce, dst, nullptr, plan);
+}
+}

@@ -1,0 +1,300 @@
+// Reductions: validation and launch planning (no element types here).
+#include <cstdlib>
+#include "reduce_dispatch.hpp"
+
+namespace dpx {
+
+int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *dst,
+                 const dpx_array_view *aux, bool empty_ok)
+{
+    if (!view_ok(src) || !view_ok(dst) || (aux && !view_ok(aux)))
+        return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (trailing <= 0 || trailing > src->nd)
+        return fail(DPX_ERR_BAD_ARGUMENT, "Trailing_dim_to_reduce must be positive, but no greater than rank "
+                                          "of the array being reduced");
+    const int ndi = src->nd - trailing;
+    if (dst->nd != ndi)
+        return fail(DPX_ERR_RANK_MISMATCH, "Destination array rank does not match input array rank and number "
+                                           "of reduced dimensions");
+    for (int d = 0; d < ndi; ++d)
+        if (src->shape[d] != dst->shape[d])
+            return fail(DPX_ERR_SHAPE_MISMATCH, "Destination shape does not match unreduced dimensions of the input shape");
+    if (!(dst->flags & DPX_WRITABLE)) return fail(DPX_ERR_NOT_WRITABLE, "output array is read-only.");
+    if (aux) {
+        if (!same_shape(aux, dst)) return fail(DPX_ERR_SHAPE_MISMATCH, "aux shape does not match destination shape");
+        if (aux->dtype != dst->dtype) return fail(DPX_ERR_BAD_DTYPE, "aux dtype does not match destination dtype");
+    }
+    const int64_t m = view_size(dst);
+    int64_t n = 1;
+    for (int d = ndi; d < src->nd; ++d) n *= src->shape[d];
+    if (m == 0) return DPX_OK;
+    if (n == 0 && !empty_ok) return fail(DPX_ERR_BAD_ARGUMENT, "reduction cannot be performed over zero-size axes");
+    if (dst->data == nullptr || (n > 0 && src->data == nullptr) || (aux && aux->data == nullptr))
+        return fail(DPX_ERR_BAD_ARGUMENT, "null data pointer");
+    if (views_overlap(src, dst) || (aux && views_overlap(aux, dst)))
+        return fail(DPX_ERR_OVERLAP, "Arrays index overlapping segments of memory");
+    int64_t lo, hi;
+    view_minmax(dst, lo, hi);
+    if (hi - lo + 1 < m)
+        return fail(DPX_ERR_NOT_AMPLE, "Memory addressed by the output array is not sufficiently ample.");
+    return DPX_OK;
+}
+
+static int env_int(const char *name, int dflt)
+{
+    const char *s = std::getenv(name);
+    return (s && *s) ? std::atoi(s) : dflt;
+}
+static int ceil_log2(int64_t v)
+{
+    int lg = 0;
+    while (((int64_t)1 << lg) < v) ++lg;
+    return lg;
+}
+static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// lanes cooperating on one output of `n` elements read `e` at a time: aim at ~8 accesses
+// per lane; more than a wave means a whole 256- or 1024-thread block
+static void rows_geometry(int64_t n, int e, int &g_log2, int &block)
+{
+    int64_t lanes = cdiv(n, (int64_t)e * 8);
+    const int forced = env_int("DPX_ROWS_G_LOG2", -1); // experiment knob
+    if (forced >= 0) lanes = (int64_t)1 << forced;
+    if (lanes <= 64) {
+        g_log2 = ceil_log2(lanes);
+        block = 256;
+    }
+    else if (lanes <= 256) {
+        g_log2 = 8;
+        block = 256;
+    }
+    else {
+        g_log2 = 10;
+        block = 1024;
+    }
+}
+
+void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
+                   const dpx_array_view *aux, bool keep_order, int in_size, bool arg)
+{
+    pl = RedPlan{};
+    const int nd = src->nd, ndi = nd - trailing;
+    int64_t m = 1, n = 1;
+    for (int d = 0; d < ndi; ++d) m *= src->shape[d];
+    for (int d = ndi; d < nd; ++d) n *= src->shape[d];
+    pl.L.m = m;
+    pl.L.n = n;
+    pl.L.splits = 1;
+    if (m == 0) {
+        pl.path = DPX_PATH_NOOP;
+        return;
+    }
+    // iteration space: src (leading dims), aux, dst collapse together
+    int64_t ishape[DPX_MAX_ND], istr[3][DPX_MAX_ND], ioff[3];
+    for (int d = 0; d < ndi; ++d) {
+        ishape[d] = src->shape[d];
+        istr[0][d] = src->strides[d];
+        istr[1][d] = aux ? aux->strides[d] : 0;
+        istr[2][d] = dst->strides[d];
+    }
+    int nd_i = collapse(ndi, 3, ishape, istr, ioff, false);
+    if (nd_i == 0) {
+        nd_i = 1;
+        ishape[0] = 1;
+        istr[0][0] = istr[1][0] = istr[2][0] = 0;
+    }
+    int64_t rshape[DPX_MAX_ND], rstr[1][DPX_MAX_ND], roff[1] = {0};
+    int nd_r = 0;
+    if (n > 0) {
+        for (int d = 0; d < trailing; ++d) {
+            rshape[d] = src->shape[ndi + d];
+            rstr[0][d] = src->strides[ndi + d];
+        }
+        nd_r = collapse(trailing, 1, rshape, rstr, roff, keep_order);
+    }
+    if (nd_r == 0) {
+        nd_r = 1;
+        rshape[0] = n > 0 ? 1 : 0;
+        rstr[0][0] = 1;
+    }
+    RedIndex &ix = pl.ix;
+    ix.nd_i = nd_i;
+    ix.nd_r = nd_r;
+    for (int d = 0; d < DPX_MAX_ND; ++d) {
+        ix.shape_i[d] = d < nd_i ? ishape[d] : 1;
+        ix.src_istr[d] = d < nd_i ? istr[0][d] : 0;
+        ix.aux_str[d] = d < nd_i ? istr[1][d] : 0;
+        ix.dst_str[d] = d < nd_i ? istr[2][d] : 0;
+        ix.shape_r[d] = d < nd_r ? rshape[d] : 1;
+        ix.src_rstr[d] = d < nd_r ? rstr[0][d] : 0;
+    }
+    pl.src_off = ioff[0] + roff[0];
+    pl.aux_off = ioff[1];
+    pl.dst_off = ioff[2];
+    if (n == 0) {
+        pl.path = DPX_PATH_RED_SMALL; // identity fill
+        pl.block = 256;
+        pl.grid = cdiv(m, 256);
+        return;
+    }
+
+    const int E = 16 / in_size;
+    const int64_t target = env_int("DPX_RED_TARGET_BLOCKS", 4 * device_cus());
+    const uintptr_t base = (uintptr_t)src->data + (uintptr_t)(pl.src_off * in_size);
+    const int last = nd_i - 1;
+    const int64_t inner = ishape[last];
+    const bool contig_red = nd_r == 1 && (rstr[0][0] == 1 || n == 1);
+    const bool cols_ok = !contig_red && nd_r == 1 && istr[0][last] == 1 && inner > 1;
+    RedLaunch &L = pl.L;
+
+    if (!cols_ok) {
+        // ---- rows / generic -------------------------------------------------------
+        bool vec = contig_red && (base % 16 == 0);
+        for (int d = 0; d < nd_i && vec; ++d)
+            if (ishape[d] > 1 && istr[0][d] % E != 0) vec = false;
+        const int e = vec ? E : 1;
+        L.vec = vec ? 1 : 0;
+        rows_geometry(n, e, L.g_log2, pl.block);
+        const int64_t G = (int64_t)1 << L.g_log2;
+        const int64_t opb = (G <= 64) ? 256 / G : 1;
+        const int64_t oblocks = cdiv(m, opb);
+        int64_t splits = 1;
+        const int64_t per_pass = G * e * 8; // elements one group covers with 8 accesses per lane
+        if (oblocks < target && n >= 2 * per_pass) splits = std::min(cdiv(target, oblocks), cdiv(n, per_pass));
+        if (arg) splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
+        int64_t chunk = cdiv(n, splits);
+        chunk = cdiv(chunk, G * e) * (G * e);
+        splits = cdiv(n, chunk);
+        L.chunk = chunk;
+        L.splits = (int32_t)splits;
+        pl.grid = oblocks * splits;
+        pl.path = !contig_red ? DPX_PATH_RED_GENERIC
+                              : (splits > 1 ? DPX_PATH_RED_ROWS_SPLIT
+                                            : (G == 1 ? DPX_PATH_RED_SMALL : DPX_PATH_RED_ROWS));
+        if (splits > 1) {
+            pl.scratch_elems = m * splits;
+            pl.fold_cols = false;
+            pl.fix = ix;
+            int64_t st = splits;
+            for (int d = nd_i - 1; d >= 0; --d) {
+                pl.fix.src_istr[d] = st;
+                st *= ishape[d];
+                pl.fix.aux_str[d] = 0;
+            }
+            pl.fix.nd_r = 1;
+            pl.fix.shape_r[0] = splits;
+            pl.fix.src_rstr[0] = 1;
+            RedLaunch &F = pl.fL;
+            F = RedLaunch{};
+            F.m = m;
+            F.n = splits;
+            F.splits = 1;
+            F.vec = 0; // set by red_finish_fold once the partial size is known
+            F.chunk = splits;
+        }
+        return;
+    }
+    // ---- cols -----------------------------------------------------------------------
+    const int64_t rstride = rstr[0][0];
+    bool vec = !arg && (base % 16 == 0) && (inner % E == 0) && (rstride % E == 0);
+    for (int d = 0; d < last && vec; ++d)
+        if (ishape[d] > 1 && istr[0][d] % E != 0) vec = false;
+    const int e = vec ? E : 1;
+    L.vec = vec ? 1 : 0;
+    L.rstride = rstride;
+    L.inner = inner;
+    int lg = std::min(8, ceil_log2(cdiv(inner, e)));
+    const int forced = env_int("DPX_COLS_TX_LOG2", -1); // experiment knob
+    if (forced >= 0 && forced <= 8) lg = std::min(lg, forced);
+    L.g_log2 = lg;
+    const int64_t TX = (int64_t)1 << lg, TY = 256 / TX;
+    L.col_blocks = cdiv(inner, TX * e);
+    const int64_t outer = m / inner;
+    const int64_t base_blocks = L.col_blocks * outer;
+    int64_t splits = 1;
+    if (base_blocks < target && n >= 2 * TY * 8) splits = std::min(cdiv(target, base_blocks), cdiv(n, TY * 8));
+    int64_t chunk = cdiv(n, splits);
+    splits = cdiv(n, chunk);
+    L.chunk = chunk;
+    L.splits = (int32_t)splits;
+    pl.block = 256;
+    pl.grid = base_blocks * splits;
+    pl.path = splits > 1 ? DPX_PATH_RED_COLS_SPLIT : DPX_PATH_RED_COLS;
+    if (splits > 1) {
+        pl.scratch_elems = m * splits;
+        pl.fold_cols = true;
+        pl.fix = ix;
+        int64_t st = 1;
+        for (int d = nd_i - 1; d >= 0; --d) {
+            pl.fix.src_istr[d] = st;
+            st *= ishape[d];
+            pl.fix.aux_str[d] = 0;
+        }
+        pl.fix.nd_r = 1;
+        pl.fix.shape_r[0] = splits;
+        pl.fix.src_rstr[0] = m;
+        RedLaunch &F = pl.fL;
+        F = RedLaunch{};
+        F.m = m;
+        F.n = splits;
+        F.splits = 1;
+        F.chunk = splits;
+        F.rstride = m;
+        F.inner = inner;
+    }
+}
+
+// Launch geometry of the fold pass, which depends on the byte size of a partial.
+void red_finish_fold(RedPlan &pl, int acc_size, bool arg)
+{
+    if (pl.L.splits <= 1) return;
+    RedLaunch &F = pl.fL;
+    const int E = 16 / acc_size;
+    if (!pl.fold_cols) {
+        const bool vec = !arg && (F.n % E == 0);
+        F.vec = vec ? 1 : 0;
+        rows_geometry(F.n, vec ? E : 1, F.g_log2, pl.fblock);
+        const int64_t G = (int64_t)1 << F.g_log2;
+        const int64_t opb = (G <= 64) ? 256 / G : 1;
+        F.chunk = cdiv(F.n, G * (vec ? E : 1)) * G * (vec ? E : 1);
+        pl.fgrid = cdiv(F.m, opb);
+    }
+    else {
+        const bool vec = !arg && (F.inner % E == 0) && (F.m % E == 0);
+        const int e = vec ? E : 1;
+        F.vec = vec ? 1 : 0;
+        const int lg = std::min(8, ceil_log2(cdiv(F.inner, e)));
+        F.g_log2 = lg;
+        F.col_blocks = cdiv(F.inner, ((int64_t)1 << lg) * e);
+        pl.fblock = 256;
+        pl.fgrid = F.col_blocks * (F.m / F.inner);
+    }
+}
+
+void red_export_plan(const RedPlan &pl, dpx_plan *out, int acc_size)
+{
+    *out = dpx_plan{};
+    out->path = pl.path;
+    if (pl.path == DPX_PATH_NOOP) return;
+    out->nd = pl.ix.nd_i;
+    out->red_nd = pl.ix.nd_r;
+    for (int d = 0; d < pl.ix.nd_i; ++d) {
+        out->shape[d] = pl.ix.shape_i[d];
+        out->strides[0][d] = pl.ix.src_istr[d];
+        out->strides[1][d] = pl.ix.dst_str[d];
+    }
+    for (int d = 0; d < pl.ix.nd_r; ++d) {
+        out->strides[2][d] = pl.ix.shape_r[d];
+        out->strides[3][d] = pl.ix.src_rstr[d];
+    }
+    out->offsets[0] = pl.src_off;
+    out->offsets[1] = pl.dst_off;
+    out->vec = pl.L.vec;
+    out->grid[0] = pl.grid;
+    out->grid[1] = out->grid[2] = 1;
+    out->block = pl.block;
+    out->splits = pl.L.splits;
+    out->scratch_bytes = pl.scratch_elems * acc_size;
+}
+
+} // namespace dpx

@@ -1,0 +1,328 @@
+/*
+ * dpnp_amd.h -- C ABI of libdpnp_amd.so: the elementwise + axis-reduction hot
+ * path of dpnp.tensor for AMD MI355X (gfx950).
+ *
+ * Every entry point replaces one family of pybind11 functions that the
+ * reference's Python layer calls in the extension modules _tensor_impl,
+ * _tensor_elementwise_impl and _tensor_reductions_impl.  The reference passes
+ * usm_ndarray objects, a sycl::queue and a list of events and gets back a pair
+ * of events; here the caller passes plain array descriptors and a hipStream_t
+ * and gets back a status code.  Work is enqueued on the given (in-order)
+ * stream and is asynchronous with respect to the host.
+ *
+ * Conventions
+ *   - all array arguments are borrowed for the duration of the call; the
+ *     caller keeps the device memory alive until the stream has passed the work;
+ *   - `dst` is always allocated by the caller; the library allocates only
+ *     scratch (partial results of multi-block reductions) from a grow-only,
+ *     per-stream pool it owns;
+ *   - strides are in ELEMENTS (as usm_ndarray.strides), may be zero
+ *     (broadcast) or negative; `data` points at the element with all indices 0;
+ *   - a return value != DPX_OK leaves `dst` untouched (all validation happens
+ *     before the first launch); dpx_last_error() gives the message of the last
+ *     failure on the calling thread;
+ *   - zero-size iteration spaces return DPX_OK without launching.
+ *
+ * citations: paths are relative to the reference tree, libtensor =
+ * dpnp/tensor/libtensor.
+ */
+#ifndef DPNP_AMD_H
+#define DPNP_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DPX_MAX_ND 12
+
+/* dtype ids: same order as typenum_t,
+ * libtensor/include/utils/type_dispatch_building.hpp:45-61 */
+typedef enum dpx_dtype {
+    DPX_BOOL = 0,
+    DPX_INT8 = 1,
+    DPX_UINT8 = 2,
+    DPX_INT16 = 3,
+    DPX_UINT16 = 4,
+    DPX_INT32 = 5,
+    DPX_UINT32 = 6,
+    DPX_INT64 = 7,
+    DPX_UINT64 = 8,
+    DPX_HALF = 9,
+    DPX_FLOAT = 10,
+    DPX_DOUBLE = 11,
+    DPX_CFLOAT = 12,
+    DPX_CDOUBLE = 13,
+    DPX_NUM_DTYPES = 14
+} dpx_dtype;
+
+/* flag bits: dpnp/include/usm_ndarray_constants.h:33-38 */
+#define DPX_C_CONTIGUOUS 1
+#define DPX_F_CONTIGUOUS 2
+#define DPX_WRITABLE 4
+
+/* array descriptor: the fields of the usm_ndarray struct the kernels glue
+ * reads (dpnp/tensor/_usmarray.pxd:81-97, dpnp/include/dpnp4pybind11.hpp:402-447) */
+typedef struct dpx_array_view {
+    void *data;                  /* device pointer, element offset applied */
+    int32_t nd;                  /* 0 <= nd <= DPX_MAX_ND */
+    int32_t dtype;               /* dpx_dtype */
+    int32_t flags;               /* DPX_C_CONTIGUOUS | DPX_F_CONTIGUOUS | DPX_WRITABLE */
+    int32_t reserved;
+    int64_t shape[DPX_MAX_ND];
+    int64_t strides[DPX_MAX_ND]; /* in elements */
+} dpx_array_view;
+
+/* status codes; the Python shim maps them to the exception classes the
+ * reference raises (libtensor/source/elementwise_functions/elementwise_functions.hpp:96-141,
+ * libtensor/source/reductions/reduction_over_axis.hpp:188-238,456-458) */
+typedef enum dpx_status {
+    DPX_OK = 0,
+    DPX_ERR_BAD_DTYPE = 1,       /* ValueError: dst dtype is not op's result type */
+    DPX_ERR_SHAPE_MISMATCH = 2,  /* ValueError */
+    DPX_ERR_RANK_MISMATCH = 3,   /* ValueError */
+    DPX_ERR_NOT_WRITABLE = 4,    /* ValueError */
+    DPX_ERR_OVERLAP = 5,         /* ValueError */
+    DPX_ERR_NOT_AMPLE = 6,       /* ValueError */
+    DPX_ERR_NOT_IMPLEMENTED = 7, /* RuntimeError */
+    DPX_ERR_HIP = 8,             /* RuntimeError */
+    DPX_ERR_BAD_ARGUMENT = 9     /* ValueError */
+} dpx_status;
+
+/* unary elementwise ops (one functor header each under
+ * libtensor/include/kernels/elementwise_functions/) */
+typedef enum dpx_unary_op {
+    DPX_U_ABS = 0,
+    DPX_U_NEGATIVE,
+    DPX_U_POSITIVE,
+    DPX_U_SQUARE,
+    DPX_U_SQRT,
+    DPX_U_EXP,
+    DPX_U_LOG,
+    DPX_U_ERF, /* dpnp/backend/kernels/elementwise_functions/erf.hpp:52-95 */
+    DPX_U_SIN,
+    DPX_U_COS,
+    DPX_U_TAN,
+    DPX_U_TANH,
+    DPX_U_EXP2,
+    DPX_U_EXPM1,
+    DPX_U_LOG2,
+    DPX_U_LOG10,
+    DPX_U_LOG1P,
+    DPX_U_RSQRT,
+    DPX_U_CBRT,
+    DPX_U_RECIPROCAL,
+    DPX_U_FLOOR,
+    DPX_U_CEIL,
+    DPX_U_TRUNC,
+    DPX_U_SIGN,
+    DPX_U_ISNAN,
+    DPX_U_ISINF,
+    DPX_U_ISFINITE,
+    DPX_U_LOGICAL_NOT,
+    DPX_U_BITWISE_INVERT,
+    DPX_U_SIGNBIT,
+    DPX_U_NUM_OPS
+} dpx_unary_op;
+
+typedef enum dpx_binary_op {
+    DPX_B_ADD = 0,
+    DPX_B_SUBTRACT,
+    DPX_B_MULTIPLY,
+    DPX_B_DIVIDE,
+    DPX_B_BITWISE_AND,
+    DPX_B_BITWISE_OR,
+    DPX_B_BITWISE_XOR,
+    DPX_B_EQUAL,
+    DPX_B_NOT_EQUAL,
+    DPX_B_LESS,
+    DPX_B_LESS_EQUAL,
+    DPX_B_GREATER,
+    DPX_B_GREATER_EQUAL,
+    DPX_B_MAXIMUM,
+    DPX_B_MINIMUM,
+    DPX_B_LOGICAL_AND,
+    DPX_B_LOGICAL_OR,
+    DPX_B_LOGICAL_XOR,
+    DPX_B_POW,
+    DPX_B_FLOOR_DIVIDE,
+    DPX_B_REMAINDER,
+    DPX_B_ATAN2,
+    DPX_B_HYPOT,
+    DPX_B_COPYSIGN,
+    DPX_B_LEFT_SHIFT,
+    DPX_B_RIGHT_SHIFT,
+    DPX_B_NUM_OPS
+} dpx_binary_op;
+
+typedef enum dpx_reduce_op {
+    DPX_R_SUM = 0,
+    DPX_R_PROD,
+    DPX_R_MAX,
+    DPX_R_MIN,
+    DPX_R_SUMSQDEV, /* sum((x - aux)^2): second pass of var, see dpx_reduce */
+    DPX_R_NUM_OPS
+} dpx_reduce_op;
+
+typedef enum dpx_search_op { DPX_S_ARGMAX = 0, DPX_S_ARGMIN = 1 } dpx_search_op;
+
+/* which kernel family a call resolves to (reported by the dpx_*_plan queries;
+ * lets the host-side dispatch be tested without a GPU) */
+typedef enum dpx_path {
+    DPX_PATH_NOOP = 0,          /* zero-size: nothing launched */
+    DPX_PATH_EW_CONTIG = 1,     /* 1-D unit-stride, 128-bit accesses */
+    DPX_PATH_EW_ROWS = 2,       /* N-D, threads vectorised along the inner dim */
+    DPX_PATH_EW_FLAT = 3,       /* N-D, one element per thread */
+    DPX_PATH_EW_TILE = 4,       /* 2-D transposing through an LDS tile */
+    DPX_PATH_RED_ROWS = 10,     /* reduced run contiguous: block or wave per output */
+    DPX_PATH_RED_ROWS_SPLIT = 11, /* ... several blocks per output + finalise pass */
+    DPX_PATH_RED_COLS = 12,     /* outputs contiguous, reduced run strided */
+    DPX_PATH_RED_COLS_SPLIT = 13, /* ... reduced run split over blocks + finalise */
+    DPX_PATH_RED_GENERIC = 14,  /* fully strided */
+    DPX_PATH_RED_SMALL = 15     /* tiny reduced run: one thread per output */
+} dpx_path;
+
+typedef struct dpx_plan {
+    int32_t path;   /* dpx_path */
+    int32_t nd;     /* dims left after stride collapsing (iteration space) */
+    int32_t red_nd; /* collapsed reduction dims (reductions only) */
+    int32_t vec;    /* elements per thread */
+    int64_t shape[DPX_MAX_ND];
+    int64_t strides[4][DPX_MAX_ND]; /* per operand, dst last */
+    int64_t offsets[4];             /* element displacement per operand */
+    int64_t grid[3];
+    int32_t block;
+    int32_t splits;        /* blocks cooperating on one output (reductions) */
+    int64_t scratch_bytes; /* pool bytes the call would use */
+} dpx_plan;
+
+/* ---- library ---------------------------------------------------------- */
+
+/* version of this ABI (bumped on incompatible change) */
+int dpx_abi_version(void);
+/* message of the last failing call on this thread ("" if none) */
+const char *dpx_last_error(void);
+/* number of bytes of element type dt, or -1 */
+int dpx_dtype_itemsize(int dt);
+/* release the scratch pool (device must be idle) */
+int dpx_release_scratch(void);
+
+/* ---- dtype queries ---------------------------------------------------- */
+
+/* result dtype of op for the exact input dtype(s), or -1 when no kernel exists:
+ * the _X_result_type functions, elementwise_functions.hpp:256-285,567-603 */
+int dpx_unary_result_type(int op, int dt);
+int dpx_binary_result_type(int op, int dt1, int dt2);
+/* 1 if `lhs op= rhs` has a kernel (py_binary_inplace_ufunc's table,
+ * elementwise_functions.hpp:612-650) */
+int dpx_binary_inplace_supported(int op, int lhs_dt, int rhs_dt);
+/* _sum_over_axis_dtype_supported & co., libtensor/source/reductions/sum.cpp:445-456 */
+int dpx_reduce_dtype_supported(int op, int src_dt, int dst_dt);
+/* argmax/argmin: any dtype -> int64, libtensor/source/reductions/argmax.cpp:77-127 */
+int dpx_search_dtype_supported(int op, int src_dt, int dst_dt);
+
+/* ---- host predicates --------------------------------------------------- */
+
+/* ti._array_overlap, libtensor/include/utils/memory_overlap.hpp:56-113 */
+int dpx_array_overlap(const dpx_array_view *a, const dpx_array_view *b);
+/* ti._same_logical_tensors, memory_overlap.hpp:115-155 */
+int dpx_same_logical(const dpx_array_view *a, const dpx_array_view *b);
+
+/* ---- elementwise ------------------------------------------------------- */
+
+/* py_unary_ufunc, elementwise_functions.hpp:77-251  (ti._exp, ti._sqrt, ...) */
+int dpx_unary(int op, const dpx_array_view *src, const dpx_array_view *dst,
+              void *stream);
+/* py_binary_ufunc, elementwise_functions.hpp:305-563  (ti._add, ti._multiply, ...).
+ * Inputs are already broadcast to dst's shape (zero strides). */
+int dpx_binary(int op, const dpx_array_view *src1, const dpx_array_view *src2,
+               const dpx_array_view *dst, void *stream);
+/* py_binary_inplace_ufunc, elementwise_functions.hpp:612-804 (ti._add_inplace, ...) */
+int dpx_binary_inplace(int op, const dpx_array_view *lhs,
+                       const dpx_array_view *rhs, void *stream);
+/* py_where, libtensor/source/where.cpp:74-247  (ti._where) */
+int dpx_where(const dpx_array_view *cond, const dpx_array_view *x1,
+              const dpx_array_view *x2, const dpx_array_view *dst,
+              void *stream);
+/* tei._divide_by_scalar, libtensor/source/elementwise_functions/true_divide.cpp:249-430;
+ * the scalar is converted to dst's real type before the division */
+int dpx_divide_by_scalar(const dpx_array_view *src, double scalar,
+                         const dpx_array_view *dst, void *stream);
+/* ti._copy_usm_ndarray_into_usm_ndarray,
+ * libtensor/source/copy_and_cast_usm_to_usm.cpp:137-216: dst = cast(src), any
+ * dtype pair, equal shapes */
+int dpx_copy_cast(const dpx_array_view *src, const dpx_array_view *dst,
+                  void *stream);
+/* dst = value (converted to dst's dtype): ti._full_usm_ndarray,
+ * libtensor/source/full_ctor.cpp. value_im is used for complex dst only. */
+int dpx_fill(const dpx_array_view *dst, double value_re, double value_im,
+             int64_t value_int, int use_int, void *stream);
+
+/* plans: the dispatch decision of the calls above without launching */
+int dpx_unary_plan(int op, const dpx_array_view *src,
+                   const dpx_array_view *dst, dpx_plan *plan);
+int dpx_binary_plan(int op, const dpx_array_view *src1,
+                    const dpx_array_view *src2, const dpx_array_view *dst,
+                    dpx_plan *plan);
+int dpx_where_plan(const dpx_array_view *cond, const dpx_array_view *x1,
+                   const dpx_array_view *x2, const dpx_array_view *dst,
+                   dpx_plan *plan);
+
+/* ---- fused chains (no counterpart in the reference, which runs them as
+ * sequences of the kernels above; results follow the unfused op order) ---- */
+
+/* dst = (lhs CMP rhs) ? x1 : x2 in one pass; cmp_op is one of the six
+ * comparison ids of dpx_binary_op.  Equivalent to ti._greater (etc.) into a
+ * bool temporary followed by ti._where. */
+int dpx_where_compare(int cmp_op, const dpx_array_view *lhs,
+                      const dpx_array_view *rhs, const dpx_array_view *x1,
+                      const dpx_array_view *x2, const dpx_array_view *dst,
+                      void *stream);
+/* Black-Scholes call/put prices (formula of examples/example_bs.py:50-78),
+ * float64 or float32, all five arrays 1-D contiguous of n elements */
+int dpx_black_scholes(const void *price, const void *strike, const void *t,
+                      double rate, double vol, void *call, void *put,
+                      int64_t n, int dtype, void *stream);
+
+/* ---- reductions --------------------------------------------------------- */
+
+/* py_reduction_over_axis / py_tree_reduction_over_axis,
+ * reduction_over_axis.hpp:174-501,508-777 (tri._sum_over_axis, _prod_over_axis,
+ * _max_over_axis, _min_over_axis).  The last `trailing_dims_to_reduce` axes of
+ * src are reduced; dst has the leading src.nd - trailing axes.
+ * op == DPX_R_SUMSQDEV additionally takes `aux` (same shape and dtype as dst,
+ * any strides): dst[i] = sum_j (src[i,j] - aux[i])^2; aux is NULL otherwise. */
+int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
+               const dpx_array_view *dst, const dpx_array_view *aux,
+               void *stream);
+/* py_search_over_axis, reduction_over_axis.hpp:781-1047 (tri._argmax_over_axis,
+ * tri._argmin_over_axis): int64 C-order flat index over the reduced axes,
+ * smallest index among equal extrema, NaN counts as the extremum (first NaN) */
+int dpx_argreduce(int op, const dpx_array_view *src,
+                  int trailing_dims_to_reduce, const dpx_array_view *dst,
+                  void *stream);
+int dpx_reduce_plan(int op, const dpx_array_view *src,
+                    int trailing_dims_to_reduce, const dpx_array_view *dst,
+                    dpx_plan *plan);
+int dpx_argreduce_plan(int op, const dpx_array_view *src,
+                       int trailing_dims_to_reduce, const dpx_array_view *dst,
+                       dpx_plan *plan);
+
+/* ---- stride collapsing (exposed for testing) ---------------------------- */
+
+/* Joint collapse of `nops` stride vectors over one shape
+ * (simplify_iteration_space*, libtensor/source/simplify_iteration_space.cpp:51-417;
+ * libtensor/include/utils/strided_iters.hpp:364-899).  strides is
+ * [nops][DPX_MAX_ND]; shape and strides are rewritten in place, offsets[nops]
+ * receives the element displacement of each operand.  keep_order != 0 only
+ * merges adjacent dims (compact_iteration, strided_iters.hpp:946-983).
+ * Returns the new number of dims. */
+int dpx_collapse(int nd, int nops, int64_t *shape, int64_t *strides,
+                 int64_t *offsets, int keep_order);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DPNP_AMD_H */
