@@ -6,6 +6,12 @@ module raises; there is no CPU or PyTorch fallback.
 import ctypes
 import os
 
+# PyTorch ships its own HIP runtime (libamdhip64.so.7).  It must be in the process before
+# libdpnp_amd.so is loaded so that both bind to the SAME runtime instance: device memory
+# allocated by torch is then valid in this library's launches, and the stream handles match.
+# Loading in the other order leaves two runtimes in the process and the second one finds no device.
+import torch  # noqa: F401,E402
+
 MAX_ND = 12
 
 (BOOL, INT8, UINT8, INT16, UINT16, INT32, UINT32, INT64, UINT64, HALF, FLOAT,

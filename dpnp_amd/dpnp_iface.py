@@ -1,0 +1,500 @@
+"""NumPy-flavoured functions over dpnp_array: the dpnp-level wrappers on the hot path.
+
+Keyword handling follows DPNPUnaryFunc / DPNPBinaryFunc
+(dpnp/dpnp_algo/dpnp_elementwise_common.py:167-235,647-739), dpnp_wrap_reduction_call
+(dpnp/dpnp_utils/dpnp_utils_reduction.py:35-53) and the public functions in
+dpnp/dpnp_iface_{mathematical,trigonometric,statistics,searching,bitwise,logic}.py:
+`where=`, `subok=`, `initial=` other than their defaults raise NotImplementedError, `dtype=`
+casts the inputs and excludes `out=`, `out is x1` runs the in-place kernel, a reduction's
+`out` of another dtype receives an unsafe cast of the result.
+"""
+import numpy as np
+
+from . import tensor as dpt
+from .dpnp_array import dpnp_array
+from .tensor import _elementwise_funcs as ef
+from .tensor import _tensor_elementwise_impl as tei
+from .tensor import _tensor_impl as ti
+from .tensor._type_utils import _default_accumulation_dtype
+from .tensor._usmarray import usm_ndarray
+
+# dtypes and constants under their NumPy names
+bool = bool_ = dpt.bool  # noqa: A001
+int8, uint8, int16, uint16 = dpt.int8, dpt.uint8, dpt.int16, dpt.uint16
+int32, uint32, int64, uint64 = dpt.int32, dpt.uint32, dpt.int64, dpt.uint64
+float16, float32, float64 = dpt.float16, dpt.float32, dpt.float64
+complex64, complex128 = dpt.complex64, dpt.complex128
+nan, inf, pi, e, newaxis = np.nan, np.inf, np.pi, np.e, None
+
+
+def is_supported_array_type(a):
+    return isinstance(a, (dpnp_array, usm_ndarray))
+
+
+def isscalar(x):
+    return np.isscalar(x)
+
+
+def get_usm_ndarray(a):
+    if isinstance(a, dpnp_array):
+        return a.get_array()
+    if isinstance(a, usm_ndarray):
+        return a
+    raise TypeError(f"An array must be any of supported type, but got {type(a)}")
+
+
+def get_usm_ndarray_or_scalar(a):
+    return a if np.isscalar(a) else get_usm_ndarray(a)
+
+
+def check_supported_arrays_type(*arrays, scalar_type=False, all_scalars=False):
+    any_is_array = False
+    for a in arrays:
+        if is_supported_array_type(a):
+            any_is_array = True
+            continue
+        if scalar_type and np.isscalar(a):
+            continue
+        raise TypeError(f"An array must be any of supported type, but got {type(a)}")
+    if len(arrays) > 1 and not (all_scalars or any_is_array):
+        raise TypeError("At least one input must be of supported array type, but got all scalars.")
+    return True
+
+
+def check_limitations(**kwargs):
+    """Raise NotImplementedError for NumPy keywords that only work at their default."""
+    defaults = {"where": True, "initial": None, "subok": True, "order": None}
+    for k, v in kwargs.items():
+        d = defaults.get(k)
+        if not (v is d or (k == "order" and v in ("C", "K", None))):
+            raise NotImplementedError(f"Parameter `{k}` is supported only with default value `{d}`, "
+                                      f"but got {v}.")
+
+
+def get_result_array(a, out=None, casting="safe"):
+    """`out` filled with `a` (cast by `casting`), or `a` wrapped when there is no `out`."""
+    if out is None:
+        return dpnp_array._create_from_usm_ndarray(a) if isinstance(a, usm_ndarray) else a
+    out_w = dpnp_array._create_from_usm_ndarray(out) if isinstance(out, usm_ndarray) else out
+    a_usm, out_usm = get_usm_ndarray(a), get_usm_ndarray(out_w)
+    if a_usm is out_usm or ti._same_logical_tensors(a_usm, out_usm):
+        return out_w
+    if out_usm.shape != a_usm.shape:
+        raise ValueError(f"Output array of shape {a_usm.shape} is needed, got {out_usm.shape}.")
+    if not np.can_cast(a_usm.dtype, out_usm.dtype, casting=casting):
+        raise TypeError(f"Cannot cast from {a_usm.dtype} to {out_usm.dtype} according to the rule {casting}.")
+    if a_usm.size:
+        ti._copy_usm_ndarray_into_usm_ndarray(src=a_usm, dst=out_usm)
+    return out_w
+
+
+# -- array creation / transfer ------------------------------------------------------------------------
+def _wrap(u):
+    return dpnp_array._create_from_usm_ndarray(u)
+
+
+def array(a, dtype=None, *, copy=True, order="K", subok=False, ndmin=0, like=None, device=None,
+          usm_type=None, sycl_queue=None):
+    check_limitations(subok=True if not subok else subok)
+    src = a.get_array() if isinstance(a, dpnp_array) else a
+    r = dpt.asarray(src, dtype=dtype, copy=True if copy else None, order=order)
+    if ndmin > r.ndim:
+        r = dpt.reshape(r, (1,) * (ndmin - r.ndim) + r.shape)
+    return _wrap(r)
+
+
+def asarray(a, dtype=None, order=None, *, device=None, usm_type=None, sycl_queue=None, copy=None, like=None):
+    src = a.get_array() if isinstance(a, dpnp_array) else a
+    return _wrap(dpt.asarray(src, dtype=dtype, copy=copy, order=order or "K"))
+
+
+def asnumpy(a, order="C"):
+    if isinstance(a, (dpnp_array, usm_ndarray)):
+        return np.asarray(dpt.asnumpy(get_usm_ndarray(a)), order=order)
+    return np.asarray(a, order=order)
+
+
+def empty(shape, *, dtype=None, order="C", like=None, device=None, usm_type="device", sycl_queue=None):
+    return _wrap(dpt.empty(shape, dtype=dtype, order=order or "C"))
+
+
+def zeros(shape, *, dtype=None, order="C", like=None, device=None, usm_type="device", sycl_queue=None):
+    return _wrap(dpt.zeros(shape, dtype=dtype, order=order or "C"))
+
+
+def ones(shape, *, dtype=None, order="C", like=None, device=None, usm_type="device", sycl_queue=None):
+    return _wrap(dpt.ones(shape, dtype=dtype, order=order or "C"))
+
+
+def full(shape, fill_value, *, dtype=None, order="C", like=None, device=None, usm_type=None, sycl_queue=None):
+    fv = fill_value.get_array() if isinstance(fill_value, dpnp_array) else fill_value
+    return _wrap(dpt.full(shape, fv, dtype=dtype, order=order or "C"))
+
+
+def empty_like(a, /, *, dtype=None, order="C", subok=False, shape=None, device=None, usm_type=None,
+               sycl_queue=None):
+    u = get_usm_ndarray(a)
+    if shape is not None:
+        return _wrap(dpt.empty(shape, dtype=dtype or u.dtype, order="C" if order in ("K", "A") else order))
+    return _wrap(dpt.empty_like(u, dtype=dtype, order=order))
+
+
+def zeros_like(a, /, *, dtype=None, order="C", subok=False, shape=None, device=None, usm_type=None,
+               sycl_queue=None):
+    r = empty_like(a, dtype=dtype, order=order, shape=shape)
+    r.fill(0)
+    return r
+
+
+def ones_like(a, /, *, dtype=None, order="C", subok=False, shape=None, device=None, usm_type=None,
+              sycl_queue=None):
+    r = empty_like(a, dtype=dtype, order=order, shape=shape)
+    r.fill(1)
+    return r
+
+
+def arange(start, /, stop=None, step=1, *, dtype=None, like=None, device=None, usm_type="device",
+           sycl_queue=None):
+    return _wrap(dpt.arange(start, stop, step, dtype=dtype))
+
+
+def broadcast_to(a, /, shape, subok=False):
+    return _wrap(dpt.broadcast_to(get_usm_ndarray(a), shape))
+
+
+def reshape(a, /, shape=None, order="C", *, copy=None):
+    return _wrap(dpt.reshape(get_usm_ndarray(a), shape, order=order or "C", copy=copy))
+
+
+def transpose(a, axes=None):
+    u = get_usm_ndarray(a)
+    return _wrap(u.T if axes is None else dpt.permute_dims(u, axes))
+
+
+def astype(x, dtype, /, *, order="K", casting="unsafe", copy=True, device=None):
+    return _wrap(dpt.astype(get_usm_ndarray(x), dtype, order=order, casting=casting, copy=copy))
+
+
+def copyto(dst, src, casting="same_kind", where=True):
+    check_limitations(where=where)
+    d = get_usm_ndarray(dst)
+    s = src if np.isscalar(src) else get_usm_ndarray(src)
+    if not np.isscalar(src) and not np.can_cast(s.dtype, d.dtype, casting=casting):
+        raise TypeError(f"Cannot cast from {s.dtype} to {d.dtype} according to the rule {casting}.")
+    d[...] = s
+
+
+def can_cast(from_, to, casting="safe"):
+    f = from_.dtype if is_supported_array_type(from_) else from_
+    return np.can_cast(f, to, casting=casting)
+
+
+def result_type(*args):
+    return dpt.result_type(*[get_usm_ndarray(a) if is_supported_array_type(a) else a for a in args])
+
+
+# -- elementwise functions ----------------------------------------------------------------------------------
+def _norm_order(order):
+    if order is None:
+        return "K"
+    if isinstance(order, str) and len(order) == 1 and order in "afkcAFKC":
+        return order.upper()
+    raise ValueError(f"order must be one of 'C', 'F', 'A', or 'K' (got '{order}')")
+
+
+def _check_ufunc_kwargs(name, where, subok, dtype, out, kwargs):
+    if kwargs:
+        raise NotImplementedError(f"Requested function={name} with kwargs={kwargs} isn't currently supported.")
+    if where is not True:
+        raise NotImplementedError(f"Requested function={name} with where={where} isn't currently supported.")
+    if subok is not True:
+        raise NotImplementedError(f"Requested function={name} with subok={subok} isn't currently supported.")
+    if dtype is not None and out is not None:
+        raise TypeError(f"Requested function={name} only takes `out` or `dtype` as an argument, "
+                        "but both were provided.")
+
+
+def _unpack_out(out, nout=1):
+    if isinstance(out, tuple):
+        if len(out) != nout:
+            raise ValueError("'out' tuple must have exactly one entry per ufunc output")
+        return out[0]
+    return out
+
+
+class DPNPUnaryFunc:
+    """NumPy-style unary ufunc over a tensor-level elementwise function."""
+
+    def __init__(self, name, tensor_fn):
+        self.name_ = self.__name__ = name
+        self._fn = tensor_fn
+        self.__doc__ = tensor_fn.__doc__
+        self.nin, self.nout = 1, 1
+
+    @property
+    def types(self):
+        return self._fn.types
+
+    def __call__(self, x, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+        _check_ufunc_kwargs(self.name_, where, subok, dtype, out, kwargs)
+        if not is_supported_array_type(x):
+            raise TypeError(f"Input array must be any of supported type, but got {type(x)}")
+        order = _norm_order(order)
+        x_usm = get_usm_ndarray(x)
+        if dtype is not None:
+            x_usm = dpt.astype(x_usm, dtype, copy=False)
+        out = _unpack_out(out)
+        out_usm = None if out is None else get_usm_ndarray(out)
+        res = self._fn(x_usm, out=out_usm, order=order)
+        if out is not None and isinstance(out, dpnp_array):
+            return out
+        return _wrap(res)
+
+
+class DPNPBinaryFunc:
+    """NumPy-style binary ufunc over a tensor-level elementwise function."""
+
+    def __init__(self, name, tensor_fn):
+        self.name_ = self.__name__ = name
+        self._fn = tensor_fn
+        self.__doc__ = tensor_fn.__doc__
+        self.nin, self.nout = 2, 1
+
+    @property
+    def types(self):
+        return self._fn.types
+
+    def __call__(self, x1, x2, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+        check_supported_arrays_type(x1, x2, scalar_type=True, all_scalars=False)
+        _check_ufunc_kwargs(self.name_, where, subok, dtype, out, kwargs)
+        u1, u2 = get_usm_ndarray_or_scalar(x1), get_usm_ndarray_or_scalar(x2)
+        u1 = u1.item() if isinstance(u1, np.generic) else u1
+        u2 = u2.item() if isinstance(u2, np.generic) else u2
+        out = _unpack_out(out)
+        out_usm = None if out is None else get_usm_ndarray(out)
+        if isinstance(x1, dpnp_array) and x1 is out and order == "K" and dtype is None:
+            self._fn._inplace_op(u1, u2)
+            return x1
+        order = _norm_order(order)
+        if dtype is not None:
+            u1 = dpt.asarray(u1, dtype=dtype) if np.isscalar(u1) else dpt.astype(u1, dtype, copy=False)
+            u2 = dpt.asarray(u2, dtype=dtype) if np.isscalar(u2) else dpt.astype(u2, dtype, copy=False)
+        res = self._fn(u1, u2, out=out_usm, order=order)
+        if out is not None and isinstance(out, dpnp_array):
+            return out
+        return _wrap(res)
+
+
+_UNARY = {
+    "abs": ef.abs, "absolute": ef.abs, "negative": ef.negative, "positive": ef.positive,
+    "square": ef.square, "sqrt": ef.sqrt, "exp": ef.exp, "log": ef.log, "erf": ef.erf, "sin": ef.sin,
+    "cos": ef.cos, "tan": ef.tan, "tanh": ef.tanh, "exp2": ef.exp2, "expm1": ef.expm1, "log2": ef.log2,
+    "log10": ef.log10, "log1p": ef.log1p, "rsqrt": ef.rsqrt, "cbrt": ef.cbrt, "reciprocal": ef.reciprocal,
+    "floor": ef.floor, "ceil": ef.ceil, "trunc": ef.trunc, "sign": ef.sign, "isnan": ef.isnan,
+    "isinf": ef.isinf, "isfinite": ef.isfinite, "logical_not": ef.logical_not, "invert": ef.bitwise_invert,
+    "bitwise_not": ef.bitwise_invert, "bitwise_invert": ef.bitwise_invert, "signbit": ef.signbit,
+}
+_BINARY = {
+    "add": ef.add, "subtract": ef.subtract, "multiply": ef.multiply, "divide": ef.divide,
+    "true_divide": ef.divide, "bitwise_and": ef.bitwise_and, "bitwise_or": ef.bitwise_or,
+    "bitwise_xor": ef.bitwise_xor, "equal": ef.equal, "not_equal": ef.not_equal, "less": ef.less,
+    "less_equal": ef.less_equal, "greater": ef.greater, "greater_equal": ef.greater_equal,
+    "maximum": ef.maximum, "minimum": ef.minimum, "logical_and": ef.logical_and,
+    "logical_or": ef.logical_or, "logical_xor": ef.logical_xor, "power": ef.pow, "pow": ef.pow,
+    "floor_divide": ef.floor_divide, "remainder": ef.remainder, "mod": ef.remainder,
+    "arctan2": ef.atan2, "atan2": ef.atan2, "hypot": ef.hypot, "copysign": ef.copysign,
+    "left_shift": ef.bitwise_left_shift, "bitwise_left_shift": ef.bitwise_left_shift,
+    "right_shift": ef.bitwise_right_shift, "bitwise_right_shift": ef.bitwise_right_shift,
+}
+for _n, _f in _UNARY.items():
+    globals()[_n] = DPNPUnaryFunc(_n, _f)
+for _n, _f in _BINARY.items():
+    globals()[_n] = DPNPBinaryFunc(_n, _f)
+
+
+def where(condition, x=None, y=None, /, *, order="K", out=None):
+    """Elements of `x` where `condition` holds, else of `y`."""
+    missing = (x is None, y is None).count(True)
+    if missing == 1:
+        raise ValueError("Must provide both 'x' and 'y' or neither.")
+    if missing == 2:
+        raise NotImplementedError("where(condition) without x and y (nonzero) is outside this library's scope")
+    ux, uy = get_usm_ndarray_or_scalar(x), get_usm_ndarray_or_scalar(y)
+    ux = ux.item() if isinstance(ux, np.generic) else ux
+    uy = uy.item() if isinstance(uy, np.generic) else uy
+    out_usm = None if out is None else get_usm_ndarray(out)
+    res = dpt.where(get_usm_ndarray(condition), ux, uy, order=order, out=out_usm)
+    return get_result_array(res, out)
+
+
+# -- reductions ---------------------------------------------------------------------------------------------
+def _wrap_reduction_call(usm_a, out, fn, res_dt, **kwargs):
+    """Run a tensor-level reduction; an `out` of another dtype gets an unsafe cast of the result."""
+    usm_out = None
+    if out is not None:
+        check_supported_arrays_type(out)
+        usm_out = get_usm_ndarray(out)
+        if usm_out.dtype != res_dt:
+            usm_out = None  # compute into a fresh array of the kernel's dtype, cast into `out` below
+    res = fn(usm_a, out=usm_out, **kwargs)
+    return get_result_array(res, out, casting="unsafe")
+
+
+def _reduction_res_dt(a, dtype):
+    return _default_accumulation_dtype(a.dtype) if dtype is None else dpt.dtype(dtype)
+
+
+def sum(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    check_limitations(initial=initial, where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.sum, _reduction_res_dt(u, dtype), axis=axis, dtype=dtype,
+                                keepdims=keepdims)
+
+
+def prod(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where=True):
+    check_limitations(initial=initial, where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.prod, _reduction_res_dt(u, dtype), axis=axis, dtype=dtype,
+                                keepdims=keepdims)
+
+
+def max(a, axis=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    check_limitations(initial=initial, where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.max, u.dtype, axis=axis, keepdims=keepdims)
+
+
+def min(a, axis=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    check_limitations(initial=initial, where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.min, u.dtype, axis=axis, keepdims=keepdims)
+
+
+amax, amin = max, min
+
+
+def _search_res_dt(out):
+    res_dt = dpt.dtype(ti.default_device_index_type())
+    if out is not None and not np.can_cast(out.dtype, res_dt, casting="safe"):
+        raise TypeError(f"Cannot cast from {out.dtype} to {res_dt} according to the rule safe.")
+    return res_dt
+
+
+def argmax(a, axis=None, out=None, *, keepdims=False):
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.argmax, _search_res_dt(out), axis=axis, keepdims=keepdims)
+
+
+def argmin(a, axis=None, out=None, *, keepdims=False):
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.argmin, _search_res_dt(out), axis=axis, keepdims=keepdims)
+
+
+def _wider_float(u, dtype):
+    """dtype to accumulate in when the caller asks for a wider floating result than the
+    input's: the statistics then run in that type end to end.  (The reference computes in
+    the input's type and casts the result, dpnp/dpnp_iface_statistics.py:1203-1205; this is
+    never less accurate.)"""
+    if dtype is None:
+        return None
+    d = dpt.dtype(dtype)
+    if u.dtype.kind == "f" and d.kind == "f" and d.itemsize > u.dtype.itemsize:
+        return d
+    return None
+
+
+def mean(a, /, axis=None, dtype=None, out=None, keepdims=False, *, where=True):
+    check_limitations(where=where)
+    u = get_usm_ndarray(a)
+    res = dpt.mean(u, axis=axis, keepdims=keepdims, dtype=_wider_float(u, dtype))
+    if dtype is not None:
+        res = dpt.astype(res, dtype, copy=False)
+    return get_result_array(res, out, casting="unsafe")
+
+
+def var(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
+        correction=None):
+    check_limitations(where=where)
+    if mean is not None:
+        raise NotImplementedError("var(..., mean=) is outside this library's scope")
+    if correction is not None:
+        if ddof != 0:
+            raise ValueError("ddof and correction can't be provided simultaneously.")
+        ddof = correction
+    if not isinstance(ddof, (int, float)):
+        raise TypeError(f"An integer or float is required, but got {type(ddof)}")
+    u = get_usm_ndarray(a)
+    res = dpt.var(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
+    result = get_result_array(res, out)
+    if out is None and dtype is not None:
+        result = result.astype(dtype, casting="same_kind")
+    return result
+
+
+def std(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
+        correction=None):
+    check_limitations(where=where)
+    if mean is not None:
+        raise NotImplementedError("std(..., mean=) is outside this library's scope")
+    if correction is not None:
+        if ddof != 0:
+            raise ValueError("ddof and correction can't be provided simultaneously.")
+        ddof = correction
+    if not isinstance(ddof, (int, float)):
+        raise TypeError(f"An integer or float is required, but got {type(ddof)}")
+    u = get_usm_ndarray(a)
+    res = dpt.std(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
+    result = get_result_array(res, out)
+    if out is None and dtype is not None:
+        result = result.astype(dtype, casting="same_kind")
+    return result
+
+
+# -- fused chains (extensions: one kernel where the reference runs a sequence) ---------------------------------
+def where_compare(cmp_name, lhs, rhs, x, y, out=None):
+    """`where(lhs CMP rhs, x, y)` in one pass; cmp_name in equal/not_equal/less/less_equal/
+    greater/greater_equal.  All four operands must share a shape after broadcasting; lhs/rhs
+    share a dtype and x/y share a dtype (scalars adopt the array operand's dtype)."""
+    arrs = [o for o in (lhs, rhs, x, y) if is_supported_array_type(o)]
+    if not arrs:
+        raise TypeError("at least one operand must be an array")
+    from .tensor._manipulation_functions import _broadcast_shape_impl
+
+    shape = _broadcast_shape_impl([get_usm_ndarray(o).shape if is_supported_array_type(o) else ()
+                                   for o in (lhs, rhs, x, y)])
+
+    def pair(a, b):
+        ua = get_usm_ndarray(a) if is_supported_array_type(a) else None
+        ub = get_usm_ndarray(b) if is_supported_array_type(b) else None
+        if ua is None and ub is None:
+            raise TypeError("each of (lhs, rhs) and (x, y) needs an array operand")
+        dt = (ua if ua is not None else ub).dtype
+        ua = dpt.full((), a, dtype=dt) if ua is None else ua
+        ub = dpt.full((), b, dtype=dt) if ub is None else ub
+        if ua.dtype != ub.dtype:
+            raise ValueError("operands of a pair must have one dtype")
+        return dpt.broadcast_to(ua, shape), dpt.broadcast_to(ub, shape)
+
+    ul, ur = pair(lhs, rhs)
+    ux, uy = pair(x, y)
+    res = dpt.empty(shape, dtype=ux.dtype) if out is None else get_usm_ndarray(out)
+    ti._where_compare(cmp_name, ul, ur, ux, uy, res)
+    return out if out is not None else _wrap(res)
+
+
+def black_scholes(price, strike, t, rate, vol, call=None, put=None):
+    """Call and put prices of European options (one fused kernel); returns (call, put)."""
+    up, us, ut = get_usm_ndarray(price), get_usm_ndarray(strike), get_usm_ndarray(t)
+    uc = dpt.empty_like(up) if call is None else get_usm_ndarray(call)
+    uq = dpt.empty_like(up) if put is None else get_usm_ndarray(put)
+    tei._black_scholes(up, us, ut, rate, vol, uc, uq)
+    return (call if call is not None else _wrap(uc)), (put if put is not None else _wrap(uq))
+
+
+def synchronize():
+    """Wait for all work queued by this library (and torch) on the current stream."""
+    dpt._device.default_queue().wait()
+
+
+__all__ = [n for n in list(globals()) if not n.startswith("_") and n not in (
+    "np", "dpt", "ef", "tei", "ti", "usm_ndarray", "dpnp_array")]

@@ -1,0 +1,127 @@
+"""Device memory and the execution stream.
+
+PyTorch is used as plumbing only: its caching allocator hands out device memory
+(a uint8 CUDA tensor per allocation) and its current stream is the hipStream_t
+every kernel of the library is enqueued on.  The allocator is stream-ordered, so
+a temporary released right after a launch is not reused before that launch ran.
+"""
+import numpy as np
+
+
+def _torch():
+    import torch
+
+    return torch
+
+
+class ExecutionPlacementError(Exception):
+    """Raised when arrays of one call live on different devices."""
+
+
+class Device:
+    """Stand-in for dpctl.SyclDevice: the one GPU this process uses."""
+
+    has_aspect_fp16 = True
+    has_aspect_fp64 = True
+    has_aspect_gpu = True
+
+    def __init__(self, index=0):
+        self.index = index
+
+    @property
+    def name(self):
+        t = _torch()
+        return t.cuda.get_device_name(self.index) if t.cuda.is_available() else "AMD GPU (not present)"
+
+    def __eq__(self, other):
+        return isinstance(other, Device) and other.index == self.index
+
+    def __hash__(self):
+        return hash(("dpnp_amd.Device", self.index))
+
+    def __repr__(self):
+        return f"<Device hip:{self.index}>"
+
+
+class Queue:
+    """Stand-in for dpctl.SyclQueue: an in-order HIP stream on one device.
+
+    The queue always denotes the stream that is current in PyTorch at call
+    time, so work submitted by this library interleaves correctly with torch
+    work of the same process.
+    """
+
+    def __init__(self, device=None):
+        self.sycl_device = device if isinstance(device, Device) else Device(0)
+
+    @property
+    def stream_ptr(self):
+        return _torch().cuda.current_stream(self.sycl_device.index).cuda_stream
+
+    def wait(self):
+        _torch().cuda.current_stream(self.sycl_device.index).synchronize()
+
+    def __eq__(self, other):
+        return isinstance(other, Queue) and other.sycl_device == self.sycl_device
+
+    def __hash__(self):
+        return hash(("dpnp_amd.Queue", self.sycl_device.index))
+
+    def __repr__(self):
+        return f"<Queue on {self.sycl_device!r}>"
+
+
+_DEFAULT_QUEUE = Queue()
+
+
+def default_queue():
+    return _DEFAULT_QUEUE
+
+
+def get_execution_queue(queues):
+    """The common queue of `queues`, or None when they differ (compute follows data)."""
+    qs = [q for q in queues if q is not None]
+    if not qs:
+        return None
+    first = qs[0]
+    return first if all(q == first for q in qs[1:]) else None
+
+
+class Event:
+    """Completion handle returned by the kernel entry points (in place of sycl::event)."""
+
+    def __init__(self, queue=None):
+        self._queue = queue or _DEFAULT_QUEUE
+
+    def wait(self):
+        self._queue.wait()
+
+
+def gpu_available():
+    t = _torch()
+    return t.cuda.is_available()
+
+
+def alloc(nbytes):
+    """A device allocation of at least `nbytes` bytes (a uint8 CUDA tensor)."""
+    t = _torch()
+    if not t.cuda.is_available():
+        raise RuntimeError("dpnp_amd needs an AMD GPU: no HIP device is visible to this process")
+    return t.empty(max(int(nbytes), 1), dtype=t.uint8, device="cuda")
+
+
+def to_device_bytes(host_bytes_array):
+    """Copy a contiguous NumPy uint8 array to a new device allocation."""
+    t = _torch()
+    if not t.cuda.is_available():
+        raise RuntimeError("dpnp_amd needs an AMD GPU: no HIP device is visible to this process")
+    if host_bytes_array.size == 0:
+        return alloc(0)
+    return t.from_numpy(host_bytes_array).to("cuda")
+
+
+def to_host_bytes(buf, byte_offset, nbytes):
+    """Copy `nbytes` bytes starting at `byte_offset` of allocation `buf` to a NumPy uint8 array."""
+    if nbytes == 0:
+        return np.empty(0, dtype=np.uint8)
+    return buf[byte_offset:byte_offset + nbytes].cpu().numpy()

@@ -1,0 +1,183 @@
+"""View-making helpers the hot path relies on: broadcast_to, permute_dims, reshape,
+squeeze, expand_dims (behaviour of dpnp/tensor/_manipulation_functions.py and
+dpnp/tensor/_reshape.py for these five)."""
+import operator
+
+from ._usmarray import usm_ndarray
+
+
+def normalize_axis_index(axis, ndim, name="axis"):
+    axis = operator.index(axis)
+    if axis < -ndim or axis >= ndim:
+        raise IndexError(f"{name} {axis} is out of bounds for array of dimension {ndim}")
+    return axis + ndim if axis < 0 else axis
+
+
+def normalize_axis_tuple(axis, ndim, argname="axis", allow_duplicate=False):
+    if not isinstance(axis, (tuple, list)):
+        axis = (axis,)
+    axes = tuple(normalize_axis_index(a, ndim, argname) for a in axis)
+    if not allow_duplicate and len(set(axes)) != len(axes):
+        raise ValueError(f"repeated axis in `{argname}` argument")
+    return axes
+
+
+def _broadcast_shape_impl(shapes):
+    nd = max((len(s) for s in shapes), default=0)
+    out = [1] * nd
+    for s in shapes:
+        for i, ext in enumerate(reversed(s)):
+            j = nd - 1 - i
+            if ext == 1 or ext == out[j]:
+                continue
+            if out[j] == 1:
+                out[j] = ext
+            else:
+                raise ValueError("shape mismatch: objects cannot be broadcast to a single shape")
+    return tuple(out)
+
+
+def broadcast_to(x, shape):
+    """A read-only-safe view of `x` with `shape`: new and stretched dims get stride 0."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    shape = tuple(shape) if isinstance(shape, (tuple, list)) else (shape,)
+    nd = len(shape)
+    if nd < x.ndim:
+        raise ValueError(f"array of shape {x.shape} cannot be broadcast to shape {shape}")
+    strides = [0] * nd
+    for i in range(x.ndim):
+        j = nd - x.ndim + i
+        if x.shape[i] == shape[j]:
+            strides[j] = x.strides[i] if shape[j] != 1 else 0
+        elif x.shape[i] == 1:
+            strides[j] = 0
+        else:
+            raise ValueError(f"array of shape {x.shape} cannot be broadcast to shape {shape}")
+    return x._view(shape, strides, x._offset)
+
+
+def permute_dims(x, axes):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    axes = normalize_axis_tuple(axes, x.ndim, "axes")
+    if sorted(axes) != list(range(x.ndim)):
+        raise ValueError("The length of the passed axes does not match to the number of usm_ndarray dimensions.")
+    return x._view([x.shape[a] for a in axes], [x.strides[a] for a in axes], x._offset)
+
+
+def expand_dims(x, axis):
+    axes = normalize_axis_tuple(axis, x.ndim + (len(axis) if isinstance(axis, (tuple, list)) else 1))
+    nd = x.ndim + len(axes)
+    sh, st = [], []
+    it_sh, it_st = iter(x.shape), iter(x.strides)
+    for d in range(nd):
+        if d in axes:
+            sh.append(1)
+            st.append(0)
+        else:
+            sh.append(next(it_sh))
+            st.append(next(it_st))
+    return x._view(sh, st, x._offset)
+
+
+def squeeze(x, axis=None):
+    if axis is None:
+        keep = [d for d in range(x.ndim) if x.shape[d] != 1]
+    else:
+        axes = normalize_axis_tuple(axis, x.ndim)
+        for a in axes:
+            if x.shape[a] != 1:
+                raise ValueError("Cannot select an axis to squeeze out which has size not equal to one.")
+        keep = [d for d in range(x.ndim) if d not in axes]
+    return x._view([x.shape[d] for d in keep], [x.strides[d] for d in keep], x._offset)
+
+
+def _reshape_strides(shape, strides, new_shape):
+    """Strides of a no-copy reshape, or None when the layout needs a copy (NumPy's rule)."""
+    old = [(s, st) for s, st in zip(shape, strides) if s != 1]
+    new_strides = [0] * len(new_shape)
+    oi = 0
+    ni = 0
+    nn = len(new_shape)
+    while ni < nn:
+        if new_shape[ni] == 1:
+            new_strides[ni] = 0
+            ni += 1
+            continue
+        if oi >= len(old):
+            return None
+        # grow groups on both sides until the element counts agree
+        np_, op_ = new_shape[ni], old[oi][0]
+        nj, oj = ni + 1, oi + 1
+        while np_ != op_:
+            if np_ < op_:
+                if nj >= nn:
+                    return None
+                np_ *= new_shape[nj]
+                nj += 1
+            else:
+                if oj >= len(old):
+                    return None
+                op_ *= old[oj][0]
+                oj += 1
+        # the old group must be internally contiguous (in units of its last stride)
+        for k in range(oi, oj - 1):
+            if old[k][1] != old[k + 1][0] * old[k + 1][1]:
+                return None
+        st = old[oj - 1][1]
+        for k in range(nj - 1, ni - 1, -1):
+            new_strides[k] = st
+            st *= new_shape[k]
+        ni, oi = nj, oj
+    return new_strides
+
+
+def reshape(x, shape, /, *, order="C", copy=None):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    if order not in ("C", "c"):
+        raise ValueError("only order='C' reshapes are supported")
+    shape = [operator.index(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,))]
+    if shape.count(-1) > 1:
+        raise ValueError("Only one dimension of the new shape may be -1")
+    if -1 in shape:
+        known = 1
+        for s in shape:
+            if s != -1:
+                known *= s
+        if known == 0 or x.size % known != 0:
+            raise ValueError(f"Can not reshape array of size {x.size} into {tuple(shape)}")
+        shape[shape.index(-1)] = x.size // known
+    n = 1
+    for s in shape:
+        n *= s
+    if n != x.size:
+        raise ValueError(f"Can not reshape array of size {x.size} into {tuple(shape)}")
+    if x.size == 0:
+        from ._usmarray import _contig_strides
+
+        return x._view(shape, _contig_strides(shape), x._offset) if not copy else _copy_reshape(x, shape)
+    st = _reshape_strides(x.shape, x.strides, shape)
+    if st is not None and not copy:
+        return x._view(shape, st, x._offset)
+    if copy is False:
+        raise ValueError("Reshaping the array requires a copy, but no copying was requested by using copy=False")
+    return _copy_reshape(x, shape)
+
+
+def _copy_reshape(x, shape):
+    from ._copy_utils import copy as _copy
+    from ._usmarray import _contig_strides
+
+    c = _copy(x, order="C")
+    return c._view(shape, _contig_strides(shape), c._offset)
+
+
+def flip(x, /, *, axis=None):
+    """View of `x` with the elements along `axis` (all axes when None) reversed."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    axes = range(x.ndim) if axis is None else normalize_axis_tuple(axis, x.ndim)
+    key = tuple(slice(None, None, -1) if d in axes else slice(None) for d in range(x.ndim))
+    return x[key]

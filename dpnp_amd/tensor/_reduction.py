@@ -1,0 +1,205 @@
+"""sum, prod, max, min, argmax, argmin over axes.
+
+Host logic of dpnp/tensor/_reduction.py:43-138,141-296,299-395 restated around one
+skeleton: move the reduced axes last (a view), allocate or validate `out`, run the
+kernel on (array, number of trailing axes, destination), undo the permutation for
+keepdims.  Result dtypes: sum/prod use the default accumulation dtype unless `dtype`
+is given; max/min keep the dtype; argmax/argmin give int64.
+"""
+import builtins
+
+from . import _tensor_impl as ti
+from . import _tensor_reductions_impl as tri
+from ._ctors import empty, empty_like
+from ._dtypes import dtype as _as_dtype
+from ._manipulation_functions import normalize_axis_tuple, permute_dims, reshape, squeeze
+from ._type_utils import _default_accumulation_dtype
+from ._usmarray import usm_ndarray
+
+
+def _move_reduced_axes_last(x, axis, int_only=False):
+    nd = x.ndim
+    if axis is None:
+        return x, tuple(range(nd)), list(range(nd))
+    if int_only:
+        if not isinstance(axis, int):
+            raise TypeError("'axis' argument expected to have type 'int' or be `None`, "
+                            f"got type {type(axis)}")
+        axis = (axis,)
+    axis = normalize_axis_tuple(axis, nd, "axis")
+    perm = [i for i in range(nd) if i not in axis] + list(axis)
+    return permute_dims(x, perm), axis, perm
+
+
+def _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap):
+    """Validate a user `out`; returns (array the kernel writes, array the user gets back)."""
+    if out is None:
+        r = empty(res_shape, dtype=res_dt)
+        return r, r
+    if not isinstance(out, usm_ndarray):
+        raise TypeError(f"output array must be of usm_ndarray type, got {type(out)}")
+    if not out.flags.writable:
+        raise ValueError("provided `out` array is read-only")
+    final_shape = res_shape if not keepdims else tuple(
+        x.shape[i] if i not in axis else 1 for i in range(x.ndim))
+    if out.shape != final_shape:
+        raise ValueError("The shape of input and output arrays are inconsistent. "
+                         f"Expected output shape is {final_shape}, got {out.shape}")
+    if res_dt != out.dtype:
+        raise ValueError(f"Output array of type {res_dt} is needed, got {out.dtype}")
+    if keepdims:
+        out = squeeze(out, axis=axis)
+    user = out
+    if guard_overlap and ti._array_overlap(x, out):
+        out = empty_like(out)
+    return out, user
+
+
+def _finish(out, user, keepdims, res_shape, red_nd, perm, nd):
+    if user is not out:
+        ti._copy_usm_ndarray_into_usm_ndarray(src=out, dst=user)
+        out = user
+    if keepdims:
+        inv = sorted(range(nd), key=lambda d: perm[d])
+        out = permute_dims(reshape(out, res_shape + (1,) * red_nd), inv)
+    return out
+
+
+def _reduction_over_axis(x, axis, dtype, keepdims, out, _reduction_fn, _dtype_supported,
+                         _default_reduction_type_fn):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    nd = x.ndim
+    arr, axis, perm = _move_reduced_axes_last(x, axis)
+    red_nd = len(axis)
+    res_shape = arr.shape[: nd - red_nd]
+    inp_dt = x.dtype
+    res_dt = _default_reduction_type_fn(inp_dt, None) if dtype is None else _as_dtype(dtype)
+    direct = _dtype_supported(inp_dt, res_dt, "device", None)
+    if dtype is None and not direct:
+        raise RuntimeError("Automatically determined reduction data type does not have direct implementation")
+    out, user = _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap=direct)
+    if red_nd == 0:
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=out)
+        return _finish(out, user, False, res_shape, red_nd, perm, nd)
+    if direct:
+        _reduction_fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)
+    elif _dtype_supported(res_dt, res_dt, "device", None):
+        # no (input, result) kernel: cast the input to the result type first
+        tmp = empty(arr.shape, dtype=res_dt)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=tmp)
+        _reduction_fn(src=tmp, trailing_dims_to_reduce=red_nd, dst=out)
+    else:
+        # reduce in the default type of the input, cast the (small) result
+        buf_dt = _default_reduction_type_fn(inp_dt, None)
+        tmp = empty(arr.shape, dtype=buf_dt)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=tmp)
+        tmp_res = empty(res_shape, dtype=buf_dt)
+        _reduction_fn(src=tmp, trailing_dims_to_reduce=red_nd, dst=tmp_res)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=tmp_res, dst=out)
+    return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
+
+
+def _comparison_over_axis(x, axis, keepdims, out, _reduction_fn):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    nd = x.ndim
+    arr, axis, perm = _move_reduced_axes_last(x, axis)
+    red_nd = len(axis)
+    if builtins.any(arr.shape[i] == 0 for i in range(nd - red_nd, nd)):
+        raise ValueError("reduction cannot be performed over zero-size axes")
+    res_shape = arr.shape[: nd - red_nd]
+    out, user = _prepare_out(x, out, axis, keepdims, res_shape, x.dtype, guard_overlap=True)
+    if red_nd == 0:
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=out)
+        return _finish(out, user, False, res_shape, red_nd, perm, nd)
+    _reduction_fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)
+    return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
+
+
+def _search_over_axis(x, axis, keepdims, out, _reduction_fn):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    nd = x.ndim
+    arr, axis, perm = _move_reduced_axes_last(x, axis, int_only=True)
+    red_nd = len(axis)
+    if builtins.any(arr.shape[i] == 0 for i in range(nd - red_nd, nd)):
+        raise ValueError("reduction cannot be performed over zero-size axes")
+    res_shape = arr.shape[: nd - red_nd]
+    res_dt = _as_dtype(ti.default_device_index_type())
+    out, user = _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap=red_nd > 0)
+    if red_nd == 0:
+        ti._full_usm_ndarray(fill_value=0, dst=out)
+        return out
+    _reduction_fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)
+    return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
+
+
+def sum(x, /, *, axis=None, dtype=None, keepdims=False, out=None):  # noqa: A001
+    """Sum of the elements of `x` over `axis` (all axes when None)."""
+    return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._sum_over_axis,
+                                tri._sum_over_axis_dtype_supported, _default_accumulation_dtype)
+
+
+def prod(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
+    """Product of the elements of `x` over `axis`."""
+    return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._prod_over_axis,
+                                tri._prod_over_axis_dtype_supported, _default_accumulation_dtype)
+
+
+def max(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
+    """Maximum over `axis`; NaN propagates."""
+    return _comparison_over_axis(x, axis, keepdims, out, tri._max_over_axis)
+
+
+def min(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
+    """Minimum over `axis`; NaN propagates."""
+    return _comparison_over_axis(x, axis, keepdims, out, tri._min_over_axis)
+
+
+def argmax(x, /, *, axis=None, keepdims=False, out=None):
+    """Index of the maximum along `axis` (flat C-order index when None); first occurrence,
+    NaN counts as the maximum."""
+    return _search_over_axis(x, axis, keepdims, out, tri._argmax_over_axis)
+
+
+def argmin(x, /, *, axis=None, keepdims=False, out=None):
+    """Index of the minimum along `axis`; first occurrence, NaN counts as the minimum."""
+    return _search_over_axis(x, axis, keepdims, out, tri._argmin_over_axis)
+
+
+def _boolean_reduction(x, axis, keepdims, out, fn):
+    """all/any through max/min of the truth values (bool max is logical or, min is and)."""
+    from ._copy_utils import astype
+    from ._dtypes import bool as _bool
+
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    b = astype(x, _bool, copy=False)
+    nd = b.ndim
+    arr, axis, perm = _move_reduced_axes_last(b, axis)
+    red_nd = len(axis)
+    res_shape = arr.shape[: nd - red_nd]
+    n = 1
+    for i in range(nd - red_nd, nd):
+        n *= arr.shape[i]
+    out, user = _prepare_out(b, out, axis, keepdims, res_shape, _bool, guard_overlap=True)
+    if red_nd == 0:
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=out)
+        return _finish(out, user, False, res_shape, red_nd, perm, nd)
+    if n == 0:
+        if out.size:
+            ti._full_usm_ndarray(fn is tri._min_over_axis, out)  # all([]) is True, any([]) is False
+    else:
+        fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)
+    return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
+
+
+def all(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
+    """True where every element along `axis` is non-zero."""
+    return _boolean_reduction(x, axis, keepdims, out, tri._min_over_axis)
+
+
+def any(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
+    """True where some element along `axis` is non-zero."""
+    return _boolean_reduction(x, axis, keepdims, out, tri._max_over_axis)

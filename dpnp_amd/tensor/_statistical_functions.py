@@ -1,0 +1,133 @@
+"""mean, var, std over axes.
+
+Results and dtypes as dpnp/tensor/_statistical_functions.py:38-321 (floating input keeps its
+dtype, integer and bool input gives float64; N - correction <= 0 gives NaN; complex input is
+rejected for var/std).  The variance is computed in two passes over the data (mean, then
+sum of squared deviations in one kernel) instead of the reference's five kernels and a
+full-size temporary; the arithmetic per element is the same (x - mean, squared, summed).
+"""
+import math
+
+from . import _tensor_elementwise_impl as tei
+from . import _tensor_impl as ti
+from . import _tensor_reductions_impl as tri
+from ._copy_utils import astype
+from ._ctors import empty, empty_like
+from ._dtypes import dtype as _as_dtype
+from ._dtypes import float64
+from ._manipulation_functions import normalize_axis_tuple, permute_dims, reshape
+from ._usmarray import usm_ndarray
+
+
+def _split_axes(x, axis):
+    nd = x.ndim
+    if axis is None:
+        axis = tuple(range(nd))
+    if not isinstance(axis, (tuple, list)):
+        axis = (axis,)
+    axis = normalize_axis_tuple(axis, nd, "axis")
+    nelems = 1
+    for a in axis:
+        nelems *= x.shape[a]
+    perm = [i for i in range(nd) if i not in axis] + list(axis)
+    return axis, perm, nelems
+
+
+def _keepdims_view(res, res_shape, red_nd, perm, nd):
+    inv = sorted(range(nd), key=lambda d: perm[d])
+    return permute_dims(reshape(res, tuple(res_shape) + (1,) * red_nd), inv)
+
+
+def _sum_as(arr, red_nd, res_shape, res_dt):
+    """Sum of the trailing axes of `arr` accumulated in res_dt."""
+    res = empty(res_shape, dtype=res_dt)
+    if tri._sum_over_axis_dtype_supported(arr.dtype, res_dt):
+        tri._sum_over_axis(src=arr, trailing_dims_to_reduce=red_nd, dst=res)
+    else:
+        tmp = empty(arr.shape, dtype=res_dt)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=tmp)
+        tri._sum_over_axis(src=tmp, trailing_dims_to_reduce=red_nd, dst=res)
+    return res
+
+
+def mean(x, axis=None, keepdims=False, *, dtype=None):
+    """Arithmetic mean over `axis`.
+
+    `dtype` (an extension used by the NumPy-flavoured front end) asks for accumulation in a
+    wider floating type than the input's, e.g. float64 for a float32 array.
+    """
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    nd = x.ndim
+    axis, perm, nelems = _split_axes(x, axis)
+    red_nd = len(axis)
+    res_dt = x.dtype if x.dtype.kind in "fc" else float64
+    if dtype is not None:
+        res_dt = _as_dtype(dtype)
+    if red_nd == 0:
+        return astype(x, res_dt, copy=True)
+    arr = permute_dims(x, perm)
+    res_shape = arr.shape[: nd - red_nd]
+    res = _sum_as(arr, red_nd, res_shape, res_dt)
+    if keepdims:
+        res = _keepdims_view(res, res_shape, red_nd, perm, nd)
+    if res.size:
+        tei._divide_by_scalar(src=res, scalar=nelems if nelems else math.nan, dst=res)
+    return res
+
+
+def _var_impl(x, axis, correction, keepdims, dtype=None):
+    nd = x.ndim
+    axis, perm, nelems = _split_axes(x, axis)
+    red_nd = len(axis)
+    res_dt = x.dtype if x.dtype.kind == "f" else float64
+    if dtype is not None:
+        res_dt = _as_dtype(dtype)
+    div = max(nelems - correction, 0)
+    div = div if div else math.nan
+    if red_nd == 0:
+        # every element is its own mean: zeros (or NaN when the divisor is not positive)
+        res = empty_like(x, dtype=res_dt)
+        if res.size:
+            ti._full_usm_ndarray(0, res)
+            tei._divide_by_scalar(src=res, scalar=div, dst=res)
+        return res
+    buf = x
+    if not tri._sumsqdev_over_axis_dtype_supported(x.dtype, res_dt):
+        buf = empty_like(x, dtype=res_dt)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=x, dst=buf)
+    arr = permute_dims(buf, perm)
+    res_shape = arr.shape[: nd - red_nd]
+    mean_ary = _sum_as(arr, red_nd, res_shape, res_dt)
+    res = empty(res_shape, dtype=res_dt)
+    if res.size:
+        tei._divide_by_scalar(src=mean_ary, scalar=nelems if nelems else math.nan, dst=mean_ary)
+        tri._sumsqdev_over_axis(src=arr, mean=mean_ary, trailing_dims_to_reduce=red_nd, dst=res)
+        tei._divide_by_scalar(src=res, scalar=div, dst=res)
+    if keepdims:
+        res = _keepdims_view(res, res_shape, red_nd, perm, nd)
+    return res
+
+
+def _check_var_args(x, correction, name):
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    if not isinstance(correction, (int, float)):
+        raise TypeError(f"Expected a Python integer or float for `correction`, got{type(x)}")
+    if x.dtype.kind == "c":
+        raise ValueError(f"`{name}` does not support complex types")
+
+
+def var(x, axis=None, correction=0.0, keepdims=False, *, dtype=None):
+    """Variance over `axis` with divisor N - correction."""
+    _check_var_args(x, correction, "var")
+    return _var_impl(x, axis, correction, keepdims, dtype)
+
+
+def std(x, axis=None, correction=0.0, keepdims=False, *, dtype=None):
+    """Standard deviation over `axis` with divisor N - correction."""
+    _check_var_args(x, correction, "std")
+    res = _var_impl(x, axis, correction, keepdims, dtype)
+    if res.size:
+        tei._sqrt(src=res, dst=res)
+    return res

@@ -1,0 +1,77 @@
+"""Drop-in for the reference's `_tensor_elementwise_impl` extension module
+(libtensor/source/elementwise_functions/elementwise_common.cpp:118-188): for every
+op `X` it exposes `_X(src[, src2], dst, sycl_queue, depends)`, `_X_result_type(dt[, dt2])`
+and, for binary ops, `_X_inplace(lhs, rhs, sycl_queue, depends)`, all backed by the C ABI.
+"""
+from .. import _lib
+from ._device import Event
+from ._dtypes import dtype_from_id, dtype_id
+from ._tensor_impl import _events, _stream
+
+lib = _lib.lib
+
+
+def _make_unary(name, op_id):
+    def fn(src, dst, sycl_queue=None, depends=()):
+        vs, vd = src._as_view(), dst._as_view()
+        _lib.check(lib.dpx_unary(op_id, vs, vd, _stream(sycl_queue)))
+        return _events(sycl_queue)
+
+    def result_type(dt):
+        return dtype_from_id(lib.dpx_unary_result_type(op_id, dtype_id(dt)))
+
+    fn.__name__ = "_" + name
+    result_type.__name__ = f"_{name}_result_type"
+    return fn, result_type
+
+
+def _make_binary(name, op_id):
+    def fn(src1, src2, dst, sycl_queue=None, depends=()):
+        v1, v2, vd = src1._as_view(), src2._as_view(), dst._as_view()
+        _lib.check(lib.dpx_binary(op_id, v1, v2, vd, _stream(sycl_queue)))
+        return _events(sycl_queue)
+
+    def result_type(dt1, dt2):
+        return dtype_from_id(lib.dpx_binary_result_type(op_id, dtype_id(dt1), dtype_id(dt2)))
+
+    def inplace(lhs, rhs, sycl_queue=None, depends=()):
+        vl, vr = lhs._as_view(), rhs._as_view()
+        _lib.check(lib.dpx_binary_inplace(op_id, vl, vr, _stream(sycl_queue)))
+        return _events(sycl_queue)
+
+    fn.__name__ = "_" + name
+    result_type.__name__ = f"_{name}_result_type"
+    inplace.__name__ = f"_{name}_inplace"
+    return fn, result_type, inplace
+
+
+for _n, _i in _lib.UNARY_ID.items():
+    _f, _r = _make_unary(_n, _i)
+    globals()["_" + _n] = _f
+    globals()[f"_{_n}_result_type"] = _r
+for _n, _i in _lib.BINARY_ID.items():
+    _f, _r, _ip = _make_binary(_n, _i)
+    globals()["_" + _n] = _f
+    globals()[f"_{_n}_result_type"] = _r
+    globals()[f"_{_n}_inplace"] = _ip
+
+
+def _divide_by_scalar(src, scalar, dst, sycl_queue=None, depends=()):
+    vs, vd = src._as_view(), dst._as_view()
+    _lib.check(lib.dpx_divide_by_scalar(vs, float(scalar), vd, _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
+def _black_scholes(price, strike, t, rate, vol, call, put, sycl_queue=None, depends=()):
+    """Fused Black-Scholes pricing over 1-D contiguous arrays (no counterpart in the reference)."""
+    arrs = (price, strike, t, call, put)
+    n = price.size
+    dt = price.dtype
+    for a in arrs:
+        if a.ndim != 1 or a.size != n or a.dtype != dt or not a.flags.c_contiguous:
+            raise ValueError("black_scholes expects five 1-D contiguous arrays of one size and dtype")
+    if not (call.flags.writable and put.flags.writable):
+        raise ValueError("output array is read-only.")
+    _lib.check(lib.dpx_black_scholes(price._pointer, strike._pointer, t._pointer, float(rate), float(vol),
+                                     call._pointer, put._pointer, n, dtype_id(dt), _stream(sycl_queue)))
+    return _events(sycl_queue)

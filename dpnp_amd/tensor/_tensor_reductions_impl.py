@@ -1,0 +1,55 @@
+"""Drop-in for the reference's `_tensor_reductions_impl` extension module
+(libtensor/source/reductions/{sum,prod,max,min,argmax,argmin}.cpp): `_X_over_axis(src,
+trailing_dims_to_reduce, dst, sycl_queue, depends)` and `_X_over_axis_dtype_supported`.
+"""
+from .. import _lib
+from ._dtypes import dtype_id
+from ._tensor_impl import _events, _stream
+
+lib = _lib.lib
+
+
+def _make_reduction(name, op_id):
+    def fn(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
+        vs, vd = src._as_view(), dst._as_view()
+        _lib.check(lib.dpx_reduce(op_id, vs, int(trailing_dims_to_reduce), vd, None, _stream(sycl_queue)))
+        return _events(sycl_queue)
+
+    def supported(arg_dtype, out_dtype, dst_usm_type=None, sycl_queue=None):
+        return bool(lib.dpx_reduce_dtype_supported(op_id, dtype_id(arg_dtype), dtype_id(out_dtype)))
+
+    fn.__name__ = f"_{name}_over_axis"
+    return fn, supported
+
+
+def _make_search(name, op_id):
+    def fn(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
+        vs, vd = src._as_view(), dst._as_view()
+        _lib.check(lib.dpx_argreduce(op_id, vs, int(trailing_dims_to_reduce), vd, _stream(sycl_queue)))
+        return _events(sycl_queue)
+
+    fn.__name__ = f"_{name}_over_axis"
+    return fn
+
+
+_sum_over_axis, _sum_over_axis_dtype_supported = _make_reduction("sum", _lib.REDUCE_ID["sum"])
+_prod_over_axis, _prod_over_axis_dtype_supported = _make_reduction("prod", _lib.REDUCE_ID["prod"])
+_max_over_axis, _max_over_axis_dtype_supported = _make_reduction("max", _lib.REDUCE_ID["max"])
+_min_over_axis, _min_over_axis_dtype_supported = _make_reduction("min", _lib.REDUCE_ID["min"])
+_argmax_over_axis = _make_search("argmax", _lib.SEARCH_ID["argmax"])
+_argmin_over_axis = _make_search("argmin", _lib.SEARCH_ID["argmin"])
+
+
+def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
+    """dst[i] = sum_j (src[i, j] - mean[i])**2: the second pass of var in one kernel
+    (the reference runs subtract, square and sum kernels over a full-size temporary,
+    dpnp/tensor/_statistical_functions.py:38-163)."""
+    vs, vm, vd = src._as_view(), mean._as_view(), dst._as_view()
+    _lib.check(lib.dpx_reduce(_lib.REDUCE_ID["sumsqdev"], vs, int(trailing_dims_to_reduce), vd, vm,
+                              _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
+def _sumsqdev_over_axis_dtype_supported(arg_dtype, out_dtype, dst_usm_type=None, sycl_queue=None):
+    return bool(lib.dpx_reduce_dtype_supported(_lib.REDUCE_ID["sumsqdev"], dtype_id(arg_dtype),
+                                               dtype_id(out_dtype)))

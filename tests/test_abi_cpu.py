@@ -1,0 +1,234 @@
+"""The C-ABI library without a GPU: it loads, exports what the header declares, answers the
+dtype queries, collapses strides, plans launches and rejects bad calls before launching."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import dpnp_amd._lib as L
+from oracle import oracle as orc
+from tests.test_oracle import random_view_strides
+
+lib = L.lib
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+NP = [np.dtype(c) for c in ("?", "i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8", "f2", "f4", "f8", "c8", "c16")]
+FAKE = 0x7F0000000000  # never dereferenced: plans and failed validations do not touch memory
+P0, P1, P2 = FAKE, FAKE + (1 << 36), FAKE + (2 << 36)  # three disjoint "allocations"
+
+
+def view(shape, strides=None, dt=L.FLOAT, ptr=FAKE, writable=True):
+    shape = list(shape)
+    if strides is None:
+        strides, acc = [0] * len(shape), 1
+        for d in range(len(shape) - 1, -1, -1):
+            strides[d] = acc
+            acc *= max(shape[d], 1)
+    return L.make_view(ptr, shape, list(strides), dt, L.WRITABLE if writable else 0)
+
+
+def test_header_symbols_are_exported():
+    text = open(os.path.join(ROOT, "include", "dpnp_amd.h")).read()
+    declared = set(re.findall(r"\b(dpx_[a-z0-9_]+)\s*\(", text))
+    assert declared, "no declarations found"
+    assert declared == set(L.SIGNATURES), declared ^ set(L.SIGNATURES)
+    for name in declared:
+        assert hasattr(lib, name)
+    assert lib.dpx_abi_version() == 1
+    assert [lib.dpx_dtype_itemsize(i) for i in range(14)] == [d.itemsize for d in NP]
+
+
+def test_op_tables_match_header_enums():
+    text = open(os.path.join(ROOT, "include", "dpnp_amd.h")).read()
+    for prefix, names in (("DPX_U_", L.UNARY_OPS), ("DPX_B_", L.BINARY_OPS), ("DPX_R_", L.REDUCE_OPS)):
+        body = re.search(r"typedef enum dpx_%s_op \{(.*?)\}" % {"DPX_U_": "unary", "DPX_B_": "binary",
+                                                                "DPX_R_": "reduce"}[prefix], text, re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        ids = [m for m in re.findall(prefix + r"([A-Z0-9_]+)", body) if m != "NUM_OPS"]
+        want = [n.upper().replace("BITWISE_LEFT_SHIFT", "LEFT_SHIFT").replace("BITWISE_RIGHT_SHIFT", "RIGHT_SHIFT")
+                for n in names]
+        assert ids == want
+
+
+def test_binary_result_types():
+    B = L.BINARY_ID
+    for i, d in enumerate(NP):
+        assert lib.dpx_binary_result_type(B["add"], i, i) == i
+        assert lib.dpx_binary_result_type(B["multiply"], i, i) == i
+        assert lib.dpx_binary_result_type(B["subtract"], i, i) == (-1 if d.kind == "b" else i)
+        assert lib.dpx_binary_result_type(B["divide"], i, i) == (i if d.kind in "fc" else -1)
+        assert lib.dpx_binary_result_type(B["bitwise_and"], i, i) == (i if d.kind in "biu" else -1)
+        assert lib.dpx_binary_result_type(B["greater"], i, i) == L.BOOL
+        assert lib.dpx_binary_result_type(B["maximum"], i, i) == i
+    # only same-dtype pairs, except int64/uint64 comparisons
+    assert lib.dpx_binary_result_type(B["add"], L.FLOAT, L.DOUBLE) == -1
+    assert lib.dpx_binary_result_type(B["less"], L.INT64, L.UINT64) == L.BOOL
+    assert lib.dpx_binary_result_type(B["less"], L.UINT64, L.INT64) == L.BOOL
+    assert lib.dpx_binary_result_type(B["less"], L.INT32, L.UINT32) == -1
+    assert lib.dpx_binary_inplace_supported(B["add"], L.FLOAT, L.FLOAT) == 1
+    assert lib.dpx_binary_inplace_supported(B["greater"], L.FLOAT, L.FLOAT) == 0
+
+
+def test_unary_result_types():
+    U = L.UNARY_ID
+    for i, d in enumerate(NP):
+        assert lib.dpx_unary_result_type(U["exp"], i) == (i if d.kind == "f" else -1)
+        assert lib.dpx_unary_result_type(U["sqrt"], i) == (i if d.kind == "f" else -1)
+        assert lib.dpx_unary_result_type(U["isnan"], i) == L.BOOL
+        want_abs = {L.CFLOAT: L.FLOAT, L.CDOUBLE: L.DOUBLE}.get(i, i)
+        assert lib.dpx_unary_result_type(U["abs"], i) == want_abs
+        assert lib.dpx_unary_result_type(U["negative"], i) == (-1 if d.kind == "b" else i)
+        assert lib.dpx_unary_result_type(U["square"], i) == (L.INT8 if d.kind == "b" else i)
+    assert lib.dpx_unary_result_type(U["erf"], L.HALF) == L.FLOAT
+    assert lib.dpx_unary_result_type(U["erf"], L.DOUBLE) == L.DOUBLE
+
+
+def test_reduction_dtype_support():
+    R = L.REDUCE_ID
+    for i, d in enumerate(NP):
+        assert lib.dpx_reduce_dtype_supported(R["sum"], i, i) == 1
+        dflt = orc.default_accumulation_dtype(d)
+        assert lib.dpx_reduce_dtype_supported(R["sum"], i, NP.index(dflt)) == 1
+        assert lib.dpx_reduce_dtype_supported(R["max"], i, i) == 1
+        assert lib.dpx_search_dtype_supported(0, i, L.INT64) == 1
+        assert lib.dpx_search_dtype_supported(0, i, L.INT32) == 0
+    assert lib.dpx_reduce_dtype_supported(R["sum"], L.FLOAT, L.DOUBLE) == 1
+    assert lib.dpx_reduce_dtype_supported(R["sum"], L.DOUBLE, L.FLOAT) == 0
+    assert lib.dpx_reduce_dtype_supported(R["max"], L.FLOAT, L.DOUBLE) == 0
+    assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.FLOAT, L.DOUBLE) == 1
+    assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.INT32, L.DOUBLE) == 0
+
+
+def c_collapse(shape, strides_list, keep_order=False):
+    nd, nops = len(shape), len(strides_list)
+    sh = (ctypes.c_int64 * L.MAX_ND)(*shape)
+    st = (ctypes.c_int64 * (L.MAX_ND * nops))()
+    for k, s in enumerate(strides_list):
+        for d, v in enumerate(s):
+            st[k * L.MAX_ND + d] = v
+    off = (ctypes.c_int64 * nops)()
+    n = lib.dpx_collapse(nd, nops, sh, st, off, 1 if keep_order else 0)
+    return list(sh[:n]), [[st[k * L.MAX_ND + d] for d in range(n)] for k in range(nops)], list(off)
+
+
+def test_collapse_matches_brute_force_and_oracle():
+    rng = np.random.default_rng(3)
+    for _ in range(400):
+        nd = int(rng.integers(1, 6))
+        shape = [int(s) for s in rng.integers(1, 5, nd)]
+        strides = [random_view_strides(rng, shape) for _k in range(int(rng.integers(1, 5)))]
+        for keep in (False, True):
+            sh, st, off = c_collapse(shape, strides, keep)
+            assert orc.address_tuples(sh, st, off) == orc.address_tuples(shape, strides)
+            osh, ost, ooff = orc.collapse(shape, strides, keep)
+            assert len(sh) == len(osh)  # both reach the same number of dims
+
+
+def test_collapse_examples():
+    assert c_collapse([3, 4, 5], [[20, 5, 1], [20, 5, 1]]) == ([60], [[1], [1]], [0, 0])
+    assert c_collapse([3, 4], [[-4, -1]]) == ([12], [[1]], [-11])
+    assert c_collapse([8192, 8192], [[1, 8192], [1, 8192]]) == ([8192 * 8192], [[1], [1]], [0, 0])  # F-contig pair
+    sh, st, _ = c_collapse([8192, 4096], [[8192, 2], [0, 1], [4096, 1]])
+    assert sh == [8192, 4096] and st == [[8192, 2], [0, 1], [4096, 1]]
+    assert c_collapse([3, 4], [[1, 3]], keep_order=True)[0] == [3, 4]
+
+
+def plan_binary(op, a, b, o):
+    p = L.Plan()
+    L.check(lib.dpx_binary_plan(L.BINARY_ID[op], a, b, o, p))
+    return p
+
+
+def test_elementwise_plans():
+    n = 1 << 20
+    p = plan_binary("add", view([n]), view([n], ptr=P1), view([n], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_contig" and p.vec == 4 and p.grid[0] == n // 1024
+    # array (+) scalar: zero-stride operand still takes the contiguous kernel
+    p = plan_binary("add", view([n]), view([n], [0], ptr=P1), view([n], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_contig"
+    # F-contiguous triple collapses to 1-D
+    p = plan_binary("add", view([64, 32], [1, 64]), view([64, 32], [1, 64]), view([64, 32], [1, 64]))
+    assert L.PATH_NAMES[p.path] == "ew_contig" and p.nd == 1
+    # reversed views collapse too
+    p = plan_binary("add", view([100], [-1], ptr=P0 + 396), view([100], [-1], ptr=P1 + 396),
+                    view([100], [-1], ptr=P2 + 396))
+    assert L.PATH_NAMES[p.path] == "ew_contig" and list(p.offsets[:3]) == [-99, -99, -99]
+    # config 4: strided x broadcast row
+    p = plan_binary("multiply", view([8192, 4096], [8192, 2]), view([8192, 4096], [0, 1], ptr=P1),
+                    view([8192, 4096], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.nd == 2 and list(p.shape[:2]) == [8192, 4096]
+    # empty
+    p = plan_binary("add", view([0, 3]), view([0, 3]), view([0, 3]))
+    assert L.PATH_NAMES[p.path] == "noop"
+
+
+def plan_reduce(op, src, trailing, dst):
+    p = L.Plan()
+    L.check(lib.dpx_reduce_plan(L.REDUCE_ID[op], src, trailing, dst, p))
+    return p
+
+
+def test_reduction_plans():
+    p = plan_reduce("sum", view([1 << 28]), 1, view([], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_rows_split" and p.splits > 1 and p.vec == 1 and p.scratch_bytes == 4 * p.splits
+    p = plan_reduce("sum", view([16384, 16384]), 1, view([16384], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_rows" and p.splits == 1 and p.grid[0] == 16384
+    # axis=0 of a C-contiguous matrix: the caller passes the transposed view
+    p = plan_reduce("sum", view([16384, 16384], [1, 16384]), 1, view([16384], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_cols_split" and p.vec == 1
+    p = plan_reduce("sum", view([1 << 20, 4]), 1, view([1 << 20], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_small", "red_rows")
+    # reduce a middle axis of (a, r, c): outputs contiguous along c
+    p = plan_reduce("max", view([8, 64, 1000], [64000, 1, 64]), 1, view([8, 64], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_rows", "red_small", "red_generic", "red_cols", "red_cols_split")
+    p = plan_reduce("sum", view([5, 0]), 1, view([5], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_small" and p.splits == 1  # identity fill
+    pa = L.Plan()
+    L.check(lib.dpx_argreduce_plan(0, view([1 << 28]), 1, view([], dt=L.INT64, ptr=P1), pa))
+    assert L.PATH_NAMES[pa.path] == "red_rows_split"
+
+
+def test_validation_errors_are_raised_before_any_launch():
+    B = L.BINARY_ID["add"]
+    a, o = view([4, 4]), view([4, 4])
+    with pytest.raises(ValueError, match="read-only"):
+        L.check(lib.dpx_binary(B, a, a, view([4, 4], writable=False), None))
+    with pytest.raises(ValueError, match="dimensions"):
+        L.check(lib.dpx_binary(B, a, a, view([16]), None))
+    with pytest.raises(ValueError, match="shapes"):
+        L.check(lib.dpx_binary(B, a, a, view([4, 5]), None))
+    with pytest.raises(ValueError, match="result type"):
+        L.check(lib.dpx_binary(B, a, a, view([4, 4], dt=L.DOUBLE), None))
+    with pytest.raises(ValueError, match="ample"):
+        L.check(lib.dpx_binary(B, a, a, view([4, 4], [0, 1]), None))
+    with pytest.raises(ValueError, match="overlapping"):
+        L.check(lib.dpx_binary(B, a, a, view([4, 4], ptr=FAKE + 4), None))
+    with pytest.raises(ValueError, match="unexpected elemental data type"):
+        L.check(lib.dpx_unary(L.UNARY_ID["exp"], view([4], dt=L.INT32), view([4], dt=L.INT32), None))
+    R = L.REDUCE_ID
+    with pytest.raises(ValueError, match="rank"):
+        L.check(lib.dpx_reduce(R["sum"], view([4, 4]), 1, view([4, 1], ptr=P1), None, None))
+    with pytest.raises(ValueError, match="Trailing"):
+        L.check(lib.dpx_reduce(R["sum"], view([4, 4]), 0, view([4, 4], ptr=P1), None, None))
+    with pytest.raises(ValueError, match="overlapping"):
+        L.check(lib.dpx_reduce(R["sum"], view([4, 4]), 1, view([4]), None, None))
+    with pytest.raises(RuntimeError, match="not supported"):
+        L.check(lib.dpx_reduce(R["sum"], view([4, 4], dt=L.DOUBLE), 1, view([4], dt=L.FLOAT, ptr=FAKE + 4096), None, None))
+    with pytest.raises(ValueError, match="zero-size"):
+        L.check(lib.dpx_reduce(R["max"], view([4, 0]), 1, view([4], ptr=FAKE + 4096), None, None))
+    with pytest.raises(ValueError, match="zero-size"):
+        L.check(lib.dpx_argreduce(0, view([4, 0]), 1, view([4], dt=L.INT64, ptr=FAKE + 4096), None))
+    # zero-size iteration spaces succeed without touching the device
+    L.check(lib.dpx_binary(B, view([0]), view([0]), view([0]), None))
+    L.check(lib.dpx_reduce(R["sum"], view([0, 4]), 1, view([0], ptr=P1), None, None))
+
+
+def test_overlap_predicates():
+    a = view([10], ptr=FAKE)
+    assert lib.dpx_array_overlap(a, view([10], ptr=FAKE + 36)) == 1
+    assert lib.dpx_array_overlap(a, view([10], ptr=FAKE + 40)) == 0
+    assert lib.dpx_array_overlap(view([5], [2], ptr=FAKE), view([5], [2], ptr=FAKE + 4)) == 1  # interleaved: ranges meet
+    assert lib.dpx_same_logical(a, view([10], ptr=FAKE)) == 1
+    assert lib.dpx_same_logical(a, view([10], [2], ptr=FAKE)) == 0
+    assert lib.dpx_same_logical(a, view([10], ptr=FAKE, dt=L.INT32)) == 0

@@ -1,0 +1,332 @@
+"""Elementwise kernels against the oracle, through the Python layer and the C ABI.
+Bar: bit-exact for integer/bool results and IEEE basic ops; <= 4 ULP for transcendentals."""
+import numpy as np
+import pytest
+
+import dpnp_amd.tensor as dpt
+from oracle import oracle as orc
+from tests.helpers import ALL, FLOATS, INTS, assert_same, assert_ulp, dev, dev_view_like, host, random_array, strided_views
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 3, 255, 1023, 1024, 1025, 4099, 70001]
+EXACT_BINARY = ["add", "subtract", "multiply", "divide", "bitwise_and", "bitwise_or", "bitwise_xor", "equal",
+                "not_equal", "less", "less_equal", "greater", "greater_equal", "maximum", "minimum",
+                "logical_and", "logical_or", "logical_xor", "floor_divide", "remainder", "copysign",
+                "bitwise_left_shift", "bitwise_right_shift"]
+ULP_BINARY = ["pow", "atan2", "hypot"]
+EXACT_UNARY = ["abs", "negative", "positive", "square", "sqrt", "floor", "ceil", "trunc", "sign", "isnan",
+               "isinf", "isfinite", "logical_not", "bitwise_invert", "signbit", "reciprocal"]
+ULP_UNARY = ["exp", "log", "erf", "sin", "cos", "tan", "tanh", "exp2", "expm1", "log2", "log10", "log1p", "cbrt",
+             "rsqrt"]
+
+
+def assert_close_complex(got, want, a, b=None):
+    """|got - want| within 8 eps of the magnitude of the operands' product (or of the result)."""
+    assert got.dtype == want.dtype and got.shape == want.shape
+    ok = np.isfinite(want)
+    with np.errstate(all="ignore"):
+        scale = np.maximum(np.abs(a) * np.abs(a if b is None else b), np.abs(np.where(ok, want, 0)))
+    err = np.abs(got[ok] - want[ok])
+    assert (err <= 8 * np.finfo(got.dtype).eps * np.maximum(scale[ok], 1e-30)).all()
+    assert (np.isnan(got[~ok]) == np.isnan(want[~ok])).all()
+
+
+def supported_binary(op, dt):
+    from dpnp_amd.tensor import _tensor_elementwise_impl as tei
+
+    return getattr(tei, f"_{op}_result_type")(dt, dt) is not None
+
+
+def supported_unary(op, dt):
+    from dpnp_amd.tensor import _tensor_elementwise_impl as tei
+
+    return getattr(tei, f"_{op}_result_type")(dt) is not None
+
+
+@pytest.mark.parametrize("d1", ALL, ids=str)
+def test_add_dtype_matrix(d1):
+    # dpnp/tests/tensor/elementwise/test_add.py:49-88
+    for d2 in ALL:
+        a, b = dpt.ones(33, dtype=d1), dpt.ones(33, dtype=d2)
+        r = dpt.add(a, b)
+        want_dt = np.result_type(d1, d2)
+        assert r.dtype == want_dt
+        want = np.ones(33, d1) + np.ones(33, d2)
+        assert_same(host(r), want.astype(want_dt))
+        r2 = dpt.add(a[::-1], b[::-1])
+        assert_same(host(r2), want.astype(want_dt))
+
+
+@pytest.mark.parametrize("op", EXACT_BINARY)
+def test_binary_exact_all_dtypes_and_sizes(op):
+    rng = np.random.default_rng(hash(op) % 2**32)
+    for dt in ALL:
+        if not supported_binary(op, dt):
+            continue
+        for n in SIZES:
+            a, b = random_array(rng, n, dt, -9, 9), random_array(rng, n, dt, -9, 9)
+            if dt.kind == "f":
+                a[rng.integers(0, n)] = np.nan
+                b[rng.integers(0, n)] = np.inf
+                if n > 3:
+                    b[rng.integers(0, n)] = 0.0
+            if "shift" in op:
+                b = np.abs(b).astype(dt) if dt.kind == "i" else b
+            got = host(getattr(dpt, op)(dev(a), dev(b)))
+            want = orc.binary(op, a, b)
+            if op in ("divide", "multiply") and dt.kind == "c":
+                # complex products are sums of two rounded products: the last bit depends on
+                # whether the compiler fuses them, so compare to a few ULP of the magnitude
+                assert_close_complex(got, want, a, b)
+            else:
+                assert_same(got, want)
+
+
+@pytest.mark.parametrize("op", ULP_BINARY)
+def test_binary_ulp(op):
+    rng = np.random.default_rng(7)
+    for dt in FLOATS:
+        a = random_array(rng, 5000, dt, 0.1, 6)
+        b = random_array(rng, 5000, dt, -4, 4)
+        got = host(getattr(dpt, op)(dev(a), dev(b)))
+        wide = np.float64 if dt.itemsize <= 4 else np.longdouble
+        f = {"pow": np.power, "atan2": np.arctan2, "hypot": np.hypot}[op]
+        assert_ulp(got, f(a.astype(wide), b.astype(wide)), 4.0)
+    for dt in INTS:
+        a = random_array(rng, 500, dt, -5, 5)
+        b = random_array(rng, 500, dt, 0, 7)
+        if op == "pow":
+            with np.errstate(over="ignore"):
+                assert_same(host(dpt.pow(dev(a), dev(b))), np.power(a, b))
+
+
+@pytest.mark.parametrize("op", EXACT_UNARY)
+def test_unary_exact(op):
+    rng = np.random.default_rng(11)
+    for dt in ALL:
+        if not supported_unary(op, dt):
+            continue
+        for n in (1, 1025, 4099):
+            a = random_array(rng, n, dt, -50, 50)
+            if dt.kind == "f" and n > 4:
+                a[:4] = [np.nan, np.inf, -np.inf, -0.0]
+            if op in ("sqrt",):
+                a = np.abs(a)
+            got = host(getattr(dpt, op)(dev(a)))
+            want = orc.unary(op, a)
+            if dt.kind == "c" and op == "abs":
+                np.testing.assert_allclose(got, want, rtol=4 * np.finfo(got.dtype).eps)
+            elif dt.kind == "c" and op == "square":
+                assert_close_complex(got, want, a)
+            elif dt == np.dtype("f2") and op in ("reciprocal",):
+                assert_ulp(got, 1 / a.astype("f8"), 1.0)
+            else:
+                assert_same(got, want)
+
+
+@pytest.mark.parametrize("op", ULP_UNARY)
+def test_unary_transcendentals_within_4_ulp(op):
+    rng = np.random.default_rng(13)
+    rng_by_op = {"exp": (-80, 80), "exp2": (-100, 100), "expm1": (-30, 30), "log": (1e-30, 1e30),
+                 "log2": (1e-30, 1e30), "log10": (1e-30, 1e30), "log1p": (-0.99, 1e10), "erf": (-6, 6),
+                 "sin": (-50, 50), "cos": (-50, 50), "tan": (-1.5, 1.5), "tanh": (-20, 20), "cbrt": (-1e10, 1e10),
+                 "rsqrt": (1e-10, 1e10)}
+    lo, hi = rng_by_op[op]
+    for dt in FLOATS:
+        if dt == np.dtype("f2"):
+            lo2, hi2 = max(lo, -10), min(hi, 10)
+            if op in ("log", "log2", "log10", "rsqrt"):
+                lo2, hi2 = 1e-3, 6e4
+        else:
+            lo2, hi2 = (max(lo, -80), min(hi, 80)) if (dt == np.dtype("f4") and op in ("exp", "exp2")) else (lo, hi)
+        n = 3000 if (dt.itemsize == 8 and op == "erf") else 20000
+        a = rng.uniform(lo2, hi2, n).astype(dt)
+        if op.startswith("log") or op == "rsqrt":
+            a = np.exp(rng.uniform(np.log(max(lo2, 1e-30)), np.log(hi2), n)).astype(dt)
+        got = host(getattr(dpt, op)(dev(a)))
+        if op == "rsqrt":
+            wide = np.float64 if dt.itemsize <= 4 else np.longdouble
+            exact = 1 / np.sqrt(a.astype(wide))
+        else:
+            exact = orc.hi_precision(op, a)
+        assert got.dtype == orc.unary_result_dtype(op, dt)
+        assert_ulp(got, exact, 4.0)
+    # special values, dpnp/tests/tensor/elementwise/test_exp.py:124-137, test_log.py:88, test_sqrt.py:94-129
+    x = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0], dtype="f4")
+    with np.errstate(all="ignore"):
+        want = {"exp": np.exp, "log": np.log, "erf": None}.get(op)
+        if want is not None:
+            got = host(getattr(dpt, op)(dev(x)))
+            np.testing.assert_array_equal(got, want(x))
+            np.testing.assert_array_equal(np.signbit(got), np.signbit(want(x)))
+
+
+def test_exp_known_answers():
+    # dpnp/tests/tensor/elementwise/test_exp.py:111-120
+    for dt in ("f2", "f4", "f8"):
+        x = (np.arange(11, dtype=dt) * np.dtype(dt).type(0.69314718055994530943)).astype(dt)
+        tol = 8 * np.finfo(dt).resolution
+        np.testing.assert_allclose(host(dpt.exp(dev(x))).astype("f8"), np.exp(x.astype("f8")), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dt", ["f4", "i4", "?", "f8", "i1", "c8"])
+def test_strided_and_broadcast_views(dt):
+    rng = np.random.default_rng(17)
+    base_a = random_array(rng, (37, 130), dt, -9, 9)
+    base_b = random_array(rng, (37, 130), dt, -9, 9)
+    for (na, va), (nb, vb) in zip(strided_views(base_a), strided_views(base_b)):
+        a, b = dev_view_like(va, base_a), dev_view_like(vb, base_b)
+        assert a.strides == tuple(s // va.itemsize for s in va.strides)
+        if dt == "c8":
+            assert_close_complex(host(dpt.multiply(a, b)), orc.binary("multiply", va, vb), va, vb)
+        else:
+            assert_same(host(dpt.multiply(a, b)), orc.binary("multiply", va, vb))
+        assert_same(host(dpt.greater(a, b)), orc.binary("greater", va, vb))
+    # row vector and column vector broadcast, scalar operand
+    row, col = random_array(rng, (1, 130), dt, -9, 9), random_array(rng, (37, 1), dt, -9, 9)
+    assert_same(host(dpt.add(dev(base_a), dev(row))), orc.binary("add", base_a, np.broadcast_to(row, base_a.shape)))
+    assert_same(host(dpt.add(dev(col), dev(base_a))), orc.binary("add", np.broadcast_to(col, base_a.shape), base_a))
+    assert_same(host(dpt.add(dev(row), dev(col))),
+                orc.binary("add", np.broadcast_to(row, (37, 130)), np.broadcast_to(col, (37, 130))))
+    if dt != "?":
+        two = np.dtype(dt).type(2)
+        assert_same(host(dpt.multiply(dev(base_a), 2)), orc.binary("multiply", base_a, np.full_like(base_a, two)))
+        assert_same(host(dpt.multiply(2, dev(base_a)[:, ::3])),
+                    orc.binary("multiply", np.full_like(base_a[:, ::3], two), base_a[:, ::3]))
+
+
+def test_nd_views_random():
+    rng = np.random.default_rng(19)
+    for _ in range(25):
+        nd = int(rng.integers(1, 6))
+        shape = tuple(int(s) for s in rng.integers(1, 9, nd))
+        big = tuple(2 * s + 1 for s in shape)
+        base_a, base_b = random_array(rng, big, "i4"), random_array(rng, big, "i4")
+
+        def rv(base):
+            perm = rng.permutation(nd)
+            v = np.transpose(base, perm)
+            v = v[tuple(slice(None, None, int(st)) for st in rng.choice([1, 2, -1, -2], nd))]
+            inv = np.argsort(perm)
+            v = np.transpose(v, inv)
+            return v[tuple(slice(0, s) for s in shape)] if all(
+                v.shape[d] >= shape[d] for d in range(nd)) else np.broadcast_to(base.ravel()[:1].reshape((1,) * nd), shape)
+
+        va, vb = rv(base_a), rv(base_b)
+        if va.shape != shape or vb.shape != shape:
+            continue
+        a = dev_view_like(va, base_a) if va.base is not None and va.strides != (0,) * nd else dev(np.ascontiguousarray(va))
+        b = dev_view_like(vb, base_b) if vb.base is not None and vb.strides != (0,) * nd else dev(np.ascontiguousarray(vb))
+        assert_same(host(dpt.subtract(a, b)), va - vb)
+        cond = random_array(rng, shape, "?")
+        assert_same(host(dpt.where(dev(cond), a, b)), np.where(cond, va, vb))
+
+
+@pytest.mark.parametrize("order", ["K", "C", "F", "A"])
+def test_result_layout(order):
+    rng = np.random.default_rng(23)
+    a = random_array(rng, (12, 20), "f4")
+    for v in (dev(a), dev(a).T, dev(a)[:, ::2], dpt.permute_dims(dev(random_array(rng, (3, 4, 5), "f4")), (1, 2, 0))):
+        r = dpt.exp(v, order=order)
+        want = np.exp(host(v))
+        assert_ulp(host(r), np.exp(host(v).astype("f8")), 4.0)
+        if order == "C":
+            assert r.flags.c_contiguous
+        elif order == "F":
+            assert r.flags.f_contiguous
+        elif order == "K" and v.flags.f_contiguous and not v.flags.c_contiguous:
+            assert r.flags.f_contiguous
+        assert r.shape == want.shape
+        r2 = dpt.add(v, v, order=order)
+        assert_same(host(r2), host(v) + host(v))
+
+
+def test_out_and_overlap():
+    rng = np.random.default_rng(29)
+    a, b = random_array(rng, 1000, "f4"), random_array(rng, 1000, "f4")
+    da, db = dev(a), dev(b)
+    out = dpt.empty(1000, dtype="f4")
+    r = dpt.add(da, db, out=out)
+    assert r is out
+    assert_same(host(out), a + b)
+    # out is an input: computed in place
+    dc = dev(a)
+    assert dpt.add(dc, db, out=dc) is dc
+    assert_same(host(dc), a + b)
+    dc = dev(b)
+    assert dpt.subtract(da, dc, out=dc) is dc
+    assert_same(host(dc), a - b)
+    # partial overlap: a temporary is used, result lands in out
+    buf = dev(np.concatenate([a, a]))
+    x, o = buf[:1000], buf[1:1001]
+    dpt.multiply(x, db, out=o)
+    assert_same(host(buf)[1:1001], a * b)
+    assert host(buf)[0] == a[0]
+    # out in a strided slice of a larger zero array leaves the neighbours untouched
+    big = dpt.zeros((1000, 2), dtype="f4")
+    dpt.exp(da, out=big[:, 1])
+    hb = host(big)
+    assert (hb[:, 0] == 0).all()
+    assert_ulp(hb[:, 1], np.exp(a.astype("f8")))
+    # in-place operators
+    dc = dev(a)
+    dc += db
+    dc *= 2
+    assert_same(host(dc), (a + b) * 2)
+    di = dev(np.arange(10, dtype="i4"))
+    with pytest.raises(ValueError):
+        di += 1.5
+    ro = dev(a)
+    ro.flags.writable = False
+    with pytest.raises(ValueError):
+        ro += db
+
+
+def test_python_scalars_follow_weak_promotion():
+    a = dev(np.arange(5, dtype="i1"))
+    assert dpt.add(a, 1).dtype == np.dtype("i1")
+    assert dpt.add(a, 1.5).dtype == np.dtype("f8")
+    f = dev(np.arange(5, dtype="f4"))
+    assert dpt.multiply(f, 2.5).dtype == np.dtype("f4")
+    assert dpt.multiply(f, 1j).dtype == np.dtype("c8")
+    assert_same(host(dpt.greater(dev(np.array([1, 200], dtype="u1")), -1)), np.array([True, True]))
+    assert_same(host(dpt.divide(dev(np.arange(4, dtype="i4")), 2)), np.arange(4) / 2)
+    with pytest.raises(OverflowError):
+        dpt.add(a, 1000)
+
+
+@pytest.mark.parametrize("src", ALL, ids=str)
+def test_astype_matrix(src):
+    rng = np.random.default_rng(31)
+    a = random_array(rng, 2051, src, -120, 120)
+    if src.kind == "f":
+        a[:3] = [-0.0, 0.25, -3.75]
+    for dst in ALL:
+        got = host(dpt.astype(dev(a), dst))
+        want = orc.cast(a, dst)
+        assert_same(got, want)
+    v = dev(a)[::-2]
+    assert_same(host(dpt.astype(v, "f8")), orc.cast(a[::-2], "f8"))
+    assert_same(host(dpt.copy(v)), a[::-2])
+
+
+def test_empty_and_zero_d():
+    z = dpt.empty((0, 5), dtype="f4")
+    assert dpt.add(z, z).shape == (0, 5)
+    assert dpt.exp(z).shape == (0, 5)
+    s = dev(np.float32(3.0))
+    assert host(dpt.add(s, s)).shape == () and float(dpt.add(s, s)) == 6.0
+    assert float(dpt.sqrt(dev(np.float64(16)))) == 4.0
+
+
+def test_unaligned_base_pointer():
+    # kernels must not assume 16-byte alignment (views such as x[1:])
+    rng = np.random.default_rng(37)
+    for dt in ("i1", "f2", "f4", "f8"):
+        a, b = random_array(rng, 5003, dt), random_array(rng, 5003, dt)
+        for k in (1, 2, 3, 5):
+            assert_same(host(dpt.add(dev(a)[k:], dev(b)[k:])), (a + b)[k:])
+            o = dpt.empty(5003, dtype=dt)
+            dpt.add(dev(a)[k:], dev(b)[:-k], out=o[k:])
+            assert_same(host(o)[k:], a[k:] + b[:-k])

@@ -1,0 +1,319 @@
+"""Pins the CPU oracle: reference known answers, closed forms, brute force, mpmath.
+Runs without a GPU."""
+import itertools
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+from oracle.oracle_c import OracleC
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+ALL = [d.str[1:] if d.kind != "b" else "?" for d in orc.ALL_DTYPES]
+
+
+def _f(v):
+    return float(v) if isinstance(v, str) else v
+
+
+# ---- elementwise -----------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ALL)
+def test_add_ones_is_two(dt):
+    # dpnp/tests/tensor/elementwise/test_add.py:49-88: ones + ones == 2 (bool: True)
+    a = np.ones(7, dtype=dt)
+    r = orc.binary("add", a, a)
+    assert r.dtype == a.dtype
+    assert (r == np.full(7, 2, dtype=dt)).all() if dt != "?" else r.all()
+
+
+@pytest.mark.parametrize("dt", ["i1", "u1", "i2", "u2"])
+@pytest.mark.parametrize("op", ["add", "subtract", "multiply", "bitwise_and", "bitwise_or", "bitwise_xor"])
+def test_integer_ops_wrap_like_python_ints(dt, op):
+    info = np.iinfo(dt)
+    vals = np.array([info.min, info.min + 1, -1 if info.min < 0 else 1, 0, 1, 2, 3, 7, info.max - 1, info.max],
+                    dtype=dt)
+    a, b = np.meshgrid(vals, vals)
+    r = orc.binary(op, a, b)
+    py = {"add": int.__add__, "subtract": int.__sub__, "multiply": int.__mul__, "bitwise_and": int.__and__,
+          "bitwise_or": int.__or__, "bitwise_xor": int.__xor__}[op]
+    bits = 8 * np.dtype(dt).itemsize
+    for x, y, z in zip(a.ravel(), b.ravel(), r.ravel()):
+        want = py(int(x), int(y)) & ((1 << bits) - 1)
+        if info.min < 0 and want >= (1 << (bits - 1)):
+            want -= 1 << bits
+        assert int(z) == want
+
+
+def test_floor_divide_and_remainder_integer_rules():
+    # floor_divide.hpp:69-86, remainder.hpp: x // 0 == 0, x % 0 == 0, Python floor semantics otherwise
+    vals = np.array([-7, -3, -1, 0, 1, 3, 7], dtype="i4")
+    a, b = np.meshgrid(vals, vals)
+    q, r = orc.binary("floor_divide", a, b), orc.binary("remainder", a, b)
+    for x, y, qq, rr in zip(a.ravel(), b.ravel(), q.ravel(), r.ravel()):
+        if y == 0:
+            assert qq == 0 and rr == 0
+        else:
+            assert qq == int(x) // int(y) and rr == int(x) % int(y)
+
+
+def test_mixed_int64_uint64_comparisons_are_exact():
+    a = np.array([-1, 0, 2**62, -2**63, 2**63 - 1], dtype="i8")
+    b = np.array([2**64 - 1, 0, 2**62, 2**63, 2**63 - 1], dtype="u8")
+    for op, f in (("less", int.__lt__), ("greater", int.__gt__), ("equal", int.__eq__),
+                  ("less_equal", int.__le__), ("greater_equal", int.__ge__), ("not_equal", int.__ne__)):
+        for x, y in ((a, b), (b, a)):
+            r = orc.binary(op, x, y)
+            assert [bool(v) for v in r] == [f(int(p), int(q)) for p, q in zip(x, y)]
+
+
+def test_bool_arithmetic_is_logical():
+    t = np.array([True, True, False, False])
+    u = np.array([True, False, True, False])
+    assert (orc.binary("add", t, u) == (t | u)).all()
+    assert (orc.binary("multiply", t, u) == (t & u)).all()
+    assert (orc.binary("bitwise_and", t, u) == (t & u)).all()
+
+
+def test_maximum_minimum_nan_rule():
+    a = np.array([np.nan, 1.0, 2.0, np.nan], dtype="f4")
+    b = np.array([1.0, np.nan, 3.0, np.nan], dtype="f4")
+    assert np.isnan(orc.binary("maximum", a, b)[[0, 1, 3]]).all() and orc.binary("maximum", a, b)[2] == 3
+    assert np.isnan(orc.binary("minimum", a, b)[[0, 1, 3]]).all() and orc.binary("minimum", a, b)[2] == 2
+
+
+def test_exp_known_answers():
+    g = GOLD["exp_powers_of_two"]
+    for dt in ("f2", "f4", "f8"):
+        x = (np.array(g["k"], dtype=dt) * np.dtype(dt).type(g["log2"])).astype(dt)
+        tol = 8 * np.finfo(dt).resolution
+        np.testing.assert_allclose(orc.unary("exp", x).astype("f8"), np.exp(x.astype("f8")), rtol=tol, atol=tol)
+    s = GOLD["exp_special"]
+    x = np.array([_f(v) for v in s["x"]], dtype="f8")
+    want = np.array([_f(v) for v in s["expected"]], dtype="f8")
+    np.testing.assert_array_equal(orc.unary("exp", x), want)
+
+
+@pytest.mark.parametrize("op", ["exp", "log", "erf"])
+def test_high_precision_evaluation_against_mpmath(op):
+    import mpmath
+
+    mpmath.mp.dps = 60
+    rng = np.random.default_rng(5)
+    x = {"exp": rng.uniform(-80, 80, 200), "log": rng.uniform(1e-30, 1e30, 200), "erf": rng.uniform(-4, 4, 200)}[op]
+    f = {"exp": mpmath.exp, "log": mpmath.log, "erf": mpmath.erf}[op]
+    for dt in ("f4", "f8"):
+        xs = x.astype(dt)
+        got = orc.unary(op, xs)
+        exact = np.array([np.longdouble(mpmath.nstr(f(mpmath.mpf(float(v))), 40)) for v in xs])
+        assert orc.ulp_error(got, exact).max() <= 0.5 + 1e-3  # the oracle rounds the exact value
+
+
+def test_cast_rules():
+    # type_utils.hpp:64-117
+    assert (orc.cast(np.array([0.0, -0.0, 0.5, np.nan]), "?") == [False, False, True, True]).all()
+    assert (orc.cast(np.array([-1.0, -3.7, 5.2], dtype="f4"), "u1") == [255, 253, 5]).all()
+    assert (orc.cast(np.array([-1.0, 2.0**31], dtype="f8"), "u4") == [2**32 - 1, 2**31]).all()
+    assert orc.cast(np.array([3 + 4j]), "f8")[0] == 3.0
+    assert orc.cast(np.array([0 + 1j]), "?")[0]
+
+
+def test_where_known_answer():
+    g = GOLD["where_basic"]
+    cond = np.array(g["cond"], dtype=bool)
+    r = orc.where(cond, np.full(cond.shape, g["x1"]), np.full(cond.shape, g["x2"]))
+    assert (r == np.array(g["expected"])).all()
+    # truthiness of non-bool conditions: any set bit except -0.0
+    assert (orc.where(np.array([0.0, -0.0, np.nan, 2.0]), np.ones(4), np.zeros(4)) == [0, 0, 1, 1]).all()
+
+
+def test_black_scholes_put_call_parity():
+    rng = np.random.default_rng(4)
+    p, s, t = rng.uniform(10, 50, 1000), rng.uniform(10, 50, 1000), rng.uniform(1, 2, 1000)
+    call, put = orc.black_scholes(p, s, t, 0.1, 0.2)
+    np.testing.assert_allclose(call - put, p - s * np.exp(-0.1 * t), rtol=1e-12, atol=1e-12)
+    # closed form of the same expression tree with the normal CDF written through erf:
+    # call = P*N(d1') - S*exp(-rT)*N(d2') with N(x) = (1 + erf(x)) / 2 applied to w1, w2
+    z = t * (0.2 * 0.2 * 2)
+    w1 = (np.log(p / s) + 0.1 * t + 0.25 * z) / np.sqrt(z)
+    w2 = (np.log(p / s) + 0.1 * t - 0.25 * z) / np.sqrt(z)
+    erf = np.vectorize(math.erf)
+    want = p * (0.5 + 0.5 * erf(w1)) - s * np.exp(-0.1 * t) * (0.5 + 0.5 * erf(w2))
+    np.testing.assert_allclose(call, want, rtol=1e-11, atol=1e-11)
+
+
+# ---- reductions ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ALL)
+def test_sum_of_ones(dt):
+    for n in GOLD["sum_ones"]["n"]:
+        r = orc.reduce("sum", np.ones(n, dtype=dt), 1)
+        assert r == n
+        assert r.dtype == orc.default_accumulation_dtype(np.dtype(dt))
+    g = GOLD["sum_strided_ones"]
+    assert orc.reduce("sum", np.ones(g["base_n"], dtype=dt)[slice(*g["slice"])], 1) == g["expected"]
+
+
+def test_sum_known_answers():
+    g = GOLD["sum_gh1391"]
+    a = np.arange(g["arange"], dtype="i4").reshape(g["shape"]).transpose(g["permute"])
+    assert (orc.reduce("sum", a, 1) == np.array(g["expected"])).all()
+    g = GOLD["sum_axis0_3x4x5"]
+    x = np.arange(g["arange"], dtype="f4").reshape(g["shape"])
+    assert (orc.reduce("sum", np.moveaxis(x, 0, -1), 1) == np.array(g["expected"], dtype="f4")).all()
+    g = GOLD["sum_flip_axis2_3x4x5"]
+    assert (orc.reduce("sum", np.flip(x, 2), 1) == np.array(g["expected"], dtype="f4")).all()
+    g = GOLD["sum_bool_dtype_gh1944"]
+    for dt in g["dtypes"]:
+        assert bool(orc.reduce("sum", np.array(g["input"], dtype=dt), 1, out_dtype="?")) is True
+    assert orc.reduce("sum", np.empty(0, dtype="u1"), 1) == 0
+    assert orc.reduce("prod", np.empty(0, dtype="f4"), 1) == 1
+
+
+def test_integer_sum_wraps():
+    x = np.full(300, 127, dtype="i1")
+    assert orc.reduce("sum", x, 1, out_dtype="i1") == np.int8((300 * 127) % 256 - 256 if (300 * 127) % 256 > 127 else (300 * 127) % 256)
+    assert orc.reduce("sum", x, 1) == 300 * 127
+
+
+def test_float_sum_is_exact_sum_rounded():
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, 4097).astype("f4")
+    assert orc.reduce("sum", x, 1) == np.float32(math.fsum(x.astype("f8")))
+
+
+def test_max_min_known_answers():
+    g = GOLD["max_axis0_arange"]
+    x = np.arange(g["arange"]).reshape(g["shape"])
+    assert (orc.reduce("max", np.moveaxis(x, 0, -1), 1) == x[-1]).all()
+    for c in GOLD["max_min_nan"]["cases"]:
+        v = np.array([_f(e) for e in c["values"]], dtype=c["dtype"])
+        assert np.isnan(orc.reduce("max", v, 1)) and np.isnan(orc.reduce("min", v, 1))
+    z = np.arange(4, dtype="c8")
+    z[0] = complex(np.nan, 0)
+    assert np.isnan(orc.reduce("max", z, 1)) and np.isnan(orc.reduce("min", z, 1))
+    with pytest.raises(ValueError):
+        orc.reduce("max", np.empty((3, 0)), 1)
+
+
+def test_argmax_known_answers():
+    g = GOLD["argmax_2x3"]
+    x = np.array(g["input"], dtype=g["dtype"])
+    assert orc.argreduce("argmax", x, 2) == g["argmax_flat"]
+    assert (orc.argreduce("argmax", x.T, 1) == g["argmax_axis0"]).all()
+    assert (orc.argreduce("argmax", x, 1) == g["argmax_axis1"]).all()
+    assert orc.argreduce("argmax", np.full(3, np.iinfo("i4").min, dtype="i4"), 1) == 0
+    assert orc.argreduce("argmin", np.full(3, np.iinfo("i4").max, dtype="i4"), 1) == 0
+    for idx in range(4):
+        for dt in ("f4", "c8"):
+            x = np.arange(4, dtype=dt)
+            x[idx] = np.nan
+            assert orc.argreduce("argmax", x, 1) == idx and orc.argreduce("argmin", x, 1) == idx
+    x = np.arange(4, dtype="c8")
+    x[2] = complex(0, np.nan)
+    assert orc.argreduce("argmax", x, 1) == 2 and orc.argreduce("argmin", x, 1) == 2
+
+
+def test_argmax_brute_force_all_patterns():
+    vals = [0.0, 1.0, -1.0, np.nan, np.inf, -np.inf]
+    for n in (1, 2, 3, 4):
+        for combo in itertools.product(vals, repeat=n):
+            x = np.array(combo, dtype="f4")
+            nan = [i for i, v in enumerate(combo) if v != v]
+            want_max = nan[0] if nan else max(range(n), key=lambda i: (combo[i], -i))
+            want_min = nan[0] if nan else min(range(n), key=lambda i: (combo[i], i))
+            assert orc.argreduce("argmax", x, 1) == want_max
+            assert orc.argreduce("argmin", x, 1) == want_min
+            assert orc.argreduce("argmax", x, 1) == np.argmax(x)  # NumPy: first NaN, first maximum
+
+
+def test_mean_var_known_answers():
+    g = GOLD["mean_3x3"]
+    x = np.arange(g["arange"], dtype=g["dtype"]).reshape(g["shape"])
+    assert orc.mean(x, 2) == g["mean"]
+    assert (orc.mean(x.T, 1) == g["mean_axis0"]).all() and (orc.mean(x, 1) == g["mean_axis1"]).all()
+    g = GOLD["var_3x3"]
+    np.testing.assert_allclose(orc.var(x, 2), g["var"], rtol=1e-6)
+    np.testing.assert_allclose(orc.var(x, 2, correction=3), g["var_corr3"], rtol=1e-6)
+    np.testing.assert_allclose(orc.var(x.T, 1), g["var_axis0"], rtol=1e-6)
+    np.testing.assert_allclose(orc.var(x.T, 1, correction=1), g["var_axis0_corr1"], rtol=1e-6)
+    np.testing.assert_allclose(orc.var(x, 1), g["var_axis1"], rtol=1e-6)
+    np.testing.assert_allclose(orc.var(x, 1, correction=1), g["var_axis1_corr1"], rtol=1e-6)
+    # test_tensor_statistical_functions.py:229-241: N - correction <= 0 gives NaN
+    assert np.isnan(orc.var(x, 2, correction=9)) and np.isnan(orc.var(x, 1, correction=3)).all()
+    assert orc.mean(np.arange(4, dtype="i4"), 1).dtype == np.dtype("f8")
+
+
+# ---- stride collapsing ----------------------------------------------------------------------------------
+def random_view_strides(rng, shape):
+    """Element strides of a random view with `shape`: permuted base layout, steps of +-1/+-2,
+    some dims broadcast (stride 0)."""
+    nd = len(shape)
+    perm = rng.permutation(nd)
+    big = [2 * s + 1 for s in shape]
+    base = np.arange(int(np.prod(big))).reshape([big[p] for p in perm])
+    v = np.transpose(base, np.argsort(perm))
+    v = v[tuple(slice(None, None, int(st)) for st in rng.choice([1, 2, -1, -2], nd))]
+    v = v[tuple(slice(0, s) for s in shape)]
+    for d in range(nd):
+        if rng.random() < 0.2:
+            one = v[tuple(slice(0, 1) if i == d else slice(None) for i in range(nd))]
+            v = np.broadcast_to(one, shape)
+    assert v.shape == tuple(shape)
+    return [st // base.itemsize for st in v.strides]
+
+
+def test_collapse_keeps_the_address_set():
+    rng = np.random.default_rng(11)
+    for _ in range(300):
+        nd = int(rng.integers(1, 5))
+        shape = [int(s) for s in rng.integers(1, 5, nd)]
+        strides = [random_view_strides(rng, shape) for _k in range(int(rng.integers(1, 4)))]
+        for keep in (False, True):
+            sh, st, off = orc.collapse(shape, strides, keep_order=keep)
+            assert orc.address_tuples(sh, st, off) == orc.address_tuples(shape, strides)
+            assert len(sh) <= nd
+
+
+def test_collapse_merges_contiguous_and_reversed():
+    assert orc.collapse([3, 4, 5], [[20, 5, 1], [20, 5, 1]])[0] == [60]
+    sh, st, off = orc.collapse([3, 4], [[-4, -1]])
+    assert sh == [12] and st == [[1]] and off == [-11]
+    sh, st, off = orc.collapse([8192, 4096], [[8192, 2], [0, 1], [4096, 1]])
+    assert sh == [8192, 4096] and st == [[8192, 2], [0, 1], [4096, 1]]
+    # keep_order: only neighbours merge, nothing is reordered or reversed
+    sh, st, off = orc.collapse([3, 4], [[1, 3]], keep_order=True)
+    assert sh == [3, 4] and st == [[1, 3]]
+
+
+# ---- promotion --------------------------------------------------------------------------------------------
+def test_promotion_matches_numpy_result_type():
+    # dpnp/tests/tensor/elementwise/test_add.py:62-65: result dtype of add == numpy.result_type
+    same = lambda a, b: a if a == b else None  # noqa: E731  (add has all 14 same-dtype pairs)
+    for d1 in orc.ALL_DTYPES:
+        for d2 in orc.ALL_DTYPES:
+            b1, b2, r = orc.promote_binary(same, d1, d2)
+            assert r == np.result_type(d1, d2), (d1, d2, r)
+
+
+# ---- C restatement vs NumPy restatement ----------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def oc():
+    return OracleC()
+
+
+@pytest.mark.parametrize("n", [1, 100, 255, 256, 257, 2048, 16384, 16385, 100003, 1 << 20])
+def test_c_port_matches_numpy_oracle(oc, n):
+    rng = np.random.default_rng(n)
+    a = rng.uniform(-1, 1, n).astype("f4")
+    b = rng.uniform(-1, 1, n).astype("f4")
+    assert np.array_equal(oc.add(a, b), orc.binary("add", a, b))
+    exact = orc.reduce("sum", a, 1)
+    assert abs(float(oc.sum(a)) - float(exact)) <= 1e-5 * max(abs(float(exact)), float(np.abs(a).sum()) * 1e-2)
+    x = rng.standard_normal(n).astype("f4")
+    x[rng.integers(0, n, max(n // 100, 1))] = x.max()
+    assert oc.argmax(x) == orc.argreduce("argmax", x, 1)
+    assert oc.argmin(x) == orc.argreduce("argmin", x, 1)
+    x[int(rng.integers(0, n))] = np.nan  # a single NaN is pinned by the reference's tests
+    assert oc.argmax(x) == orc.argreduce("argmax", x, 1) == oc.argmin(x)
