@@ -7,10 +7,12 @@
 //
 // Layout choices for MI355X:
 //   * every thread moves 16 bytes of the widest operand per access
-//     (global_load_dwordx4 / global_store_dwordx4, non-temporal), 256 threads per
-//     block and exactly one access per operand per thread: many short-lived
-//     waves keep the HBM queues full and the hardware dispatcher walks the
-//     arrays front to back, which measured faster than grid-stride loops;
+//     (global_load_dwordx4 / global_store_dwordx4, non-temporal) and makes exactly
+//     one access per operand; contiguous kernels run one wave (64 threads) per
+//     block: many short-lived waves keep the HBM queues full and the hardware
+//     dispatcher walks the arrays front to back.  Measured on MI355X for
+//     c = a + b over 2^28 floats: 64-thread blocks 6.6-6.8 TB/s, 256-thread
+//     blocks 6.3-6.5 TB/s, grid-stride loops 5.3-6.0 TB/s, no NT hint -5 %;
 //   * shape and strides of the collapsed iteration space travel in the kernel
 //     argument segment (no device-side metadata buffers to allocate or free);
 //   * strided kernels keep threads adjacent along the innermost output
@@ -22,7 +24,9 @@
 
 namespace dpx {
 
-constexpr int EW_BLOCK = 256;
+constexpr int EW_BLOCK = 256;       // upper bound of threads per block
+constexpr int EW_CONTIG_BLOCK = 64; // default for contiguous kernels: one wave
+constexpr int EW_ROWS_BLOCK = 256;  // default for strided kernels
 
 // operand access mode along the inner dimension (2 bits per operand)
 enum : uint32_t { MODE_STRIDED = 0, MODE_VEC = 1, MODE_BCAST = 2 };
@@ -52,13 +56,13 @@ template <class T, int E> DPX_D pack<T, E> splat(T v)
 }
 
 // ---- contiguous ---------------------------------------------------------------
-// grid.x * 256 * E >= n.  bcast bit i set: input i is a single element.
+// grid.x * blockDim.x * E >= n.  bcast bit i set: input i is a single element.
 template <bool VEC, class Fn, class Out, class... Ins, size_t... I>
 DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
                           const InPtrs<sizeof...(Ins)> &in, std::index_sequence<I...>)
 {
     constexpr int E = ew_traits<Out, Ins...>::E;
-    const int64_t block_base = (int64_t)blockIdx.x * (EW_BLOCK * E);
+    const int64_t block_base = (int64_t)blockIdx.x * ((int)blockDim.x * E);
     if constexpr (VEC) {
         const int64_t base = block_base + (int64_t)threadIdx.x * E;
         if (base + E <= n) {
@@ -82,7 +86,7 @@ DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
     else {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int64_t i = block_base + e * EW_BLOCK + threadIdx.x;
+            const int64_t i = block_base + e * (int)blockDim.x + threadIdx.x;
             if (i < n)
                 out[i] = to_storage<Out>(fn(to_value(
                     load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, u
 }
 
 // ---- strided, vectorised along the inner dimension -----------------------------
-// Block = TY rows x TX threads (TX = 1 << tx_log2, TX * TY = 256); a thread owns E
+// Block = TY rows x TX threads (TX = 1 << tx_log2, TX * TY = blockDim.x); a thread owns E
 // consecutive inner positions of one row.  ix.strides[k] for inputs k < N,
 // ix.strides[N] for the output.  modes: 2 bits per operand, output at bit 2*N.
 template <class Fn, class Out, class... Ins, size_t... I>
@@ -114,7 +118,7 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     const int ty = threadIdx.x >> tx_log2;
     const int64_t rb = (int64_t)blockIdx.x / col_blocks;
     const int64_t cb = (int64_t)blockIdx.x - rb * col_blocks;
-    const int64_t row = rb * (EW_BLOCK >> tx_log2) + ty;
+    const int64_t row = rb * ((int)blockDim.x >> tx_log2) + ty;
     const int inner = ix.nd - 1;
     const int64_t ncols = ix.shape[inner];
     const int64_t col0 = ((cb << tx_log2) + tx) * E;
@@ -192,6 +196,7 @@ struct EwPlan {
     uint32_t bcast;
     uint32_t modes;
     int tx_log2;
+    int block; // threads per block
     int64_t nrows, col_blocks, grid;
 };
 
@@ -220,10 +225,10 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
     if (pl.path == DPX_PATH_EW_CONTIG) {
         if (pl.vec)
             hipLaunchKernelGGL((ew_contig_kernel<true, Fn, Out, Ins...>), dim3((unsigned)pl.grid),
-                               dim3(EW_BLOCK), 0, stream, fn, pl.n, pl.bcast, out, in);
+                               dim3(pl.block), 0, stream, fn, pl.n, pl.bcast, out, in);
         else
             hipLaunchKernelGGL((ew_contig_kernel<false, Fn, Out, Ins...>),
-                               dim3((unsigned)pl.grid), dim3(EW_BLOCK), 0, stream, fn, pl.n,
+                               dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, fn, pl.n,
                                pl.bcast, out, in);
     }
     else {
@@ -235,7 +240,7 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
             for (int k = 0; k <= N; ++k) ix.strides[k][d] = d < pl.nd ? pl.strides[k][d] : 0;
         }
         hipLaunchKernelGGL((ew_rows_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid),
-                           dim3(EW_BLOCK), 0, stream, fn, ix, out, in, pl.modes, pl.tx_log2,
+                           dim3(pl.block), 0, stream, fn, ix, out, in, pl.modes, pl.tx_log2,
                            pl.nrows, pl.col_blocks);
     }
     return hipGetLastError();

@@ -1,4 +1,5 @@
 // Elementwise calls: validation and the choice of kernel, independent of element types.
+#include <cstdlib>
 #include "ew.hpp"
 #include "host.hpp"
 
@@ -32,6 +33,14 @@ int ew_validate(int nops, const dpx_array_view *const *views, int64_t &n)
     return DPX_OK;
 }
 
+// block-size override for experiments: a power of two in [64, 256], else the default
+static int env_block(const char *name, int dflt)
+{
+    const char *s = std::getenv(name);
+    const int v = (s && *s) ? std::atoi(s) : dflt;
+    return (v == 64 || v == 128 || v == 256) ? v : dflt;
+}
+
 void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
 {
     const dpx_array_view *dst = views[nops - 1];
@@ -40,6 +49,7 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     pl.vec = false;
     pl.bcast = pl.modes = 0;
     pl.tx_log2 = 0;
+    pl.block = EW_CONTIG_BLOCK;
     pl.nrows = pl.col_blocks = pl.grid = 0;
     for (int k = 0; k < 5; ++k) pl.offsets[k] = 0;
     if (pl.n == 0) {
@@ -75,7 +85,8 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
             if (k + 1 < nops && pl.strides[k][0] == 0 && pl.n > 1) pl.bcast |= 1u << k;
             else pl.vec = pl.vec && aligned(k);
         }
-        pl.grid = (pl.n + (int64_t)EW_BLOCK * E - 1) / ((int64_t)EW_BLOCK * E);
+        pl.block = env_block("DPX_EW_CONTIG_BLOCK", EW_CONTIG_BLOCK);
+        pl.grid = (pl.n + (int64_t)pl.block * E - 1) / ((int64_t)pl.block * E);
         return;
     }
     const int inner = pl.nd - 1;
@@ -94,10 +105,12 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         pl.modes |= mode << (2 * k);
     }
     const int64_t per_row = (ncols + E - 1) / E; // threads wanted along a row
-    int lg = 0;
-    while (lg < 8 && ((int64_t)1 << lg) < per_row) ++lg;
+    pl.block = env_block("DPX_EW_ROWS_BLOCK", EW_ROWS_BLOCK);
+    int lg = 0, lg_max = 0;
+    while ((1 << lg_max) < pl.block) ++lg_max;
+    while (lg < lg_max && ((int64_t)1 << lg) < per_row) ++lg;
     pl.tx_log2 = lg;
-    const int64_t tx = (int64_t)1 << lg, ty = EW_BLOCK / tx;
+    const int64_t tx = (int64_t)1 << lg, ty = pl.block / tx;
     pl.col_blocks = (per_row + tx - 1) / tx;
     pl.grid = pl.col_blocks * ((pl.nrows + ty - 1) / ty);
 }
@@ -114,7 +127,7 @@ void ew_export_plan(const EwPlan &pl, dpx_plan *out)
     for (int k = 0; k < pl.nops && k < 4; ++k) out->offsets[k] = pl.offsets[k];
     out->grid[0] = pl.grid;
     out->grid[1] = out->grid[2] = 1;
-    out->block = EW_BLOCK;
+    out->block = pl.block;
 }
 
 } // namespace dpx

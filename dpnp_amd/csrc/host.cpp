@@ -176,6 +176,12 @@ void *scratch_get(hipStream_t stream, size_t bytes)
         b.p = nullptr;
         return nullptr;
     }
+    // callers rely on fresh blocks being zero (ticket counters) and keep them zero
+    if (hipMemsetAsync(b.p, 0, want, stream) != hipSuccess) {
+        (void)hipFree(b.p);
+        b.p = nullptr;
+        return nullptr;
+    }
     b.bytes = want;
     return b.p;
 }

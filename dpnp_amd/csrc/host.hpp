@@ -31,6 +31,7 @@ int collapse(int nd, int nops, int64_t *shape, int64_t (*strides)[DPX_MAX_ND],
 
 // Scratch for partial results, owned by the library: one grow-only block per stream.
 // Work on one stream is ordered, so reuse by the next call on that stream is safe.
+// A newly allocated block is zero-filled (on the stream).
 void *scratch_get(hipStream_t stream, size_t bytes);
 int scratch_release_all();
 

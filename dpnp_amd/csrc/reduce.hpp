@@ -15,9 +15,12 @@
 //     dimension, so every load is a coalesced 16-byte pack of adjacent columns;
 //     TY thread rows walk down the reduced axis and meet in LDS.
 //   * when there are too few outputs to fill 256 CUs the reduced run is split
-//     over several blocks; partials go to scratch and a second launch of the
-//     same kernels folds them.  Partition and fold order are fixed functions of
-//     the shapes: results are bit-reproducible run to run, no atomics anywhere.
+//     over several blocks.  Pass one leaves a partial per block in scratch; the
+//     block that finishes last for an output (found with a ticket counter) runs
+//     pass two in the same launch: it folds that output's partials in index
+//     order.  Partition and fold order are fixed functions of the shapes, so
+//     results are bit-reproducible run to run; no value is ever accumulated
+//     with an atomic.
 #pragma once
 #include "ops.hpp"
 #include "types.hpp"
@@ -195,10 +198,96 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
 // ================================ rows kernel ================================================
 // Linear block id = oblock * splits + split.  G = 1 << g_log2 lanes per output
 // (G <= 64, several outputs per block) or the whole block (G == blockDim.x).
+// Folds r over the G lanes of a group (G <= 64: shuffles only) or over the whole block
+// (wave shuffles, then the wave leaders' values through LDS in wave order).  The result is
+// valid in lane 0 of the group / thread 0 of the block.
+template <class P> DPX_D typename P::Acc group_reduce(typename P::Acc r, bool whole_block, int G)
+{
+    using Acc = typename P::Acc;
+    const int wl = whole_block ? 64 : G;
+    for (int off = wl >> 1; off > 0; off >>= 1) r = P::combine(r, shfl_down_any(r, off));
+    if (whole_block) {
+        __shared__ Acc sm[16];
+        __syncthreads(); // sm may still be read by a previous call
+        const int w = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) sm[w] = r;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int nw = blockDim.x >> 6;
+            for (int i = 1; i < nw; ++i) r = P::combine(r, sm[i]);
+        }
+    }
+    return r;
+}
+
+// ---- cross-block hand-off ------------------------------------------------------------------
+// A partial travels between blocks through agent-scope atomics only: the producer writes it
+// with atomic exchanges (performed at the device's coherence point, so no cache has to be
+// written back), takes its ticket with an atomic add whose address depends on the values
+// the exchanges returned (the add cannot issue before the exchanges have completed), and
+// the one block that draws the last ticket invalidates its caches once and reads the
+// partials.  A release fence per block instead (L2 write-back) cost 15-30 % of kernel time.
+template <class T> struct Slot {
+    static constexpr int W = ((int)sizeof(T) + 3) / 4;
+    uint32_t w[W];
+};
+
+// Stores v into *p; returns 0, available only once the store has completed device-wide.
+template <class T> DPX_D uint32_t slot_publish(Slot<T> *p, const T &v)
+{
+    union {
+        Slot<T> s;
+        T t;
+    } u;
+#pragma unroll
+    for (int i = 0; i < Slot<T>::W; ++i) u.s.w[i] = 0;
+    u.t = v;
+    uint32_t tok = 0;
+#pragma unroll
+    for (int i = 0; i < Slot<T>::W; ++i)
+        tok |= __hip_atomic_exchange(&p->w[i], u.s.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t zero;
+    asm volatile("v_and_b32 %0, 0, %1" : "=v"(zero) : "v"(tok));
+    return zero;
+}
+template <class T> DPX_D T slot_read(const Slot<T> *p)
+{
+    union {
+        Slot<T> s;
+        T t;
+    } u;
+#pragma unroll
+    for (int i = 0; i < Slot<T>::W; ++i) u.s.w[i] = p->w[i];
+    return u.t;
+}
+
+// Called by every thread of a block; `zero` is what slot_publish returned in this thread
+// (0 in threads that published nothing).  True, for all threads, in the block that took
+// the last of `splits` tickets for this counter: every partial of the output is then
+// readable.  The counter is left at zero for the next launch.
+DPX_D bool last_block_of(unsigned *counter, int splits, uint32_t zero)
+{
+    __shared__ unsigned sh_zero;
+    __shared__ int is_last;
+    if (threadIdx.x == 0) sh_zero = 0;
+    __syncthreads();
+    atomicOr(&sh_zero, zero); // consumes `zero`: waits for this thread's exchanges
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned t = __hip_atomic_fetch_add(counter + sh_zero, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (t == (unsigned)(splits - 1));
+        if (is_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const bool last = is_last != 0;
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return last;
+}
+
 template <class P, bool CONTIG>
 __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
-                                                       typename P::Out *dst, typename P::Acc *partial,
-                                                       const typename P::Aux *aux)
+                                                       typename P::Out *dst, Slot<typename P::Acc> *partial,
+                                                       const typename P::Aux *aux, unsigned *counters)
 {
     using In = typename P::In;
     using Acc = typename P::Acc;
@@ -264,40 +353,64 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L
     }
     Acc r = P::combine(P::combine(acc[0], acc[1]), P::combine(acc[2], acc[3]));
     static_assert(RED_U == 4);
-
-    const int wl = whole_block ? 64 : G; // lanes to fold with shuffles
-    for (int off = wl >> 1; off > 0; off >>= 1) r = P::combine(r, shfl_down_any(r, off));
-    if (whole_block) {
-        __shared__ Acc sm[16];
-        const int w = threadIdx.x >> 6;
-        if ((threadIdx.x & 63) == 0) sm[w] = r;
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            const int nw = blockDim.x >> 6;
-            for (int i = 1; i < nw; ++i) r = P::combine(r, sm[i]);
-        }
+    r = group_reduce<P>(r, whole_block, G);
+    if (L.splits == 1) {
+        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = P::post(r);
+        return;
     }
-    if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) {
-        if (L.splits == 1) dst[dof] = P::post(r);
-        else partial[o * L.splits + split] = r;
-    }
+    // split mode (always a whole block per output): pass two by the last block to finish
+    uint32_t zero = 0;
+    if (threadIdx.x == 0) zero = slot_publish(partial + o * L.splits + split, r);
+    if (!last_block_of(counters + o, L.splits, zero)) return;
+    Acc v = P::identity();
+    for (int i = threadIdx.x; i < L.splits; i += blockDim.x) v = P::combine(v, slot_read(partial + o * L.splits + i));
+    v = group_reduce<P>(v, true, G);
+    if (threadIdx.x == 0) dst[dof] = P::post(v);
 }
 
 // ================================ cols kernel ================================================
 // Iteration space: outer dims (0 .. nd_i-2) x inner dim (nd_i-1, src stride 1).
-// Block = TY x TX threads, TX = 1 << g_log2 along the inner dim, E_ columns per thread
-// (E_ = 16 / sizeof(In) when L.vec, else 1).  Linear block id = (outer * splits + split) *
-// col_blocks + col_block.  Partials are laid out [split][output] so the fold pass is again
-// a coalesced column reduction.
+// Block = TY x TX threads, TX = 1 << g_log2 along the inner dim, TY = blockDim.x / TX rows,
+// ecnt columns per thread (ecnt = 16 / sizeof(In) when L.vec, else 1).
+// Linear block id = (outer * splits + split) * col_blocks + col_block.
+// Partials are laid out [split][output] (coalesced to write and to fold).
+constexpr int COLS_MAX_BLOCK = 1024;
+
+// elements of LDS scratch per thread and loads in flight per thread: wide inputs keep 4
+// packs in flight, 1- and 2-byte inputs (8 or 16 accumulators per pack) keep 2
+template <class In> struct cols_cfg {
+    static constexpr int E = 16 / (int)sizeof(In);
+    static constexpr int U = E >= 8 ? 2 : 4;
+};
+
+// combines acc over the TY thread rows of the block; result valid for ty == 0
+template <class P, int E> DPX_D void cols_block_combine(typename P::Acc (&v)[E], typename P::Acc *sm, int tx, int ty,
+                                                        int TX, int TY)
+{
+    __syncthreads(); // sm may still be read by a previous call
+#pragma unroll
+    for (int e = 0; e < E; ++e) sm[threadIdx.x * E + e] = v[e];
+    __syncthreads();
+    if (ty == 0) {
+        for (int y = 1; y < TY; ++y)
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = P::combine(v[e], sm[(y * TX + tx) * E + e]);
+    }
+}
+
 template <class P>
-__global__ __launch_bounds__(256) void red_cols_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
-                                                      typename P::Out *dst, typename P::Acc *partial,
-                                                      const typename P::Aux *aux)
+__global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, RedLaunch L,
+                                                                 const typename P::In *src, typename P::Out *dst,
+                                                                 Slot<typename P::Acc> *partial,
+                                                                 const typename P::Aux *aux, unsigned *counters)
 {
     using In = typename P::In;
     using Acc = typename P::Acc;
-    constexpr int E = 16 / (int)sizeof(In);
-    const int TX = 1 << L.g_log2, TY = 256 >> L.g_log2;
+    constexpr int E = cols_cfg<In>::E;
+    constexpr int U = cols_cfg<In>::U;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Acc *sm = reinterpret_cast<Acc *>(smem_raw);
+    const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
     const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> L.g_log2;
     int64_t b = blockIdx.x;
     const int64_t cb = b % L.col_blocks;
@@ -308,9 +421,9 @@ __global__ __launch_bounds__(256) void red_cols_kernel(RedIndex ix, RedLaunch L,
     const int64_t col0 = (cb * TX + tx) * ecnt;
     const bool active = col0 < L.inner;
 
-    Acc acc[RED_U][E];
+    Acc acc[U][E];
 #pragma unroll
-    for (int u = 0; u < RED_U; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[u][e] = P::identity();
 
@@ -328,10 +441,10 @@ __global__ __launch_bounds__(256) void red_cols_kernel(RedIndex ix, RedLaunch L,
         }
     }
     const int last = ix.nd_i - 1;
-    Acc a[E];
-#pragma unroll
-    for (int e = 0; e < E; ++e) a[e] = P::identity();
     if (active) {
+        Acc a[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) a[e] = P::identity();
         if constexpr (P::has_aux) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
@@ -342,12 +455,12 @@ __global__ __launch_bounds__(256) void red_cols_kernel(RedIndex ix, RedLaunch L,
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         int64_t r = beg + ty;
         if (L.vec) {
-            for (; r + (RED_U - 1) * TY < end; r += RED_U * TY) {
-                pack<In, E> v[RED_U];
+            for (; r + (U - 1) * TY < end; r += U * TY) {
+                pack<In, E> v[U];
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u) v[u] = load_pack<In, E>(p + (r + u * TY) * L.rstride);
+                for (int u = 0; u < U; ++u) v[u] = load_pack<In, E>(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u)
+                for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], P::pre(v[u].v[e], a[e]));
             }
@@ -358,32 +471,56 @@ __global__ __launch_bounds__(256) void red_cols_kernel(RedIndex ix, RedLaunch L,
             }
         }
         else {
-            for (; r + (RED_U - 1) * TY < end; r += RED_U * TY) {
-                In v[RED_U];
+            for (; r + (U - 1) * TY < end; r += U * TY) {
+                In v[U];
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
+                for (int u = 0; u < U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u) acc[u][0] = P::combine(acc[u][0], P::pre(v[u], a[0]));
+                for (int u = 0; u < U; ++u) acc[u][0] = P::combine(acc[u][0], P::pre(v[u], a[0]));
             }
             for (; r < end; r += TY) acc[0][0] = P::combine(acc[0][0], P::pre(load_one(p + r * L.rstride), a[0]));
         }
     }
-    static_assert(RED_U == 4);
-    __shared__ Acc sm[256 * E];
+    Acc v[E];
 #pragma unroll
-    for (int e = 0; e < E; ++e)
-        sm[threadIdx.x * E + e] = P::combine(P::combine(acc[0][e], acc[1][e]), P::combine(acc[2][e], acc[3][e]));
-    __syncthreads();
+    for (int e = 0; e < E; ++e) {
+        v[e] = acc[0][e];
+#pragma unroll
+        for (int u = 1; u < U; ++u) v[e] = P::combine(v[e], acc[u][e]);
+    }
+    cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
+    const int64_t out0 = outer * L.inner + col0; // flat output index of this thread's first column
+    if (L.splits == 1) {
+        if (ty == 0 && active) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e]);
+        }
+        return;
+    }
+    uint32_t zero = 0;
     if (ty == 0 && active) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-            if (e < ecnt && col0 + e < L.inner) {
-                Acc r = sm[tx * E + e];
-                for (int y = 1; y < TY; ++y) r = P::combine(r, sm[(y * TX + tx) * E + e]);
-                if (L.splits == 1) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(r);
-                else partial[(int64_t)split * L.m + outer * L.inner + col0 + e] = r;
-            }
+        for (int e = 0; e < E; ++e)
+            if (e < ecnt && col0 + e < L.inner) zero |= slot_publish(partial + (int64_t)split * L.m + out0 + e, v[e]);
+    }
+    if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
+    // pass two: thread row ty folds splits ty, ty + TY, ... in increasing order
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = P::identity();
+    if (active) {
+        for (int sidx = ty; sidx < L.splits; sidx += TY) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (e < ecnt && col0 + e < L.inner)
+                    v[e] = P::combine(v[e], slot_read(partial + (int64_t)sidx * L.m + out0 + e));
         }
+    }
+    cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
+    if (ty == 0 && active) {
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e]);
     }
 }
 
@@ -435,13 +572,37 @@ template <bool IS_MAX, class T> DPX_D void arg_merge(T &v, int64_t &i, T ov, int
     }
 }
 
-// FIRST: reads src, position = index along the reduced run; otherwise reads the partial
-// (value, position) pairs of the previous pass, laid out [output][split].
-// Linear block id = oblock * splits + split, lanes per output as in red_rows_kernel.
-template <class T, bool IS_MAX, bool CONTIG, bool FIRST>
-__global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L, const T *src,
-                                                       const int64_t *src_idx, int64_t *dst, T *pval,
-                                                       int64_t *pidx)
+// Folds (value, position) pairs like group_reduce; result valid in lane 0 / thread 0.
+template <bool IS_MAX, class VT> DPX_D void arg_group_reduce(VT &best, int64_t &bidx, bool whole_block, int G)
+{
+    const int wl = whole_block ? 64 : G;
+    for (int off = wl >> 1; off > 0; off >>= 1) {
+        const VT ov = shfl_down_any(best, off);
+        const int64_t oi = shfl_down_any(bidx, off);
+        arg_merge<IS_MAX, VT>(best, bidx, ov, oi);
+    }
+    if (whole_block) {
+        __shared__ VT smv[16];
+        __shared__ int64_t smi[16];
+        __syncthreads();
+        const int w = threadIdx.x >> 6;
+        if ((threadIdx.x & 63) == 0) {
+            smv[w] = best;
+            smi[w] = bidx;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int nw = blockDim.x >> 6;
+            for (int i = 1; i < nw; ++i) arg_merge<IS_MAX, VT>(best, bidx, smv[i], smi[i]);
+        }
+    }
+}
+
+// Position = index along the reduced run.  Linear block id = oblock * splits + split, lanes
+// per output as in red_rows_kernel; partial (value, position) pairs laid out [output][split].
+template <class T, bool IS_MAX, bool CONTIG>
+__global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst,
+                                                       Slot<T> *pval, Slot<int64_t> *pidx, unsigned *counters)
 {
     using VT = value_of_t<T>;
     constexpr int E = 16 / (int)sizeof(T);
@@ -461,12 +622,7 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         const T *p = src + so;
-        if constexpr (!FIRST) {
-            const int64_t *pi = src_idx + so;
-            for (int64_t pos = beg + lane; pos < end; pos += G)
-                arg_merge<IS_MAX, VT>(best, bidx, to_value(load_one(p + pos)), pi[pos]);
-        }
-        else if constexpr (CONTIG) {
+        if constexpr (CONTIG) {
             uint32_t bl = 0; // position relative to beg; chunk < 2^32 by construction
             bool have = false;
             if (L.vec) {
@@ -548,43 +704,35 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
             }
         }
     }
-    const int wl = whole_block ? 64 : G;
-    for (int off = wl >> 1; off > 0; off >>= 1) {
-        const VT ov = shfl_down_any(best, off);
-        const int64_t oi = shfl_down_any(bidx, off);
-        arg_merge<IS_MAX, VT>(best, bidx, ov, oi);
+    arg_group_reduce<IS_MAX, VT>(best, bidx, whole_block, G);
+    if (L.splits == 1) {
+        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = bidx;
+        return;
     }
-    if (whole_block) {
-        __shared__ VT smv[16];
-        __shared__ int64_t smi[16];
-        const int w = threadIdx.x >> 6;
-        if ((threadIdx.x & 63) == 0) {
-            smv[w] = best;
-            smi[w] = bidx;
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            const int nw = blockDim.x >> 6;
-            for (int i = 1; i < nw; ++i) arg_merge<IS_MAX, VT>(best, bidx, smv[i], smi[i]);
-        }
+    uint32_t zero = 0;
+    if (threadIdx.x == 0) {
+        zero = slot_publish(pval + o * L.splits + split, to_storage<T>(best));
+        zero |= slot_publish(pidx + o * L.splits + split, bidx);
     }
-    if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) {
-        if (L.splits == 1) dst[dof] = bidx;
-        else {
-            pval[o * L.splits + split] = to_storage<T>(best);
-            pidx[o * L.splits + split] = bidx;
-        }
-    }
+    if (!last_block_of(counters + o, L.splits, zero)) return;
+    best = VT{};
+    bidx = ARG_NONE;
+    for (int i = threadIdx.x; i < L.splits; i += blockDim.x)
+        arg_merge<IS_MAX, VT>(best, bidx, to_value(slot_read(pval + o * L.splits + i)),
+                              slot_read(pidx + o * L.splits + i));
+    arg_group_reduce<IS_MAX, VT>(best, bidx, true, G);
+    if (threadIdx.x == 0) dst[dof] = bidx;
 }
 
 // Column variant (reduced axis strided by L.rstride, outputs contiguous).  One column per
-// thread; partials laid out [split][output].
-template <class T, bool IS_MAX, bool FIRST>
-__global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L, const T *src,
-                                                      const int64_t *src_idx, int64_t *dst, T *pval,
-                                                      int64_t *pidx)
+// thread, 256 threads per block; partials laid out [split][output].
+template <class T, bool IS_MAX>
+__global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst,
+                                                      Slot<T> *pval, Slot<int64_t> *pidx, unsigned *counters)
 {
     using VT = value_of_t<T>;
+    __shared__ VT smv[256];
+    __shared__ int64_t smi[256];
     const int TX = 1 << L.g_log2, TY = 256 >> L.g_log2;
     const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> L.g_log2;
     int64_t b = blockIdx.x;
@@ -611,49 +759,57 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
         const T *p = src + so + col;
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
-        if constexpr (FIRST) {
-            int64_t r = beg + ty;
-            for (; r + (RED_U - 1) * TY < end; r += RED_U * TY) {
-                T v[RED_U];
+        int64_t r = beg + ty;
+        for (; r + (RED_U - 1) * TY < end; r += RED_U * TY) {
+            T v[RED_U];
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
+            for (int u = 0; u < RED_U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                for (int u = 0; u < RED_U; ++u) {
-                    const VT x = to_value(v[u]);
-                    if (bidx == ARG_NONE || arg_better<IS_MAX, VT>(x, best)) {
-                        best = x;
-                        bidx = r + u * TY;
-                    }
-                }
-            }
-            for (; r < end; r += TY) {
-                const VT x = to_value(load_one(p + r * L.rstride));
+            for (int u = 0; u < RED_U; ++u) {
+                const VT x = to_value(v[u]);
                 if (bidx == ARG_NONE || arg_better<IS_MAX, VT>(x, best)) {
                     best = x;
-                    bidx = r;
+                    bidx = r + u * TY;
                 }
             }
         }
-        else {
-            const int64_t *pi = src_idx + so + col;
-            for (int64_t r = beg + ty; r < end; r += TY)
-                arg_merge<IS_MAX, VT>(best, bidx, to_value(load_one(p + r * L.rstride)), pi[r * L.rstride]);
+        for (; r < end; r += TY) {
+            const VT x = to_value(load_one(p + r * L.rstride));
+            if (bidx == ARG_NONE || arg_better<IS_MAX, VT>(x, best)) {
+                best = x;
+                bidx = r;
+            }
         }
     }
-    __shared__ VT smv[256];
-    __shared__ int64_t smi[256];
-    smv[threadIdx.x] = best;
-    smi[threadIdx.x] = bidx;
-    __syncthreads();
+    auto combine_rows = [&]() {
+        __syncthreads();
+        smv[threadIdx.x] = best;
+        smi[threadIdx.x] = bidx;
+        __syncthreads();
+        if (ty == 0)
+            for (int y = 1; y < TY; ++y) arg_merge<IS_MAX, VT>(best, bidx, smv[y * TX + tx], smi[y * TX + tx]);
+    };
+    combine_rows();
+    const int last = ix.nd_i - 1;
+    const int64_t out = outer * L.inner + col;
+    if (L.splits == 1) {
+        if (ty == 0 && active) dst[dof + col * ix.dst_str[last]] = bidx;
+        return;
+    }
+    uint32_t zero = 0;
     if (ty == 0 && active) {
-        for (int y = 1; y < TY; ++y) arg_merge<IS_MAX, VT>(best, bidx, smv[y * TX + tx], smi[y * TX + tx]);
-        const int last = ix.nd_i - 1;
-        if (L.splits == 1) dst[dof + col * ix.dst_str[last]] = bidx;
-        else {
-            pval[(int64_t)split * L.m + outer * L.inner + col] = to_storage<T>(best);
-            pidx[(int64_t)split * L.m + outer * L.inner + col] = bidx;
-        }
+        zero = slot_publish(pval + (int64_t)split * L.m + out, to_storage<T>(best));
+        zero |= slot_publish(pidx + (int64_t)split * L.m + out, bidx);
     }
+    if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
+    best = VT{};
+    bidx = ARG_NONE;
+    if (active)
+        for (int sidx = ty; sidx < L.splits; sidx += TY)
+            arg_merge<IS_MAX, VT>(best, bidx, to_value(slot_read(pval + (int64_t)sidx * L.m + out)),
+                                  slot_read(pidx + (int64_t)sidx * L.m + out));
+    combine_rows();
+    if (ty == 0 && active) dst[dof + col * ix.dst_str[last]] = bidx;
 }
 
 } // namespace dpx

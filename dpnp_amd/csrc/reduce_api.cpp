@@ -45,7 +45,6 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
         if (op == DPX_R_SUMSQDEV && dst->dtype == DPX_HALF) acc = 4;
-        red_finish_fold(pl, acc, false);
         red_export_plan(pl, plan_out, acc);
         return DPX_OK;
     }
@@ -69,7 +68,6 @@ static int argreduce_call(int op, const dpx_array_view *src, int trailing, const
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, nullptr, true, itemsize_of(src->dtype), true);
     if (plan_out) {
-        red_finish_fold(pl, itemsize_of(src->dtype), true);
         red_export_plan(pl, plan_out, itemsize_of(src->dtype) + 8);
         return DPX_OK;
     }

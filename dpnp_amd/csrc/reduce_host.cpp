@@ -53,8 +53,15 @@ static int ceil_log2(int64_t v)
 }
 static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Measured on MI355X (2^28 floats): HBM streams best when each CU runs about 8 waves with
+// 4 x 16-byte loads in flight per lane (85-87 % of peak); 16 or 32 waves per CU, or
+// 1024-thread blocks, lose 5-10 points, and a grid that is not a multiple of the CU count
+// loses as much to the tail.  Hence: 256-thread blocks, two per CU when a reduction has to
+// be split.
+static int64_t red_target_blocks() { return env_int("DPX_RED_TARGET_BLOCKS", 2 * device_cus()); }
+
 // lanes cooperating on one output of `n` elements read `e` at a time: aim at ~8 accesses
-// per lane; more than a wave means a whole 256- or 1024-thread block
+// per lane; more than a wave means a whole 256-thread block
 static void rows_geometry(int64_t n, int e, int &g_log2, int &block)
 {
     int64_t lanes = cdiv(n, (int64_t)e * 8);
@@ -64,13 +71,13 @@ static void rows_geometry(int64_t n, int e, int &g_log2, int &block)
         g_log2 = ceil_log2(lanes);
         block = 256;
     }
-    else if (lanes <= 256) {
-        g_log2 = 8;
-        block = 256;
+    else if (forced >= 7 && forced <= 10) {
+        g_log2 = forced;
+        block = 1 << forced;
     }
     else {
-        g_log2 = 10;
-        block = 1024;
+        g_log2 = 8;
+        block = 256;
     }
 }
 
@@ -139,7 +146,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
 
     const int E = 16 / in_size;
-    const int64_t target = env_int("DPX_RED_TARGET_BLOCKS", 4 * device_cus());
+    const int64_t target = red_target_blocks();
     const uintptr_t base = (uintptr_t)src->data + (uintptr_t)(pl.src_off * in_size);
     const int last = nd_i - 1;
     const int64_t inner = ishape[last];
@@ -160,8 +167,11 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         const int64_t oblocks = cdiv(m, opb);
         int64_t splits = 1;
         const int64_t per_pass = G * e * 8; // elements one group covers with 8 accesses per lane
-        if (oblocks < target && n >= 2 * per_pass) splits = std::min(cdiv(target, oblocks), cdiv(n, per_pass));
-        if (arg) splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
+        // splitting needs a whole block per output (G > 64) and one ticket counter per output
+        if (G > 64 && oblocks < target && oblocks <= RED_MAX_TICKETS && n >= 2 * per_pass)
+            splits = std::min(cdiv(target, oblocks), cdiv(n, per_pass));
+        if (arg && G > 64 && oblocks <= RED_MAX_TICKETS)
+            splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
         int64_t chunk = cdiv(n, splits);
         chunk = cdiv(chunk, G * e) * (G * e);
         splits = cdiv(n, chunk);
@@ -171,27 +181,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         pl.path = !contig_red ? DPX_PATH_RED_GENERIC
                               : (splits > 1 ? DPX_PATH_RED_ROWS_SPLIT
                                             : (G == 1 ? DPX_PATH_RED_SMALL : DPX_PATH_RED_ROWS));
-        if (splits > 1) {
-            pl.scratch_elems = m * splits;
-            pl.fold_cols = false;
-            pl.fix = ix;
-            int64_t st = splits;
-            for (int d = nd_i - 1; d >= 0; --d) {
-                pl.fix.src_istr[d] = st;
-                st *= ishape[d];
-                pl.fix.aux_str[d] = 0;
-            }
-            pl.fix.nd_r = 1;
-            pl.fix.shape_r[0] = splits;
-            pl.fix.src_rstr[0] = 1;
-            RedLaunch &F = pl.fL;
-            F = RedLaunch{};
-            F.m = m;
-            F.n = splits;
-            F.splits = 1;
-            F.vec = 0; // set by red_finish_fold once the partial size is known
-            F.chunk = splits;
-        }
+        if (splits > 1) pl.scratch_elems = m * splits;
         return;
     }
     // ---- cols -----------------------------------------------------------------------
@@ -203,72 +193,37 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     L.vec = vec ? 1 : 0;
     L.rstride = rstride;
     L.inner = inner;
-    int lg = std::min(8, ceil_log2(cdiv(inner, e)));
+    // TX threads side by side cover 512 contiguous bytes of a row (32 x 16 B); up to 16 thread
+    // rows walk down the reduced axis: 512-thread blocks, one per CU when splitting
+    int lg = std::min(arg ? 6 : 5, ceil_log2(cdiv(inner, e)));
     const int forced = env_int("DPX_COLS_TX_LOG2", -1); // experiment knob
-    if (forced >= 0 && forced <= 8) lg = std::min(lg, forced);
+    if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(inner, e)), forced);
     L.g_log2 = lg;
-    const int64_t TX = (int64_t)1 << lg, TY = 256 / TX;
+    const int64_t TX = (int64_t)1 << lg;
+    int block = 256;
+    if (!arg) {
+        int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
+        block = (int)std::min<int64_t>(512, std::max<int64_t>(64, TX * ty));
+        const int fb = env_int("DPX_COLS_BLOCK", 0); // experiment knob
+        if (fb == 256 || fb == 512 || fb == 1024) block = fb;
+        if (block < TX) block = (int)TX;
+    }
+    const int64_t TY = block / TX;
     L.col_blocks = cdiv(inner, TX * e);
     const int64_t outer = m / inner;
     const int64_t base_blocks = L.col_blocks * outer;
+    const int64_t want = std::max<int64_t>(target * 256 / block, 1); // same number of threads in flight
     int64_t splits = 1;
-    if (base_blocks < target && n >= 2 * TY * 8) splits = std::min(cdiv(target, base_blocks), cdiv(n, TY * 8));
+    if (base_blocks < want && base_blocks <= RED_MAX_TICKETS && n >= 2 * TY * 8)
+        splits = std::min(cdiv(want, base_blocks), cdiv(n, TY * 8));
     int64_t chunk = cdiv(n, splits);
     splits = cdiv(n, chunk);
     L.chunk = chunk;
     L.splits = (int32_t)splits;
-    pl.block = 256;
+    pl.block = block;
     pl.grid = base_blocks * splits;
     pl.path = splits > 1 ? DPX_PATH_RED_COLS_SPLIT : DPX_PATH_RED_COLS;
-    if (splits > 1) {
-        pl.scratch_elems = m * splits;
-        pl.fold_cols = true;
-        pl.fix = ix;
-        int64_t st = 1;
-        for (int d = nd_i - 1; d >= 0; --d) {
-            pl.fix.src_istr[d] = st;
-            st *= ishape[d];
-            pl.fix.aux_str[d] = 0;
-        }
-        pl.fix.nd_r = 1;
-        pl.fix.shape_r[0] = splits;
-        pl.fix.src_rstr[0] = m;
-        RedLaunch &F = pl.fL;
-        F = RedLaunch{};
-        F.m = m;
-        F.n = splits;
-        F.splits = 1;
-        F.chunk = splits;
-        F.rstride = m;
-        F.inner = inner;
-    }
-}
-
-// Launch geometry of the fold pass, which depends on the byte size of a partial.
-void red_finish_fold(RedPlan &pl, int acc_size, bool arg)
-{
-    if (pl.L.splits <= 1) return;
-    RedLaunch &F = pl.fL;
-    const int E = 16 / acc_size;
-    if (!pl.fold_cols) {
-        const bool vec = !arg && (F.n % E == 0);
-        F.vec = vec ? 1 : 0;
-        rows_geometry(F.n, vec ? E : 1, F.g_log2, pl.fblock);
-        const int64_t G = (int64_t)1 << F.g_log2;
-        const int64_t opb = (G <= 64) ? 256 / G : 1;
-        F.chunk = cdiv(F.n, G * (vec ? E : 1)) * G * (vec ? E : 1);
-        pl.fgrid = cdiv(F.m, opb);
-    }
-    else {
-        const bool vec = !arg && (F.inner % E == 0) && (F.m % E == 0);
-        const int e = vec ? E : 1;
-        F.vec = vec ? 1 : 0;
-        const int lg = std::min(8, ceil_log2(cdiv(F.inner, e)));
-        F.g_log2 = lg;
-        F.col_blocks = cdiv(F.inner, ((int64_t)1 << lg) * e);
-        pl.fblock = 256;
-        pl.fgrid = F.col_blocks * (F.m / F.inner);
-    }
+    if (splits > 1) pl.scratch_elems = m * splits;
 }
 
 void red_export_plan(const RedPlan &pl, dpx_plan *out, int acc_size)
@@ -294,7 +249,7 @@ void red_export_plan(const RedPlan &pl, dpx_plan *out, int acc_size)
     out->grid[1] = out->grid[2] = 1;
     out->block = pl.block;
     out->splits = pl.L.splits;
-    out->scratch_bytes = pl.scratch_elems * acc_size;
+    out->scratch_bytes = pl.scratch_elems ? (int64_t)RED_COUNTER_BYTES + pl.scratch_elems * ((acc_size + 3) / 4 * 4) : 0;
 }
 
 } // namespace dpx
