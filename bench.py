@@ -57,6 +57,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ops", default="add,sum_axis1,sum_axis0,argmax",
+                    help="subset of add,sum_axis1,sum_axis0,argmax,copy to run (profiling runs); the metric is "
+                         "the default set")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -87,12 +90,19 @@ def main():
     M = a.reshape(side, side)
     r1, r0 = dpnp.empty(side, dtype="f4"), dpnp.empty(side, dtype="f4")
     idx = dpnp.empty((), dtype="i8")
-    ops = [
+    all_ops = [
         ("add", lambda: dpnp.add(a, b, out=c), 12 * n),
         ("sum_axis1", lambda: dpnp.sum(M, axis=1, out=r1), 4 * n + 4 * side),
         ("sum_axis0", lambda: dpnp.sum(M, axis=0, out=r0), 4 * n + 4 * side),
         ("argmax", lambda: dpnp.argmax(x, out=idx), 4 * n + 8),
+        # plain copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        ("copy", lambda: dpnp.copyto(c, a), 8 * n),
     ]
+    wanted = [w for w in args.ops.split(",") if w]
+    ops = [o for o in all_ops if o[0] in wanted]
+    if not ops or len(ops) != len(wanted):
+        print(f"--ops: unknown op in {wanted}", file=sys.stderr)
+        sys.exit(2)
     step_bytes = sum(nb for _, _, nb in ops)
 
     def step(events=None):
@@ -124,7 +134,7 @@ def main():
         ms = sum(ev[s][k][0].elapsed_time(ev[s][k][1]) for s in range(args.steps)) / args.steps
         per_op[name] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4),
                         "elements/s": round(n / ms * 1e3)}
-    add_ms = per_op["add"]["ms"]
+    add_ms = per_op["add"]["ms"] if "add" in per_op else float("nan")
     out = {
         "metric": "achieved HBM GB/s for fp32 add, axis-sum, argmax at 2^28 elements",
         "value": round(step_bytes / ms_per_step / 1e6, 1),
@@ -138,7 +148,8 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic (seeded uniform[-1,1) and normal(0,1), resident in HBM)",
-        "config": {"workload": "fp32 add 2^28 + sum axis=-1 and axis=0 over 16384x16384 + argmax 2^28 (->int64)",
+        "config": {"workload": "fp32 add 2^28 + sum axis=-1 and axis=0 over 16384x16384 + argmax 2^28 (->int64)"
+                   if args.ops == ap.get_default("ops") else "subset: " + args.ops,
                    "bytes_per_step": step_bytes, "frac_of_hbm_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4)},
         "per_op": per_op,
         "roofline": {"bound": "hbm", "kernel": "ew_contig_kernel<add,f32> (c = a + b, 2^28 elements)",
