@@ -29,7 +29,7 @@ constexpr int EW_CONTIG_BLOCK = 64; // default for contiguous kernels: one wave
 constexpr int EW_ROWS_BLOCK = 256;  // default for strided kernels
 
 // operand access mode along the inner dimension (2 bits per operand)
-enum : uint32_t { MODE_STRIDED = 0, MODE_VEC = 1, MODE_BCAST = 2 };
+enum : uint32_t { MODE_STRIDED = 0, MODE_VEC = 1, MODE_BCAST = 2, MODE_VEC2 = 3 };
 
 template <int NOPS> struct NdIndex {
     int32_t nd; // >= 1; the last dim is the inner one
@@ -116,18 +116,29 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     constexpr int E = ew_traits<Out, Ins...>::E;
     const int tx = threadIdx.x & ((1 << tx_log2) - 1);
     const int ty = threadIdx.x >> tx_log2;
-    const int64_t rb = (int64_t)blockIdx.x / col_blocks;
-    const int64_t cb = (int64_t)blockIdx.x - rb * col_blocks;
-    const int64_t row = rb * ((int)blockDim.x >> tx_log2) + ty;
+    // blockIdx.x < 2^31 and col_blocks <= gridDim.x: 32-bit division
+    const uint32_t rb = blockIdx.x / (uint32_t)col_blocks;
+    const uint32_t cb = blockIdx.x - rb * (uint32_t)col_blocks;
+    const int64_t row = (int64_t)rb * ((int)blockDim.x >> tx_log2) + ty;
     const int inner = ix.nd - 1;
     const int64_t ncols = ix.shape[inner];
-    const int64_t col0 = ((cb << tx_log2) + tx) * E;
+    const int64_t col0 = (((int64_t)cb << tx_log2) + tx) * E;
     if (row >= nrows || col0 >= ncols) return;
 
     int64_t off[N + 1];
 #pragma unroll
     for (int k = 0; k <= N; ++k) off[k] = col0 * ix.strides[k][inner];
-    {
+    if (nrows <= 0x7fffffff) { // the usual case: 32-bit div/mod chain
+        uint32_t r = (uint32_t)row;
+        for (int d = inner - 1; d >= 0; --d) {
+            const uint32_t q = (d == 0) ? 0u : r / (uint32_t)ix.shape[d];
+            const int64_t i = r - q * (uint32_t)ix.shape[d];
+#pragma unroll
+            for (int k = 0; k <= N; ++k) off[k] += i * ix.strides[k][d];
+            r = q;
+        }
+    }
+    else {
         int64_t r = row;
         for (int d = inner - 1; d >= 0; --d) {
             const int64_t q = (d == 0) ? 0 : r / ix.shape[d];
@@ -147,6 +158,16 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         }
         else if (mode == MODE_BCAST) {
             r = splat<T, E>(load_one(p + o));
+        }
+        else if (mode == MODE_VEC2 && cnt == E && col0 + E < ncols) {
+            // stride 2 (x[:, ::2], real/imag parts): two contiguous 16-byte loads, keep every
+            // other element.  The loads reach one element past the last one used, which lies
+            // inside the view for every pack but the last of a row (that one goes scalar).
+            if constexpr (E >= 2) {
+                const pack<T, E> lo = load_pack<T, E>(p + o), hi = load_pack<T, E>(p + o + E);
+#pragma unroll
+                for (int e = 0; e < E; ++e) r.v[e] = (2 * e < E) ? lo.v[(2 * e) % E] : hi.v[(2 * e) % E];
+            }
         }
         else {
 #pragma unroll
@@ -182,6 +203,91 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_rows_kernel(Fn fn,
                                   std::index_sequence_for<Ins...>{});
 }
 
+// ---- transposing through an LDS tile ------------------------------------------------------
+// For calls where the output is contiguous along the inner dim but some inputs are
+// contiguous along another dim `dT` (op(A.T, out=C), op(A.T, B), ...).  A block owns a
+// TS x TS tile of the (dT, inner) plane: inputs flagged in `tmask` are read with threads
+// side by side along dT (coalesced for them) into padded LDS tiles, then every thread
+// computes with threads side by side along the inner dim (coalesced for the output and
+// the other inputs).  Remaining dims are batch dims decoded from the block index.
+template <class Out, class... Ins> struct tile_traits {
+    static constexpr int TS = max_sizeof<Out, Ins...>() <= 4 ? 64 : 32;
+};
+
+template <class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out *out,
+                        const InPtrs<sizeof...(Ins)> &in, uint32_t tmask, int dT, int64_t tiles_t,
+                        int64_t tiles_i, unsigned char *smem, std::index_sequence<I...>)
+{
+    constexpr int N = sizeof...(Ins);
+    constexpr int TS = tile_traits<Out, Ins...>::TS;
+    constexpr int STEP = EW_BLOCK / TS;
+    constexpr size_t sizes[N] = {(size_t)TS * (TS + 1) * sizeof(Ins)...};
+    const int inner = ix.nd - 1;
+    int64_t b = blockIdx.x;
+    const int64_t ti = b % tiles_i;
+    b /= tiles_i;
+    const int64_t tt = b % tiles_t;
+    b /= tiles_t;
+    int64_t off[N + 1];
+#pragma unroll
+    for (int k = 0; k <= N; ++k) off[k] = 0;
+    for (int d = inner - 1; d >= 0; --d) {
+        if (d == dT) continue;
+        const int64_t q = b / ix.shape[d];
+        const int64_t i = b - q * ix.shape[d];
+#pragma unroll
+        for (int k = 0; k <= N; ++k) off[k] += i * ix.strides[k][d];
+        b = q;
+    }
+    const int64_t i0 = tt * TS, j0 = ti * TS;
+    const int64_t ni = ix.shape[dT], nj = ix.shape[inner];
+    const int lo = threadIdx.x % TS, hi = threadIdx.x / TS;
+    // phase 1: transposed inputs -> LDS, threads adjacent along dT
+    auto stage = [&](auto *p, int k, size_t lds_off) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        if (!((tmask >> k) & 1u)) return;
+        T *tile = reinterpret_cast<T *>(smem + lds_off);
+        if (i0 + lo < ni) {
+            const int64_t base = off[k] + (i0 + lo) * ix.strides[k][dT];
+            for (int bb = hi; bb < TS; bb += STEP)
+                if (j0 + bb < nj) tile[bb * (TS + 1) + lo] = load_one(p + base + (j0 + bb) * ix.strides[k][inner]);
+        }
+    };
+    size_t lds_off[N];
+    {
+        size_t acc = 0;
+        for (int k = 0; k < N; ++k) {
+            lds_off[k] = acc;
+            acc += (sizes[k] + 15) & ~(size_t)15;
+        }
+    }
+    (stage((const Ins *)in.p[I], (int)I, lds_off[I]), ...);
+    __syncthreads();
+    // phase 2: compute, threads adjacent along the inner dim
+    if (j0 + lo >= nj) return;
+    auto fetch = [&](auto *p, int k, size_t l_off, int aa) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        if ((tmask >> k) & 1u) return reinterpret_cast<const T *>(smem + l_off)[lo * (TS + 1) + aa];
+        return load_one(p + off[k] + (i0 + aa) * ix.strides[k][dT] + (j0 + lo) * ix.strides[k][inner]);
+    };
+    for (int aa = hi; aa < TS; aa += STEP) {
+        if (i0 + aa >= ni) break;
+        out[off[N] + (i0 + aa) * ix.strides[N][dT] + (j0 + lo) * ix.strides[N][inner]] =
+            to_storage<Out>(fn(to_value(fetch((const Ins *)in.p[I], (int)I, lds_off[I], aa))...));
+    }
+}
+
+template <class Fn, class Out, class... Ins>
+__global__ __launch_bounds__(EW_BLOCK) void ew_tile_kernel(Fn fn, NdIndex<sizeof...(Ins) + 1> ix, Out *out,
+                                                          InPtrs<sizeof...(Ins)> in, uint32_t tmask, int dT,
+                                                          int64_t tiles_t, int64_t tiles_i)
+{
+    extern __shared__ __align__(16) unsigned char ew_tile_smem[];
+    ew_tile_body<Fn, Out, Ins...>(fn, ix, out, in, tmask, dT, tiles_t, tiles_i, ew_tile_smem,
+                                  std::index_sequence_for<Ins...>{});
+}
+
 // ---- host-side plan (element-type independent) ----------------------------------
 struct EwPlan {
     int path; // dpx_path
@@ -198,6 +304,10 @@ struct EwPlan {
     int tx_log2;
     int block; // threads per block
     int64_t nrows, col_blocks, grid;
+    // tile path
+    uint32_t tmask; // inputs staged through LDS
+    int dT;         // the dim those inputs are contiguous along
+    int64_t tiles_t, tiles_i;
 };
 
 // fills path/nd/shape/strides/offsets from (already validated) views
@@ -205,6 +315,8 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views);
 // fills the launch parameters for E elements per thread and the operands' item sizes
 // and (displaced) base pointers
 void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs);
+// tile geometry for tile side TS (call after ew_finish_plan when pl.path == DPX_PATH_EW_TILE)
+void ew_finish_tile_plan(EwPlan &pl, int TS);
 
 // dry != 0: only fill the launch parameters of pl
 template <class Fn, class Out, class... Ins>
@@ -218,6 +330,9 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
     for (int k = 0; k <= N; ++k)
         ptrs[k] = (const char *)views[k]->data + pl.offsets[k] * sizes[k];
     ew_finish_plan(pl, E, sizes, ptrs);
+    if constexpr (N >= 1) {
+        if (pl.path == DPX_PATH_EW_TILE) ew_finish_tile_plan(pl, tile_traits<Out, Ins...>::TS);
+    }
     if (pl.path == DPX_PATH_NOOP || dry) return hipSuccess;
     InPtrs<N> in;
     for (int k = 0; k < N; ++k) in.p[k] = ptrs[k];
@@ -238,6 +353,17 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
         for (int d = 0; d < DPX_MAX_ND; ++d) {
             ix.shape[d] = d < pl.nd ? pl.shape[d] : 1;
             for (int k = 0; k <= N; ++k) ix.strides[k][d] = d < pl.nd ? pl.strides[k][d] : 0;
+        }
+        if (pl.path == DPX_PATH_EW_TILE) {
+            if constexpr (N >= 1) {
+                using TT = tile_traits<Out, Ins...>;
+                size_t smem = 0;
+                const size_t sz[N] = {(size_t)TT::TS * (TT::TS + 1) * sizeof(Ins)...};
+                for (int k = 0; k < N; ++k) smem += (sz[k] + 15) & ~(size_t)15;
+                hipLaunchKernelGGL((ew_tile_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(EW_BLOCK), smem,
+                                   stream, fn, ix, out, in, pl.tmask, pl.dT, pl.tiles_t, pl.tiles_i);
+            }
+            return hipGetLastError();
         }
         hipLaunchKernelGGL((ew_rows_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid),
                            dim3(pl.block), 0, stream, fn, ix, out, in, pl.modes, pl.tx_log2,

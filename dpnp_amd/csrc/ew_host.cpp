@@ -71,6 +71,44 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     for (int k = 0; k + 1 < nops && contig; ++k)
         contig = pl.strides[k][0] == 1 || pl.strides[k][0] == 0;
     pl.path = contig ? DPX_PATH_EW_CONTIG : DPX_PATH_EW_ROWS;
+    pl.tmask = 0;
+    pl.dT = -1;
+    if (contig || pl.nd < 2 || nops < 2) return;
+    // Transposed operands: the output runs along the inner dim, some input runs along another
+    // dim dT (stride 1 there, a long stride along the inner dim).  All such inputs must agree
+    // on dT; the others are read in output orientation.
+    const int inner = pl.nd - 1;
+    if (pl.strides[nops - 1][inner] != 1 || pl.shape[inner] < 16) return;
+    int dT = -1;
+    uint32_t tmask = 0;
+    for (int k = 0; k + 1 < nops; ++k) {
+        const int64_t si = pl.strides[k][inner];
+        if (si == 0 || si == 1 || si == -1 || si == 2) continue; // row oriented (or a cheap stride)
+        int d1 = -1;
+        for (int d = 0; d < inner; ++d)
+            if (pl.strides[k][d] == 1 && pl.shape[d] >= 16) d1 = d;
+        if (d1 < 0) continue;         // strided both ways: nothing to gain from staging
+        if (dT >= 0 && d1 != dT) return; // two different orientations: keep the generic kernel
+        dT = d1;
+        tmask |= 1u << k;
+    }
+    if (tmask) {
+        pl.path = DPX_PATH_EW_TILE;
+        pl.tmask = tmask;
+        pl.dT = dT;
+    }
+}
+
+void ew_finish_tile_plan(EwPlan &pl, int TS)
+{
+    const int inner = pl.nd - 1;
+    pl.block = EW_BLOCK;
+    pl.tiles_t = (pl.shape[pl.dT] + TS - 1) / TS;
+    pl.tiles_i = (pl.shape[inner] + TS - 1) / TS;
+    int64_t batch = 1;
+    for (int d = 0; d < inner; ++d)
+        if (d != pl.dT) batch *= pl.shape[d];
+    pl.grid = batch * pl.tiles_t * pl.tiles_i;
 }
 
 void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs)
@@ -89,6 +127,7 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         pl.grid = (pl.n + (int64_t)pl.block * E - 1) / ((int64_t)pl.block * E);
         return;
     }
+    if (pl.path == DPX_PATH_EW_TILE) return; // geometry set by ew_finish_tile_plan
     const int inner = pl.nd - 1;
     const int64_t ncols = pl.shape[inner];
     pl.nrows = pl.n / ncols;
@@ -97,8 +136,8 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         uint32_t mode = MODE_STRIDED;
         const int64_t s = pl.strides[k][inner];
         if (s == 0 && k + 1 < nops) mode = MODE_BCAST;
-        else if (s == 1 && aligned(k)) {
-            mode = MODE_VEC;
+        else if ((s == 1 || (s == 2 && E >= 2 && k + 1 < nops)) && aligned(k)) {
+            mode = s == 1 ? MODE_VEC : MODE_VEC2;
             for (int d = 0; d < inner; ++d)
                 if (pl.strides[k][d] % E != 0) mode = MODE_STRIDED;
         }

@@ -47,6 +47,10 @@ static int where_call(const dpx_array_view *cond, const dpx_array_view *x1, cons
 template <class Cmp, class T, class S> struct WhereCmpFn {
     DPX_D S operator()(V<T> l, V<T> r, S a, S b) const { return Cmp::template apply<T>(l, r) ? a : b; }
 };
+// where(x CMP r, x, b): the compared array is also the first choice, read once
+template <class Cmp, class T> struct WhereCmpSelfFn {
+    DPX_D T operator()(T x, T r, T b) const { return Cmp::template apply<T>(x, r) ? x : b; }
+};
 
 static int where_compare_call(int cmp_op, const dpx_array_view *lhs, const dpx_array_view *rhs,
                               const dpx_array_view *x1, const dpx_array_view *x2,
@@ -69,11 +73,14 @@ static int where_compare_call(int cmp_op, const dpx_array_view *lhs, const dpx_a
     int64_t n = 0;
     if (int rc = ew_validate(5, views, n)) return rc;
     int rc = DPX_ERR_NOT_IMPLEMENTED;
+    const bool self = views_same_logical(lhs, x1);
+    const dpx_array_view *views3[4] = {lhs, rhs, x2, dst};
     auto with_cmp = [&](auto cmptag) {
         using Cmp = typename decltype(cmptag)::type;
         auto with_t = [&](auto ttag) {
             using T = typename decltype(ttag)::type;
-            if (vs == 4) rc = run_ew<WhereCmpFn<Cmp, T, uint32_t>, uint32_t, T, T, uint32_t, uint32_t>({}, views, (hipStream_t)stream, nullptr);
+            if (self) rc = run_ew<WhereCmpSelfFn<Cmp, T>, T, T, T, T>({}, views3, (hipStream_t)stream, nullptr);
+            else if (vs == 4) rc = run_ew<WhereCmpFn<Cmp, T, uint32_t>, uint32_t, T, T, uint32_t, uint32_t>({}, views, (hipStream_t)stream, nullptr);
             else rc = run_ew<WhereCmpFn<Cmp, T, uint64_t>, uint64_t, T, T, uint64_t, uint64_t>({}, views, (hipStream_t)stream, nullptr);
         };
         if (dt == DPX_FLOAT) with_t(tag<float>{});
