@@ -46,7 +46,23 @@ def _operand_dtype(o):
         return WeakFloatingType(o)
     if isinstance(o, complex):
         return WeakComplexType(o)
-    return None
+    a = _foreign_as_numpy(o)
+    return None if a is None else _as_dtype(a.dtype)
+
+
+def _foreign_as_numpy(o):
+    """NumPy form of an operand that is neither an array of this package nor a Python/NumPy
+    scalar (ctypes scalars, objects with the buffer protocol, nested sequences); None if it has
+    no numeric interpretation."""
+    if isinstance(o, (usm_ndarray, np.ndarray, np.generic, bool, int, float, complex)) or o is None:
+        return None
+    try:
+        a = np.asarray(o)
+    except Exception:
+        return None
+    if a.dtype.kind not in "biufc" or a.dtype.itemsize > 16:
+        return None
+    return a
 
 
 def _operand_shape(o):
@@ -54,7 +70,8 @@ def _operand_shape(o):
         return tuple(o.shape)
     if isinstance(o, (bool, int, float, complex, np.generic)):
         return ()
-    return None
+    a = _foreign_as_numpy(o)
+    return None if a is None else tuple(a.shape)
 
 
 def _as_device_array(o, dt):
@@ -65,6 +82,10 @@ def _as_device_array(o, dt):
         from ._copy_utils import from_numpy
 
         return from_numpy(o, dtype=dt)
+    if not isinstance(o, (bool, int, float, complex, np.generic)):
+        from ._copy_utils import from_numpy
+
+        return from_numpy(_foreign_as_numpy(o), dtype=dt)
     v = o.item() if isinstance(o, np.generic) else o
     if dt.kind in "iu" and isinstance(v, int):
         info = np.iinfo(dt)
@@ -136,6 +157,8 @@ class UnaryElementwiseFunc:
             if r is not None:
                 out.append(f"{dt}->{r.char}")
         return out
+
+    types_ = types
 
     def __call__(self, x, /, *, out=None, order="K"):
         if not isinstance(x, usm_ndarray):
@@ -224,6 +247,8 @@ class BinaryElementwiseFunc:
             if r is not None:
                 out.append(f"{dt}{dt}->{r.char}")
         return out
+
+    types_ = types
 
     def _resolve(self, o1, o2):
         is_arr1, is_arr2 = isinstance(o1, usm_ndarray), isinstance(o2, usm_ndarray)
