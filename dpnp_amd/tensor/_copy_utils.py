@@ -11,7 +11,7 @@ from ._usmarray import usm_ndarray
 
 
 def _empty(shape, dtype, order="C"):
-    return usm_ndarray(shape, dtype=dtype, order=order)
+    return usm_ndarray._new_contiguous(tuple(shape), _as_dtype(dtype), order)
 
 
 def _like_strides(shape, stride_lists, dt):

@@ -56,7 +56,7 @@ class Queue:
 
     @property
     def stream_ptr(self):
-        return _torch().cuda.current_stream(self.sycl_device.index).cuda_stream
+        return current_stream_ptr(self.sycl_device.index)
 
     def wait(self):
         _torch().cuda.current_stream(self.sycl_device.index).synchronize()
@@ -69,6 +69,19 @@ class Queue:
 
     def __repr__(self):
         return f"<Queue on {self.sycl_device!r}>"
+
+
+_raw_stream = None
+
+
+def current_stream_ptr(device_index=0):
+    """hipStream_t (as an integer) of torch's current stream on the device."""
+    global _raw_stream
+    if _raw_stream is None:
+        t = _torch()
+        fast = getattr(t._C, "_cuda_getCurrentRawStream", None)
+        _raw_stream = fast if fast is not None else (lambda i: t.cuda.current_stream(i).cuda_stream)
+    return _raw_stream(device_index)
 
 
 _DEFAULT_QUEUE = Queue()
@@ -102,12 +115,18 @@ def gpu_available():
     return t.cuda.is_available()
 
 
+_alloc_state = {}
+
+
 def alloc(nbytes):
     """A device allocation of at least `nbytes` bytes (a uint8 CUDA tensor)."""
-    t = _torch()
-    if not t.cuda.is_available():
-        raise RuntimeError("dpnp_amd needs an AMD GPU: no HIP device is visible to this process")
-    return t.empty(max(int(nbytes), 1), dtype=t.uint8, device="cuda")
+    st = _alloc_state
+    if not st:
+        t = _torch()
+        if not t.cuda.is_available():
+            raise RuntimeError("dpnp_amd needs an AMD GPU: no HIP device is visible to this process")
+        st["empty"], st["u8"], st["dev"] = t.empty, t.uint8, t.device("cuda", t.cuda.current_device())
+    return st["empty"](nbytes if nbytes > 0 else 1, dtype=st["u8"], device=st["dev"])
 
 
 def to_device_bytes(host_bytes_array):

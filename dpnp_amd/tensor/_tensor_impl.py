@@ -16,10 +16,11 @@ def _events(q):
     return e, e
 
 
-def _stream(q):
-    from ._device import default_queue
+from ._device import current_stream_ptr as _current_stream_ptr
 
-    return (q or default_queue()).stream_ptr
+
+def _stream(q):
+    return _current_stream_ptr(0) if q is None else q.stream_ptr
 
 
 def _where(condition, x1, x2, dst, sycl_queue=None, depends=()):

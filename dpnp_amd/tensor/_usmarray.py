@@ -155,6 +155,22 @@ class usm_ndarray:
                          (self._offset + hi + 1) * dt.itemsize > self._buf.numel()):
                 raise ValueError("shape, strides and offset address memory outside the allocation")
 
+    @staticmethod
+    def _new_contiguous(shape, dt, order="C"):
+        """Freshly allocated C- or F-contiguous array (arguments already normalised)."""
+        r = usm_ndarray.__new__(usm_ndarray)
+        size = 1
+        for s in shape:
+            size *= s
+        r._shape = shape
+        r._strides = _contig_strides(shape, order)
+        r._dtype = dt
+        r._offset = 0
+        r._writable = True
+        r._buf = _device.alloc(size * dt.itemsize)
+        r._base = None
+        return r
+
     # -- construction of views -------------------------------------------------------------
     def _view(self, shape, strides, offset, dtype=None):
         r = usm_ndarray.__new__(usm_ndarray)
@@ -178,6 +194,7 @@ class usm_ndarray:
 
         r = reshape(self, new_shape, copy=False)
         self._shape, self._strides = r._shape, r._strides
+        self.__dict__.pop("_cview", None)
 
     @property
     def strides(self):
@@ -238,12 +255,18 @@ class usm_ndarray:
     def _element_offset(self):
         return self._offset
 
-    def _as_view(self, writable=None):
-        """The C descriptor of this array (borrowed; valid while `self` is alive)."""
-        c, f = _contig_flags(self._shape, self._strides)
-        w = self._writable if writable is None else writable
-        flags = (_lib.C_CONTIGUOUS if c else 0) | (_lib.F_CONTIGUOUS if f else 0) | (_lib.WRITABLE if w else 0)
-        return _lib.make_view(self._pointer, self._shape, self._strides, dtype_id(self._dtype), flags)
+    def _as_view(self):
+        """The C descriptor of this array (borrowed; valid while `self` is alive).  Built once:
+        shape, strides, offset and allocation of an array object never change; only the
+        writable bit may."""
+        v = self.__dict__.get("_cview")
+        if v is None:
+            c, f = _contig_flags(self._shape, self._strides)
+            flags = (_lib.C_CONTIGUOUS if c else 0) | (_lib.F_CONTIGUOUS if f else 0)
+            v = _lib.make_view(self._pointer, self._shape, self._strides, dtype_id(self._dtype), flags)
+            self._cview = v
+        v.flags = (v.flags & ~_lib.WRITABLE) | (_lib.WRITABLE if self._writable else 0)
+        return v
 
     @property
     def T(self):
