@@ -26,14 +26,15 @@ UNARY_OPS = [
     "abs", "negative", "positive", "square", "sqrt", "exp", "log", "erf", "sin",
     "cos", "tan", "tanh", "exp2", "expm1", "log2", "log10", "log1p", "rsqrt",
     "cbrt", "reciprocal", "floor", "ceil", "trunc", "sign", "isnan", "isinf",
-    "isfinite", "logical_not", "bitwise_invert", "signbit",
+    "isfinite", "logical_not", "bitwise_invert", "signbit", "asin", "acos", "atan", "sinh",
+    "cosh", "asinh", "acosh", "atanh", "round", "conj", "real", "imag", "proj", "angle",
 ]
 BINARY_OPS = [
     "add", "subtract", "multiply", "divide", "bitwise_and", "bitwise_or",
     "bitwise_xor", "equal", "not_equal", "less", "less_equal", "greater",
     "greater_equal", "maximum", "minimum", "logical_and", "logical_or",
     "logical_xor", "pow", "floor_divide", "remainder", "atan2", "hypot",
-    "copysign", "bitwise_left_shift", "bitwise_right_shift",
+    "copysign", "bitwise_left_shift", "bitwise_right_shift", "logaddexp", "nextafter",
 ]
 REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev"]
 SEARCH_OPS = ["argmax", "argmin"]
@@ -43,7 +44,7 @@ REDUCE_ID = {n: i for i, n in enumerate(REDUCE_OPS)}
 SEARCH_ID = {n: i for i, n in enumerate(SEARCH_OPS)}
 
 PATH_NAMES = {
-    0: "noop", 1: "ew_contig", 2: "ew_rows", 3: "ew_flat", 4: "ew_tile",
+    0: "noop", 1: "ew_contig", 2: "ew_rows", 4: "ew_tile",
     10: "red_rows", 11: "red_rows_split", 12: "red_cols", 13: "red_cols_split",
     14: "red_generic", 15: "red_small",
 }

@@ -100,6 +100,15 @@ DPX_FP_FN1(m_cbrt, ::cbrtf, ::cbrt)
 DPX_FP_FN1(m_floor, ::floorf, ::floor)
 DPX_FP_FN1(m_ceil, ::ceilf, ::ceil)
 DPX_FP_FN1(m_trunc, ::truncf, ::trunc)
+DPX_FP_FN1(m_rint, ::rintf, ::rint)
+DPX_FP_FN1(m_asin, ::asinf, ::asin)
+DPX_FP_FN1(m_acos, ::acosf, ::acos)
+DPX_FP_FN1(m_atan, ::atanf, ::atan)
+DPX_FP_FN1(m_sinh, ::sinhf, ::sinh)
+DPX_FP_FN1(m_cosh, ::coshf, ::cosh)
+DPX_FP_FN1(m_asinh, ::asinhf, ::asinh)
+DPX_FP_FN1(m_acosh, ::acoshf, ::acosh)
+DPX_FP_FN1(m_atanh, ::atanhf, ::atanh)
 #undef DPX_FP_FN1
 #define DPX_FP_FN2(NAME, F32, F64)                                          \
     template <class T> DPX_D T NAME(T x, T y)                               \
@@ -113,6 +122,7 @@ DPX_FP_FN2(m_atan2, ::atan2f, ::atan2)
 DPX_FP_FN2(m_hypot, ::hypotf, ::hypot)
 DPX_FP_FN2(m_copysign, ::copysignf, ::copysign)
 DPX_FP_FN2(m_fmod, ::fmodf, ::fmod)
+DPX_FP_FN2(m_nextafter, ::nextafterf, ::nextafter)
 #undef DPX_FP_FN2
 
 template <class T> DPX_D bool m_signbit(T x)
@@ -126,6 +136,54 @@ template <class T> DPX_D bool m_isinf(T x)
     if constexpr (is_fp_v<T>) { T a = x < T(0) ? -x : x; return a == (T)__builtin_inff(); }
     else return false;
 }
+
+// ---- complex elementary functions (textbook formulas on the real functions above; the
+// reference gets these from the SYCL complex library, results agree to rounding error for
+// finite arguments of moderate size) -----------------------------------------------------------
+template <class R> DPX_D cplx<R> c_exp(cplx<R> z)
+{
+    const R e = m_exp(z.re);
+    if (z.im == R(0)) return {e, z.im};
+    return {e * m_cos(z.im), e * m_sin(z.im)};
+}
+template <class R> DPX_D cplx<R> c_log(cplx<R> z) { return {m_log(m_hypot(z.re, z.im)), m_atan2(z.im, z.re)}; }
+template <class R> DPX_D cplx<R> c_sqrt(cplx<R> z)
+{
+    if (z.re == R(0) && z.im == R(0)) return {R(0), z.im};
+    if (m_isinf(z.im)) return {(R)__builtin_inff(), z.im};
+    const R ar = z.re < R(0) ? -z.re : z.re;
+    const R t = m_sqrt((ar + m_hypot(z.re, z.im)) * R(0.5));
+    if (z.re >= R(0)) return {t, z.im / (t + t)};
+    const R ai = z.im < R(0) ? -z.im : z.im;
+    return {ai / (t + t), m_copysign(t, z.im)};
+}
+template <class R> DPX_D cplx<R> c_sinh(cplx<R> z)
+{
+    if (z.im == R(0)) return {m_sinh(z.re), z.im};
+    return {m_sinh(z.re) * m_cos(z.im), m_cosh(z.re) * m_sin(z.im)};
+}
+template <class R> DPX_D cplx<R> c_cosh(cplx<R> z)
+{
+    if (z.im == R(0)) return {m_cosh(z.re), z.re * z.im};
+    return {m_cosh(z.re) * m_cos(z.im), m_sinh(z.re) * m_sin(z.im)};
+}
+template <class R> DPX_D cplx<R> c_tanh(cplx<R> z)
+{
+    // Kahan's formulation: no cancellation near the poles at x = 0, y = pi/2 + k pi
+    const R ax = z.re < R(0) ? -z.re : z.re;
+    if (ax > R(20)) return {m_copysign(R(1), z.re), m_copysign(R(0), m_sin(z.im + z.im))};
+    const R t = m_tan(z.im);
+    const R beta = R(1) + t * t;
+    const R s = m_sinh(z.re);
+    const R rho = m_sqrt(R(1) + s * s);
+    if (m_isinf(t)) return {rho / s, R(1) / t};
+    const R d = R(1) + beta * s * s;
+    return {beta * rho * s / d, t / d};
+}
+// sin z = -i sinh(iz), cos z = cosh(iz), tan z = -i tanh(iz)
+template <class R> DPX_D cplx<R> c_sin(cplx<R> z) { const cplx<R> w = c_sinh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+template <class R> DPX_D cplx<R> c_cos(cplx<R> z) { return c_cosh(cplx<R>{-z.im, z.re}); }
+template <class R> DPX_D cplx<R> c_tan(cplx<R> z) { const cplx<R> w = c_tanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
 
 template <class T> using V = value_of_t<T>;
 
@@ -285,11 +343,17 @@ struct RemainderOp { // remainder.hpp: Python-style modulo, x % 0 == 0 for ints
     }
 };
 struct PowOp { // pow.hpp: ints by repeated squaring (negative exponent -> 0), fp via pow
-    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T> || is_cplx_v<T>;
     template <class T> using out = T;
     template <class T> DPX_D static T apply(T a, T b)
     {
-        if constexpr (is_int_v<T>) {
+        if constexpr (is_cplx_v<T>) {
+            using R = real_of_t<T>;
+            if (b.re == R(0) && b.im == R(0)) return T{R(1), R(0)};
+            if (a.re == R(0) && a.im == R(0)) return T{R(0), R(0)};
+            return c_exp(b * c_log(a));
+        }
+        else if constexpr (is_int_v<T>) {
             if constexpr (std::is_signed_v<T>) {
                 if (b < 0) return (a == 1) ? T(1) : ((a == -1) ? ((b & 1) ? T(-1) : T(1)) : T(0));
             }
@@ -383,13 +447,24 @@ struct SquareOp { // square.hpp:64-90; bool -> int8
         template <class T> using out = T;                          \
         template <class T> DPX_D static T apply(T x) { return EXPR; } \
     };
-DPX_FP_UNARY(SqrtOp, m_sqrt(x))
-DPX_FP_UNARY(ExpOp, m_exp(x))
-DPX_FP_UNARY(LogOp, m_log(x))
-DPX_FP_UNARY(SinOp, m_sin(x))
-DPX_FP_UNARY(CosOp, m_cos(x))
-DPX_FP_UNARY(TanOp, m_tan(x))
-DPX_FP_UNARY(TanhOp, m_tanh(x))
+// same, with a complex form CEXPR
+#define DPX_FPC_UNARY(NAME, EXPR, CEXPR)                                        \
+    struct NAME {                                                               \
+        template <class T> static constexpr bool ok = is_fp_v<T> || is_cplx_v<T>; \
+        template <class T> using out = T;                                       \
+        template <class T> DPX_D static T apply(T x)                            \
+        {                                                                       \
+            if constexpr (is_cplx_v<T>) return CEXPR;                           \
+            else return EXPR;                                                   \
+        }                                                                       \
+    };
+DPX_FPC_UNARY(SqrtOp, m_sqrt(x), c_sqrt(x))
+DPX_FPC_UNARY(ExpOp, m_exp(x), c_exp(x))
+DPX_FPC_UNARY(LogOp, m_log(x), c_log(x))
+DPX_FPC_UNARY(SinOp, m_sin(x), c_sin(x))
+DPX_FPC_UNARY(CosOp, m_cos(x), c_cos(x))
+DPX_FPC_UNARY(TanOp, m_tan(x), c_tan(x))
+DPX_FPC_UNARY(TanhOp, m_tanh(x), c_tanh(x))
 DPX_FP_UNARY(Exp2Op, m_exp2(x))
 DPX_FP_UNARY(Expm1Op, m_expm1(x))
 DPX_FP_UNARY(Log2Op, m_log2(x))
@@ -397,8 +472,17 @@ DPX_FP_UNARY(Log10Op, m_log10(x))
 DPX_FP_UNARY(Log1pOp, m_log1p(x))
 DPX_FP_UNARY(RsqrtOp, T(1) / m_sqrt(x))
 DPX_FP_UNARY(CbrtOp, m_cbrt(x))
-DPX_FP_UNARY(ReciprocalOp, T(1) / x)
+DPX_FPC_UNARY(ReciprocalOp, T(1) / x, (T{real_of_t<T>(1), real_of_t<T>(0)} / x))
+DPX_FPC_UNARY(SinhOp, m_sinh(x), c_sinh(x))
+DPX_FPC_UNARY(CoshOp, m_cosh(x), c_cosh(x))
+DPX_FP_UNARY(AsinOp, m_asin(x))
+DPX_FP_UNARY(AcosOp, m_acos(x))
+DPX_FP_UNARY(AtanOp, m_atan(x))
+DPX_FP_UNARY(AsinhOp, m_asinh(x))
+DPX_FP_UNARY(AcoshOp, m_acosh(x))
+DPX_FP_UNARY(AtanhOp, m_atanh(x))
 #undef DPX_FP_UNARY
+#undef DPX_FPC_UNARY
 struct ErfOp { // dpnp/backend/kernels/elementwise_functions/erf.hpp:52-95; f2 -> f4
     template <class T> static constexpr bool ok = is_fp_v<T>;
     template <class T> using out = std::conditional_t<std::is_same_v<T, half_t>, float, T>;
@@ -417,12 +501,18 @@ template <int WHICH> struct RoundOp { // floor.hpp / ceil.hpp / trunc.hpp: ident
         else return x;
     }
 };
-struct SignOp { // sign.hpp:63-110 (real types; NaN -> NaN)
-    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
+struct SignOp { // sign.hpp:63-110 (NaN -> NaN; complex: z / |z|, 0 for 0)
+    template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T> || is_cplx_v<T>;
     template <class T> using out = T;
     template <class T> DPX_D static T apply(T x)
     {
-        if constexpr (is_uint_v<T>) return (T)(x > 0);
+        if constexpr (is_cplx_v<T>) {
+            using R = real_of_t<T>;
+            if (x.re == R(0) && x.im == R(0)) return T{R(0), R(0)};
+            const R a = m_hypot(x.re, x.im);
+            return T{x.re / a, x.im / a};
+        }
+        else if constexpr (is_uint_v<T>) return (T)(x > 0);
         else if constexpr (is_fp_v<T>) return (x != x) ? x : (T)((T(0) < x) - (x < T(0)));
         else return (T)((T(0) < x) - (x < T(0)));
     }
@@ -466,6 +556,84 @@ struct SignbitOp {
     template <class T> DPX_D static bool apply(T x) { return m_signbit(x); }
 };
 
+struct RoundOp2 { // round.hpp:74-96: rint (ties to even) on floats and complex parts, identity on ints
+    template <class T> static constexpr bool ok = !is_bool_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if constexpr (is_cplx_v<T>) return T{m_rint(x.re), m_rint(x.im)};
+        else if constexpr (is_fp_v<T>) return m_rint(x);
+        else return x;
+    }
+};
+struct ConjOp { // conj.hpp: bool -> int8, real types unchanged
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = std::conditional_t<is_bool_v<T>, int8_t, T>;
+    template <class T> DPX_D static V<out<T>> apply(V<T> x)
+    {
+        if constexpr (is_bool_v<T>) return (int8_t)(x ? 1 : 0);
+        else if constexpr (is_cplx_v<T>) return T{x.re, -x.im};
+        else return x;
+    }
+};
+template <bool IMAG> struct PartOp { // real.hpp / imag.hpp: complex -> its real type, others unchanged (imag: zero)
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = real_of_t<T>;
+    template <class T> DPX_D static V<out<T>> apply(V<T> x)
+    {
+        if constexpr (is_cplx_v<T>) return IMAG ? x.im : x.re;
+        else if constexpr (IMAG) return V<T>(0);
+        else return x;
+    }
+};
+struct ProjOp { // proj.hpp: complex only; infinities map to (inf, copysign(0, im))
+    template <class T> static constexpr bool ok = is_cplx_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        using R = real_of_t<T>;
+        if (m_isinf(x.re) || m_isinf(x.im)) return T{(R)__builtin_inff(), m_copysign(R(0), x.im)};
+        return x;
+    }
+};
+struct AngleOp { // angle.hpp: complex -> real, atan2(im, re)
+    template <class T> static constexpr bool ok = is_cplx_v<T>;
+    template <class T> using out = real_of_t<T>;
+    template <class T> DPX_D static real_of_t<T> apply(T x) { return m_atan2(x.im, x.re); }
+};
+struct LogaddexpOp { // logaddexp.hpp with libtensor/include/utils/math_utils.hpp:129-150
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x, T y)
+    {
+        if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x, (float)y);
+        if (x == y) return x + m_log(T(2)); // also handles equal infinities
+        const T d = x - y;
+        if (d > T(0)) return x + m_log1p(m_exp(-d));
+        if (d <= T(0)) return y + m_log1p(m_exp(d));
+        return d; // NaN
+    }
+};
+struct NextafterOp {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x, T y)
+    {
+        if constexpr (std::is_same_v<T, half_t>) {
+            // step in half precision: operate on the 16-bit pattern
+            if (x != x || y != y) return x + y;
+            if (x == y) return y;
+            union { half_t h; uint16_t u; } v;
+            v.h = x;
+            if (x == half_t(0)) { v.u = (uint16_t)((y < half_t(0)) ? 0x8001 : 0x0001); return v.h; }
+            const bool up = (x < y) == (x > half_t(0));
+            v.u = (uint16_t)(up ? v.u + 1 : v.u - 1);
+            return v.h;
+        }
+        else return m_nextafter(x, y);
+    }
+};
+
 // op id -> op struct; f(tag<Op>{}) is called for a valid id
 template <class F> inline bool for_binary_op(int op, F &&f)
 {
@@ -496,6 +664,8 @@ template <class F> inline bool for_binary_op(int op, F &&f)
     case DPX_B_COPYSIGN: f(tag<CopysignOp>{}); return true;
     case DPX_B_LEFT_SHIFT: f(tag<ShiftOp<true>>{}); return true;
     case DPX_B_RIGHT_SHIFT: f(tag<ShiftOp<false>>{}); return true;
+    case DPX_B_LOGADDEXP: f(tag<LogaddexpOp>{}); return true;
+    case DPX_B_NEXTAFTER: f(tag<NextafterOp>{}); return true;
     default: return false;
     }
 }
@@ -532,6 +702,20 @@ template <class F> inline bool for_unary_op(int op, F &&f)
     case DPX_U_LOGICAL_NOT: f(tag<LogicalNotOp>{}); return true;
     case DPX_U_BITWISE_INVERT: f(tag<InvertOp>{}); return true;
     case DPX_U_SIGNBIT: f(tag<SignbitOp>{}); return true;
+    case DPX_U_ASIN: f(tag<AsinOp>{}); return true;
+    case DPX_U_ACOS: f(tag<AcosOp>{}); return true;
+    case DPX_U_ATAN: f(tag<AtanOp>{}); return true;
+    case DPX_U_SINH: f(tag<SinhOp>{}); return true;
+    case DPX_U_COSH: f(tag<CoshOp>{}); return true;
+    case DPX_U_ASINH: f(tag<AsinhOp>{}); return true;
+    case DPX_U_ACOSH: f(tag<AcoshOp>{}); return true;
+    case DPX_U_ATANH: f(tag<AtanhOp>{}); return true;
+    case DPX_U_ROUND: f(tag<RoundOp2>{}); return true;
+    case DPX_U_CONJ: f(tag<ConjOp>{}); return true;
+    case DPX_U_REAL: f(tag<PartOp<false>>{}); return true;
+    case DPX_U_IMAG: f(tag<PartOp<true>>{}); return true;
+    case DPX_U_PROJ: f(tag<ProjOp>{}); return true;
+    case DPX_U_ANGLE: f(tag<AngleOp>{}); return true;
     default: return false;
     }
 }

@@ -293,6 +293,10 @@ _UNARY = {
     "floor": ef.floor, "ceil": ef.ceil, "trunc": ef.trunc, "sign": ef.sign, "isnan": ef.isnan,
     "isinf": ef.isinf, "isfinite": ef.isfinite, "logical_not": ef.logical_not, "invert": ef.bitwise_invert,
     "bitwise_not": ef.bitwise_invert, "bitwise_invert": ef.bitwise_invert, "signbit": ef.signbit,
+    "arcsin": ef.asin, "asin": ef.asin, "arccos": ef.acos, "acos": ef.acos, "arctan": ef.atan, "atan": ef.atan,
+    "sinh": ef.sinh, "cosh": ef.cosh, "arcsinh": ef.asinh, "asinh": ef.asinh, "arccosh": ef.acosh,
+    "acosh": ef.acosh, "arctanh": ef.atanh, "atanh": ef.atanh, "rint": ef.round, "conj": ef.conj,
+    "conjugate": ef.conj, "real": ef.real, "imag": ef.imag, "proj": ef.proj, "angle": ef.angle,
 }
 _BINARY = {
     "add": ef.add, "subtract": ef.subtract, "multiply": ef.multiply, "divide": ef.divide,
@@ -305,6 +309,7 @@ _BINARY = {
     "arctan2": ef.atan2, "atan2": ef.atan2, "hypot": ef.hypot, "copysign": ef.copysign,
     "left_shift": ef.bitwise_left_shift, "bitwise_left_shift": ef.bitwise_left_shift,
     "right_shift": ef.bitwise_right_shift, "bitwise_right_shift": ef.bitwise_right_shift,
+    "logaddexp": ef.logaddexp, "nextafter": ef.nextafter,
 }
 for _n, _f in _UNARY.items():
     globals()[_n] = DPNPUnaryFunc(_n, _f)

@@ -36,7 +36,7 @@ from ._dtypes import (
     uint64,
 )
 from ._elementwise_funcs import *  # noqa: F401,F403
-from ._elementwise_funcs import abs, pow  # noqa: A004
+from ._elementwise_funcs import abs, pow, round  # noqa: A004
 from ._manipulation_functions import (
     broadcast_to,
     expand_dims,

@@ -52,6 +52,20 @@ isfinite = _unary("isfinite", "Elementwise test for finiteness.")
 logical_not = _unary("logical_not", "Elementwise logical negation.")
 bitwise_invert = _unary("bitwise_invert", "Elementwise bit inversion.")
 signbit = _unary("signbit", "Elementwise test of the sign bit.")
+asin = _unary("asin", "Elementwise inverse sine.")
+acos = _unary("acos", "Elementwise inverse cosine.")
+atan = _unary("atan", "Elementwise inverse tangent.")
+sinh = _unary("sinh", "Elementwise hyperbolic sine.")
+cosh = _unary("cosh", "Elementwise hyperbolic cosine.")
+asinh = _unary("asinh", "Elementwise inverse hyperbolic sine.")
+acosh = _unary("acosh", "Elementwise inverse hyperbolic cosine.")
+atanh = _unary("atanh", "Elementwise inverse hyperbolic tangent.")
+round = _unary("round", "Elementwise rounding to the nearest integer, ties to even.")  # noqa: A001
+conj = _unary("conj", "Elementwise complex conjugate.")
+real = _unary("real", "Elementwise real part.")
+imag = _unary("imag", "Elementwise imaginary part.")
+proj = _unary("proj", "Elementwise projection onto the Riemann sphere.")
+angle = _unary("angle", "Elementwise argument of a complex number.")
 
 add = _binary("add", "add(x1, x2, /, *, out=None, order='K'): elementwise sum.")
 subtract = _binary("subtract", "Elementwise difference.", acceptance_fn=_acceptance_fn_subtract)
@@ -81,3 +95,5 @@ hypot = _binary("hypot", "Elementwise hypotenuse.", inplace=False)
 copysign = _binary("copysign", "Elementwise copysign.", inplace=False)
 bitwise_left_shift = _binary("bitwise_left_shift", "Elementwise left shift.")
 bitwise_right_shift = _binary("bitwise_right_shift", "Elementwise right shift.")
+logaddexp = _binary("logaddexp", "Elementwise log(exp(x1) + exp(x2)).", inplace=False)
+nextafter = _binary("nextafter", "Next representable value after x1 towards x2.", inplace=False)

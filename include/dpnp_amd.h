@@ -124,6 +124,20 @@ typedef enum dpx_unary_op {
     DPX_U_LOGICAL_NOT,
     DPX_U_BITWISE_INVERT,
     DPX_U_SIGNBIT,
+    DPX_U_ASIN,
+    DPX_U_ACOS,
+    DPX_U_ATAN,
+    DPX_U_SINH,
+    DPX_U_COSH,
+    DPX_U_ASINH,
+    DPX_U_ACOSH,
+    DPX_U_ATANH,
+    DPX_U_ROUND,
+    DPX_U_CONJ,
+    DPX_U_REAL,
+    DPX_U_IMAG,
+    DPX_U_PROJ,
+    DPX_U_ANGLE,
     DPX_U_NUM_OPS
 } dpx_unary_op;
 
@@ -154,6 +168,8 @@ typedef enum dpx_binary_op {
     DPX_B_COPYSIGN,
     DPX_B_LEFT_SHIFT,
     DPX_B_RIGHT_SHIFT,
+    DPX_B_LOGADDEXP,
+    DPX_B_NEXTAFTER,
     DPX_B_NUM_OPS
 } dpx_binary_op;
 
@@ -174,12 +190,11 @@ typedef enum dpx_path {
     DPX_PATH_NOOP = 0,          /* zero-size: nothing launched */
     DPX_PATH_EW_CONTIG = 1,     /* 1-D unit-stride, 128-bit accesses */
     DPX_PATH_EW_ROWS = 2,       /* N-D, threads vectorised along the inner dim */
-    DPX_PATH_EW_FLAT = 3,       /* N-D, one element per thread */
-    DPX_PATH_EW_TILE = 4,       /* 2-D transposing through an LDS tile */
+    DPX_PATH_EW_TILE = 4,       /* inputs contiguous along another dim than the output: LDS tile */
     DPX_PATH_RED_ROWS = 10,     /* reduced run contiguous: block or wave per output */
-    DPX_PATH_RED_ROWS_SPLIT = 11, /* ... several blocks per output + finalise pass */
+    DPX_PATH_RED_ROWS_SPLIT = 11, /* ... several blocks per output, folded by the last one */
     DPX_PATH_RED_COLS = 12,     /* outputs contiguous, reduced run strided */
-    DPX_PATH_RED_COLS_SPLIT = 13, /* ... reduced run split over blocks + finalise */
+    DPX_PATH_RED_COLS_SPLIT = 13, /* ... reduced run split over blocks, folded by the last one */
     DPX_PATH_RED_GENERIC = 14,  /* fully strided */
     DPX_PATH_RED_SMALL = 15     /* tiny reduced run: one thread per output */
 } dpx_path;

@@ -193,6 +193,10 @@ def binary(op, a, b):
             return _shift(a, b, True)
         if op == "bitwise_right_shift":
             return _shift(a, b, False)
+        if op == "logaddexp":           # math_utils.hpp:129-150
+            return np.logaddexp(a.astype(np.longdouble), b.astype(np.longdouble)).astype(a.dtype)
+        if op == "nextafter":
+            return np.nextafter(a, b)
     raise KeyError(op)
 
 
@@ -200,10 +204,10 @@ def unary_result_dtype(op, dt):
     dt = np.dtype(dt)
     if op in ("isnan", "isinf", "isfinite", "logical_not", "signbit"):
         return np.dtype("?")
-    if op == "abs":
+    if op in ("abs", "real", "imag", "angle"):
         return np.dtype({"c8": "f4", "c16": "f8"}.get(dt.str[1:], dt))
-    if op == "square" and dt.kind == "b":
-        return np.dtype("i1")           # square.hpp type map: bool -> int8
+    if op in ("square", "conj") and dt.kind == "b":
+        return np.dtype("i1")           # square.hpp / conj.hpp type maps: bool -> int8
     if op == "erf" and dt == np.dtype("f2"):
         return np.dtype("f4")           # dpnp/backend/extensions/ufunc/elementwise_functions/erf_funcs.cpp:74-84
     return dt
@@ -248,19 +252,39 @@ def unary(op, a):
             return ~a
         if op == "signbit":
             return np.signbit(a)
+        if op == "round":               # round.hpp:74-96: rint, ties to even; ints unchanged
+            return np.rint(a).astype(a.dtype) if k in "fc" else a.copy()
+        if op == "conj":
+            return np.conj(a).astype(out_dt)
+        if op == "real":
+            return np.real(a).astype(out_dt)
+        if op == "imag":
+            return np.imag(a).astype(out_dt)
+        if op == "angle":
+            return np.angle(a).astype(out_dt)
+        if op == "proj":                # proj.hpp: infinities collapse to (inf, copysign(0, im))
+            inf = np.isinf(a.real) | np.isinf(a.imag)
+            out = a.copy()
+            out.real[inf] = np.inf
+            out.imag[inf] = np.copysign(0.0, a.imag[inf])
+            return out
     raise KeyError(op)
 
 
 _HI = {"exp": np.exp, "log": np.log, "sin": np.sin, "cos": np.cos, "tan": np.tan, "tanh": np.tanh,
        "exp2": np.exp2, "expm1": np.expm1, "log2": np.log2, "log10": np.log10, "log1p": np.log1p,
-       "cbrt": np.cbrt, "erf": None}
+       "cbrt": np.cbrt, "erf": None, "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan,
+       "sinh": np.sinh, "cosh": np.cosh, "asinh": np.arcsinh, "acosh": np.arccosh, "atanh": np.arctanh}
 
 
 def hi_precision(op, a):
     """op(a) in a precision well above a.dtype's (float64 for <= float32 input, long double
     for float64 input; erf through mpmath-free math.erf in float64 / mpmath for float64)."""
     a = np.asarray(a)
-    wide = np.float64 if a.dtype.itemsize <= 4 else np.longdouble
+    if a.dtype.kind == "c":
+        wide = np.complex128 if a.dtype.itemsize <= 8 else np.clongdouble
+    else:
+        wide = np.float64 if a.dtype.itemsize <= 4 else np.longdouble
     x = a.astype(wide)
     with np.errstate(all="ignore"):
         if op == "erf":

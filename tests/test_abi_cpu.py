@@ -73,8 +73,12 @@ def test_binary_result_types():
 def test_unary_result_types():
     U = L.UNARY_ID
     for i, d in enumerate(NP):
-        assert lib.dpx_unary_result_type(U["exp"], i) == (i if d.kind == "f" else -1)
-        assert lib.dpx_unary_result_type(U["sqrt"], i) == (i if d.kind == "f" else -1)
+        assert lib.dpx_unary_result_type(U["exp"], i) == (i if d.kind in "fc" else -1)
+        assert lib.dpx_unary_result_type(U["sqrt"], i) == (i if d.kind in "fc" else -1)
+        assert lib.dpx_unary_result_type(U["cbrt"], i) == (i if d.kind == "f" else -1)
+        assert lib.dpx_unary_result_type(U["real"], i) == {L.CFLOAT: L.FLOAT, L.CDOUBLE: L.DOUBLE}.get(i, i)
+        assert lib.dpx_unary_result_type(U["angle"], i) == {L.CFLOAT: L.FLOAT, L.CDOUBLE: L.DOUBLE}.get(i, -1)
+        assert lib.dpx_unary_result_type(U["round"], i) == (-1 if d.kind == "b" else i)
         assert lib.dpx_unary_result_type(U["isnan"], i) == L.BOOL
         want_abs = {L.CFLOAT: L.FLOAT, L.CDOUBLE: L.DOUBLE}.get(i, i)
         assert lib.dpx_unary_result_type(U["abs"], i) == want_abs

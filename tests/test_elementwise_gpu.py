@@ -16,9 +16,10 @@ EXACT_BINARY = ["add", "subtract", "multiply", "divide", "bitwise_and", "bitwise
                 "bitwise_left_shift", "bitwise_right_shift"]
 ULP_BINARY = ["pow", "atan2", "hypot"]
 EXACT_UNARY = ["abs", "negative", "positive", "square", "sqrt", "floor", "ceil", "trunc", "sign", "isnan",
-               "isinf", "isfinite", "logical_not", "bitwise_invert", "signbit", "reciprocal"]
+               "isinf", "isfinite", "logical_not", "bitwise_invert", "signbit", "reciprocal", "round", "conj",
+               "real", "imag", "proj"]
 ULP_UNARY = ["exp", "log", "erf", "sin", "cos", "tan", "tanh", "exp2", "expm1", "log2", "log10", "log1p", "cbrt",
-             "rsqrt"]
+             "rsqrt", "asin", "acos", "atan", "sinh", "cosh", "asinh", "acosh", "atanh"]
 
 
 def assert_close_complex(got, want, a, b=None):
@@ -111,14 +112,21 @@ def test_unary_exact(op):
             a = random_array(rng, n, dt, -50, 50)
             if dt.kind == "f" and n > 4:
                 a[:4] = [np.nan, np.inf, -np.inf, -0.0]
-            if op in ("sqrt",):
+            if op in ("sqrt",) and dt.kind != "c":
                 a = np.abs(a)
+            if op == "proj" and n > 4:
+                a[:2] = [complex(np.inf, -1.0), complex(2.0, -np.inf)]
             got = host(getattr(dpt, op)(dev(a)))
             want = orc.unary(op, a)
-            if dt.kind == "c" and op == "abs":
-                np.testing.assert_allclose(got, want, rtol=4 * np.finfo(got.dtype).eps)
+            if dt.kind == "c" and op in ("abs", "sign", "sqrt", "reciprocal"):
+                if op == "sqrt":
+                    want = np.sqrt(a.astype("c16")).astype(dt)
+                np.testing.assert_allclose(got, want, rtol=8 * np.finfo(got.dtype).eps)
             elif dt.kind == "c" and op == "square":
                 assert_close_complex(got, want, a)
+            elif op == "proj":
+                assert_same(got, want)
+                assert_same(np.signbit(got.imag), np.signbit(want.imag))
             elif dt == np.dtype("f2") and op in ("reciprocal",):
                 assert_ulp(got, 1 / a.astype("f8"), 1.0)
             else:
@@ -131,11 +139,14 @@ def test_unary_transcendentals_within_4_ulp(op):
     rng_by_op = {"exp": (-80, 80), "exp2": (-100, 100), "expm1": (-30, 30), "log": (1e-30, 1e30),
                  "log2": (1e-30, 1e30), "log10": (1e-30, 1e30), "log1p": (-0.99, 1e10), "erf": (-6, 6),
                  "sin": (-50, 50), "cos": (-50, 50), "tan": (-1.5, 1.5), "tanh": (-20, 20), "cbrt": (-1e10, 1e10),
-                 "rsqrt": (1e-10, 1e10)}
+                 "rsqrt": (1e-10, 1e10), "asin": (-1, 1), "acos": (-1, 1), "atan": (-1e3, 1e3), "sinh": (-20, 20),
+                 "cosh": (-20, 20), "asinh": (-1e6, 1e6), "acosh": (1, 1e6), "atanh": (-0.999, 0.999)}
     lo, hi = rng_by_op[op]
     for dt in FLOATS:
         if dt == np.dtype("f2"):
             lo2, hi2 = max(lo, -10), min(hi, 10)
+            if op == "acosh":
+                lo2, hi2 = 1, 1000
             if op in ("log", "log2", "log10", "rsqrt"):
                 lo2, hi2 = 1e-3, 6e4
         else:
@@ -330,3 +341,47 @@ def test_unaligned_base_pointer():
             o = dpt.empty(5003, dtype=dt)
             dpt.add(dev(a)[k:], dev(b)[:-k], out=o[k:])
             assert_same(host(o)[k:], a[k:] + b[:-k])
+
+
+@pytest.mark.parametrize("op", ["exp", "log", "sqrt", "sin", "cos", "tan", "tanh", "sinh", "cosh"])
+def test_complex_elementary_functions(op):
+    rng = np.random.default_rng(97)
+    for dt, rtol in (("c8", 4e-6), ("c16", 8e-15)):
+        a = (rng.uniform(-3, 3, 4000) + 1j * rng.uniform(-3, 3, 4000)).astype(dt)
+        got = host(getattr(dpt, op)(dev(a)))
+        want = getattr(np, op)(a.astype("c16" if dt == "c8" else np.clongdouble))
+        assert got.dtype == np.dtype(dt)
+        # log: the real part log|z| vanishes on the unit circle, measure against |z|-scale there
+        scale = np.maximum(np.abs(want), 1.0 if op == "log" else 1e-3)
+        err = np.abs(got - want) / scale
+        assert float(err.max()) <= rtol, float(err.max())
+    z = np.array([0j, 1 + 0j, -1 + 0j, 1j, -4 + 0j], dtype="c16")
+    np.testing.assert_allclose(host(dpt.sqrt(dev(z))), np.sqrt(z), rtol=1e-15, atol=0)
+    np.testing.assert_allclose(host(dpt.exp(dev(z))), np.exp(z), rtol=1e-15, atol=1e-16)
+    np.testing.assert_allclose(host(dpt.pow(dev(z[1:]), dev(np.full(4, 2 + 0j)))), z[1:] ** 2, rtol=1e-14, atol=1e-15)
+
+
+def test_angle_logaddexp_nextafter():
+    rng = np.random.default_rng(101)
+    z = (rng.standard_normal(3000) + 1j * rng.standard_normal(3000)).astype("c8")
+    got = host(dpt.angle(dev(z)))
+    assert got.dtype == np.dtype("f4")
+    assert_ulp(got, np.angle(z.astype("c16")), 4.0)
+    for dt in FLOATS:
+        a, b = random_array(rng, 5000, dt, -30, 30), random_array(rng, 5000, dt, -30, 30)
+        a[:4] = [np.inf, -np.inf, np.nan, 1.0]
+        b[:4] = [np.inf, -np.inf, 1.0, 1.0]
+        got = host(dpt.logaddexp(dev(a), dev(b)))
+        wide = np.float64 if dt.itemsize <= 4 else np.longdouble
+        with np.errstate(all="ignore"):
+            want = np.logaddexp(a.astype(wide), b.astype(wide))
+            # max(x, y) + log1p(exp(-|x - y|)) (the reference's formula) cancels when the result is
+            # near zero: the error is a few ULPs of the operands, not of the result
+            scale = np.maximum(np.maximum(np.abs(a), np.abs(b)).astype(wide), np.abs(want))
+            fin = np.isfinite(want)
+            assert (np.abs(got[fin].astype(wide) - want[fin]) <= 4 * np.finfo(dt).eps * scale[fin]).all()
+            assert_same(got[~fin], want[~fin].astype(dt))
+        x, y = random_array(rng, 3000, dt, -5, 5), random_array(rng, 3000, dt, -5, 5)
+        x[:6] = [0.0, 0.0, -0.0, 1.0, np.inf, np.nan]
+        y[:6] = [1.0, -1.0, 0.0, 1.0, 0.0, 0.0]
+        assert_same(host(dpt.nextafter(dev(x), dev(y))), np.nextafter(x, y))

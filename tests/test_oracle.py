@@ -317,3 +317,18 @@ def test_c_port_matches_numpy_oracle(oc, n):
     assert oc.argmin(x) == orc.argreduce("argmin", x, 1)
     x[int(rng.integers(0, n))] = np.nan  # a single NaN is pinned by the reference's tests
     assert oc.argmax(x) == orc.argreduce("argmax", x, 1) == oc.argmin(x)
+
+
+def test_round_conj_parts_proj_rules():
+    # round.hpp:74-96 (rint: ties to even), conj.hpp / real.hpp / imag.hpp / proj.hpp type maps
+    assert (orc.unary("round", np.array([0.5, 1.5, 2.5, -0.5, -1.5], dtype="f4")) == [0, 2, 2, -0.0, -2]).all()
+    assert (orc.unary("round", np.array([3, -4], dtype="i2")) == [3, -4]).all()
+    assert orc.unary("conj", np.array([True])).dtype == np.dtype("i1")
+    assert orc.unary("conj", np.array([1 + 2j], dtype="c8"))[0] == 1 - 2j
+    assert orc.unary("real", np.array([1 + 2j], dtype="c16")).dtype == np.dtype("f8")
+    assert orc.unary("imag", np.array([5], dtype="i4"))[0] == 0
+    p = orc.unary("proj", np.array([complex(-np.inf, -2.0), 1 + 1j]))
+    assert p[0].real == np.inf and np.signbit(p[0].imag) and p[1] == 1 + 1j
+    # logaddexp closed forms: log(e^x + e^x) = x + log 2; one operand at -inf leaves the other
+    assert orc.binary("logaddexp", np.array([3.0]), np.array([3.0]))[0] == 3.0 + np.log(2.0)
+    assert orc.binary("logaddexp", np.array([-np.inf]), np.array([7.0]))[0] == 7.0
