@@ -36,7 +36,7 @@ BINARY_OPS = [
     "logical_xor", "pow", "floor_divide", "remainder", "atan2", "hypot",
     "copysign", "bitwise_left_shift", "bitwise_right_shift", "logaddexp", "nextafter",
 ]
-REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev"]
+REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot"]
 SEARCH_OPS = ["argmax", "argmin"]
 UNARY_ID = {n: i for i, n in enumerate(UNARY_OPS)}
 BINARY_ID = {n: i for i, n in enumerate(BINARY_OPS)}

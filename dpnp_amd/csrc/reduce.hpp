@@ -121,13 +121,16 @@ template <class In, class Out> DPX_D acc_of_t<Out> in_to_acc(In x)
     else return (Acc)convert<Out, In>(x);
 }
 
-enum { K_SUM = 0, K_PROD = 1, K_MAX = 2, K_MIN = 3, K_SUMSQDEV = 4 };
+enum { K_SUM = 0, K_PROD = 1, K_MAX = 2, K_MIN = 3, K_SUMSQDEV = 4, K_LOGSUMEXP = 5, K_HYPOT = 6 };
 
 template <int KIND, class T> DPX_D T red_identity()
 {
-    if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV) {
+    if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV || KIND == K_HYPOT) {
         if constexpr (is_cplx_v<T>) return T{0, 0};
         else return T(0);
+    }
+    else if constexpr (KIND == K_LOGSUMEXP) {
+        return -(T)__builtin_inff();
     }
     else if constexpr (KIND == K_PROD) {
         if constexpr (is_cplx_v<T>) return T{1, 0};
@@ -183,6 +186,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         }
         else if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV) return a + b;
         else if constexpr (KIND == K_PROD) return a * b;
+        else if constexpr (KIND == K_LOGSUMEXP) return LogaddexpOp::apply<Acc>(a, b);
+        else if constexpr (KIND == K_HYPOT) return m_hypot(a, b);
         else if constexpr (KIND == K_MAX) return max_nan(a, b);
         else return min_nan(a, b);
     }

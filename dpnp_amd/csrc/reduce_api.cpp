@@ -12,6 +12,8 @@ int sum_acc_size(int, int);
 int prod_acc_size(int, int);
 int minmax_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 int arg_run_any(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int fpred_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+bool fpred_pair_supported(int, int);
 
 static bool reduce_supported(int op, int s, int d)
 {
@@ -22,6 +24,8 @@ static bool reduce_supported(int op, int s, int d)
     case DPX_R_MAX:
     case DPX_R_MIN: return s == d;
     case DPX_R_SUMSQDEV: return sqdev_pair_supported(s, d);
+    case DPX_R_LOGSUMEXP:
+    case DPX_R_HYPOT: return fpred_pair_supported(s, d);
     default: return false;
     }
 }
@@ -35,7 +39,7 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         return fail(DPX_ERR_BAD_ARGUMENT, "aux must be given for DPX_R_SUMSQDEV and only for it");
     if (!reduce_supported(op, src->dtype, dst->dtype))
         return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
-    const bool empty_ok = op == DPX_R_SUM || op == DPX_R_PROD || op == DPX_R_SUMSQDEV;
+    const bool empty_ok = op != DPX_R_MAX && op != DPX_R_MIN;
     if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false);
@@ -44,7 +48,7 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if (op == DPX_R_SUM || op == DPX_R_SUMSQDEV) acc = sum_acc_size(src->dtype, dst->dtype) ? sum_acc_size(src->dtype, dst->dtype) : acc;
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
-        if (op == DPX_R_SUMSQDEV && dst->dtype == DPX_HALF) acc = 4;
+        if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
         red_export_plan(pl, plan_out, acc);
         return DPX_OK;
     }
@@ -54,6 +58,8 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     case DPX_R_PROD: return prod_run(pl, src, dst, s);
     case DPX_R_MAX: return minmax_run(true, pl, src, dst, s);
     case DPX_R_MIN: return minmax_run(false, pl, src, dst, s);
+    case DPX_R_LOGSUMEXP: return fpred_run(true, pl, src, dst, s);
+    case DPX_R_HYPOT: return fpred_run(false, pl, src, dst, s);
     default: return sqdev_run(pl, src, dst, aux, s);
     }
 }

@@ -378,6 +378,35 @@ def min(a, axis=None, out=None, keepdims=False, initial=None, where=True):  # no
 amax, amin = max, min
 
 
+def all(a, /, axis=None, out=None, keepdims=False, *, where=True):  # noqa: A001
+    check_limitations(where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.all, dpt.bool, axis=axis, keepdims=keepdims)
+
+
+def any(a, /, axis=None, out=None, keepdims=False, *, where=True):  # noqa: A001
+    check_limitations(where=where)
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.any, dpt.bool, axis=axis, keepdims=keepdims)
+
+
+def count_nonzero(a, axis=None, *, keepdims=False, out=None):
+    u = get_usm_ndarray(a)
+    return _wrap_reduction_call(u, out, dpt.count_nonzero, dpt.int64, axis=axis, keepdims=keepdims)
+
+
+def logsumexp(x, /, *, axis=None, out=None, dtype=None, keepdims=False):
+    u = get_usm_ndarray(x)
+    res_dt = dpt.dtype(dtype) if dtype is not None else (u.dtype if u.dtype.kind == "f" else dpt.float64)
+    return _wrap_reduction_call(u, out, dpt.logsumexp, res_dt, axis=axis, dtype=dtype, keepdims=keepdims)
+
+
+def reduce_hypot(x, /, *, axis=None, out=None, dtype=None, keepdims=False):
+    u = get_usm_ndarray(x)
+    res_dt = dpt.dtype(dtype) if dtype is not None else (u.dtype if u.dtype.kind == "f" else dpt.float64)
+    return _wrap_reduction_call(u, out, dpt.reduce_hypot, res_dt, axis=axis, dtype=dtype, keepdims=keepdims)
+
+
 def _search_res_dt(out):
     res_dt = dpt.dtype(ti.default_device_index_type())
     if out is not None and not np.can_cast(out.dtype, res_dt, casting="safe"):

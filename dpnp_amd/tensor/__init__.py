@@ -45,7 +45,19 @@ from ._manipulation_functions import (
     reshape,
     squeeze,
 )
-from ._reduction import all, any, argmax, argmin, max, min, prod, sum  # noqa: A004
+from ._reduction import (  # noqa: A004
+    all,
+    any,
+    argmax,
+    argmin,
+    count_nonzero,
+    logsumexp,
+    max,
+    min,
+    prod,
+    reduce_hypot,
+    sum,
+)
 from ._search_functions import where
 from ._statistical_functions import mean, std, var
 from ._type_utils import can_cast, result_type

@@ -13,7 +13,7 @@ from . import _tensor_reductions_impl as tri
 from ._ctors import empty, empty_like
 from ._dtypes import dtype as _as_dtype
 from ._manipulation_functions import normalize_axis_tuple, permute_dims, reshape, squeeze
-from ._type_utils import _default_accumulation_dtype
+from ._type_utils import _default_accumulation_dtype, _default_accumulation_dtype_fp_types
 from ._usmarray import usm_ndarray
 
 
@@ -76,7 +76,7 @@ def _reduction_over_axis(x, axis, dtype, keepdims, out, _reduction_fn, _dtype_su
     inp_dt = x.dtype
     res_dt = _default_reduction_type_fn(inp_dt, None) if dtype is None else _as_dtype(dtype)
     direct = _dtype_supported(inp_dt, res_dt, "device", None)
-    if dtype is None and not direct:
+    if dtype is None and not direct and not _dtype_supported(res_dt, res_dt, "device", None):
         raise RuntimeError("Automatically determined reduction data type does not have direct implementation")
     out, user = _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap=direct)
     if red_nd == 0:
@@ -203,3 +203,29 @@ def all(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
 def any(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
     """True where some element along `axis` is non-zero."""
     return _boolean_reduction(x, axis, keepdims, out, tri._max_over_axis)
+
+
+def logsumexp(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
+    """log(sum(exp(x))) over `axis`, combined pairwise with logaddexp (no overflow)."""
+    return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._logsumexp_over_axis,
+                                lambda i, o, u=None, q=None: i.kind != "c" and o.kind != "c"
+                                and tri._logsumexp_over_axis_dtype_supported(i, o),
+                                _default_accumulation_dtype_fp_types)
+
+
+def reduce_hypot(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
+    """sqrt(sum(x**2)) over `axis`, combined pairwise with hypot (no overflow)."""
+    return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._hypot_over_axis,
+                                lambda i, o, u=None, q=None: i.kind != "c" and o.kind != "c"
+                                and tri._hypot_over_axis_dtype_supported(i, o),
+                                _default_accumulation_dtype_fp_types)
+
+
+def count_nonzero(x, /, *, axis=None, keepdims=False, out=None):
+    """Number of non-zero elements over `axis` (int64)."""
+    from ._copy_utils import astype
+    from ._dtypes import bool as _bool
+
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
+    return sum(astype(x, _bool, copy=False), axis=axis, dtype="i8", keepdims=keepdims, out=out)

@@ -36,6 +36,8 @@ _sum_over_axis, _sum_over_axis_dtype_supported = _make_reduction("sum", _lib.RED
 _prod_over_axis, _prod_over_axis_dtype_supported = _make_reduction("prod", _lib.REDUCE_ID["prod"])
 _max_over_axis, _max_over_axis_dtype_supported = _make_reduction("max", _lib.REDUCE_ID["max"])
 _min_over_axis, _min_over_axis_dtype_supported = _make_reduction("min", _lib.REDUCE_ID["min"])
+_logsumexp_over_axis, _logsumexp_over_axis_dtype_supported = _make_reduction("logsumexp", _lib.REDUCE_ID["logsumexp"])
+_hypot_over_axis, _hypot_over_axis_dtype_supported = _make_reduction("hypot", _lib.REDUCE_ID["hypot"])
 _argmax_over_axis = _make_search("argmax", _lib.SEARCH_ID["argmax"])
 _argmin_over_axis = _make_search("argmin", _lib.SEARCH_ID["argmin"])
 

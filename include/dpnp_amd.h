@@ -179,6 +179,8 @@ typedef enum dpx_reduce_op {
     DPX_R_MAX,
     DPX_R_MIN,
     DPX_R_SUMSQDEV, /* sum((x - aux)^2): second pass of var, see dpx_reduce */
+    DPX_R_LOGSUMEXP, /* log(sum(exp(x))), libtensor/source/reductions/logsumexp.cpp */
+    DPX_R_HYPOT,     /* sqrt(sum(x^2)) by pairwise hypot, libtensor/source/reductions/reduce_hypot.cpp */
     DPX_R_NUM_OPS
 } dpx_reduce_op;
 

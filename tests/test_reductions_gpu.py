@@ -253,3 +253,25 @@ def test_all_any():
     assert_same(host(dpt.any(dev(a), axis=1)), a.any(axis=1))
     assert_same(host(dpt.all(dev(a), axis=1)), a.all(axis=1))
     assert bool(dpt.all(dpt.empty((0,)))) and not bool(dpt.any(dpt.empty((0,))))
+
+
+def test_logsumexp_hypot_count_nonzero():
+    # dpnp/tests/tensor/test_usm_ndarray_reductions.py (logsumexp / reduce_hypot sections)
+    rng = np.random.default_rng(103)
+    for dt, rtol in (("f4", 1e-5), ("f8", 1e-12)):
+        a = (rng.standard_normal((7, 3001)) * 20).astype(dt)
+        want = np.log(np.sum(np.exp(a.astype(np.longdouble)), axis=1))
+        np.testing.assert_allclose(host(dpt.logsumexp(dev(a), axis=1)).astype(np.longdouble), want, rtol=rtol)
+        big = np.full(1000, 1000.0, dtype=dt)  # exp overflows, the pairwise combine does not
+        np.testing.assert_allclose(float(dpt.logsumexp(dev(big))), 1000.0 + np.log(1000.0), rtol=rtol)
+        want = np.sqrt(np.sum(a.astype(np.longdouble) ** 2, axis=0))
+        np.testing.assert_allclose(host(dpt.reduce_hypot(dev(a), axis=0)).astype(np.longdouble), want, rtol=rtol)
+        huge = np.full(100, np.finfo(dt).max / 100, dtype=dt)  # the squares overflow, the result does not
+        assert np.isfinite(float(dpt.reduce_hypot(dev(huge))))
+    assert float(dpt.logsumexp(dpt.empty((0,), dtype="f4"))) == -np.inf
+    assert float(dpt.reduce_hypot(dpt.empty((0,), dtype="f4"))) == 0.0
+    assert dpt.logsumexp(dpt.ones(5, dtype="i4")).dtype == np.dtype("f8")
+    np.testing.assert_allclose(float(dpt.logsumexp(dpt.ones(5, dtype="i4"))), 1 + np.log(5), rtol=1e-14)
+    m = rng.integers(-1, 2, (40, 50)).astype("i1")
+    assert_same(host(dpt.count_nonzero(dev(m), axis=0)), np.count_nonzero(m, axis=0).astype("i8"))
+    assert int(dpt.count_nonzero(dev(m))) == int(np.count_nonzero(m))
