@@ -53,6 +53,153 @@ def cpu_baseline(n_log2=26, repeats=5):
 
 PRIME_STEPS = 24
 
+WORKLOADS = {
+    "metric": "fp32 add 2^28 + sum axis=-1 and axis=0 over 16384x16384 + argmax 2^28 (->int64)",
+    "cfg1": "fp32 add of two 2^24 arrays, then sum of the result",
+    "cfg2": "fp32 16384x16384: sum and max along axis=1 and axis=0",
+    "cfg3": "fp32 2^28 normal(0,1), 1 % duplicated extrema, 0.1 % NaN: argmax, argmin, mean and var accumulated in fp64 "
+            "(fp32 input and fp64 input)",
+    "cfg4": "8192x8192 fp32 views A[:, ::2], A.T and a (1,4096) row: multiply, exp, where(A>0, A, B); int32 bitwise_and",
+    "cfg5": "Black-Scholes over 2^26 fp64 options, call and put: one fused kernel, and the chain of elementwise calls",
+}
+
+
+def _device_array(dpnp, torch, t):
+    """A dpnp array holding the bytes of torch tensor t (handed over by a byte copy, before timing)."""
+    names = {torch.float32: "f4", torch.float64: "f8", torch.int32: "i4", torch.bool: "?"}
+    arr = dpnp.empty(tuple(t.shape), dtype=names[t.dtype])
+    nbytes = t.numel() * t.element_size()
+    arr.get_array()._buf[:nbytes].copy_(t.contiguous().view(-1).view(torch.uint8))
+    return arr
+
+
+def build_workload(name, dpnp, torch):
+    """-> (ops, dtype, data): ops = [(label, callable, algorithmic bytes, elements)].
+    Algorithmic bytes = every input element read once + every output element written once."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def uniform(shape, lo=-1.0, hi=1.0, dtype=torch.float32):
+        t = torch.rand(shape, device="cuda", generator=g, dtype=dtype) * (hi - lo) + lo
+        return _device_array(dpnp, torch, t)
+
+    def normal(shape):
+        return _device_array(dpnp, torch, torch.randn(shape, device="cuda", generator=g))
+
+    if name == "metric":
+        n, side = 1 << 28, 1 << 14
+        a, b, x = uniform(n), uniform(n), normal(n)
+        c = dpnp.empty(n, dtype="f4")
+        M = a.reshape(side, side)
+        r1, r0 = dpnp.empty(side, dtype="f4"), dpnp.empty(side, dtype="f4")
+        idx = dpnp.empty((), dtype="i8")
+        ops = [
+            ("add", lambda: dpnp.add(a, b, out=c), 12 * n, n),
+            ("sum_axis1", lambda: dpnp.sum(M, axis=1, out=r1), 4 * n + 4 * side, n),
+            ("sum_axis0", lambda: dpnp.sum(M, axis=0, out=r0), 4 * n + 4 * side, n),
+            ("argmax", lambda: dpnp.argmax(x, out=idx), 4 * n + 8, n),
+            # plain copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters (--ops copy)
+            ("copy", lambda: dpnp.copyto(c, a), 8 * n, n),
+        ]
+        return ops, "f32", "synthetic (seeded uniform[-1,1) and normal(0,1), resident in HBM)"
+    if name == "cfg1":
+        n = 1 << 24
+        a, b = uniform(n), uniform(n)
+        c, s = dpnp.empty(n, dtype="f4"), dpnp.empty((), dtype="f4")
+        ops = [("add", lambda: dpnp.add(a, b, out=c), 12 * n, n),
+               ("sum", lambda: dpnp.sum(c, out=s), 4 * n + 4, n)]
+        return ops, "f32", "synthetic (seeded uniform[-1,1), resident in HBM)"
+    if name == "cfg2":
+        side = 1 << 14
+        n = side * side
+        M = uniform((side, side))
+        r = [dpnp.empty(side, dtype="f4") for _ in range(4)]
+        nb = 4 * n + 4 * side
+        ops = [("sum_axis1", lambda: dpnp.sum(M, axis=1, out=r[0]), nb, n),
+               ("max_axis1", lambda: dpnp.max(M, axis=1, out=r[1]), nb, n),
+               ("sum_axis0", lambda: dpnp.sum(M, axis=0, out=r[2]), nb, n),
+               ("max_axis0", lambda: dpnp.max(M, axis=0, out=r[3]), nb, n)]
+        return ops, "f32", "synthetic (seeded uniform[-1,1), resident in HBM)"
+    if name == "cfg3":
+        n = 1 << 28
+        t = torch.randn(n, device="cuda", generator=g)
+        pick = torch.randint(0, n, (n // 100,), device="cuda", generator=g)
+        t[pick] = t.max()
+        pick = torch.randint(0, n, (n // 100,), device="cuda", generator=g)
+        t[pick] = t.min()
+        clean = _device_array(dpnp, torch, t)
+        clean64 = _device_array(dpnp, torch, t.double())
+        pick = torch.randint(0, n, (n // 1000,), device="cuda", generator=g)
+        t[pick] = float("nan")
+        x = _device_array(dpnp, torch, t)
+        del t, pick
+        i0, i1 = dpnp.empty((), dtype="i8"), dpnp.empty((), dtype="i8")
+        m = [dpnp.empty((), dtype="f8") for _ in range(4)]
+        ops = [("argmax_nan", lambda: dpnp.argmax(x, out=i0), 4 * n + 8, n),
+               ("argmin_nan", lambda: dpnp.argmin(x, out=i1), 4 * n + 8, n),
+               ("argmax", lambda: dpnp.argmax(clean, out=i0), 4 * n + 8, n),
+               ("mean_f32_acc64", lambda: dpnp.mean(clean, dtype="f8", out=m[0]), 4 * n + 8, n),
+               ("var_f32_acc64", lambda: dpnp.var(clean, dtype="f8", out=m[1]), 2 * 4 * n + 8, n),  # two passes
+               ("mean_f64", lambda: dpnp.mean(clean64, out=m[2]), 8 * n + 8, n),
+               ("var_f64", lambda: dpnp.var(clean64, out=m[3]), 2 * 8 * n + 8, n)]
+        return ops, "f32 (fp64 accumulation)", "synthetic (seeded normal(0,1) with planted extrema / NaN, resident in HBM)"
+    if name == "cfg4":
+        side = 8192
+        A, B = normal((side, side)), normal((1, side // 2))
+        ints = [_device_array(dpnp, torch, torch.randint(-2**31, 2**31, (side, side), device="cuda", generator=g,
+                                                         dtype=torch.int64).to(torch.int32)) for _ in range(2)]
+        V1, V2 = A[:, ::2], A.T
+        h = side * side // 2
+        o_half = dpnp.empty((side, side // 2), dtype="f4")
+        o_f = dpnp.empty((side, side), dtype="f4").T  # F-contiguous, the layout order="K" gives exp(A.T)
+        o_c = dpnp.empty((side, side), dtype="f4")
+        o_b = dpnp.empty((side, side // 2), dtype="?")
+        o_i = dpnp.empty((side, side), dtype="i4")
+        o_ih = dpnp.empty((side, side // 2), dtype="i4")
+
+        def where_unfused():
+            dpnp.greater(V1, 0, out=o_b)
+            dpnp.where(o_b, V1, B, out=o_half)
+
+        ops = [("multiply_V1_B", lambda: dpnp.multiply(V1, B, out=o_half), 8 * h + 4 * (side // 2), h),
+               ("exp_V1", lambda: dpnp.exp(V1, out=o_half), 8 * h, h),
+               ("exp_AT_keep_layout", lambda: dpnp.exp(V2, out=o_f), 8 * 2 * h, 2 * h),
+               ("exp_AT_to_C", lambda: dpnp.exp(V2, out=o_c), 8 * 2 * h, 2 * h),
+               ("where_greater_fused", lambda: dpnp.where_compare("greater", V1, 0, V1, B, out=o_half),
+                8 * h + 4 * (side // 2), h),
+               ("where_greater_two_calls", where_unfused, (4 + 1) * h + (1 + 4 + 4) * h + 4 * (side // 2), h),
+               ("bitwise_and", lambda: dpnp.bitwise_and(ints[0], ints[1], out=o_i), 12 * 2 * h, 2 * h),
+               ("bitwise_and_V1", lambda: dpnp.bitwise_and(ints[0][:, ::2], ints[1][:, ::2], out=o_ih), 12 * h, h)]
+        return ops, "f32/i32/bool", "synthetic (seeded normal(0,1), uniform int32, resident in HBM)"
+    if name == "cfg5":
+        n = 1 << 26
+        price = uniform(n, 10.0, 50.0, torch.float64)
+        strike = uniform(n, 10.0, 50.0, torch.float64)
+        t = uniform(n, 1.0, 2.0, torch.float64)
+        call, put = dpnp.empty(n, dtype="f8"), dpnp.empty(n, dtype="f8")
+        r, vol = 0.1, 0.2
+
+        def chain():
+            # the expression tree of the reference's example (examples/example_bs.py:50-78), one call per node
+            a = dpnp.log(price / strike)
+            b = t * (-r)
+            z = t * (vol * vol * 2)
+            c = 0.25 * z
+            y = 1.0 / dpnp.sqrt(z)
+            w1 = (a - b + c) * y
+            w2 = (a - b - c) * y
+            d1 = 0.5 + 0.5 * dpnp.erf(w1)
+            d2 = 0.5 + 0.5 * dpnp.erf(w2)
+            se = dpnp.exp(b) * strike
+            res = price * d1 - se * d2
+            dpnp.copyto(call, res)
+            dpnp.subtract(res, price, out=put)
+            dpnp.add(put, se, out=put)
+
+        ops = [("black_scholes_fused", lambda: dpnp.black_scholes(price, strike, t, r, vol, call=call, put=put), 40 * n, n),
+               ("black_scholes_chain", chain, 40 * n, n)]
+        return ops, "f64", "synthetic (seeded uniform price, strike [10,50), T [1,2), resident in HBM)"
+    raise SystemExit(f"--workload: unknown workload {name!r} (one of {', '.join(WORKLOADS)})")
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -61,9 +208,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--dump-steps", action="store_true", help="print every step's per-op times to stderr")
-    ap.add_argument("--ops", default="add,sum_axis1,sum_axis0,argmax",
-                    help="subset of add,sum_axis1,sum_axis0,argmax,copy to run (profiling runs); the metric is "
-                         "the default set")
+    ap.add_argument("--workload", default="metric",
+                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5, "
+                         "measured the same way")
+    ap.add_argument("--ops", default=None,
+                    help="comma-separated subset of the workload's ops (profiling runs); 'copy' in the metric "
+                         "workload is a plain copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -76,43 +226,21 @@ def main():
         sys.exit(1)
     import dpnp_amd as dpnp
 
-    n = 1 << 28
-    side = 1 << 14
-    g = torch.Generator(device="cuda").manual_seed(0)
-
-    def uniform(count):
-        t = torch.rand(count, device="cuda", generator=g, dtype=torch.float32) * 2 - 1
-        arr = dpnp.empty(count, dtype="f4")
-        # hand the synthetic data over through a byte copy; no torch compute in the timed region
-        arr.get_array()._buf[: count * 4].copy_(t.view(torch.uint8))
-        return arr
-
-    a, b = uniform(n), uniform(n)
-    x = dpnp.empty(n, dtype="f4")
-    x.get_array()._buf[: n * 4].copy_(torch.randn(n, device="cuda", generator=g).view(torch.uint8))
-    c = dpnp.empty(n, dtype="f4")
-    M = a.reshape(side, side)
-    r1, r0 = dpnp.empty(side, dtype="f4"), dpnp.empty(side, dtype="f4")
-    idx = dpnp.empty((), dtype="i8")
-    all_ops = [
-        ("add", lambda: dpnp.add(a, b, out=c), 12 * n),
-        ("sum_axis1", lambda: dpnp.sum(M, axis=1, out=r1), 4 * n + 4 * side),
-        ("sum_axis0", lambda: dpnp.sum(M, axis=0, out=r0), 4 * n + 4 * side),
-        ("argmax", lambda: dpnp.argmax(x, out=idx), 4 * n + 8),
-        # plain copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
-        ("copy", lambda: dpnp.copyto(c, a), 8 * n),
-    ]
-    wanted = [w for w in args.ops.split(",") if w]
-    ops = [o for o in all_ops if o[0] in wanted]
-    if not ops or len(ops) != len(wanted):
-        print(f"--ops: unknown op in {wanted}", file=sys.stderr)
-        sys.exit(2)
-    step_bytes = sum(nb for _, _, nb in ops)
+    all_ops, dtype, data = build_workload(args.workload, dpnp, torch)
+    if args.ops is None:
+        ops = [o for o in all_ops if o[0] != "copy"]
+    else:
+        wanted = [w for w in args.ops.split(",") if w]
+        ops = [o for o in all_ops if o[0] in wanted]
+        if not ops or len(ops) != len(wanted):
+            print(f"--ops: unknown op in {wanted}; {args.workload} has {[o[0] for o in all_ops]}", file=sys.stderr)
+            sys.exit(2)
+    step_bytes = sum(o[2] for o in ops)
 
     host_us = []
 
     def step(events=None):
-        for k, (_, fn, _) in enumerate(ops):
+        for k, (_, fn, _, _) in enumerate(ops):
             if events is not None:
                 events[k][0].record()
             if args.dump_steps:
@@ -148,18 +276,25 @@ def main():
     gpu_ms = t_begin.elapsed_time(t_end)
     ms_per_step = max(gpu_ms, wall * 1e3) / args.steps
     per_op = {}
-    for k, (name, _, nb) in enumerate(ops):
+    for k, (name, _, nb, nel) in enumerate(ops):
         ms = sum(ev[s][k][0].elapsed_time(ev[s][k][1]) for s in range(args.steps)) / args.steps
         per_op[name] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4),
-                        "elements/s": round(n / ms * 1e3)}
+                        "elements/s": round(nel / ms * 1e3)}
     if args.dump_steps:
         for s in range(args.steps):
             print(s, " ".join("%s=%.4f(host %.0fus)" % (ops[k][0], ev[s][k][0].elapsed_time(ev[s][k][1]),
                                                          host_us[s * len(ops) + k]) for k in range(len(ops))),
                   file=sys.stderr)
-    add_ms = per_op["add"]["ms"] if "add" in per_op else float("nan")
+    # the roofline object describes the op with the largest share of the step
+    dom = max(range(len(ops)), key=lambda k: per_op[ops[k][0]]["ms"])
+    dom_name, _, dom_bytes, _ = ops[dom]
+    dom_ms = per_op[dom_name]["ms"]
+    kernel = ("ew_contig_kernel<add,f32> (c = a + b, 2^28 elements)" if (args.workload, dom_name) == ("metric", "add")
+              else f"{args.workload}:{dom_name}")
+    workload = WORKLOADS[args.workload] if args.ops is None else f"{args.workload}, subset: {args.ops}"
     out = {
-        "metric": "achieved HBM GB/s for fp32 add, axis-sum, argmax at 2^28 elements",
+        "metric": "achieved HBM GB/s for fp32 add, axis-sum, argmax at 2^28 elements" if args.workload == "metric"
+                  else f"achieved HBM GB/s (algorithmic bytes / time), configuration {args.workload}",
         "value": round(step_bytes / ms_per_step / 1e6, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -169,20 +304,20 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic (seeded uniform[-1,1) and normal(0,1), resident in HBM)",
-        "config": {"workload": "fp32 add 2^28 + sum axis=-1 and axis=0 over 16384x16384 + argmax 2^28 (->int64)"
-                   if args.ops == ap.get_default("ops") else "subset: " + args.ops,
-                   "bytes_per_step": step_bytes, "frac_of_hbm_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4)},
+        "dtype": dtype,
+        "data": data,
+        "config": {"workload": workload, "bytes_per_step": step_bytes,
+                   "frac_of_hbm_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4)},
         "per_op": per_op,
-        "roofline": {"bound": "hbm", "kernel": "ew_contig_kernel<add,f32> (c = a + b, 2^28 elements)",
-                     "achieved": round(12 * n / add_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(12 * n / add_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
+        "roofline": {"bound": "hbm", "kernel": kernel,
+                     "achieved": round(dom_bytes / dom_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None},
     }
     traffic_file = os.path.join(ROOT, "profiles", "add_f32_2p28_traffic.json")
-    if os.path.exists(traffic_file):  # HBM bytes per launch from the committed rocprofv3 --pmc summary
+    if (args.workload, dom_name) == ("metric", "add") and os.path.exists(traffic_file):
+        # HBM bytes per launch from the committed rocprofv3 --pmc summary
         out["roofline"]["traffic"] = json.load(open(traffic_file)).get("bytes_per_launch")
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload == "metric":
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 

@@ -99,18 +99,6 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     }
 }
 
-void ew_finish_tile_plan(EwPlan &pl, int TS)
-{
-    const int inner = pl.nd - 1;
-    pl.block = EW_BLOCK;
-    pl.tiles_t = (pl.shape[pl.dT] + TS - 1) / TS;
-    pl.tiles_i = (pl.shape[inner] + TS - 1) / TS;
-    int64_t batch = 1;
-    for (int d = 0; d < inner; ++d)
-        if (d != pl.dT) batch *= pl.shape[d];
-    pl.grid = batch * pl.tiles_t * pl.tiles_i;
-}
-
 void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs)
 {
     if (pl.path == DPX_PATH_NOOP) return;
@@ -127,8 +115,35 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         pl.grid = (pl.n + (int64_t)pl.block * E - 1) / ((int64_t)pl.block * E);
         return;
     }
-    if (pl.path == DPX_PATH_EW_TILE) return; // geometry set by ew_finish_tile_plan
     const int inner = pl.nd - 1;
+    if (pl.path == DPX_PATH_EW_TILE) {
+        // tile = 64 positions along dT x (512 bytes / widest itemsize) positions along the inner dim
+        const int64_t TI = 64, TJ = 32 * E;
+        pl.modes = 0;
+        for (int k = 0; k < nops; ++k) {
+            uint32_t mode = MODE_STRIDED;
+            const bool staged = k + 1 < nops && ((pl.tmask >> k) & 1u);
+            // elements per 16-byte access of this operand and the dim those accesses run along
+            const int64_t ve = staged ? 16 / itemsize[k] : E;
+            const int run = staged ? pl.dT : inner;
+            if (pl.strides[k][run] == 0 && !staged && k + 1 < nops) mode = MODE_BCAST;
+            else if (pl.strides[k][run] == 1 && ((uintptr_t)ptrs[k] % (uintptr_t)(ve * itemsize[k])) == 0 &&
+                     (!staged || pl.shape[run] % ve == 0)) {
+                mode = MODE_VEC;
+                for (int d = 0; d < pl.nd; ++d)
+                    if (d != run && pl.strides[k][d] % ve != 0) mode = MODE_STRIDED;
+            }
+            pl.modes |= mode << (2 * k);
+        }
+        pl.block = EW_BLOCK;
+        pl.tiles_t = (pl.shape[pl.dT] + TI - 1) / TI;
+        pl.tiles_i = (pl.shape[inner] + TJ - 1) / TJ;
+        int64_t batch = 1;
+        for (int d = 0; d < inner; ++d)
+            if (d != pl.dT) batch *= pl.shape[d];
+        pl.grid = batch * pl.tiles_t * pl.tiles_i;
+        return;
+    }
     const int64_t ncols = pl.shape[inner];
     pl.nrows = pl.n / ncols;
     pl.modes = 0;

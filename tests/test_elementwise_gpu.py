@@ -385,3 +385,97 @@ def test_angle_logaddexp_nextafter():
         x[:6] = [0.0, 0.0, -0.0, 1.0, np.inf, np.nan]
         y[:6] = [1.0, -1.0, 0.0, 1.0, 0.0, 0.0]
         assert_same(host(dpt.nextafter(dev(x), dev(y))), np.nextafter(x, y))
+
+
+# ---- transposed operands (LDS tile kernel) ----------------------------------------------------
+def _plan_path(fn_name, *arrays):
+    """Kernel the library would use for these operands (last one is the output)."""
+    import dpnp_amd._lib as L
+
+    p = L.Plan()
+    views = [dpt.broadcast_to(a, arrays[-1].shape)._as_view() for a in arrays]
+    if len(arrays) == 2:
+        L.check(L.lib.dpx_unary_plan(L.UNARY_ID[fn_name], views[0], views[1], p))
+    else:
+        L.check(L.lib.dpx_binary_plan(L.BINARY_ID[fn_name], views[0], views[1], views[2], p))
+    return L.PATH_NAMES[p.path]
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "f2", "i4", "f4", "i8", "f8", "c8", "c16"])
+@pytest.mark.parametrize("shape", [(64, 128), (200, 333), (17, 1000), (1000, 19), (129, 513)])
+def test_transposed_input_all_widths(dt, shape):
+    """out (C-contiguous) = op(A.T): full tiles, ragged edges, lengths that are not a multiple of
+    the 16-byte pack (element-wise staging), every item size."""
+    rng = np.random.default_rng(101)
+    a = random_array(rng, shape[::-1], dt, -50, 50)
+    d = dev(a)
+    out = dpt.empty(shape, dtype=dt)
+    if dt == "?":
+        dpt.logical_not(d.T, out=out)
+        assert _plan_path("logical_not", d.T, out) == "ew_tile"
+        assert_same(host(out), ~a.T)
+    else:
+        dpt.negative(d.T, out=out)
+        assert _plan_path("negative", d.T, out) == "ew_tile"
+        assert_same(host(out), orc.unary("negative", np.ascontiguousarray(a.T)))
+    if dt != "?":  # allocation by the call itself
+        assert_same(host(dpt.positive(d.T, order="C")), np.ascontiguousarray(a.T))
+
+
+def test_transposed_binary_mixed_operands():
+    rng = np.random.default_rng(103)
+    m, n = 150, 260
+    a = random_array(rng, (n, m), "f4")        # used as a.T: transposed
+    b = random_array(rng, (m, n), "f4")        # row oriented
+    row = random_array(rng, (1, n), "f4")      # broadcast along dT
+    col = random_array(rng, (m, 1), "f4")      # broadcast along the inner dim
+    b2 = random_array(rng, (m, 2 * n), "f4")   # stride 2 along the inner dim
+    c = random_array(rng, (n, m), "f4")        # second transposed operand
+    da, db, drow, dcol, db2, dc = map(dev, (a, b, row, col, b2, c))
+    out = dpt.empty((m, n), dtype="f4")
+    for name, x, y, hx, hy in [
+        ("add", da.T, db, a.T, b),
+        ("subtract", db, da.T, b, a.T),
+        ("multiply", da.T, drow, a.T, np.broadcast_to(row, (m, n))),
+        ("multiply", dcol, da.T, np.broadcast_to(col, (m, n)), a.T),
+        ("add", da.T, db2[:, ::2], a.T, b2[:, ::2]),
+        ("subtract", da.T, dc.T, a.T, c.T),
+        ("add", da.T, da.T, a.T, a.T),
+    ]:
+        getattr(dpt, name)(x, y, out=out)
+        assert _plan_path(name, x, y, out) == "ew_tile", name
+        assert_same(host(out), orc.binary(name, np.ascontiguousarray(hx), np.ascontiguousarray(hy)))
+    # mixed item sizes: comparison of a transposed float matrix writes bools
+    ob = dpt.empty((m, n), dtype="?")
+    dpt.greater(da.T, db, out=ob)
+    assert _plan_path("greater", da.T, db, ob) == "ew_tile"
+    assert_same(host(ob), a.T > b)
+    # float64 against transposed float32 after promotion in Python: cast kernel + tile kernel
+    d8 = dev(b.astype("f8"))
+    assert_same(host(dpt.add(da.T, d8, order="C")), a.T.astype("f8") + b.astype("f8"))
+    # where with a transposed condition and transposed branches
+    cond = random_array(rng, (n, m), "?")
+    assert_same(host(dpt.where(dev(cond).T, da.T, db, order="C")), np.where(cond.T, a.T, b))
+    assert_same(host(dpt.where(dev(cond).T, da.T, dc.T, order="C")), np.where(cond.T, a.T, c.T))
+
+
+def test_transposed_with_batch_dims_offsets_and_strided_output():
+    rng = np.random.default_rng(107)
+    a = random_array(rng, (3, 70, 5, 90), "i4")
+    d = dev(a)
+    # swap the two long axes, keep the short ones as batch dims
+    v, hv = dpt.permute_dims(d, (0, 3, 2, 1)), np.transpose(a, (0, 3, 2, 1))
+    assert_same(host(dpt.multiply(v, 3, order="C")), hv * np.int32(3))
+    # views that start inside the allocation: 16-byte alignment is lost for some of them
+    for lo in (1, 2, 3, 4):
+        w, hw = d[0, lo:, 0, lo:].T, a[0, lo:, 0, lo:].T
+        out = dpt.empty(hw.shape, dtype="i4")
+        dpt.negative(w, out=out)
+        assert_same(host(out), -hw)
+    # output that is a row-contiguous slice of a wider matrix
+    big = dpt.zeros((90, 200), dtype="i4")
+    src, hsrc = d[1, :, 2, :].T, a[1, :, 2, :].T      # (90, 70)
+    dpt.negative(src, out=big[:, 7:77])
+    want = np.zeros((90, 200), dtype="i4")
+    want[:, 7:77] = -hsrc
+    assert_same(host(big), want)
