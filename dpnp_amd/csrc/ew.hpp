@@ -30,6 +30,9 @@ constexpr int EW_ROWS_BLOCK = 256;  // default for strided kernels
 
 // operand access mode along the inner dimension (2 bits per operand)
 enum : uint32_t { MODE_STRIDED = 0, MODE_VEC = 1, MODE_BCAST = 2, MODE_VEC2 = 3 };
+// bit MODE_KEEP_SHIFT + k of `modes`: input k is read more than once (a broadcast dim), so its
+// loads are ordinary cached ones instead of non-temporal
+constexpr int MODE_KEEP_SHIFT = 16;
 
 template <int NOPS> struct NdIndex {
     int32_t nd; // >= 1; the last dim is the inner one
@@ -103,6 +106,42 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, u
                                          std::index_sequence_for<Ins...>{});
 }
 
+// Stride-2 operand (x[:, ::2], real or imaginary parts) read by a whole wave: the lane's E
+// elements x[0], x[2], ..., x[2E-2] start at `lane_ptr`; lanes are 2E elements apart.  The wave
+// reads its 2 KiB run with two lane-interleaved 16-byte loads (each instruction covers 1 KiB
+// without holes) and the lanes then pull the two packs that hold their elements from their
+// neighbours' registers.  All 64 lanes of the wave must make the call.  Measured on MI355X
+// against two loads at a 32-byte lane pitch: 6.4 vs 5.9 TB/s of physical traffic.
+template <class T, int E> DPX_D pack<T, E> load_stride2_wave(const T *lane_ptr)
+{
+    static_assert(E >= 2 && sizeof(T) * E == 16);
+    const int lane = threadIdx.x & 63;
+    const T *wp = lane_ptr - (int64_t)lane * 2 * E;
+    const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + lane * E));
+    const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + (64 + lane) * E));
+    const int s = (2 * lane) & 63;
+    const bool first = lane < 32;
+    union {
+        u32x4 r;
+        pack<T, E> p;
+    } lo, hi;
+    lo.r = u32x4{0, 0, 0, 0};
+    hi.r = u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        // dwords that hold an element of even index
+        if (sizeof(T) >= 4 && ((d * 4 / (int)sizeof(T)) & 1)) continue;
+        const uint32_t a0 = __shfl(a[d], s), b0 = __shfl(b[d], s);
+        const uint32_t a1 = __shfl(a[d], s + 1), b1 = __shfl(b[d], s + 1);
+        lo.r[d] = first ? a0 : b0;
+        hi.r[d] = first ? a1 : b1;
+    }
+    pack<T, E> r;
+#pragma unroll
+    for (int e = 0; e < E; ++e) r.v[e] = (2 * e < E) ? lo.p.v[(2 * e) % E] : hi.p.v[(2 * e) % E];
+    return r;
+}
+
 // ---- strided, vectorised along the inner dimension -----------------------------
 // Block = TY rows x TX threads (TX = 1 << tx_log2, TX * TY = blockDim.x); a thread owns E
 // consecutive inner positions of one row.  ix.strides[k] for inputs k < N,
@@ -149,12 +188,16 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         }
     }
     const int cnt = (ncols - col0 < E) ? (int)(ncols - col0) : E;
+    // the 64 lanes of this wave lie in one row and every one of them has a full pack that is
+    // not the last of the row
+    const bool wave_full = tx_log2 >= 6 && col0 - (int64_t)(threadIdx.x & 63) * E + 64 * E < ncols;
     std::tuple<pack<Ins, E>...> v;
-    auto load_operand = [&](auto *p, int64_t o, int64_t st, uint32_t mode) {
+    auto load_operand = [&](auto *p, int64_t o, int64_t st, uint32_t mode, bool keep) {
         using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
         pack<T, E> r;
         if (mode == MODE_VEC && cnt == E) {
-            r = load_pack<T, E>(p + o);
+            // an operand that is re-read along a broadcast dim stays in cache
+            r = keep ? load_pack<T, E, false>(p + o) : load_pack<T, E>(p + o);
         }
         else if (mode == MODE_BCAST) {
             r = splat<T, E>(load_one(p + o));
@@ -164,9 +207,18 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
             // other element.  The loads reach one element past the last one used, which lies
             // inside the view for every pack but the last of a row (that one goes scalar).
             if constexpr (E >= 2) {
-                const pack<T, E> lo = load_pack<T, E>(p + o), hi = load_pack<T, E>(p + o + E);
+                bool done = false;
+                if constexpr (sizeof(T) * E == 16) {
+                    if (wave_full) {
+                        r = load_stride2_wave<T, E>(p + o);
+                        done = true;
+                    }
+                }
+                if (!done) {
+                    const pack<T, E> lo = load_pack<T, E>(p + o), hi = load_pack<T, E>(p + o + E);
 #pragma unroll
-                for (int e = 0; e < E; ++e) r.v[e] = (2 * e < E) ? lo.v[(2 * e) % E] : hi.v[(2 * e) % E];
+                    for (int e = 0; e < E; ++e) r.v[e] = (2 * e < E) ? lo.v[(2 * e) % E] : hi.v[(2 * e) % E];
+                }
             }
         }
         else {
@@ -176,7 +228,7 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         return r;
     };
     ((std::get<I>(v) = load_operand((const Ins *)in.p[I], off[I], ix.strides[I][inner],
-                                    (modes >> (2 * I)) & 3u)),
+                                    (modes >> (2 * I)) & 3u, (modes >> (MODE_KEEP_SHIFT + I)) & 1u)),
      ...);
     pack<Out, E> r;
 #pragma unroll
@@ -331,7 +383,8 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         }
         const uint32_t mode = (modes >> (2 * k)) & 3u;
         const T *q = p + col[k] + i * ix.strides[k][dT];
-        if (mode == MODE_VEC && cnt == E) return load_pack<T, E>(q);
+        if (mode == MODE_VEC && cnt == E)
+            return ((modes >> (MODE_KEEP_SHIFT + k)) & 1u) ? load_pack<T, E, false>(q) : load_pack<T, E>(q);
         if (mode == MODE_BCAST) return splat<T, E>(load_one(q));
         const int64_t st = ix.strides[k][inner];
 #pragma unroll

@@ -99,6 +99,16 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     }
 }
 
+// bits MODE_KEEP_SHIFT + k for inputs with a broadcast (stride 0, extent > 1) dim
+static uint32_t keep_bits(const EwPlan &pl)
+{
+    uint32_t bits = 0;
+    for (int k = 0; k + 1 < pl.nops; ++k)
+        for (int d = 0; d < pl.nd; ++d)
+            if (pl.strides[k][d] == 0 && pl.shape[d] > 1) bits |= 1u << (MODE_KEEP_SHIFT + k);
+    return bits;
+}
+
 void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs)
 {
     if (pl.path == DPX_PATH_NOOP) return;
@@ -135,6 +145,7 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
             }
             pl.modes |= mode << (2 * k);
         }
+        pl.modes |= keep_bits(pl);
         pl.block = EW_BLOCK;
         pl.tiles_t = (pl.shape[pl.dT] + TI - 1) / TI;
         pl.tiles_i = (pl.shape[inner] + TJ - 1) / TJ;
@@ -158,6 +169,7 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         }
         pl.modes |= mode << (2 * k);
     }
+    pl.modes |= keep_bits(pl);
     const int64_t per_row = (ncols + E - 1) / E; // threads wanted along a row
     pl.block = env_block("DPX_EW_ROWS_BLOCK", EW_ROWS_BLOCK);
     int lg = 0, lg_max = 0;

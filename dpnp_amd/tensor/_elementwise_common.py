@@ -7,12 +7,15 @@ allocated result (order "K" keeps the operands' layout), the exception raised fo
 misuse, aliasing rules for `out` (same view: computed in place; partial overlap: computed
 into a temporary then copied).
 """
+from collections import OrderedDict
+
 import numpy as np
 
 from . import _tensor_impl as ti
 from ._copy_utils import _empty_like_orderK, _empty_like_pair_orderK
 from ._ctors import empty, empty_like, full
 from ._device import ExecutionPlacementError  # noqa: F401  (re-exported)
+from ._device import current_stream_ptr
 from ._dtypes import dtype as _as_dtype
 from ._manipulation_functions import _broadcast_shape_impl, broadcast_to
 from ._type_utils import (
@@ -91,7 +94,27 @@ def _as_device_array(o, dt):
         info = np.iinfo(dt)
         if not (info.min <= v <= info.max):
             raise OverflowError(f"Python integer {v} out of bounds for {dt}")
-    return full((), v, dtype=dt)
+    # 0-d constants recur (x * 2, x > 0, ...): keep the most recent ones on the device instead of
+    # launching a fill kernel per call.  Keyed by the bit pattern (so -0.0 and 0.0, and NaN
+    # payloads, stay apart) and by the stream the fill was queued on.
+    try:
+        key = (dt.char, np.asarray(v, dtype=dt).tobytes(), current_stream_ptr())
+    except (OverflowError, TypeError, ValueError):
+        return full((), v, dtype=dt)
+    hit = _SCALAR_CACHE.get(key)
+    if hit is not None:
+        _SCALAR_CACHE.move_to_end(key)
+        return hit
+    arr = full((), v, dtype=dt)
+    arr.flags.writable = False
+    _SCALAR_CACHE[key] = arr
+    if len(_SCALAR_CACHE) > _SCALAR_CACHE_MAX:
+        _SCALAR_CACHE.popitem(last=False)
+    return arr
+
+
+_SCALAR_CACHE = OrderedDict()
+_SCALAR_CACHE_MAX = 128
 
 
 def _norm_order(order):
