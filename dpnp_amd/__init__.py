@@ -9,7 +9,9 @@ from . import _lib  # noqa: F401  (loads libdpnp_amd.so or raises)
 from . import tensor  # noqa: F401
 from .dpnp_iface import *  # noqa: F401,F403
 from .dpnp_iface import __all__ as _iface_all
+from .dpnp_iface_nanfunctions import *  # noqa: F401,F403
+from .dpnp_iface_nanfunctions import __all__ as _nan_all
 from .dpnp_array import dpnp_array as ndarray
 
-__all__ = list(_iface_all) + ["ndarray", "tensor"]
+__all__ = list(_iface_all) + list(_nan_all) + ["ndarray", "tensor"]
 __version__ = "0.1.0"

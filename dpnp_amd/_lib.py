@@ -36,8 +36,9 @@ BINARY_OPS = [
     "logical_xor", "pow", "floor_divide", "remainder", "atan2", "hypot",
     "copysign", "bitwise_left_shift", "bitwise_right_shift", "logaddexp", "nextafter",
 ]
-REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot"]
-SEARCH_OPS = ["argmax", "argmin"]
+REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot",
+              "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev"]
+SEARCH_OPS = ["argmax", "argmin", "nanargmax", "nanargmin"]
 UNARY_ID = {n: i for i, n in enumerate(UNARY_OPS)}
 BINARY_ID = {n: i for i, n in enumerate(BINARY_OPS)}
 REDUCE_ID = {n: i for i, n in enumerate(REDUCE_OPS)}

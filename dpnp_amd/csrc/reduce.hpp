@@ -121,7 +121,12 @@ template <class In, class Out> DPX_D acc_of_t<Out> in_to_acc(In x)
     else return (Acc)convert<Out, In>(x);
 }
 
-enum { K_SUM = 0, K_PROD = 1, K_MAX = 2, K_MIN = 3, K_SUMSQDEV = 4, K_LOGSUMEXP = 5, K_HYPOT = 6 };
+enum {
+    K_SUM = 0, K_PROD = 1, K_MAX = 2, K_MIN = 3, K_SUMSQDEV = 4, K_LOGSUMEXP = 5, K_HYPOT = 6,
+    // NaN-ignoring forms: a NaN element contributes the identity (0, 1, nothing, not counted)
+    K_NANSUM = 7, K_NANPROD = 8, K_NANMAX = 9, K_NANMIN = 10, K_NANCOUNT = 11, K_NANSUMSQDEV = 12
+};
+constexpr bool kind_is_minmax(int k) { return k == K_MAX || k == K_MIN || k == K_NANMAX || k == K_NANMIN; }
 
 template <int KIND, class T> DPX_D T red_identity()
 {
@@ -154,15 +159,19 @@ template <int KIND, class T> DPX_D T red_identity()
 template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy {
     using In = In_;
     using Out = Out_;
-    using Acc = std::conditional_t<(KIND == K_MAX || KIND == K_MIN),
-                                   std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>;
+    using Acc = std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>,
+                                   acc_of_t<Out_>>;
     using Aux = Out_;
-    static constexpr bool has_aux = (KIND == K_SUMSQDEV) && !FINAL;
+    static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV) && !FINAL;
     static constexpr int kind = KIND;
     DPX_D static Acc identity()
     {
         if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
         else if constexpr (is_bool_v<Out>) return KIND == K_PROD ? 1 : 0;
+        else if constexpr (KIND == K_NANMAX || KIND == K_NANMIN) return (Acc)__builtin_nanf(""); // "nothing yet"
+        else if constexpr (KIND == K_NANSUM || KIND == K_NANCOUNT || KIND == K_NANSUMSQDEV)
+            return red_identity<K_SUM, Acc>();
+        else if constexpr (KIND == K_NANPROD) return red_identity<K_PROD, Acc>();
         else return red_identity<KIND, Acc>();
     }
     DPX_D static Acc pre(In x, Acc aux)
@@ -172,7 +181,13 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
             const Acc d = in_to_acc<In, Out>(x) - aux;
             return d * d;
         }
-        else if constexpr (KIND == K_MAX || KIND == K_MIN) {
+        else if constexpr (KIND == K_NANSUMSQDEV) {
+            const Acc d = in_to_acc<In, Out>(x) - aux;
+            return isnan_(x) ? Acc(0) : d * d;
+        }
+        else if constexpr (KIND == K_NANSUM || KIND == K_NANPROD) return isnan_(x) ? identity() : in_to_acc<In, Out>(x);
+        else if constexpr (KIND == K_NANCOUNT) return isnan_(x) ? Acc(0) : Acc(1);
+        else if constexpr (kind_is_minmax(KIND)) {
             if constexpr (is_bool_v<Out>) return (int32_t)(x.v != 0);
             else return x; // In == Out
         }
@@ -184,11 +199,15 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
             if constexpr (KIND == K_PROD || KIND == K_MIN) return a & b;
             else return a | b;
         }
-        else if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV) return a + b;
-        else if constexpr (KIND == K_PROD) return a * b;
+        else if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV || KIND == K_NANSUM || KIND == K_NANCOUNT ||
+                           KIND == K_NANSUMSQDEV)
+            return a + b;
+        else if constexpr (KIND == K_PROD || KIND == K_NANPROD) return a * b;
         else if constexpr (KIND == K_LOGSUMEXP) return LogaddexpOp::apply<Acc>(a, b);
         else if constexpr (KIND == K_HYPOT) return m_hypot(a, b);
         else if constexpr (KIND == K_MAX) return max_nan(a, b);
+        else if constexpr (KIND == K_NANMAX) return isnan_(a) ? b : (isnan_(b) ? a : (a > b ? a : b));
+        else if constexpr (KIND == K_NANMIN) return isnan_(a) ? b : (isnan_(b) ? a : (a < b ? a : b));
         else return min_nan(a, b);
     }
     DPX_D static Out post(Acc a) { return acc_to_out<Acc, Out>(a); }

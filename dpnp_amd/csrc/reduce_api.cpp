@@ -14,6 +14,13 @@ int minmax_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, 
 int arg_run_any(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 int fpred_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 bool fpred_pair_supported(int, int);
+bool nan_pair_supported(int, int, int);
+int nan_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+int nan_acc_size(int, const dpx_array_view *, const dpx_array_view *);
+int nanarg_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+
+static bool is_nan_op(int op) { return op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV; }
+static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV; }
 
 static bool reduce_supported(int op, int s, int d)
 {
@@ -26,7 +33,7 @@ static bool reduce_supported(int op, int s, int d)
     case DPX_R_SUMSQDEV: return sqdev_pair_supported(s, d);
     case DPX_R_LOGSUMEXP:
     case DPX_R_HYPOT: return fpred_pair_supported(s, d);
-    default: return false;
+    default: return is_nan_op(op) && nan_pair_supported(op, s, d);
     }
 }
 
@@ -35,11 +42,11 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
 {
     if (op < 0 || op >= DPX_R_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown reduction op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
-    if ((op == DPX_R_SUMSQDEV) != (aux != nullptr))
-        return fail(DPX_ERR_BAD_ARGUMENT, "aux must be given for DPX_R_SUMSQDEV and only for it");
+    if (takes_aux(op) != (aux != nullptr))
+        return fail(DPX_ERR_BAD_ARGUMENT, "aux must be given for the squared-deviation ops and only for them");
     if (!reduce_supported(op, src->dtype, dst->dtype))
         return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
-    const bool empty_ok = op != DPX_R_MAX && op != DPX_R_MIN;
+    const bool empty_ok = op != DPX_R_MAX && op != DPX_R_MIN && op != DPX_R_NANMAX && op != DPX_R_NANMIN;
     if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false);
@@ -49,10 +56,12 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
         if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
+        if (is_nan_op(op)) acc = nan_acc_size(op, src, dst);
         red_export_plan(pl, plan_out, acc);
         return DPX_OK;
     }
     hipStream_t s = (hipStream_t)stream;
+    if (is_nan_op(op)) return nan_run(op, pl, src, dst, aux, s);
     switch (op) {
     case DPX_R_SUM: return sum_run(pl, src, dst, s);
     case DPX_R_PROD: return prod_run(pl, src, dst, s);
@@ -64,12 +73,20 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     }
 }
 
+static bool search_supported(int op, int s, int d)
+{
+    if (s < 0 || s >= DPX_NUM_DTYPES || d != DPX_INT64) return false;
+    if (op == DPX_S_ARGMAX || op == DPX_S_ARGMIN) return true;
+    if (op == DPX_S_NANARGMAX || op == DPX_S_NANARGMIN) return s == DPX_HALF || s == DPX_FLOAT || s == DPX_DOUBLE;
+    return false;
+}
+
 static int argreduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
                           void *stream, dpx_plan *plan_out)
 {
-    if (op != DPX_S_ARGMAX && op != DPX_S_ARGMIN) return fail(DPX_ERR_BAD_ARGUMENT, "unknown search op id");
+    if (op < 0 || op > DPX_S_NANARGMIN) return fail(DPX_ERR_BAD_ARGUMENT, "unknown search op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
-    if (dst->dtype != DPX_INT64) return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
+    if (!search_supported(op, src->dtype, dst->dtype)) return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
     if (int rc = red_validate(src, trailing, dst, nullptr, false)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, nullptr, true, itemsize_of(src->dtype), true);
@@ -77,6 +94,8 @@ static int argreduce_call(int op, const dpx_array_view *src, int trailing, const
         red_export_plan(pl, plan_out, itemsize_of(src->dtype) + 8);
         return DPX_OK;
     }
+    if (op == DPX_S_NANARGMAX || op == DPX_S_NANARGMIN)
+        return nanarg_run(op == DPX_S_NANARGMAX, pl, src, dst, (hipStream_t)stream);
     return arg_run_any(op == DPX_S_ARGMAX, pl, src, dst, (hipStream_t)stream);
 }
 
@@ -85,13 +104,7 @@ static int argreduce_call(int op, const dpx_array_view *src, int trailing, const
 using namespace dpx;
 extern "C" {
 int dpx_reduce_dtype_supported(int op, int src_dt, int dst_dt) { return reduce_supported(op, src_dt, dst_dt) ? 1 : 0; }
-int dpx_search_dtype_supported(int op, int src_dt, int dst_dt)
-{
-    return ((op == DPX_S_ARGMAX || op == DPX_S_ARGMIN) && src_dt >= 0 && src_dt < DPX_NUM_DTYPES &&
-            dst_dt == DPX_INT64)
-               ? 1
-               : 0;
-}
+int dpx_search_dtype_supported(int op, int src_dt, int dst_dt) { return search_supported(op, src_dt, dst_dt) ? 1 : 0; }
 int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
                const dpx_array_view *aux, void *stream)
 {
@@ -101,9 +114,10 @@ int dpx_reduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_redu
                     dpx_plan *plan)
 {
     if (!plan) return fail(DPX_ERR_BAD_ARGUMENT, "plan is null");
-    // a plan for DPX_R_SUMSQDEV is that of DPX_R_SUM with the same dtypes
-    return reduce_call(op == DPX_R_SUMSQDEV ? DPX_R_SUM : op, src, trailing_dims_to_reduce, dst, nullptr, nullptr,
-                       plan);
+    // a plan for a squared-deviation op is that of the matching sum with the same dtypes
+    if (op == DPX_R_SUMSQDEV) op = DPX_R_SUM;
+    if (op == DPX_R_NANSUMSQDEV) op = DPX_R_NANSUM;
+    return reduce_call(op, src, trailing_dims_to_reduce, dst, nullptr, nullptr, plan);
 }
 int dpx_argreduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
                   void *stream)

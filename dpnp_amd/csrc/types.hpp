@@ -153,12 +153,30 @@ template <class T> struct value_of {
 template <> struct value_of<bool_t> {
     using type = bool;
 };
+// A floating element read as "NaN loses": NaN becomes -inf for a maximum search and +inf for a
+// minimum search (nanargmax / nanargmin replace NaN this way before searching,
+// dpnp/dpnp_iface_nanfunctions.py:195,279).
+template <class T, bool IS_MAX> struct nanskip {
+    T v;
+};
+template <class T> struct is_nanskip : std::false_type {};
+template <class T, bool M> struct is_nanskip<nanskip<T, M>> : std::true_type {
+    static constexpr bool is_max = M;
+};
+template <class T, bool M> struct value_of<nanskip<T, M>> {
+    using type = T;
+};
 template <class T> using value_of_t = typename value_of<T>::type;
 
 template <class T> DPX_HD value_of_t<T> to_value(const T &s)
 {
     if constexpr (is_bool_v<T>)
         return s.v != 0;
+    else if constexpr (is_nanskip<T>::value) {
+        using V = value_of_t<T>;
+        const V inf = (V)__builtin_inff();
+        return (s.v != s.v) ? (is_nanskip<T>::is_max ? -inf : inf) : s.v;
+    }
     else
         return s;
 }
@@ -166,6 +184,8 @@ template <class T> DPX_HD T to_storage(const value_of_t<T> &v)
 {
     if constexpr (is_bool_v<T>)
         return bool_t{(uint8_t)(v ? 1 : 0)};
+    else if constexpr (is_nanskip<T>::value)
+        return T{v};
     else
         return v;
 }

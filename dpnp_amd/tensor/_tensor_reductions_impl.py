@@ -42,13 +42,25 @@ _argmax_over_axis = _make_search("argmax", _lib.SEARCH_ID["argmax"])
 _argmin_over_axis = _make_search("argmin", _lib.SEARCH_ID["argmin"])
 
 
-def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
+# NaN-ignoring forms (no counterpart among the reference's extension functions: dpnp builds
+# nansum, nanmax, ... from a masked copy and the plain reductions,
+# dpnp/dpnp_iface_nanfunctions.py:48-116)
+_nansum_over_axis, _nansum_over_axis_dtype_supported = _make_reduction("nansum", _lib.REDUCE_ID["nansum"])
+_nanprod_over_axis, _nanprod_over_axis_dtype_supported = _make_reduction("nanprod", _lib.REDUCE_ID["nanprod"])
+_nanmax_over_axis, _nanmax_over_axis_dtype_supported = _make_reduction("nanmax", _lib.REDUCE_ID["nanmax"])
+_nanmin_over_axis, _nanmin_over_axis_dtype_supported = _make_reduction("nanmin", _lib.REDUCE_ID["nanmin"])
+_nancount_over_axis, _nancount_over_axis_dtype_supported = _make_reduction("nancount", _lib.REDUCE_ID["nancount"])
+_nanargmax_over_axis = _make_search("nanargmax", _lib.SEARCH_ID["nanargmax"])
+_nanargmin_over_axis = _make_search("nanargmin", _lib.SEARCH_ID["nanargmin"])
+
+
+def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None, depends=(), nan=False):
     """dst[i] = sum_j (src[i, j] - mean[i])**2: the second pass of var in one kernel
     (the reference runs subtract, square and sum kernels over a full-size temporary,
     dpnp/tensor/_statistical_functions.py:38-163)."""
     vs, vm, vd = src._as_view(), mean._as_view(), dst._as_view()
-    _lib.check(lib.dpx_reduce(_lib.REDUCE_ID["sumsqdev"], vs, int(trailing_dims_to_reduce), vd, vm,
-                              _stream(sycl_queue)))
+    op = _lib.REDUCE_ID["nansumsqdev" if nan else "sumsqdev"]
+    _lib.check(lib.dpx_reduce(op, vs, int(trailing_dims_to_reduce), vd, vm, _stream(sycl_queue)))
     return _events(sycl_queue)
 
 

@@ -181,10 +181,28 @@ typedef enum dpx_reduce_op {
     DPX_R_SUMSQDEV, /* sum((x - aux)^2): second pass of var, see dpx_reduce */
     DPX_R_LOGSUMEXP, /* log(sum(exp(x))), libtensor/source/reductions/logsumexp.cpp */
     DPX_R_HYPOT,     /* sqrt(sum(x^2)) by pairwise hypot, libtensor/source/reductions/reduce_hypot.cpp */
+    /* NaN-ignoring forms, floating inputs only.  The reference composes them from a masked copy
+     * and the plain reduction (dpnp/dpnp_iface_nanfunctions.py:48-116,509-518,600-636,1318-1390);
+     * here NaN elements are replaced as they are read.  NANMAX / NANMIN give NaN for a run that
+     * holds nothing but NaN; NANCOUNT counts the elements that are not NaN (int64 result);
+     * NANSUMSQDEV is SUMSQDEV with NaN elements contributing zero. */
+    DPX_R_NANSUM,
+    DPX_R_NANPROD,
+    DPX_R_NANMAX,
+    DPX_R_NANMIN,
+    DPX_R_NANCOUNT,
+    DPX_R_NANSUMSQDEV,
     DPX_R_NUM_OPS
 } dpx_reduce_op;
 
-typedef enum dpx_search_op { DPX_S_ARGMAX = 0, DPX_S_ARGMIN = 1 } dpx_search_op;
+typedef enum dpx_search_op {
+    DPX_S_ARGMAX = 0,
+    DPX_S_ARGMIN = 1,
+    /* NaN elements never win (real floating inputs): dpnp.nanargmax / nanargmin,
+     * dpnp/dpnp_iface_nanfunctions.py:119-284 */
+    DPX_S_NANARGMAX = 2,
+    DPX_S_NANARGMIN = 3
+} dpx_search_op;
 
 /* which kernel family a call resolves to (reported by the dpx_*_plan queries;
  * lets the host-side dispatch be tested without a GPU) */
@@ -309,7 +327,7 @@ int dpx_black_scholes(const void *price, const void *strike, const void *t,
  * reduction_over_axis.hpp:174-501,508-777 (tri._sum_over_axis, _prod_over_axis,
  * _max_over_axis, _min_over_axis).  The last `trailing_dims_to_reduce` axes of
  * src are reduced; dst has the leading src.nd - trailing axes.
- * op == DPX_R_SUMSQDEV additionally takes `aux` (same shape and dtype as dst,
+ * op == DPX_R_SUMSQDEV (and DPX_R_NANSUMSQDEV) additionally takes `aux` (same shape and dtype as dst,
  * any strides): dst[i] = sum_j (src[i,j] - aux[i])^2; aux is NULL otherwise. */
 int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
                const dpx_array_view *dst, const dpx_array_view *aux,

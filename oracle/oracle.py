@@ -471,6 +471,91 @@ def var(a, trailing, correction=0.0, out_dtype=None):
 
 
 # ---------------------------------------------------------------------------------------------
+# NaN-ignoring reductions: dpnp/dpnp_iface_nanfunctions.py
+# ---------------------------------------------------------------------------------------------
+def _replace_nan(a, val):
+    """dpnp/dpnp_iface_nanfunctions.py:78-116: (copy of `a` with NaNs overwritten by val, mask of
+    the NaNs) for inexact input, (a, None) otherwise or when there is no NaN."""
+    a = np.asarray(a)
+    if a.dtype.kind not in "fc":
+        return a, None
+    mask = np.isnan(a)
+    if not mask.any():
+        return a, None
+    b = a.copy()
+    b[mask] = val
+    return b, mask
+
+
+def nan_reduce(op, a, trailing, out_dtype=None):
+    """nansum / nanprod / nanmax / nanmin over the last `trailing` axes.
+    nansum, nanprod (dpnp_iface_nanfunctions.py:922,1026): NaN -> 1 / 0, then the plain reduction.
+    nanmax, nanmin (:509-518, :825-834): NaN -> -inf / +inf, plain reduction, NaN written where the
+    whole run was NaN.  Returns (result, all_nan_seen)."""
+    a = np.asarray(a)
+    if op in ("nansum", "nanprod"):
+        b, _ = _replace_nan(a, 0.0 if op == "nansum" else 1.0)
+        return reduce(op[3:], b, trailing, out_dtype), False
+    b, mask = _replace_nan(a, -np.inf if op == "nanmax" else np.inf)
+    res = reduce(op[3:], b, trailing)
+    if mask is None:
+        return res, False
+    m2, _, _ = _split(mask, trailing)
+    bad = m2.all(axis=-1)
+    res = np.where(bad, np.nan, res).astype(res.dtype)
+    return res, bool(bad.any())
+
+
+def nan_argreduce(op, a, trailing):
+    """nanargmax / nanargmin (dpnp_iface_nanfunctions.py:195-200, 279-284): NaN -> -inf / +inf, then
+    argmax / argmin; a run of NaNs only raises ValueError."""
+    b, mask = _replace_nan(a, -np.inf if op == "nanargmax" else np.inf)
+    if mask is not None:
+        m2, _, _ = _split(mask, trailing)
+        if m2.all(axis=-1).any():
+            raise ValueError("All-NaN slice encountered")
+    return argreduce(op[3:], b, trailing)
+
+
+def nanmean(a, trailing, out_dtype=None):
+    """dpnp_iface_nanfunctions.py:600-636: sum of the non-NaN elements / their number."""
+    a = np.asarray(a)
+    b, mask = _replace_nan(a, 0)
+    if mask is None:
+        return mean(a, trailing, out_dtype)
+    dt = np.dtype(out_dtype) if out_dtype else a.dtype
+    m2, lead, n = _split(mask, trailing)
+    cnt = (~m2).sum(axis=-1)
+    b2, _, _ = _split(b, trailing)
+    if dt.kind == "c":
+        s = _fsum(b2.real, lead) + 1j * _fsum(b2.imag, lead)
+    else:
+        s = _fsum(b2, lead)
+    with np.errstate(all="ignore"):
+        return (s / cnt).astype(dt)
+
+
+def nanvar(a, trailing, ddof=0, out_dtype=None):
+    """dpnp_iface_nanfunctions.py:1318-1391 for real input: mean of the non-NaN elements, squared
+    deviations with the NaN positions zeroed, divided by (count - ddof); NaN where that is <= 0."""
+    a = np.asarray(a)
+    b, mask = _replace_nan(a, 0)
+    if mask is None:
+        return var(a, trailing, ddof, out_dtype)
+    dt = np.dtype(out_dtype) if out_dtype else a.dtype
+    m2, lead, n = _split(mask, trailing)
+    b2 = _split(b, trailing)[0].astype(np.longdouble)
+    cnt = (~m2).sum(axis=-1, keepdims=True)
+    with np.errstate(all="ignore"):
+        avg = b2.sum(axis=-1, keepdims=True) / cnt
+        dev = np.where(m2, 0, b2 - avg)
+        dof = cnt[..., 0] - ddof
+        res = (dev * dev).sum(axis=-1) / dof
+    res = np.where(dof <= 0, np.nan, res)
+    return res.astype(dt)
+
+
+# ---------------------------------------------------------------------------------------------
 # stride collapsing: libtensor/include/utils/strided_iters.hpp:364-899,946-983
 # ---------------------------------------------------------------------------------------------
 def address_tuples(shape, strides_list, offsets=None):

@@ -4,6 +4,7 @@ import itertools
 import json
 import math
 import os
+import warnings
 
 import numpy as np
 import pytest
@@ -332,3 +333,37 @@ def test_round_conj_parts_proj_rules():
     # logaddexp closed forms: log(e^x + e^x) = x + log 2; one operand at -inf leaves the other
     assert orc.binary("logaddexp", np.array([3.0]), np.array([3.0]))[0] == 3.0 + np.log(2.0)
     assert orc.binary("logaddexp", np.array([-np.inf]), np.array([7.0]))[0] == 7.0
+
+
+# ---- NaN-ignoring reductions: the restated composition against NumPy's nan-functions ----------
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+def test_oracle_nan_functions_match_numpy(dt):
+    rng = np.random.default_rng(5)
+    a = rng.uniform(-5, 5, (6, 9, 4)).astype(dt)
+    a[rng.random(a.shape) < 0.3] = np.nan
+    a[1, :, 2] = np.nan
+    for trailing, axis in ((1, -1), (2, (1, 2)), (3, None)):
+        for name in ("nansum", "nanprod", "nanmax", "nanmin"):
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore", RuntimeWarning)
+                want = getattr(np, name)(a.astype("f8"), axis=axis)
+            got, _ = orc.nan_reduce(name, a, trailing)
+            np.testing.assert_allclose(got, want, rtol=2e-6 if dt == "f4" else 1e-13, equal_nan=True)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", RuntimeWarning)
+            np.testing.assert_allclose(orc.nanmean(a, trailing), np.nanmean(a.astype("f8"), axis=axis),
+                                       rtol=2e-6 if dt == "f4" else 1e-13, equal_nan=True)
+            np.testing.assert_allclose(orc.nanvar(a, trailing, 1), np.nanvar(a.astype("f8"), axis=axis, ddof=1),
+                                       rtol=2e-5 if dt == "f4" else 1e-12, equal_nan=True)
+    b = a.copy()
+    b[..., 0] = rng.uniform(-5, 5, b.shape[:-1]).astype(dt)  # no run of NaNs only
+    assert_equal = np.testing.assert_array_equal
+    assert_equal(orc.nan_argreduce("nanargmax", b, 1), np.nanargmax(b, axis=-1))
+    assert_equal(orc.nan_argreduce("nanargmin", b, 1), np.nanargmin(b, axis=-1))
+    with pytest.raises(ValueError):
+        orc.nan_argreduce("nanargmax", a, 1)
+    # reference docstring values (dpnp/dpnp_iface_nanfunctions.py:583-590,1301-1306)
+    c = np.array([[1, np.nan], [3, 4]])
+    assert orc.nanmean(c, 2) == pytest.approx(2.6666666666666665)
+    np.testing.assert_allclose(orc.nanvar(c.T, 1), [1.0, 0.0])
+    assert orc.nanvar(c, 2) == pytest.approx(1.5555555555555556)

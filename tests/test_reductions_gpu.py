@@ -3,10 +3,12 @@ results bit-exact; float32 sums within 1e-5 and float64 sums within 1e-12 of the
 (relative to the sum of magnitudes, since the reference's summation order is unspecified)."""
 import json
 import os
+import warnings
 
 import numpy as np
 import pytest
 
+import dpnp_amd as dpnp
 import dpnp_amd.tensor as dpt
 from oracle import oracle as orc
 from tests.helpers import ALL, assert_same, dev, dev_view_like, host, random_array
@@ -275,3 +277,166 @@ def test_logsumexp_hypot_count_nonzero():
     m = rng.integers(-1, 2, (40, 50)).astype("i1")
     assert_same(host(dpt.count_nonzero(dev(m), axis=0)), np.count_nonzero(m, axis=0).astype("i8"))
     assert int(dpt.count_nonzero(dev(m))) == int(np.count_nonzero(m))
+
+
+# ---- NaN-ignoring reductions (one-pass kernels behind dpnp.nansum, nanmax, ...) ---------------
+def _with_nans(rng, shape, dt, frac=0.2):
+    a = random_array(rng, shape, dt, -10, 10)
+    a[rng.random(shape) < frac] = np.nan
+    return a
+
+
+@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
+@pytest.mark.parametrize("axis", [None, 0, 1, -1, (0, 2)])
+def test_nan_reductions_against_oracle(dt, axis):
+    rng = np.random.default_rng(211)
+    a = _with_nans(rng, (7, 33, 20), dt)
+    a[3, :, 5] = np.nan       # all-NaN runs along axis 1
+    d = dpnp.array(a)
+    for name in ("nansum", "nanprod", "nanmax", "nanmin"):
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", RuntimeWarning)
+            got = getattr(dpnp, name)(d, axis=axis).asnumpy()
+            want_np = getattr(np, name)(a.astype("f8") if name == "nanprod" else a, axis=axis)
+        ax = tuple(range(a.ndim)) if axis is None else (axis if isinstance(axis, tuple) else (axis % a.ndim,))
+        moved = np.moveaxis(a, ax, tuple(range(a.ndim - len(ax), a.ndim)))
+        want, _ = orc.nan_reduce(name, moved, len(ax))
+        assert got.dtype == a.dtype and got.shape == np.shape(want_np)
+        if name in ("nanmax", "nanmin"):
+            assert_same(got, want)
+            assert_same(got, np.asarray(want_np, dtype=dt))
+        else:
+            scale = (np.nansum(np.abs(moved.astype("f8")), axis=tuple(range(moved.ndim - len(ax), moved.ndim)))
+                     if name == "nansum" else np.abs(np.asarray(want, dtype="f8")))
+            tol = {"f2": 2e-3, "f4": 1e-5, "f8": 1e-12}[dt]
+            ok = np.abs(got.astype("f8") - np.asarray(want, dtype="f8")) <= tol * np.maximum(scale, 1e-30)
+            both_inf = np.isinf(got) & (got == np.asarray(want, dtype=dt))
+            assert np.all(ok | both_inf), name
+
+
+def test_nan_extrema_all_nan_warns_and_arg_raises():
+    a = np.arange(12, dtype="f4").reshape(2, 2, 3)
+    a[:, :, 2] = np.nan
+    d = dpnp.array(a)
+    with pytest.warns(RuntimeWarning, match="All-NaN slice"):
+        r = dpnp.nanmax(d, axis=0)
+    assert_same(r.asnumpy(), np.array([[0 + 6, 7, np.nan], [9, 10, np.nan]], dtype="f4"))
+    with pytest.raises(ValueError, match="All-NaN slice"):
+        dpnp.nanargmax(d, axis=0)
+    with pytest.raises(ValueError, match="All-NaN slice"):
+        dpnp.nanargmin(d, axis=0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert_same(dpnp.nanmin(d, axis=2).asnumpy(), np.nanmin(a, axis=2))  # no all-NaN run: no warning
+
+
+@pytest.mark.parametrize("func", ["nanargmin", "nanargmax"])
+@pytest.mark.parametrize("axis", [None, 0, 1, -1, 2, -2])
+@pytest.mark.parametrize("keepdims", [False, True])
+@pytest.mark.parametrize("dt", ["f4", "f8", "c8"])
+def test_nanarg_reference_basic(func, axis, keepdims, dt):
+    # dpnp/tests/test_nanfunctions.py:33-43
+    a = np.arange(768, dtype=dt).reshape((4, 4, 6, 8))
+    a[2:3, 2, 3:4, 4] = np.nan
+    got = getattr(dpnp, func)(dpnp.array(a), axis=axis, keepdims=keepdims).asnumpy()
+    assert_same(got, np.asarray(getattr(np, func)(a, axis=axis, keepdims=keepdims), dtype="i8"))
+
+
+def test_nanarg_ties_infinities_and_large():
+    rng = np.random.default_rng(223)
+    # -inf present together with NaN: NaN reads as -inf, the first of either wins
+    a = np.array([np.nan, -np.inf, 3.0, 3.0, np.nan], dtype="f4")
+    assert int(dpnp.nanargmax(dpnp.array(a))) == 2
+    assert int(dpnp.nanargmin(dpnp.array(a))) == 1
+    b = np.array([np.nan, -np.inf, -np.inf], dtype="f8")
+    assert int(dpnp.nanargmax(dpnp.array(b))) == int(orc.nan_argreduce("nanargmax", b, 1)) == 0
+    # long 1-D input: split over blocks
+    n = 3_000_003
+    x = rng.standard_normal(n).astype("f4")
+    x[rng.choice(n, n // 50, replace=False)] = np.nan
+    x[rng.choice(n, 100, replace=False)] = np.nanmax(x)
+    d = dpnp.array(x)
+    assert int(dpnp.nanargmax(d)) == int(np.nanargmax(x))
+    assert int(dpnp.nanargmin(d)) == int(np.nanargmin(x))
+    assert float(dpnp.nanmax(d)) == float(np.nanmax(x))
+    s, want = float(dpnp.nansum(d)), float(np.nansum(x.astype("f8")))
+    assert abs(s - want) <= 1e-5 * float(np.nansum(np.abs(x.astype("f8"))))
+    m = x.reshape(3, -1)[:, :1_000_000].T.copy()      # (1000000, 3): column reductions over a long axis
+    dm = dpnp.array(m)
+    assert_same(dpnp.nanargmax(dm, axis=0).asnumpy(), np.nanargmax(m, axis=0))
+    assert_same(dpnp.nanmin(dm, axis=0).asnumpy(), np.nanmin(m, axis=0))
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+@pytest.mark.parametrize("axis", [None, 0, 1, (0, 1)])
+@pytest.mark.parametrize("keepdims", [False, True])
+def test_nanmean_nanvar_nanstd(dt, axis, keepdims):
+    rng = np.random.default_rng(227)
+    a = _with_nans(rng, (19, 23, 5), dt, 0.3)
+    a[:, 4, 1] = np.nan
+    a[2, :, :] = np.nan
+    d = dpnp.array(a)
+    tol = {"f4": 2e-5, "f8": 1e-12}[dt]
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        for name, kw in (("nanmean", {}), ("nanvar", {}), ("nanvar", {"ddof": 1}), ("nanstd", {"ddof": 2})):
+            got = getattr(dpnp, name)(d, axis=axis, keepdims=keepdims, **kw).asnumpy()
+            want = getattr(np, name)(a.astype("f8"), axis=axis, keepdims=keepdims, **kw)
+            assert got.dtype == a.dtype and got.shape == np.shape(want), name
+            np.testing.assert_allclose(got, want, rtol=tol * 20, atol=tol, equal_nan=True, err_msg=name)
+    # the oracle's restatement of the reference's composition agrees as well
+    ax = tuple(range(3)) if axis is None else (axis if isinstance(axis, tuple) else (axis,))
+    moved = np.moveaxis(a, ax, tuple(range(3 - len(ax), 3)))
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        np.testing.assert_allclose(dpnp.nanvar(d, axis=axis).asnumpy(), orc.nanvar(moved, len(ax)),
+                                   rtol=tol * 20, atol=tol, equal_nan=True)
+        np.testing.assert_allclose(dpnp.nanmean(d, axis=axis).asnumpy(), orc.nanmean(moved, len(ax)),
+                                   rtol=tol * 20, atol=tol, equal_nan=True)
+
+
+def test_nan_functions_arguments_and_other_dtypes():
+    a = np.array([[1, np.nan], [3, 4]], dtype="f8")
+    d = dpnp.array(a)
+    # docstring examples of the reference (dpnp_iface_nanfunctions.py:583-590, 1301-1306)
+    np.testing.assert_allclose(float(dpnp.nanmean(d)), 2.6666666666666665, rtol=1e-15)
+    assert_same(dpnp.nanmean(d, axis=0).asnumpy(), np.array([2.0, 4.0]))
+    np.testing.assert_allclose(float(dpnp.nanvar(d)), 1.5555555555555556, rtol=1e-14)
+    assert_same(dpnp.nanvar(d, axis=0).asnumpy(), np.array([1.0, 0.0]))
+    np.testing.assert_allclose(float(dpnp.nanstd(d)), 1.247219128924647, rtol=1e-14)
+    # integer input takes the plain functions
+    i = dpnp.array(np.arange(12, dtype="i4").reshape(3, 4))
+    assert int(dpnp.nansum(i)) == 66 and dpnp.nansum(i).dtype == np.dtype("i8")
+    assert int(dpnp.nanargmax(i)) == 11 and int(dpnp.nanmax(i)) == 11
+    assert float(dpnp.nanmean(i)) == 5.5
+    # out=, dtype=
+    out = dpnp.empty(2, dtype="f8")
+    assert dpnp.nansum(d, axis=1, out=out) is out
+    assert_same(out.asnumpy(), np.array([1.0, 7.0]))
+    assert dpnp.nansum(dpnp.array(a.astype("f4")), dtype="f8").dtype == np.dtype("f8")
+    oi = dpnp.empty(2, dtype="i8")
+    assert dpnp.nanargmin(d, axis=0, out=oi) is oi
+    assert_same(oi.asnumpy(), np.array([0, 1]))
+    with pytest.raises(TypeError):
+        dpnp.nanmean(d, dtype="i4")
+    with pytest.raises(TypeError):
+        dpnp.nanmean(d, out=dpnp.empty((), dtype="i4"))
+    with pytest.raises(NotImplementedError):
+        dpnp.nanmean(d, where=False)
+    with pytest.raises(TypeError):
+        dpnp.nanargmax(d, axis=0, out=dpnp.empty(2, dtype="f4"))
+    # complex sums skip NaN in either part
+    c = np.array([1 + 2j, np.nan + 1j, 3 - 1j, 2 + np.nan * 1j], dtype="c8")
+    assert complex(dpnp.nansum(dpnp.array(c))) == 4 + 1j
+    assert complex(dpnp.nanprod(dpnp.array(c))) == (1 + 2j) * (3 - 1j)
+    np.testing.assert_allclose(complex(dpnp.nanmean(dpnp.array(c))), 2 + 0.5j)
+    # mean= keyword of nanvar (dpnp/tests/test_nanfunctions.py:716-717)
+    b = np.array([[14, 8, np.nan, 10], [7, 9, 10, 11], [np.nan, 15, 5, 10]])
+    db = dpnp.array(b)
+    mu = dpnp.nanmean(db, axis=1, keepdims=True)
+    np.testing.assert_allclose(dpnp.nanvar(db, axis=1, mean=mu).asnumpy(), [6.22222222, 2.1875, 16.66666667], rtol=1e-8)
+    # empty input
+    e = dpnp.array(np.zeros((0, 3), dtype="f4"))
+    assert_same(dpnp.nansum(e, axis=0).asnumpy(), np.zeros(3, dtype="f4"))
+    with pytest.raises(ValueError):
+        dpnp.nanmax(e, axis=0)
