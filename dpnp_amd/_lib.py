@@ -28,6 +28,8 @@ UNARY_OPS = [
     "cbrt", "reciprocal", "floor", "ceil", "trunc", "sign", "isnan", "isinf",
     "isfinite", "logical_not", "bitwise_invert", "signbit", "asin", "acos", "atan", "sinh",
     "cosh", "asinh", "acosh", "atanh", "round", "conj", "real", "imag", "proj", "angle",
+    "fabs", "degrees", "radians", "sinc", "spacing", "bitwise_count", "erfc", "erfcx", "erfinv",
+    "erfcinv", "i0",
 ]
 BINARY_OPS = [
     "add", "subtract", "multiply", "divide", "bitwise_and", "bitwise_or",
@@ -35,6 +37,7 @@ BINARY_OPS = [
     "greater_equal", "maximum", "minimum", "logical_and", "logical_or",
     "logical_xor", "pow", "floor_divide", "remainder", "atan2", "hypot",
     "copysign", "bitwise_left_shift", "bitwise_right_shift", "logaddexp", "nextafter",
+    "fmax", "fmin", "fmod", "logaddexp2", "heaviside", "gcd", "lcm",
 ]
 REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot",
               "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev"]
@@ -104,6 +107,8 @@ SIGNATURES = {
     "dpx_binary_inplace": (_i, [_i, _VP, _VP, _vp]),
     "dpx_where": (_i, [_VP, _VP, _VP, _VP, _vp]),
     "dpx_divide_by_scalar": (_i, [_VP, _d, _VP, _vp]),
+    "dpx_nan_to_num": (_i, [_VP, _d, _d, _d, _VP, _vp]),
+    "dpx_isclose": (_i, [_VP, _VP, _d, _d, _i, _VP, _vp]),
     "dpx_copy_cast": (_i, [_VP, _VP, _vp]),
     "dpx_fill": (_i, [_VP, _d, _d, _i64, _i, _vp]),
     "dpx_unary_plan": (_i, [_i, _VP, _VP, _PP]),

@@ -129,6 +129,90 @@ static int divide_by_scalar_call(const dpx_array_view *src, double scalar, const
     }
 }
 
+// ---- nan_to_num: dpnp/backend/kernels/elementwise_functions/nan_to_num.hpp:44-104 (scalar
+// replacement values; complex elements are treated part by part) ---------------------------------
+template <class T> struct NanToNumFn {
+    using R = real_of_t<T>;
+    R nan, posinf, neginf;
+    DPX_D R one(R v) const { return (v != v) ? nan : (m_isinf(v) ? (v > R(0) ? posinf : neginf) : v); }
+    DPX_D T operator()(T x) const
+    {
+        if constexpr (is_cplx_v<T>) return T{one(x.re), one(x.im)};
+        else return one(x);
+    }
+};
+
+static int nan_to_num_call(const dpx_array_view *src, double nan, double posinf, double neginf,
+                           const dpx_array_view *dst, void *stream)
+{
+    if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (src->dtype != dst->dtype)
+        return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    const dpx_array_view *views[2] = {src, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(2, views, n)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (src->dtype) {
+    case DPX_HALF:
+        return run_ew<NanToNumFn<half_t>, half_t, half_t>({(half_t)nan, (half_t)posinf, (half_t)neginf}, views, s, nullptr);
+    case DPX_FLOAT:
+        return run_ew<NanToNumFn<float>, float, float>({(float)nan, (float)posinf, (float)neginf}, views, s, nullptr);
+    case DPX_DOUBLE: return run_ew<NanToNumFn<double>, double, double>({nan, posinf, neginf}, views, s, nullptr);
+    case DPX_CFLOAT:
+        return run_ew<NanToNumFn<c64>, c64, c64>({(float)nan, (float)posinf, (float)neginf}, views, s, nullptr);
+    case DPX_CDOUBLE: return run_ew<NanToNumFn<c128>, c128, c128>({nan, posinf, neginf}, views, s, nullptr);
+    default: return fail(DPX_ERR_NOT_IMPLEMENTED, "nan_to_num: only floating and complex types");
+    }
+}
+
+// ---- isclose: dpnp/backend/kernels/elementwise_functions/isclose.hpp:47-92 (scalar tolerances) ---
+template <class T> struct IsCloseFn {
+    using R = real_of_t<T>;
+    R rtol, atol;
+    bool equal_nan;
+    DPX_D static bool finite(R v) { return v == v && !m_isinf(v); }
+    DPX_D bool operator()(T a, T b) const
+    {
+        if constexpr (is_cplx_v<T>) {
+            if (finite(a.re) && finite(a.im) && finite(b.re) && finite(b.im))
+                return m_hypot(a.re - b.re, a.im - b.im) <= atol + rtol * m_hypot(b.re, b.im);
+            if (a.re != a.re && a.im != a.im && b.re != b.re && b.im != b.im) return equal_nan;
+            return a == b;
+        }
+        else {
+            if (finite(a) && finite(b)) {
+                const R d = a - b;
+                return (d < R(0) ? -d : d) <= atol + rtol * (b < R(0) ? -b : b);
+            }
+            if (a != a && b != b) return equal_nan;
+            return a == b;
+        }
+    }
+};
+
+static int isclose_call(const dpx_array_view *a, const dpx_array_view *b, double rtol, double atol, int equal_nan,
+                        const dpx_array_view *dst, void *stream)
+{
+    if (!view_ok(a) || !view_ok(b) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (a->dtype != b->dtype) return fail(DPX_ERR_BAD_DTYPE, "Input arrays must have the same data type");
+    if (dst->dtype != DPX_BOOL) return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    const dpx_array_view *views[3] = {a, b, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(3, views, n)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const bool en = equal_nan != 0;
+    switch (a->dtype) {
+    case DPX_HALF:
+        return run_ew<IsCloseFn<half_t>, bool_t, half_t, half_t>({(half_t)rtol, (half_t)atol, en}, views, s, nullptr);
+    case DPX_FLOAT:
+        return run_ew<IsCloseFn<float>, bool_t, float, float>({(float)rtol, (float)atol, en}, views, s, nullptr);
+    case DPX_DOUBLE: return run_ew<IsCloseFn<double>, bool_t, double, double>({rtol, atol, en}, views, s, nullptr);
+    case DPX_CFLOAT: return run_ew<IsCloseFn<c64>, bool_t, c64, c64>({(float)rtol, (float)atol, en}, views, s, nullptr);
+    case DPX_CDOUBLE: return run_ew<IsCloseFn<c128>, bool_t, c128, c128>({rtol, atol, en}, views, s, nullptr);
+    default: return fail(DPX_ERR_NOT_IMPLEMENTED, "isclose: only floating and complex types");
+    }
+}
+
 // ---- fill ----------------------------------------------------------------------------------------------
 template <class T> struct FillFn {
     T v;
@@ -236,6 +320,16 @@ int dpx_where_compare(int cmp_op, const dpx_array_view *lhs, const dpx_array_vie
 int dpx_divide_by_scalar(const dpx_array_view *src, double scalar, const dpx_array_view *dst, void *stream)
 {
     return divide_by_scalar_call(src, scalar, dst, stream);
+}
+int dpx_nan_to_num(const dpx_array_view *src, double nan, double posinf, double neginf, const dpx_array_view *dst,
+                   void *stream)
+{
+    return nan_to_num_call(src, nan, posinf, neginf, dst, stream);
+}
+int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol, double atol, int equal_nan,
+                const dpx_array_view *dst, void *stream)
+{
+    return isclose_call(a, b, rtol, atol, equal_nan, dst, stream);
 }
 int dpx_fill(const dpx_array_view *dst, double value_re, double value_im, int64_t value_int, int use_int,
              void *stream)

@@ -109,6 +109,12 @@ DPX_FP_FN1(m_cosh, ::coshf, ::cosh)
 DPX_FP_FN1(m_asinh, ::asinhf, ::asinh)
 DPX_FP_FN1(m_acosh, ::acoshf, ::acosh)
 DPX_FP_FN1(m_atanh, ::atanhf, ::atanh)
+DPX_FP_FN1(m_erfc, ::erfcf, ::erfc)
+DPX_FP_FN1(m_erfcx, ::erfcxf, ::erfcx)
+DPX_FP_FN1(m_erfinv, ::erfinvf, ::erfinv)
+DPX_FP_FN1(m_erfcinv, ::erfcinvf, ::erfcinv)
+DPX_FP_FN1(m_i0, ::cyl_bessel_i0f, ::cyl_bessel_i0)
+DPX_FP_FN1(m_sinpi, ::sinpif, ::sinpi)
 #undef DPX_FP_FN1
 #define DPX_FP_FN2(NAME, F32, F64)                                          \
     template <class T> DPX_D T NAME(T x, T y)                               \
@@ -123,6 +129,8 @@ DPX_FP_FN2(m_hypot, ::hypotf, ::hypot)
 DPX_FP_FN2(m_copysign, ::copysignf, ::copysign)
 DPX_FP_FN2(m_fmod, ::fmodf, ::fmod)
 DPX_FP_FN2(m_nextafter, ::nextafterf, ::nextafter)
+DPX_FP_FN2(m_fmax, ::fmaxf, ::fmax)
+DPX_FP_FN2(m_fmin, ::fminf, ::fmin)
 #undef DPX_FP_FN2
 
 template <class T> DPX_D bool m_signbit(T x)
@@ -634,88 +642,268 @@ struct NextafterOp {
     }
 };
 
-// op id -> op struct; f(tag<Op>{}) is called for a valid id
+
+struct FabsOp { // fabs.hpp: real floating types
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x) { return m_copysign(x, T(1)); }
+};
+template <bool TO_DEG> struct DegreesOp { // degrees.hpp / radians.hpp
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x);
+        else {
+            constexpr T k = TO_DEG ? T(57.295779513082320876798154814105170332) : T(0.017453292519943295769236907684886127134);
+            return x * k;
+        }
+    }
+};
+struct SincOp { // sinc.hpp: sin(pi x) / (pi x), 1 at 0
+    template <class T> static constexpr bool ok = is_fp_v<T> || is_cplx_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if constexpr (is_cplx_v<T>) {
+            using R = real_of_t<T>;
+            constexpr R pi = R(3.1415926535897932384626433832795029);
+            const T y{pi * x.re, pi * x.im};
+            if (y.re == R(0) && y.im == R(0)) return T{R(1), R(0)};
+            return c_sin(y) / y;
+        }
+        else if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x);
+        else {
+            constexpr T pi = T(3.1415926535897932384626433832795029);
+            const T y = pi * x;
+            if (y == T(0)) return T(1);
+            return m_sinpi(x) / y;
+        }
+    }
+};
+struct SpacingOp { // spacing.hpp: distance to the next representable value away from zero
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x)
+    {
+        if (x != x) return x;
+        if (m_isinf(x)) return (T)__builtin_nanf("");
+        const T inf = (T)__builtin_inff();
+        // float16 steps towards +inf whatever the sign (as NumPy does)
+        if constexpr (std::is_same_v<T, half_t>) return NextafterOp::apply<T>(x, inf) - x;
+        else return m_nextafter(x, m_copysign(inf, x)) - x;
+    }
+};
+struct BitCountOp { // bitwise_count.hpp: set bits of |x| -> uint8
+    template <class T> static constexpr bool ok = is_int_v<T>;
+    template <class T> using out = uint8_t;
+    template <class T> DPX_D static uint8_t apply(T x)
+    {
+        using U = std::make_unsigned_t<T>;
+        const U u = x < T(0) ? (U)0 - (U)x : (U)x;
+        return (uint8_t)__popcll((unsigned long long)u);
+    }
+};
+// erf.hpp:52-95 (erfc, erfcx, erfinv, erfcinv) and i0.hpp; float16 input computes and returns float32
+// for the erf family
+template <int WHICH> struct ErfFamilyOp {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = std::conditional_t<std::is_same_v<T, half_t>, float, T>;
+    template <class T> DPX_D static out<T> apply(T x)
+    {
+        const out<T> v = (out<T>)x;
+        if constexpr (WHICH == 0) return m_erfc(v);
+        else if constexpr (WHICH == 1) return m_erfcx(v);
+        else if constexpr (WHICH == 2) return m_erfinv(v);
+        else return m_erfcinv(v);
+    }
+};
+struct I0Op {
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x) { return m_i0(x); }
+};
+
+// ---- functions of the reference's ufunc extension (dpnp/backend/extensions/ufunc) -------------
+template <bool IS_MAX> struct FmaxOp { // dpnp/backend/kernels/elementwise_functions/fmax.hpp, fmin.hpp: NaN loses
+    template <class T> static constexpr bool ok = true;
+    template <class T> using out = T;
+    template <class T> DPX_D static V<T> apply(V<T> a, V<T> b)
+    {
+        if constexpr (is_cplx_v<T>) {
+            // fmax.hpp: keep a when b holds a NaN or a >= b (lexicographic order)
+            if constexpr (IS_MAX) return (isnan_(b.re) || isnan_(b.im) || c_greater_eq(a, b)) ? a : b;
+            else return (isnan_(b.re) || isnan_(b.im) || c_less_eq(a, b)) ? a : b;
+        }
+        else if constexpr (is_fp_v<T>) return IS_MAX ? m_fmax(a, b) : m_fmin(a, b);
+        else if constexpr (is_bool_v<T>) return IS_MAX ? (a || b) : (a && b);
+        else return IS_MAX ? (a >= b ? a : b) : (a <= b ? a : b);
+    }
+};
+struct FmodOp { // fmod.hpp: C remainder (sign of the dividend); integer x fmod 0 == 0; bool -> int8
+    template <class T> static constexpr bool ok = !is_cplx_v<T>;
+    template <class T> using out = std::conditional_t<is_bool_v<T>, int8_t, T>;
+    template <class T> DPX_D static out<T> apply(V<T> a, V<T> b)
+    {
+        if constexpr (is_fp_v<T>) return m_fmod(a, b);
+        else if constexpr (is_bool_v<T>) return (int8_t)0; // {0,1} % 1 == 0 and x % 0 == 0
+        else {
+            if (b == T(0)) return T(0);
+            if constexpr (std::is_signed_v<T>)
+                if (b == T(-1)) return T(0); // also keeps INT_MIN % -1 away from the hardware division
+            return (T)(a % b);
+        }
+    }
+};
+struct Logaddexp2Op { // logaddexp2.hpp: log2(2**x + 2**y)
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T x, T y)
+    {
+        if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x, (float)y);
+        constexpr T log2e = T(1.442695040888963407359924681001892137);
+        if (x == y) return x + T(1); // also equal infinities
+        const T d = x - y;
+        if (d > T(0)) return x + log2e * m_log1p(m_exp2(-d));
+        if (d <= T(0)) return y + log2e * m_log1p(m_exp2(d));
+        return d; // NaN
+    }
+};
+struct HeavisideOp { // heaviside.hpp: NaN -> NaN, 0 -> second argument, else x > 0
+    template <class T> static constexpr bool ok = is_fp_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        if (a != a) return a;
+        if (a == T(0)) return b;
+        return a > T(0) ? T(1) : T(0);
+    }
+};
+template <bool LCM> struct GcdOp { // gcd.hpp / lcm.hpp: integers; the result is non-negative
+    template <class T> static constexpr bool ok = is_int_v<T>;
+    template <class T> using out = T;
+    template <class T> DPX_D static T apply(T a, T b)
+    {
+        using U = std::make_unsigned_t<T>;
+        U x = a < T(0) ? (U)0 - (U)a : (U)a, y = b < T(0) ? (U)0 - (U)b : (U)b;
+        const U ax = x, ay = y;
+        while (y != 0) {
+            const U t = x % y;
+            x = y;
+            y = t;
+        }
+        if constexpr (!LCM) return (T)x;
+        else return x == 0 ? T(0) : (T)(ax / x * ay);
+    }
+};
+
+// op id -> op struct; f(tag<Op>{}) is called for a valid id.  A translation unit built with
+// -DDPX_GROUP=g -DDPX_NGROUPS=n instantiates f only for the ids with id % n == g (the others
+// still return true, without a call), so the kernels of an op are compiled exactly once.
+#ifdef DPX_GROUP
+constexpr bool op_in_group(int id) { return id % DPX_NGROUPS == DPX_GROUP; }
+#else
+constexpr bool op_in_group(int) { return true; }
+#endif
 template <class F> inline bool for_binary_op(int op, F &&f)
 {
     switch (op) {
-    case DPX_B_ADD: f(tag<AddOp>{}); return true;
-    case DPX_B_SUBTRACT: f(tag<SubOp>{}); return true;
-    case DPX_B_MULTIPLY: f(tag<MulOp>{}); return true;
-    case DPX_B_DIVIDE: f(tag<DivOp>{}); return true;
-    case DPX_B_BITWISE_AND: f(tag<BitOp<0>>{}); return true;
-    case DPX_B_BITWISE_OR: f(tag<BitOp<1>>{}); return true;
-    case DPX_B_BITWISE_XOR: f(tag<BitOp<2>>{}); return true;
-    case DPX_B_EQUAL: f(tag<CmpOp<0>>{}); return true;
-    case DPX_B_NOT_EQUAL: f(tag<CmpOp<1>>{}); return true;
-    case DPX_B_LESS: f(tag<CmpOp<2>>{}); return true;
-    case DPX_B_LESS_EQUAL: f(tag<CmpOp<3>>{}); return true;
-    case DPX_B_GREATER: f(tag<CmpOp<4>>{}); return true;
-    case DPX_B_GREATER_EQUAL: f(tag<CmpOp<5>>{}); return true;
-    case DPX_B_MAXIMUM: f(tag<MaxOp>{}); return true;
-    case DPX_B_MINIMUM: f(tag<MinOp>{}); return true;
-    case DPX_B_LOGICAL_AND: f(tag<LogicalOp<0>>{}); return true;
-    case DPX_B_LOGICAL_OR: f(tag<LogicalOp<1>>{}); return true;
-    case DPX_B_LOGICAL_XOR: f(tag<LogicalOp<2>>{}); return true;
-    case DPX_B_POW: f(tag<PowOp>{}); return true;
-    case DPX_B_FLOOR_DIVIDE: f(tag<FloorDivOp>{}); return true;
-    case DPX_B_REMAINDER: f(tag<RemainderOp>{}); return true;
-    case DPX_B_ATAN2: f(tag<Atan2Op>{}); return true;
-    case DPX_B_HYPOT: f(tag<HypotOp>{}); return true;
-    case DPX_B_COPYSIGN: f(tag<CopysignOp>{}); return true;
-    case DPX_B_LEFT_SHIFT: f(tag<ShiftOp<true>>{}); return true;
-    case DPX_B_RIGHT_SHIFT: f(tag<ShiftOp<false>>{}); return true;
-    case DPX_B_LOGADDEXP: f(tag<LogaddexpOp>{}); return true;
-    case DPX_B_NEXTAFTER: f(tag<NextafterOp>{}); return true;
+    case DPX_B_ADD: if constexpr (op_in_group(DPX_B_ADD)) f(tag<AddOp>{}); return true;
+    case DPX_B_SUBTRACT: if constexpr (op_in_group(DPX_B_SUBTRACT)) f(tag<SubOp>{}); return true;
+    case DPX_B_MULTIPLY: if constexpr (op_in_group(DPX_B_MULTIPLY)) f(tag<MulOp>{}); return true;
+    case DPX_B_DIVIDE: if constexpr (op_in_group(DPX_B_DIVIDE)) f(tag<DivOp>{}); return true;
+    case DPX_B_BITWISE_AND: if constexpr (op_in_group(DPX_B_BITWISE_AND)) f(tag<BitOp<0>>{}); return true;
+    case DPX_B_BITWISE_OR: if constexpr (op_in_group(DPX_B_BITWISE_OR)) f(tag<BitOp<1>>{}); return true;
+    case DPX_B_BITWISE_XOR: if constexpr (op_in_group(DPX_B_BITWISE_XOR)) f(tag<BitOp<2>>{}); return true;
+    case DPX_B_EQUAL: if constexpr (op_in_group(DPX_B_EQUAL)) f(tag<CmpOp<0>>{}); return true;
+    case DPX_B_NOT_EQUAL: if constexpr (op_in_group(DPX_B_NOT_EQUAL)) f(tag<CmpOp<1>>{}); return true;
+    case DPX_B_LESS: if constexpr (op_in_group(DPX_B_LESS)) f(tag<CmpOp<2>>{}); return true;
+    case DPX_B_LESS_EQUAL: if constexpr (op_in_group(DPX_B_LESS_EQUAL)) f(tag<CmpOp<3>>{}); return true;
+    case DPX_B_GREATER: if constexpr (op_in_group(DPX_B_GREATER)) f(tag<CmpOp<4>>{}); return true;
+    case DPX_B_GREATER_EQUAL: if constexpr (op_in_group(DPX_B_GREATER_EQUAL)) f(tag<CmpOp<5>>{}); return true;
+    case DPX_B_MAXIMUM: if constexpr (op_in_group(DPX_B_MAXIMUM)) f(tag<MaxOp>{}); return true;
+    case DPX_B_MINIMUM: if constexpr (op_in_group(DPX_B_MINIMUM)) f(tag<MinOp>{}); return true;
+    case DPX_B_LOGICAL_AND: if constexpr (op_in_group(DPX_B_LOGICAL_AND)) f(tag<LogicalOp<0>>{}); return true;
+    case DPX_B_LOGICAL_OR: if constexpr (op_in_group(DPX_B_LOGICAL_OR)) f(tag<LogicalOp<1>>{}); return true;
+    case DPX_B_LOGICAL_XOR: if constexpr (op_in_group(DPX_B_LOGICAL_XOR)) f(tag<LogicalOp<2>>{}); return true;
+    case DPX_B_POW: if constexpr (op_in_group(DPX_B_POW)) f(tag<PowOp>{}); return true;
+    case DPX_B_FLOOR_DIVIDE: if constexpr (op_in_group(DPX_B_FLOOR_DIVIDE)) f(tag<FloorDivOp>{}); return true;
+    case DPX_B_REMAINDER: if constexpr (op_in_group(DPX_B_REMAINDER)) f(tag<RemainderOp>{}); return true;
+    case DPX_B_ATAN2: if constexpr (op_in_group(DPX_B_ATAN2)) f(tag<Atan2Op>{}); return true;
+    case DPX_B_HYPOT: if constexpr (op_in_group(DPX_B_HYPOT)) f(tag<HypotOp>{}); return true;
+    case DPX_B_COPYSIGN: if constexpr (op_in_group(DPX_B_COPYSIGN)) f(tag<CopysignOp>{}); return true;
+    case DPX_B_LEFT_SHIFT: if constexpr (op_in_group(DPX_B_LEFT_SHIFT)) f(tag<ShiftOp<true>>{}); return true;
+    case DPX_B_RIGHT_SHIFT: if constexpr (op_in_group(DPX_B_RIGHT_SHIFT)) f(tag<ShiftOp<false>>{}); return true;
+    case DPX_B_LOGADDEXP: if constexpr (op_in_group(DPX_B_LOGADDEXP)) f(tag<LogaddexpOp>{}); return true;
+    case DPX_B_NEXTAFTER: if constexpr (op_in_group(DPX_B_NEXTAFTER)) f(tag<NextafterOp>{}); return true;
+    case DPX_B_FMAX: if constexpr (op_in_group(DPX_B_FMAX)) f(tag<FmaxOp<true>>{}); return true;
+    case DPX_B_FMIN: if constexpr (op_in_group(DPX_B_FMIN)) f(tag<FmaxOp<false>>{}); return true;
+    case DPX_B_FMOD: if constexpr (op_in_group(DPX_B_FMOD)) f(tag<FmodOp>{}); return true;
+    case DPX_B_LOGADDEXP2: if constexpr (op_in_group(DPX_B_LOGADDEXP2)) f(tag<Logaddexp2Op>{}); return true;
+    case DPX_B_HEAVISIDE: if constexpr (op_in_group(DPX_B_HEAVISIDE)) f(tag<HeavisideOp>{}); return true;
+    case DPX_B_GCD: if constexpr (op_in_group(DPX_B_GCD)) f(tag<GcdOp<false>>{}); return true;
+    case DPX_B_LCM: if constexpr (op_in_group(DPX_B_LCM)) f(tag<GcdOp<true>>{}); return true;
     default: return false;
     }
 }
 template <class F> inline bool for_unary_op(int op, F &&f)
 {
     switch (op) {
-    case DPX_U_ABS: f(tag<AbsOp>{}); return true;
-    case DPX_U_NEGATIVE: f(tag<NegOp>{}); return true;
-    case DPX_U_POSITIVE: f(tag<PosOp>{}); return true;
-    case DPX_U_SQUARE: f(tag<SquareOp>{}); return true;
-    case DPX_U_SQRT: f(tag<SqrtOp>{}); return true;
-    case DPX_U_EXP: f(tag<ExpOp>{}); return true;
-    case DPX_U_LOG: f(tag<LogOp>{}); return true;
-    case DPX_U_ERF: f(tag<ErfOp>{}); return true;
-    case DPX_U_SIN: f(tag<SinOp>{}); return true;
-    case DPX_U_COS: f(tag<CosOp>{}); return true;
-    case DPX_U_TAN: f(tag<TanOp>{}); return true;
-    case DPX_U_TANH: f(tag<TanhOp>{}); return true;
-    case DPX_U_EXP2: f(tag<Exp2Op>{}); return true;
-    case DPX_U_EXPM1: f(tag<Expm1Op>{}); return true;
-    case DPX_U_LOG2: f(tag<Log2Op>{}); return true;
-    case DPX_U_LOG10: f(tag<Log10Op>{}); return true;
-    case DPX_U_LOG1P: f(tag<Log1pOp>{}); return true;
-    case DPX_U_RSQRT: f(tag<RsqrtOp>{}); return true;
-    case DPX_U_CBRT: f(tag<CbrtOp>{}); return true;
-    case DPX_U_RECIPROCAL: f(tag<ReciprocalOp>{}); return true;
-    case DPX_U_FLOOR: f(tag<RoundOp<0>>{}); return true;
-    case DPX_U_CEIL: f(tag<RoundOp<1>>{}); return true;
-    case DPX_U_TRUNC: f(tag<RoundOp<2>>{}); return true;
-    case DPX_U_SIGN: f(tag<SignOp>{}); return true;
-    case DPX_U_ISNAN: f(tag<FpClassOp<0>>{}); return true;
-    case DPX_U_ISINF: f(tag<FpClassOp<1>>{}); return true;
-    case DPX_U_ISFINITE: f(tag<FpClassOp<2>>{}); return true;
-    case DPX_U_LOGICAL_NOT: f(tag<LogicalNotOp>{}); return true;
-    case DPX_U_BITWISE_INVERT: f(tag<InvertOp>{}); return true;
-    case DPX_U_SIGNBIT: f(tag<SignbitOp>{}); return true;
-    case DPX_U_ASIN: f(tag<AsinOp>{}); return true;
-    case DPX_U_ACOS: f(tag<AcosOp>{}); return true;
-    case DPX_U_ATAN: f(tag<AtanOp>{}); return true;
-    case DPX_U_SINH: f(tag<SinhOp>{}); return true;
-    case DPX_U_COSH: f(tag<CoshOp>{}); return true;
-    case DPX_U_ASINH: f(tag<AsinhOp>{}); return true;
-    case DPX_U_ACOSH: f(tag<AcoshOp>{}); return true;
-    case DPX_U_ATANH: f(tag<AtanhOp>{}); return true;
-    case DPX_U_ROUND: f(tag<RoundOp2>{}); return true;
-    case DPX_U_CONJ: f(tag<ConjOp>{}); return true;
-    case DPX_U_REAL: f(tag<PartOp<false>>{}); return true;
-    case DPX_U_IMAG: f(tag<PartOp<true>>{}); return true;
-    case DPX_U_PROJ: f(tag<ProjOp>{}); return true;
-    case DPX_U_ANGLE: f(tag<AngleOp>{}); return true;
+    case DPX_U_ABS: if constexpr (op_in_group(DPX_U_ABS)) f(tag<AbsOp>{}); return true;
+    case DPX_U_NEGATIVE: if constexpr (op_in_group(DPX_U_NEGATIVE)) f(tag<NegOp>{}); return true;
+    case DPX_U_POSITIVE: if constexpr (op_in_group(DPX_U_POSITIVE)) f(tag<PosOp>{}); return true;
+    case DPX_U_SQUARE: if constexpr (op_in_group(DPX_U_SQUARE)) f(tag<SquareOp>{}); return true;
+    case DPX_U_SQRT: if constexpr (op_in_group(DPX_U_SQRT)) f(tag<SqrtOp>{}); return true;
+    case DPX_U_EXP: if constexpr (op_in_group(DPX_U_EXP)) f(tag<ExpOp>{}); return true;
+    case DPX_U_LOG: if constexpr (op_in_group(DPX_U_LOG)) f(tag<LogOp>{}); return true;
+    case DPX_U_ERF: if constexpr (op_in_group(DPX_U_ERF)) f(tag<ErfOp>{}); return true;
+    case DPX_U_SIN: if constexpr (op_in_group(DPX_U_SIN)) f(tag<SinOp>{}); return true;
+    case DPX_U_COS: if constexpr (op_in_group(DPX_U_COS)) f(tag<CosOp>{}); return true;
+    case DPX_U_TAN: if constexpr (op_in_group(DPX_U_TAN)) f(tag<TanOp>{}); return true;
+    case DPX_U_TANH: if constexpr (op_in_group(DPX_U_TANH)) f(tag<TanhOp>{}); return true;
+    case DPX_U_EXP2: if constexpr (op_in_group(DPX_U_EXP2)) f(tag<Exp2Op>{}); return true;
+    case DPX_U_EXPM1: if constexpr (op_in_group(DPX_U_EXPM1)) f(tag<Expm1Op>{}); return true;
+    case DPX_U_LOG2: if constexpr (op_in_group(DPX_U_LOG2)) f(tag<Log2Op>{}); return true;
+    case DPX_U_LOG10: if constexpr (op_in_group(DPX_U_LOG10)) f(tag<Log10Op>{}); return true;
+    case DPX_U_LOG1P: if constexpr (op_in_group(DPX_U_LOG1P)) f(tag<Log1pOp>{}); return true;
+    case DPX_U_RSQRT: if constexpr (op_in_group(DPX_U_RSQRT)) f(tag<RsqrtOp>{}); return true;
+    case DPX_U_CBRT: if constexpr (op_in_group(DPX_U_CBRT)) f(tag<CbrtOp>{}); return true;
+    case DPX_U_RECIPROCAL: if constexpr (op_in_group(DPX_U_RECIPROCAL)) f(tag<ReciprocalOp>{}); return true;
+    case DPX_U_FLOOR: if constexpr (op_in_group(DPX_U_FLOOR)) f(tag<RoundOp<0>>{}); return true;
+    case DPX_U_CEIL: if constexpr (op_in_group(DPX_U_CEIL)) f(tag<RoundOp<1>>{}); return true;
+    case DPX_U_TRUNC: if constexpr (op_in_group(DPX_U_TRUNC)) f(tag<RoundOp<2>>{}); return true;
+    case DPX_U_SIGN: if constexpr (op_in_group(DPX_U_SIGN)) f(tag<SignOp>{}); return true;
+    case DPX_U_ISNAN: if constexpr (op_in_group(DPX_U_ISNAN)) f(tag<FpClassOp<0>>{}); return true;
+    case DPX_U_ISINF: if constexpr (op_in_group(DPX_U_ISINF)) f(tag<FpClassOp<1>>{}); return true;
+    case DPX_U_ISFINITE: if constexpr (op_in_group(DPX_U_ISFINITE)) f(tag<FpClassOp<2>>{}); return true;
+    case DPX_U_LOGICAL_NOT: if constexpr (op_in_group(DPX_U_LOGICAL_NOT)) f(tag<LogicalNotOp>{}); return true;
+    case DPX_U_BITWISE_INVERT: if constexpr (op_in_group(DPX_U_BITWISE_INVERT)) f(tag<InvertOp>{}); return true;
+    case DPX_U_SIGNBIT: if constexpr (op_in_group(DPX_U_SIGNBIT)) f(tag<SignbitOp>{}); return true;
+    case DPX_U_ASIN: if constexpr (op_in_group(DPX_U_ASIN)) f(tag<AsinOp>{}); return true;
+    case DPX_U_ACOS: if constexpr (op_in_group(DPX_U_ACOS)) f(tag<AcosOp>{}); return true;
+    case DPX_U_ATAN: if constexpr (op_in_group(DPX_U_ATAN)) f(tag<AtanOp>{}); return true;
+    case DPX_U_SINH: if constexpr (op_in_group(DPX_U_SINH)) f(tag<SinhOp>{}); return true;
+    case DPX_U_COSH: if constexpr (op_in_group(DPX_U_COSH)) f(tag<CoshOp>{}); return true;
+    case DPX_U_ASINH: if constexpr (op_in_group(DPX_U_ASINH)) f(tag<AsinhOp>{}); return true;
+    case DPX_U_ACOSH: if constexpr (op_in_group(DPX_U_ACOSH)) f(tag<AcoshOp>{}); return true;
+    case DPX_U_ATANH: if constexpr (op_in_group(DPX_U_ATANH)) f(tag<AtanhOp>{}); return true;
+    case DPX_U_ROUND: if constexpr (op_in_group(DPX_U_ROUND)) f(tag<RoundOp2>{}); return true;
+    case DPX_U_CONJ: if constexpr (op_in_group(DPX_U_CONJ)) f(tag<ConjOp>{}); return true;
+    case DPX_U_REAL: if constexpr (op_in_group(DPX_U_REAL)) f(tag<PartOp<false>>{}); return true;
+    case DPX_U_IMAG: if constexpr (op_in_group(DPX_U_IMAG)) f(tag<PartOp<true>>{}); return true;
+    case DPX_U_PROJ: if constexpr (op_in_group(DPX_U_PROJ)) f(tag<ProjOp>{}); return true;
+    case DPX_U_ANGLE: if constexpr (op_in_group(DPX_U_ANGLE)) f(tag<AngleOp>{}); return true;
+    case DPX_U_FABS: if constexpr (op_in_group(DPX_U_FABS)) f(tag<FabsOp>{}); return true;
+    case DPX_U_DEGREES: if constexpr (op_in_group(DPX_U_DEGREES)) f(tag<DegreesOp<true>>{}); return true;
+    case DPX_U_RADIANS: if constexpr (op_in_group(DPX_U_RADIANS)) f(tag<DegreesOp<false>>{}); return true;
+    case DPX_U_SINC: if constexpr (op_in_group(DPX_U_SINC)) f(tag<SincOp>{}); return true;
+    case DPX_U_SPACING: if constexpr (op_in_group(DPX_U_SPACING)) f(tag<SpacingOp>{}); return true;
+    case DPX_U_BITWISE_COUNT: if constexpr (op_in_group(DPX_U_BITWISE_COUNT)) f(tag<BitCountOp>{}); return true;
+    case DPX_U_ERFC: if constexpr (op_in_group(DPX_U_ERFC)) f(tag<ErfFamilyOp<0>>{}); return true;
+    case DPX_U_ERFCX: if constexpr (op_in_group(DPX_U_ERFCX)) f(tag<ErfFamilyOp<1>>{}); return true;
+    case DPX_U_ERFINV: if constexpr (op_in_group(DPX_U_ERFINV)) f(tag<ErfFamilyOp<2>>{}); return true;
+    case DPX_U_ERFCINV: if constexpr (op_in_group(DPX_U_ERFCINV)) f(tag<ErfFamilyOp<3>>{}); return true;
+    case DPX_U_I0: if constexpr (op_in_group(DPX_U_I0)) f(tag<I0Op>{}); return true;
     default: return false;
     }
 }

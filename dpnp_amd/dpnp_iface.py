@@ -8,6 +8,8 @@ dpnp/dpnp_iface_{mathematical,trigonometric,statistics,searching,bitwise,logic}.
 casts the inputs and excludes `out=`, `out is x1` runs the in-place kernel, a reduction's
 `out` of another dtype receives an unsafe cast of the result.
 """
+import builtins as _builtins
+
 import numpy as np
 
 from . import tensor as dpt
@@ -297,6 +299,9 @@ _UNARY = {
     "sinh": ef.sinh, "cosh": ef.cosh, "arcsinh": ef.asinh, "asinh": ef.asinh, "arccosh": ef.acosh,
     "acosh": ef.acosh, "arctanh": ef.atanh, "atanh": ef.atanh, "rint": ef.round, "conj": ef.conj,
     "conjugate": ef.conj, "real": ef.real, "imag": ef.imag, "proj": ef.proj, "angle": ef.angle,
+    "fabs": ef.fabs, "degrees": ef.degrees, "rad2deg": ef.degrees, "radians": ef.radians, "deg2rad": ef.radians,
+    "sinc": ef.sinc, "spacing": ef.spacing, "bitwise_count": ef.bitwise_count, "erfc": ef.erfc, "erfcx": ef.erfcx,
+    "erfinv": ef.erfinv, "erfcinv": ef.erfcinv, "i0": ef.i0,
 }
 _BINARY = {
     "add": ef.add, "subtract": ef.subtract, "multiply": ef.multiply, "divide": ef.divide,
@@ -309,12 +314,101 @@ _BINARY = {
     "arctan2": ef.atan2, "atan2": ef.atan2, "hypot": ef.hypot, "copysign": ef.copysign,
     "left_shift": ef.bitwise_left_shift, "bitwise_left_shift": ef.bitwise_left_shift,
     "right_shift": ef.bitwise_right_shift, "bitwise_right_shift": ef.bitwise_right_shift,
-    "logaddexp": ef.logaddexp, "nextafter": ef.nextafter,
+    "logaddexp": ef.logaddexp, "nextafter": ef.nextafter, "fmax": ef.fmax, "fmin": ef.fmin, "fmod": ef.fmod,
+    "logaddexp2": ef.logaddexp2, "heaviside": ef.heaviside, "gcd": ef.gcd, "lcm": ef.lcm,
 }
 for _n, _f in _UNARY.items():
     globals()[_n] = DPNPUnaryFunc(_n, _f)
 for _n, _f in _BINARY.items():
     globals()[_n] = DPNPBinaryFunc(_n, _f)
+
+
+def float_power(x1, x2, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+    """x1 ** x2 computed in at least float64 (complex128 for complex operands), as
+    dpnp.float_power (dpnp/dpnp_iface_mathematical.py:1952-2030)."""
+    _check_ufunc_kwargs("float_power", where, subok, dtype, out, kwargs)
+    if dtype is not None:
+        tgt = dpt.dtype(dtype)
+    else:
+        kinds = [get_usm_ndarray(v).dtype if is_supported_array_type(v) else np.result_type(v) for v in (x1, x2)]
+        tgt = dpt.dtype("c16" if _builtins.any(k.kind == "c" for k in kinds) else "f8")
+    if tgt.kind not in "fc":
+        raise TypeError(f"float_power needs a floating or complex result type, got {tgt}")
+    return globals()["power"](x1, x2, out=out, order=order, dtype=tgt)
+
+
+def divmod(x1, x2, /, out1=None, out2=None, *, out=(None, None), where=True, order="K", dtype=None,  # noqa: A001
+           subok=True, **kwargs):
+    """(x1 // x2, x1 % x2): dpnp.divmod (dpnp/dpnp_iface_mathematical.py:1619-1700); the reference
+    runs one two-output kernel, here the two existing kernels run back to back."""
+    o1, o2 = (out1, out2) if (out1 is not None or out2 is not None) else tuple(out)
+    q = globals()["floor_divide"](x1, x2, out=o1, where=where, order=order, dtype=dtype, subok=subok, **kwargs)
+    r = globals()["remainder"](x1, x2, out=o2, where=where, order=order, dtype=dtype, subok=subok, **kwargs)
+    return q, r
+
+
+def modf(x, /, out1=None, out2=None, *, out=(None, None), where=True, order="K", dtype=None, subok=True,
+         **kwargs):
+    """(fractional part, integral part), both with the sign of x: dpnp.modf
+    (dpnp/dpnp_iface_mathematical.py:3494-3560)."""
+    o1, o2 = (out1, out2) if (out1 is not None or out2 is not None) else tuple(out)
+    u = get_usm_ndarray(x)
+    if u.dtype.kind not in "f":
+        if u.dtype.kind == "c":
+            raise ValueError("modf does not support complex input")
+        x = astype(x, "f8" if u.dtype.itemsize >= 4 else ("f4" if u.dtype.itemsize == 2 else "f2"))
+    whole = globals()["trunc"](x, out=o2, where=where, order=order, dtype=dtype, subok=subok, **kwargs)
+    frac = globals()["subtract"](x, whole, out=o1, order=order)
+    # inf - inf is NaN but the fractional part of an infinity is a zero; zeros keep the sign of x
+    fu = get_usm_ndarray(frac)
+    xu = get_usm_ndarray(x)
+    fixed = dpt.where(dpt.isinf(xu), dpt.asarray(0, dtype=fu.dtype), fu)
+    dpt.copysign(fixed, xu, out=fu)
+    return frac, whole
+
+
+def nan_to_num(x, copy=True, nan=0.0, posinf=None, neginf=None):
+    """NaN -> `nan`, +inf -> `posinf` (largest finite value by default), -inf -> `neginf`:
+    dpnp.nan_to_num (dpnp/dpnp_iface_mathematical.py:3584-3760), scalar replacement values."""
+    check_supported_arrays_type(x)
+    u = get_usm_ndarray(x)
+    if u.dtype.kind not in "fc":
+        return _wrap(dpt.copy(u)) if copy else get_result_array(x)
+    for v in (nan, posinf, neginf):
+        if v is not None and not isinstance(v, (int, float)):
+            raise NotImplementedError("nan_to_num with array replacement values is outside this library's scope")
+    real_dt = np.dtype("f" + str(u.dtype.itemsize // 2)) if u.dtype.kind == "c" else u.dtype
+    info = np.finfo(real_dt)
+    hi = float(info.max) if posinf is None else posinf
+    lo = float(info.min) if neginf is None else neginf
+    if copy:
+        out = dpt.empty_like(u)
+    else:
+        if not u.flags.writable:
+            raise ValueError("copy is required for read-only array `x`")
+        out = u
+    if u.size:
+        tei._nan_to_num(u, nan, hi, lo, out)
+    return _wrap(out) if copy else get_result_array(x)
+
+
+def isclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
+    """|a - b| <= atol + rtol * |b| elementwise, infinities equal to themselves, NaNs equal when
+    equal_nan: dpnp.isclose with scalar tolerances (dpnp/dpnp_iface_logic.py:824-960)."""
+    check_supported_arrays_type(a, b, scalar_type=True)
+    if not (np.isscalar(rtol) and np.isscalar(atol)):
+        raise NotImplementedError("isclose with array tolerances is outside this library's scope")
+    dt = result_type(a, b, 1.0)
+    ua = dpt.asarray(a, dtype=dt) if np.isscalar(a) else dpt.astype(get_usm_ndarray(a), dt, copy=False)
+    ub = dpt.asarray(b, dtype=dt) if np.isscalar(b) else dpt.astype(get_usm_ndarray(b), dt, copy=False)
+    rtol = rtol.real if isinstance(rtol, complex) else rtol
+    atol = atol.real if isinstance(atol, complex) else atol
+    shape = np.broadcast_shapes(ua.shape, ub.shape)
+    ua, ub = dpt.broadcast_to(ua, shape), dpt.broadcast_to(ub, shape)
+    out = dpt.empty(shape, dtype="?")
+    if out.size:
+        tei._isclose_scalar(ua, ub, rtol, atol, True if equal_nan else False, out)
+    return _wrap(out)
 
 
 def where(condition, x=None, y=None, /, *, order="K", out=None):

@@ -97,3 +97,24 @@ bitwise_left_shift = _binary("bitwise_left_shift", "Elementwise left shift.")
 bitwise_right_shift = _binary("bitwise_right_shift", "Elementwise right shift.")
 logaddexp = _binary("logaddexp", "Elementwise log(exp(x1) + exp(x2)).", inplace=False)
 nextafter = _binary("nextafter", "Next representable value after x1 towards x2.", inplace=False)
+
+# functions of the reference's ufunc extension module (dpnp/backend/extensions/ufunc), which the
+# dpnp layer wraps the same way as the tensor functions above
+fabs = _unary("fabs", "Elementwise absolute value of a floating array.")
+degrees = _unary("degrees", "Radians to degrees.")
+radians = _unary("radians", "Degrees to radians.")
+sinc = _unary("sinc", "Normalised sinc, sin(pi x) / (pi x).")
+spacing = _unary("spacing", "Distance to the nearest adjacent number.")
+bitwise_count = _unary("bitwise_count", "Number of set bits of the absolute value.")
+erfc = _unary("erfc", "Complementary error function.")
+erfcx = _unary("erfcx", "Scaled complementary error function exp(x**2) erfc(x).")
+erfinv = _unary("erfinv", "Inverse of the error function.")
+erfcinv = _unary("erfcinv", "Inverse of the complementary error function.")
+i0 = _unary("i0", "Modified Bessel function of the first kind, order 0.")
+fmax = _binary("fmax", "Elementwise maximum; a NaN operand is ignored.", inplace=False)
+fmin = _binary("fmin", "Elementwise minimum; a NaN operand is ignored.", inplace=False)
+fmod = _binary("fmod", "Elementwise C remainder (sign of the dividend).", inplace=False)
+logaddexp2 = _binary("logaddexp2", "Elementwise log2(2**x1 + 2**x2).", inplace=False)
+heaviside = _binary("heaviside", "Heaviside step function; x2 where x1 == 0.", inplace=False)
+gcd = _binary("gcd", "Elementwise greatest common divisor.", inplace=False)
+lcm = _binary("lcm", "Elementwise lowest common multiple.", inplace=False)

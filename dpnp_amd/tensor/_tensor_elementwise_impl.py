@@ -62,6 +62,21 @@ def _divide_by_scalar(src, scalar, dst, sycl_queue=None, depends=()):
     return _events(sycl_queue)
 
 
+def _nan_to_num(src, nan, posinf, neginf, dst, sycl_queue=None, depends=()):
+    """ufi._nan_to_num of the reference's ufunc extension
+    (dpnp/backend/extensions/ufunc/elementwise_functions/nan_to_num.cpp): scalar replacements."""
+    vs, vd = src._as_view(), dst._as_view()
+    _lib.check(lib.dpx_nan_to_num(vs, float(nan), float(posinf), float(neginf), vd, _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
+def _isclose_scalar(a, b, rtol, atol, equal_nan, dst, sycl_queue=None, depends=()):
+    """ufi._isclose_scalar (dpnp/backend/extensions/ufunc/elementwise_functions/isclose.cpp)."""
+    va, vb, vd = a._as_view(), b._as_view(), dst._as_view()
+    _lib.check(lib.dpx_isclose(va, vb, float(rtol), float(atol), int(bool(equal_nan)), vd, _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
 def _black_scholes(price, strike, t, rate, vol, call, put, sycl_queue=None, depends=()):
     """Fused Black-Scholes pricing over 1-D contiguous arrays (no counterpart in the reference)."""
     arrs = (price, strike, t, call, put)

@@ -138,6 +138,20 @@ typedef enum dpx_unary_op {
     DPX_U_IMAG,
     DPX_U_PROJ,
     DPX_U_ANGLE,
+    /* the reference's ufunc extension, dpnp/backend/extensions/ufunc/elementwise_functions/:
+     * fabs.cpp, degrees.cpp, radians.cpp, sinc.cpp, spacing.cpp, bitwise_count.cpp,
+     * erf_funcs.cpp, i0.cpp */
+    DPX_U_FABS,
+    DPX_U_DEGREES,
+    DPX_U_RADIANS,
+    DPX_U_SINC,
+    DPX_U_SPACING,
+    DPX_U_BITWISE_COUNT,
+    DPX_U_ERFC,
+    DPX_U_ERFCX,
+    DPX_U_ERFINV,
+    DPX_U_ERFCINV,
+    DPX_U_I0,
     DPX_U_NUM_OPS
 } dpx_unary_op;
 
@@ -170,6 +184,15 @@ typedef enum dpx_binary_op {
     DPX_B_RIGHT_SHIFT,
     DPX_B_LOGADDEXP,
     DPX_B_NEXTAFTER,
+    /* the reference's ufunc extension, dpnp/backend/extensions/ufunc/elementwise_functions/:
+     * fmax.cpp, fmin.cpp, fmod.cpp, logaddexp2.cpp, heaviside.cpp, gcd.cpp, lcm.cpp */
+    DPX_B_FMAX,
+    DPX_B_FMIN,
+    DPX_B_FMOD,
+    DPX_B_LOGADDEXP2,
+    DPX_B_HEAVISIDE,
+    DPX_B_GCD,
+    DPX_B_LCM,
     DPX_B_NUM_OPS
 } dpx_binary_op;
 
@@ -285,6 +308,20 @@ int dpx_where(const dpx_array_view *cond, const dpx_array_view *x1,
  * the scalar is converted to dst's real type before the division */
 int dpx_divide_by_scalar(const dpx_array_view *src, double scalar,
                          const dpx_array_view *dst, void *stream);
+
+/* dst = x with NaN replaced by `nan`, +inf by `posinf`, -inf by `neginf` (complex: part by part);
+ * float16/32/64 and complex, src and dst of one dtype.  Replaces the contiguous and strided
+ * nan_to_num calls of dpnp/backend/extensions/ufunc/elementwise_functions/nan_to_num.cpp
+ * (kernels: dpnp/backend/kernels/elementwise_functions/nan_to_num.hpp:44-104). */
+int dpx_nan_to_num(const dpx_array_view *src, double nan, double posinf,
+                   double neginf, const dpx_array_view *dst, void *stream);
+/* dst (bool) = |a - b| <= atol + rtol * |b| for finite pairs, equal_nan for two NaNs, a == b
+ * otherwise; a and b of one floating or complex dtype.  Replaces
+ * dpnp/backend/extensions/ufunc/elementwise_functions/isclose.cpp
+ * (kernels: dpnp/backend/kernels/elementwise_functions/isclose.hpp:47-92). */
+int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol,
+                double atol, int equal_nan, const dpx_array_view *dst,
+                void *stream);
 /* ti._copy_usm_ndarray_into_usm_ndarray,
  * libtensor/source/copy_and_cast_usm_to_usm.cpp:137-216: dst = cast(src), any
  * dtype pair, equal shapes */

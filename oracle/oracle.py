@@ -197,6 +197,30 @@ def binary(op, a, b):
             return np.logaddexp(a.astype(np.longdouble), b.astype(np.longdouble)).astype(a.dtype)
         if op == "nextafter":
             return np.nextafter(a, b)
+        # ---- dpnp/backend/kernels/elementwise_functions/*.hpp (the ufunc extension) ----
+        if op in ("fmax", "fmin"):      # fmax.hpp / fmin.hpp: a NaN operand loses
+            if k == "c":                # keep a when b holds a NaN or a >= b (a <= b) lexicographically
+                bn = np.isnan(b.real) | np.isnan(b.imag)
+                keep = bn | _cplx_cmp(a, b, ">=" if op == "fmax" else "<=")
+                return np.where(keep, a, b)
+            if k == "b":
+                return (a | b) if op == "fmax" else (a & b)
+            return (np.fmax if op == "fmax" else np.fmin)(a, b)
+        if op == "fmod":                # fmod.hpp: C remainder; integer x fmod 0 == 0; bool -> int8
+            if k == "b":
+                return np.zeros(a.shape, dtype="i1")
+            if k in "iu":
+                safe = np.where(b == 0, 1, b)
+                return np.where(b == 0, 0, np.fmod(a, safe)).astype(a.dtype)
+            return np.fmod(a, b)
+        if op == "logaddexp2":          # logaddexp2.hpp
+            return np.logaddexp2(a.astype(np.longdouble), b.astype(np.longdouble)).astype(a.dtype)
+        if op == "heaviside":           # heaviside.hpp
+            return np.heaviside(a, b)
+        if op == "gcd":                 # gcd.hpp: std::gcd
+            return np.gcd(a, b)
+        if op == "lcm":                 # lcm.hpp: std::lcm
+            return np.lcm(a, b)
     raise KeyError(op)
 
 
@@ -208,8 +232,10 @@ def unary_result_dtype(op, dt):
         return np.dtype({"c8": "f4", "c16": "f8"}.get(dt.str[1:], dt))
     if op in ("square", "conj") and dt.kind == "b":
         return np.dtype("i1")           # square.hpp / conj.hpp type maps: bool -> int8
-    if op == "erf" and dt == np.dtype("f2"):
+    if op in ("erf", "erfc", "erfcx", "erfinv", "erfcinv") and dt == np.dtype("f2"):
         return np.dtype("f4")           # dpnp/backend/extensions/ufunc/elementwise_functions/erf_funcs.cpp:74-84
+    if op == "bitwise_count":
+        return np.dtype("u1")           # bitwise_count.cpp:72-82
     return dt
 
 
@@ -262,6 +288,32 @@ def unary(op, a):
             return np.imag(a).astype(out_dt)
         if op == "angle":
             return np.angle(a).astype(out_dt)
+        # ---- dpnp/backend/kernels/elementwise_functions/*.hpp (the ufunc extension) ----
+        if op == "fabs":
+            return np.fabs(a)
+        if op in ("degrees", "radians"):
+            return getattr(np, op)(a.astype(np.longdouble)).astype(a.dtype)
+        if op == "sinc":                # sinc.hpp:52-72
+            wide = np.clongdouble if k == "c" else np.longdouble
+            return np.sinc(a.astype(wide)).astype(a.dtype)
+        if op == "spacing":             # spacing.hpp: float16 always steps towards +inf
+            if a.dtype == np.dtype("f2"):
+                out = (np.nextafter(a, np.float16(np.inf)) - a).astype("f2")
+                out[np.isinf(a)] = np.nan
+                return out
+            # nextafter(x, copysign(inf, x)) - x: equals numpy.spacing except at -0.0, where the
+            # step is taken downwards (numpy gives +tiny there)
+            out = np.nextafter(a, np.copysign(np.inf, a).astype(a.dtype)) - a
+            out[np.isinf(a)] = np.nan
+            return out.astype(a.dtype)
+        if op == "bitwise_count":       # bitwise_count.hpp: popcount(|x|)
+            mag = np.abs(a.astype(object)) if k == "i" else a.astype(object)
+            return np.array([bin(int(v)).count("1") for v in mag.ravel()], dtype="u1").reshape(a.shape)
+        if op in ("erfc", "erfcx", "erfinv", "erfcinv", "i0"):
+            import scipy.special as sp
+
+            x = a.astype(np.float64)
+            return getattr(sp, op)(x).astype(out_dt)
         if op == "proj":                # proj.hpp: infinities collapse to (inf, copysign(0, im))
             inf = np.isinf(a.real) | np.isinf(a.imag)
             out = a.copy()

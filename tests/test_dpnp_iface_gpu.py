@@ -130,3 +130,80 @@ def test_black_scholes_entry_point():
     r = P * d1 - Se * d2
     assert_same(call.asnumpy(), r.asnumpy())  # fused == unfused, bit for bit
     assert_same(put.asnumpy(), (r - P + Se).asnumpy())
+
+
+# ---- dpnp-level functions built on the ufunc extension kernels ---------------------------------
+def test_nan_to_num_reference_examples():
+    # docstring of dpnp.nan_to_num, dpnp/dpnp_iface_mathematical.py:3640-3670
+    x = np.array([np.inf, -np.inf, np.nan, -128, 128])
+    d = dpnp.array(x)
+    np.testing.assert_array_equal(dpnp.nan_to_num(d).asnumpy(), np.nan_to_num(x))
+    np.testing.assert_array_equal(dpnp.nan_to_num(d, nan=-9999, posinf=33333333, neginf=33333333).asnumpy(),
+                                  np.nan_to_num(x, nan=-9999, posinf=33333333, neginf=33333333))
+    y = np.array([complex(np.inf, np.nan), np.nan, complex(np.nan, np.inf)])
+    np.testing.assert_array_equal(dpnp.nan_to_num(dpnp.array(y), nan=111111, posinf=222222).asnumpy(),
+                                  np.nan_to_num(y, nan=111111, posinf=222222))
+    for dt in ("f2", "f4", "c8"):
+        z = x.astype(dt)
+        np.testing.assert_array_equal(dpnp.nan_to_num(dpnp.array(z)).asnumpy(), np.nan_to_num(z))
+    i = dpnp.array(np.arange(4))
+    assert dpnp.nan_to_num(i) is not i and dpnp.nan_to_num(i, copy=False) is i
+    w = dpnp.array(x)
+    assert dpnp.nan_to_num(w, copy=False) is w
+    np.testing.assert_array_equal(w.asnumpy(), np.nan_to_num(x))
+    # strided input
+    s = dpnp.array(np.tile(x, 7))[::3]
+    np.testing.assert_array_equal(dpnp.nan_to_num(s).asnumpy(), np.nan_to_num(np.tile(x, 7)[::3]))
+
+
+def test_isclose_reference_examples():
+    # docstring of dpnp.isclose, dpnp/dpnp_iface_logic.py:870-900
+    cases = [([1e10, 1e-7], [1.00001e10, 1e-8], {}), ([1e10, 1e-8], [1.00001e10, 1e-9], {}),
+             ([1e10, 1e-8], [1.0001e10, 1e-9], {}), ([1.0, np.nan], [1.0, np.nan], {}),
+             ([1.0, np.nan], [1.0, np.nan], {"equal_nan": True}), ([0.0, 0.0], [1e-8, 1e-7], {}),
+             ([0.0, 0.0], [1e-100, 1e-7], {"atol": 0.0}), ([1e-10, 1e-10], [1e-20, 0.0], {}),
+             ([1e-10, 1e-10], [1e-20, 0.999999e-10], {"atol": 0.0}),
+             ([np.inf, -np.inf, np.inf], [np.inf, np.inf, 1.0], {})]
+    for a, b, kw in cases:
+        got = dpnp.isclose(dpnp.array(a), dpnp.array(b), **kw).asnumpy()
+        np.testing.assert_array_equal(got, np.isclose(np.array(a), np.array(b), **kw))
+    rng = np.random.default_rng(401)
+    a = rng.standard_normal((40, 50)).astype("f4")
+    b = a + rng.standard_normal((1, 50)).astype("f4") * 1e-5
+    np.testing.assert_array_equal(dpnp.isclose(dpnp.array(a), dpnp.array(b)[0:1]).asnumpy(), np.isclose(a, b[0:1]))
+    np.testing.assert_array_equal(dpnp.isclose(dpnp.array(a), 0.5, atol=0.1).asnumpy(), np.isclose(a, 0.5, atol=0.1))
+    z = (a + 1j * a.T[:40, :40].repeat(2, axis=1)[:, :50]).astype("c8")
+    np.testing.assert_array_equal(dpnp.isclose(dpnp.array(z), dpnp.array(z * (1 + 1e-6))).asnumpy(),
+                                  np.isclose(z, z * (1 + 1e-6)))
+    ints = np.arange(10)
+    np.testing.assert_array_equal(dpnp.isclose(dpnp.array(ints), dpnp.array(ints + 1), atol=1).asnumpy(),
+                                  np.isclose(ints, ints + 1, atol=1))
+
+
+def test_float_power_divmod_modf_aliases():
+    rng = np.random.default_rng(403)
+    a = rng.integers(1, 9, 50).astype("i4")
+    b = rng.integers(-3, 4, 50).astype("i4")
+    r = dpnp.float_power(dpnp.array(a), dpnp.array(b))
+    assert r.dtype == np.dtype("f8")
+    np.testing.assert_allclose(r.asnumpy(), np.float_power(a, b), rtol=1e-15)
+    x = rng.uniform(-20, 20, 300).astype("f4")
+    y = rng.uniform(-5, 5, 300).astype("f4")
+    q, m = dpnp.divmod(dpnp.array(x), dpnp.array(y))
+    wq, wm = np.divmod(x, y)
+    np.testing.assert_array_equal(q.asnumpy(), wq)
+    np.testing.assert_allclose(m.asnumpy(), wm, rtol=1e-6, atol=1e-6)
+    qi, mi = dpnp.divmod(dpnp.array(a), dpnp.array(np.where(b == 0, 1, b).astype("i4")))
+    wqi, wmi = np.divmod(a, np.where(b == 0, 1, b).astype("i4"))
+    np.testing.assert_array_equal(qi.asnumpy(), wqi)
+    np.testing.assert_array_equal(mi.asnumpy(), wmi)
+    v = np.array([2.5, -2.5, 0.0, -0.0, np.inf, -np.inf, np.nan, 7.0], dtype="f8")
+    f, w = dpnp.modf(dpnp.array(v))
+    wf, ww = np.modf(v)
+    np.testing.assert_array_equal(f.asnumpy(), wf)
+    np.testing.assert_array_equal(w.asnumpy(), ww)
+    np.testing.assert_array_equal(np.signbit(f.asnumpy()), np.signbit(wf))
+    np.testing.assert_allclose(dpnp.rad2deg(dpnp.array(x)).asnumpy(), np.rad2deg(x), rtol=1e-6)
+    np.testing.assert_allclose(dpnp.deg2rad(dpnp.array(x)).asnumpy(), np.deg2rad(x), rtol=1e-6)
+    np.testing.assert_array_equal(dpnp.fmax(dpnp.array(x), np.float32(0.5)).asnumpy(), np.fmax(x, np.float32(0.5)))
+    np.testing.assert_array_equal(dpnp.gcd(dpnp.array(a), 6).asnumpy(), np.gcd(a, 6))

@@ -479,3 +479,116 @@ def test_transposed_with_batch_dims_offsets_and_strided_output():
     want = np.zeros((90, 200), dtype="i4")
     want[:, 7:77] = -hsrc
     assert_same(host(big), want)
+
+
+# ---- functions of the reference's ufunc extension ----------------------------------------------
+@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
+def test_extension_unary_float(dt):
+    rng = np.random.default_rng(301)
+    a = random_array(rng, 5000, dt, -6, 6)
+    a[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5]
+    d = dev(a)
+    assert_same(host(dpt.fabs(d)), orc.unary("fabs", a))
+    sp = host(dpt.spacing(d))
+    assert_same(sp, orc.unary("spacing", a))
+    tol = 4.0
+    for name in ("degrees", "radians"):
+        assert_ulp(host(getattr(dpt, name)(d)), getattr(np, name)(a.astype(np.longdouble)), 1.0)
+    import mpmath
+
+    mpmath.mp.dps = 40  # sin(pi x) near its zeros needs the exact argument: numpy.sinc rounds pi * x first
+    fin = np.isfinite(a)
+    exact = np.array([np.longdouble(str(mpmath.sincpi(mpmath.mpf(float(v))))) for v in a[fin]], dtype=np.longdouble)
+    got = host(dpt.sinc(d))
+    assert_ulp(got[fin], exact, tol if dt != "f2" else 1.0)
+    assert np.all(np.isnan(got[np.isnan(a)])) and np.all(got[np.isinf(a)] == 0) | np.all(np.isnan(got[np.isinf(a)]))
+    mp_fn = {"erfc": mpmath.erfc, "erfcx": lambda v: mpmath.exp(v * v) * mpmath.erfc(v),
+             "i0": lambda v: mpmath.besseli(0, v)}
+    for name in ("erfc", "erfcx", "i0"):
+        x = (a if name != "erfcx" else np.clip(a, -3, 6))[:1200]   # erfcx grows like exp(x^2) for negative x
+        got = host(getattr(dpt, name)(dev(x)))
+        assert got.dtype == orc.unary_result_dtype(name, dt), name
+        fin = np.isfinite(x)
+        # mpmath at 40 digits (scipy's float64 erfc is tens of ULPs off in the far tail)
+        exact = np.array([np.longdouble(str(mp_fn[name](mpmath.mpf(float(v))))) for v in x[fin]], dtype=np.longdouble)
+        assert_ulp(got[fin], exact, 8.0 if name == "i0" and dt == "f8" else tol)
+        if name == "i0":
+            assert np.all(got[np.isinf(x)] == np.inf) and np.all(np.isnan(got[np.isnan(x)]))
+        elif name == "erfc":
+            assert_same(got[~fin], np.array([0.0, 2.0, np.nan], dtype=got.dtype))
+    p = random_array(rng, 3000, dt, -0.999, 0.999)
+    assert_ulp(host(dpt.erfinv(dev(p))), orc.unary("erfinv", p).astype(np.longdouble), 8.0)
+    q = random_array(rng, 3000, dt, 0.001, 1.999)
+    assert_ulp(host(dpt.erfcinv(dev(q))), orc.unary("erfcinv", q).astype(np.longdouble), 8.0)
+    # outside the domain: NaN; at the ends: infinities
+    e = host(dpt.erfinv(dev(np.array([-1.0, 1.0, 2.0], dtype=dt))))
+    assert e[0] == -np.inf and e[1] == np.inf and np.isnan(e[2])
+
+
+def test_extension_sinc_complex_and_bitwise_count():
+    rng = np.random.default_rng(303)
+    for dt in ("c8", "c16"):
+        z = random_array(rng, 2000, dt, -3, 3)
+        z[0] = 0
+        got = host(dpt.sinc(dev(z)))
+        want = np.sinc(z.astype(np.clongdouble))
+        np.testing.assert_allclose(got, want.astype(dt), rtol=2e-5 if dt == "c8" else 1e-13)
+    for dt in ("i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8"):
+        info = np.iinfo(dt)
+        a = rng.integers(info.min, info.max, 4000, dtype=dt, endpoint=True)
+        a[:3] = [info.min, info.max, 0]
+        r = dpt.bitwise_count(dev(a))
+        assert r.dtype == np.dtype("u1")
+        assert_same(host(r), orc.unary("bitwise_count", a))
+    with pytest.raises((ValueError, TypeError)):
+        dpt.bitwise_count(dev(np.ones(3, dtype="f4")))
+
+
+@pytest.mark.parametrize("dt", [d for d in ALL])
+def test_extension_fmax_fmin_all_types(dt):
+    rng = np.random.default_rng(307)
+    a, b = random_array(rng, 3000, dt), random_array(rng, 3000, dt)
+    if np.dtype(dt).kind in "fc":
+        a[::7] = np.nan
+        b[::11] = np.nan
+        if np.dtype(dt).kind == "c":
+            a[1::13] = complex(1, np.nan)
+    for name in ("fmax", "fmin"):
+        assert_same(host(getattr(dpt, name)(dev(a), dev(b))), orc.binary(name, a, b))
+
+
+def test_extension_binary_misc():
+    rng = np.random.default_rng(311)
+    for dt in ("i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8"):
+        a, b = random_array(rng, 4000, dt, -120, 120), random_array(rng, 4000, dt, -12, 12)
+        info = np.iinfo(dt)
+        a[:2] = [info.min, info.max]
+        b[:2] = [-1 if info.min < 0 else 1, 0]
+        assert_same(host(dpt.fmod(dev(a), dev(b))), orc.binary("fmod", a, b))
+        a2, b2 = a.copy(), b.copy()
+        if info.min < 0:
+            a2[a2 == info.min] = 0   # |INT_MIN| is not representable
+        assert_same(host(dpt.gcd(dev(a2), dev(b2))), orc.binary("gcd", a2, b2))
+        small = (a2 % 50).astype(dt) if info.max < 10**5 else a2
+        small_b = (b2 % 11).astype(dt)
+        if info.max >= 10**5:
+            assert_same(host(dpt.lcm(dev(small), dev(small_b))), orc.binary("lcm", small, small_b))
+    r = dpt.fmod(dev(np.array([True, False])), dev(np.array([True, True])))
+    assert r.dtype == np.dtype("i1") and host(r).tolist() == [0, 0]
+    for dt in ("f2", "f4", "f8"):
+        a, b = random_array(rng, 4000, dt, -30, 30), random_array(rng, 4000, dt, -30, 30)
+        a[:6] = [0.0, -0.0, np.nan, np.inf, -np.inf, 2.0]
+        b[:6] = [0.5, 0.25, 1.0, 1.0, np.inf, np.nan]
+        assert_same(host(dpt.heaviside(dev(a), dev(b))), orc.binary("heaviside", a, b))
+        fm = host(dpt.fmod(dev(a), dev(b)))
+        np.testing.assert_array_equal(fm, np.fmod(a, b))
+        got = host(dpt.logaddexp2(dev(a), dev(b)))
+        with np.errstate(all="ignore"):
+            want = np.logaddexp2(a.astype(np.longdouble), b.astype(np.longdouble))
+        ok = np.isfinite(want)
+        # the reference's formula max + log2(1 + 2**-|d|) cancels near zero: ULPs of the operands
+        scale = np.maximum(np.maximum(np.abs(a), np.abs(b)).astype(np.longdouble), np.abs(want))
+        assert (np.abs(got[ok].astype(np.longdouble) - want[ok]) <= 4 * np.finfo(dt).eps * scale[ok]).all()
+        assert np.array_equal(np.isnan(got), np.isnan(want.astype(dt)))
+    with pytest.raises((ValueError, TypeError)):
+        dpt.gcd(dev(np.ones(3, dtype="f4")), dev(np.ones(3, dtype="f4")))

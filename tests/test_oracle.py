@@ -367,3 +367,34 @@ def test_oracle_nan_functions_match_numpy(dt):
     assert orc.nanmean(c, 2) == pytest.approx(2.6666666666666665)
     np.testing.assert_allclose(orc.nanvar(c.T, 1), [1.0, 0.0])
     assert orc.nanvar(c, 2) == pytest.approx(1.5555555555555556)
+
+
+# ---- functions of the ufunc extension: the oracle's entries against independent evaluations ----
+def test_oracle_extension_functions_known_values():
+    import mpmath
+
+    mpmath.mp.dps = 40
+    x = np.array([-2.5, -0.3, 0.0, 0.7, 3.0], dtype="f8")
+    for name, ref in (("erfc", mpmath.erfc), ("i0", lambda v: mpmath.besseli(0, v)),
+                      ("erfcx", lambda v: mpmath.exp(v * v) * mpmath.erfc(v))):
+        want = np.array([float(ref(mpmath.mpf(float(v)))) for v in x])
+        np.testing.assert_allclose(orc.unary(name, x), want, rtol=1e-14)
+    p = np.array([-0.9, -0.2, 0.0, 0.5, 0.99], dtype="f8")
+    np.testing.assert_allclose([math.erf(v) for v in orc.unary("erfinv", p)], p, rtol=1e-14, atol=1e-16)
+    q = np.array([0.01, 0.5, 1.0, 1.7], dtype="f8")
+    np.testing.assert_allclose([math.erfc(v) for v in orc.unary("erfcinv", q)], q, rtol=1e-13)
+    # closed forms
+    assert orc.unary("sinc", np.array([0.0, 0.5, 1.0], dtype="f8")).tolist() == pytest.approx([1.0, 2 / math.pi, 0.0],
+                                                                                           abs=1e-16)
+    assert orc.unary("degrees", np.array([math.pi], dtype="f8"))[0] == 180.0
+    assert orc.unary("bitwise_count", np.array([0, 1, -1, 127, -128], dtype="i1")).tolist() == [0, 1, 1, 7, 1]
+    assert orc.unary("spacing", np.array([1.0], dtype="f4"))[0] == np.finfo("f4").eps
+    assert orc.unary("spacing", np.array([-1.0], dtype="f2"))[0] == np.float16(2.0 ** -11)  # towards +inf
+    assert orc.binary("fmod", np.array([-7, 7, 5], dtype="i4"), np.array([3, -3, 0], dtype="i4")).tolist() == [-1, 1, 0]
+    assert orc.binary("gcd", np.array([12, -12, 0], dtype="i4"), np.array([18, 18, 0], dtype="i4")).tolist() == [6, 6, 0]
+    assert orc.binary("lcm", np.array([4, -4, 0], dtype="i4"), np.array([6, 6, 5], dtype="i4")).tolist() == [12, 12, 0]
+    nan = np.nan
+    assert np.array_equal(orc.binary("fmax", np.array([1.0, nan, nan]), np.array([nan, 2.0, nan])),
+                          np.array([1.0, 2.0, nan]), equal_nan=True)
+    assert orc.binary("heaviside", np.array([-1.0, 0.0, 2.0]), np.array([0.5, 0.5, 0.5])).tolist() == [0.0, 0.5, 1.0]
+    assert orc.binary("logaddexp2", np.array([3.0]), np.array([3.0]))[0] == 4.0
