@@ -110,6 +110,8 @@ SIGNATURES = {
     "dpx_nan_to_num": (_i, [_VP, _d, _d, _d, _VP, _vp]),
     "dpx_isclose": (_i, [_VP, _VP, _d, _d, _i, _VP, _vp]),
     "dpx_copy_cast": (_i, [_VP, _VP, _vp]),
+    "dpx_copy_from_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
+    "dpx_copy_to_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
     "dpx_fill": (_i, [_VP, _d, _d, _i64, _i, _vp]),
     "dpx_unary_plan": (_i, [_i, _VP, _VP, _PP]),
     "dpx_binary_plan": (_i, [_i, _VP, _VP, _VP, _PP]),

@@ -134,13 +134,22 @@ def to_device_bytes(host_bytes_array):
     t = _torch()
     if not t.cuda.is_available():
         raise RuntimeError("dpnp_amd needs an AMD GPU: no HIP device is visible to this process")
-    if host_bytes_array.size == 0:
-        return alloc(0)
-    return t.from_numpy(host_bytes_array).to("cuda")
+    n = int(host_bytes_array.size)
+    buf = alloc(n)
+    if n:
+        from .. import _lib
+
+        _lib.check(_lib.lib.dpx_copy_from_host(buf.data_ptr(), host_bytes_array.ctypes.data, n,
+                                               current_stream_ptr()))
+    return buf
 
 
 def to_host_bytes(buf, byte_offset, nbytes):
     """Copy `nbytes` bytes starting at `byte_offset` of allocation `buf` to a NumPy uint8 array."""
-    if nbytes == 0:
-        return np.empty(0, dtype=np.uint8)
-    return buf[byte_offset:byte_offset + nbytes].cpu().numpy()
+    out = np.empty(nbytes, dtype=np.uint8)
+    if nbytes:
+        from .. import _lib
+
+        _lib.check(_lib.lib.dpx_copy_to_host(out.ctypes.data, buf.data_ptr() + byte_offset, nbytes,
+                                             current_stream_ptr()))
+    return out

@@ -327,6 +327,19 @@ int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol,
  * dtype pair, equal shapes */
 int dpx_copy_cast(const dpx_array_view *src, const dpx_array_view *dst,
                   void *stream);
+
+/* Contiguous byte copies between pageable host memory and device memory, staged through a
+ * pool of pinned buffers filled and drained by several host threads.  Replaces the
+ * sycl::queue::memcpy calls behind dpnp.asarray / dpnp.asnumpy
+ * (libtensor/source/copy_numpy_ndarray_into_usm_ndarray.cpp:60-190 for the contiguous
+ * same-dtype case, dpnp/tensor/_copy_utils.py:54-135).
+ * dpx_copy_from_host returns once src_host has been read (the device side completes in
+ * stream order); dpx_copy_to_host is enqueued on `stream` and returns when dst_host holds
+ * the data. */
+int dpx_copy_from_host(void *dst_device, const void *src_host, size_t nbytes,
+                       void *stream);
+int dpx_copy_to_host(void *dst_host, const void *src_device, size_t nbytes,
+                     void *stream);
 /* dst = value (converted to dst's dtype): ti._full_usm_ndarray,
  * libtensor/source/full_ctor.cpp. value_im is used for complex dst only. */
 int dpx_fill(const dpx_array_view *dst, double value_re, double value_im,

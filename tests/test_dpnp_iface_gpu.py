@@ -207,3 +207,39 @@ def test_float_power_divmod_modf_aliases():
     np.testing.assert_allclose(dpnp.deg2rad(dpnp.array(x)).asnumpy(), np.deg2rad(x), rtol=1e-6)
     np.testing.assert_array_equal(dpnp.fmax(dpnp.array(x), np.float32(0.5)).asnumpy(), np.fmax(x, np.float32(0.5)))
     np.testing.assert_array_equal(dpnp.gcd(dpnp.array(a), 6).asnumpy(), np.gcd(a, 6))
+
+
+# ---- host <-> device transfers through the pinned staging pool ------------------------------------
+@pytest.mark.parametrize("nbytes", [1, 4095, (1 << 20) + 1, (16 << 20), (16 << 20) + 7, 5 * (16 << 20) + 12345])
+def test_staged_transfers_round_trip(nbytes):
+    rng = np.random.default_rng(nbytes % 1000)
+    h = rng.integers(0, 256, nbytes, dtype=np.uint8)
+    d = dpnp.array(h)
+    back = d.asnumpy()
+    assert back.dtype == h.dtype and np.array_equal(back, h)
+    # a second upload reuses the staging buffers while the first download may still be pending
+    h2 = h[::-1].copy()
+    d2 = dpnp.array(h2)
+    assert np.array_equal((d2 + np.uint8(1)).asnumpy(), h2 + np.uint8(1))
+    assert np.array_equal(d.asnumpy(), h)
+
+
+def test_transfer_entry_points_through_the_c_abi():
+    import ctypes
+
+    import torch
+
+    import dpnp_amd._lib as L
+
+    n = (3 << 20) + 5
+    h = np.random.default_rng(7).integers(0, 256, n, dtype=np.uint8)
+    buf = torch.empty(n, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    L.check(L.lib.dpx_copy_from_host(buf.data_ptr(), h.ctypes.data, n, stream))
+    assert np.array_equal(buf.cpu().numpy(), h)
+    out = np.zeros(n, dtype=np.uint8)
+    L.check(L.lib.dpx_copy_to_host(out.ctypes.data, buf.data_ptr(), n, stream))
+    assert np.array_equal(out, h)
+    assert L.lib.dpx_copy_to_host(out.ctypes.data, buf.data_ptr(), 0, stream) == 0
+    assert L.lib.dpx_copy_from_host(None, h.ctypes.data, 8, stream) != 0  # null pointer: an error, no crash
+    assert b"null" in L.lib.dpx_last_error()
