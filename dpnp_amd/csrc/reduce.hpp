@@ -46,7 +46,7 @@ struct RedLaunch {
     int32_t splits;   // blocks cooperating on one output
     int32_t g_log2;   // rows: log2(lanes per output); cols: log2(threads along columns)
     int32_t vec;      // 16-byte packs allowed
-    int32_t pad;
+    int32_t tgroup;   // rows: blocks per first-level ticket group (0: one ticket counter per output)
     int64_t rstride;  // cols: stride of the reduced axis
     int64_t inner;    // cols: length of the inner (contiguous) iteration dim
     int64_t col_blocks;
@@ -308,6 +308,60 @@ DPX_D bool last_block_of(unsigned *counter, int splits, uint32_t zero)
     return last;
 }
 
+// The same with two levels of tickets, for outputs that many blocks share: atomics on one
+// address are served one at a time (about 10 ns each on MI355X, 5 us for 512 blocks that
+// finish together), so blocks draw their ticket from a counter per group of `tgroup` blocks
+// and only the last block of a group draws from the output's counter.  `group_counters`
+// holds the groups of this output, RED_GROUP_PITCH words apart (separate cache lines).
+constexpr int RED_GROUP_PITCH = 32;
+DPX_D bool last_block_of_grouped(unsigned *counter, unsigned *group_counters, int split, int splits, int tgroup,
+                                 uint32_t zero)
+{
+    __shared__ unsigned sh_zero2;
+    __shared__ int is_last2;
+    if (threadIdx.x == 0) sh_zero2 = 0;
+    __syncthreads();
+    atomicOr(&sh_zero2, zero);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int g = split / tgroup, ng = (splits + tgroup - 1) / tgroup;
+        const int in_g = (g == ng - 1) ? splits - g * tgroup : tgroup;
+        unsigned *c1 = group_counters + (size_t)g * RED_GROUP_PITCH;
+        const unsigned t = __hip_atomic_fetch_add(c1 + sh_zero2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int last = 0;
+        if (t == (unsigned)(in_g - 1)) {
+            __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the second ticket's address depends on the first ticket: it is drawn after it
+            uint32_t z2;
+            asm volatile("v_and_b32 %0, 0, %1" : "=v"(z2) : "v"(t));
+            const unsigned t2 = __hip_atomic_fetch_add(counter + z2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (t2 == (unsigned)(ng - 1)) {
+                __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = 1;
+            }
+        }
+        is_last2 = last;
+    }
+    __syncthreads();
+    const bool last = is_last2 != 0;
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return last;
+}
+// scratch layout: [RED_MAX_TICKETS output counters | RED_MAX_GROUPS group counters, RED_GROUP_PITCH
+// words apart | partials]; the pool hands out zeroed memory and the kernels leave every counter at
+// zero again
+constexpr int64_t RED_MAX_TICKETS = 16384;
+constexpr int64_t RED_MAX_GROUPS = 512;
+constexpr size_t RED_COUNTER_BYTES = (RED_MAX_TICKETS + RED_MAX_GROUPS * RED_GROUP_PITCH) * sizeof(unsigned);
+// ticket of block `split` of output `o` under the launch's scheme
+DPX_D bool last_block_of_output(unsigned *counters, const RedLaunch &L, int64_t o, int split, uint32_t zero)
+{
+    if (L.tgroup == 0) return last_block_of(counters + o, L.splits, zero);
+    const int ng = (L.splits + L.tgroup - 1) / L.tgroup;
+    return last_block_of_grouped(counters + o, counters + RED_MAX_TICKETS + (o * ng) * RED_GROUP_PITCH, split,
+                                 L.splits, L.tgroup, zero);
+}
+
 template <class P, bool CONTIG>
 __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
                                                        typename P::Out *dst, Slot<typename P::Acc> *partial,
@@ -385,7 +439,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L
     // split mode (always a whole block per output): pass two by the last block to finish
     uint32_t zero = 0;
     if (threadIdx.x == 0) zero = slot_publish(partial + o * L.splits + split, r);
-    if (!last_block_of(counters + o, L.splits, zero)) return;
+    if (!last_block_of_output(counters, L, o, split, zero)) return;
     Acc v = P::identity();
     for (int i = threadIdx.x; i < L.splits; i += blockDim.x) v = P::combine(v, slot_read(partial + o * L.splits + i));
     v = group_reduce<P>(v, true, G);
@@ -738,7 +792,7 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
         zero = slot_publish(pval + o * L.splits + split, to_storage<T>(best));
         zero |= slot_publish(pidx + o * L.splits + split, bidx);
     }
-    if (!last_block_of(counters + o, L.splits, zero)) return;
+    if (!last_block_of_output(counters, L, o, split, zero)) return;
     best = VT{};
     bidx = ARG_NONE;
     for (int i = threadIdx.x; i < L.splits; i += blockDim.x)

@@ -6,10 +6,6 @@
 
 namespace dpx {
 
-// scratch layout: [ticket counters | partials]; the pool hands out zeroed memory and the
-// kernels leave every counter at zero again
-constexpr int64_t RED_MAX_TICKETS = 16384;
-constexpr size_t RED_COUNTER_BYTES = RED_MAX_TICKETS * sizeof(unsigned);
 
 struct RedPlan {
     int path; // dpx_path

@@ -177,6 +177,9 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         splits = cdiv(n, chunk);
         L.chunk = chunk;
         L.splits = (int32_t)splits;
+        // many blocks per output: two levels of tickets (groups of 32 blocks), while the group
+        // counters of all outputs fit their table
+        L.tgroup = (splits >= 128 && m * cdiv(splits, 32) <= RED_MAX_GROUPS) ? 32 : 0;
         pl.grid = oblocks * splits;
         pl.path = !contig_red ? DPX_PATH_RED_GENERIC
                               : (splits > 1 ? DPX_PATH_RED_ROWS_SPLIT

@@ -176,7 +176,7 @@ def plan_reduce(op, src, trailing, dst):
 def test_reduction_plans():
     p = plan_reduce("sum", view([1 << 28]), 1, view([], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_rows_split" and p.splits > 1 and p.vec == 1
-    assert p.scratch_bytes == 65536 + 4 * p.splits  # ticket counters + one float partial per block
+    assert p.scratch_bytes == 131072 + 4 * p.splits  # ticket counters (outputs + groups) + one float partial per block
     p = plan_reduce("sum", view([16384, 16384]), 1, view([16384], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_rows" and p.splits == 1 and p.grid[0] == 16384
     # axis=0 of a C-contiguous matrix: the caller passes the transposed view
