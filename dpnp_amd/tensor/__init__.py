@@ -62,6 +62,8 @@ from ._search_functions import where
 from ._statistical_functions import mean, std, var
 from ._type_utils import can_cast, result_type
 from ._usmarray import usm_ndarray
+from ._array_api import __array_api_version__, __array_namespace_info__  # noqa: E402
+from ._testing import allclose  # noqa: E402
 
 e = 2.718281828459045
 pi = 3.141592653589793

@@ -227,6 +227,8 @@ def _default_accumulation_dtype_fp_types(inp_dt, q=None):
     k = inp_dt.kind
     if k in "biu":
         return dt_.float64  # the device has fp64, so ints never settle for float32
+    if k == "c":
+        raise ValueError("function not defined for complex types")
     return inp_dt
 
 

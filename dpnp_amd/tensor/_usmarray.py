@@ -91,6 +91,12 @@ class Flags:
             raise KeyError(f"Unknown flag name: {name}")
         return getattr(self, table[name])
 
+    def __setitem__(self, name, value):
+        # only the writable flag can be changed (dpnp/tensor/_flags.pyx: "W" / "WRITABLE")
+        if name not in ("W", "WRITABLE"):
+            raise ValueError("Only writable ('W' or 'WRITABLE') flag can be set")
+        self.writable = value
+
     def __repr__(self):
         return (f"  C_CONTIGUOUS : {self.c_contiguous}\n  F_CONTIGUOUS : {self.f_contiguous}\n"
                 f"  WRITABLE : {self.writable}")
