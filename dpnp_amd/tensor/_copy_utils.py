@@ -58,13 +58,24 @@ def _empty_like_pair_orderK(x1, x2, dt, res_shape):
 
 
 def _empty_like_triple_orderK(x1, x2, x3, dt, res_shape):
+    """Layout of a result of three operands (dpnp/tensor/_copy_utils.py:914-987): two operands of
+    the full shape decide when the third has fewer dims; else C if any operand is C-contiguous,
+    F if all are F-contiguous, else dims nested by the operands' strides."""
+    res_shape = tuple(res_shape)
+    nd = len(res_shape)
+    if x1.shape == res_shape and x2.shape == res_shape and nd > x3.ndim:
+        return _empty_like_pair_orderK(x1, x2, dt, res_shape)
+    if x2.shape == res_shape and x3.shape == res_shape and nd > x1.ndim:
+        return _empty_like_pair_orderK(x2, x3, dt, res_shape)
+    if x1.shape == res_shape and x3.shape == res_shape and nd > x2.ndim:
+        return _empty_like_pair_orderK(x1, x3, dt, res_shape)
     arrs = [x1, x2, x3]
-    if any(a.flags.c_contiguous and a.shape == tuple(res_shape) for a in arrs):
+    if any(a.flags.c_contiguous for a in arrs):
         return _empty(res_shape, dt, "C")
-    if all(a.flags.f_contiguous and a.shape == tuple(res_shape) for a in arrs):
+    if all(a.flags.f_contiguous for a in arrs):
         return _empty(res_shape, dt, "F")
     b = [broadcast_to(a, res_shape) for a in arrs]
-    return _like_strides(tuple(res_shape), [a.strides for a in b], dt) if len(res_shape) else _empty(res_shape, dt)
+    return _like_strides(res_shape, [a.strides for a in b], dt) if nd else _empty(res_shape, dt)
 
 
 def _copy_into(src, dst):

@@ -74,7 +74,11 @@ def _operand_shape(o):
     if isinstance(o, (bool, int, float, complex, np.generic)):
         return ()
     a = _foreign_as_numpy(o)
-    return None if a is None else tuple(a.shape)
+    if a is not None:
+        return tuple(a.shape)
+    # anything else counts as a scalar here and is rejected by the dtype check that follows
+    # (`_get_shape`, dpnp/tensor/_scalar_utils.py:108-115)
+    return getattr(o, "shape", ())
 
 
 def _as_device_array(o, dt):
