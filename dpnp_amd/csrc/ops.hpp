@@ -162,7 +162,7 @@ template <class R> DPX_D cplx<R> c_sqrt(cplx<R> z)
     const R ar = z.re < R(0) ? -z.re : z.re;
     const R t = m_sqrt((ar + m_hypot(z.re, z.im)) * R(0.5));
     if (z.re >= R(0)) return {t, z.im / (t + t)};
-    const R ai = z.im < R(0) ? -z.im : z.im;
+    const R ai = m_copysign(z.im, R(1)); // |im| also for -0.0: the real part of a root is never -0.0
     return {ai / (t + t), m_copysign(t, z.im)};
 }
 template <class R> DPX_D cplx<R> c_sinh(cplx<R> z)
@@ -192,6 +192,52 @@ template <class R> DPX_D cplx<R> c_tanh(cplx<R> z)
 template <class R> DPX_D cplx<R> c_sin(cplx<R> z) { const cplx<R> w = c_sinh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
 template <class R> DPX_D cplx<R> c_cos(cplx<R> z) { return c_cosh(cplx<R>{-z.im, z.re}); }
 template <class R> DPX_D cplx<R> c_tan(cplx<R> z) { const cplx<R> w = c_tanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+
+// Inverse functions after W. Kahan, "Branch cuts for complex elementary functions" (1987): the
+// square roots of 1 -/+ z (or z -/+ 1) carry the branch cuts, signed zeros pick the side.
+template <class R> DPX_D cplx<R> c_asin(cplx<R> z)
+{
+    const cplx<R> s1 = c_sqrt(cplx<R>{R(1) - z.re, -z.im}), s2 = c_sqrt(cplx<R>{R(1) + z.re, z.im});
+    return {m_atan2(z.re, s1.re * s2.re - s1.im * s2.im), m_asinh(s1.re * s2.im - s1.im * s2.re)};
+}
+template <class R> DPX_D cplx<R> c_acos(cplx<R> z)
+{
+    const cplx<R> s1 = c_sqrt(cplx<R>{R(1) - z.re, -z.im}), s2 = c_sqrt(cplx<R>{R(1) + z.re, z.im});
+    return {R(2) * m_atan2(s1.re, s2.re), m_asinh(s2.re * s1.im - s2.im * s1.re)};
+}
+template <class R> DPX_D cplx<R> c_acosh(cplx<R> z)
+{
+    const cplx<R> t1 = c_sqrt(cplx<R>{z.re - R(1), z.im}), t2 = c_sqrt(cplx<R>{z.re + R(1), z.im});
+    return {m_asinh(t1.re * t2.re + t1.im * t2.im), R(2) * m_atan2(t1.im, t2.re)};
+}
+// asinh z = -i asin(iz)
+template <class R> DPX_D cplx<R> c_asinh(cplx<R> z) { const cplx<R> w = c_asin(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+template <class R> DPX_D cplx<R> c_atanh(cplx<R> z)
+{
+    // odd function: work in the right half plane
+    const bool neg = m_signbit(z.re);
+    const R x = neg ? -z.re : z.re, y = neg ? -z.im : z.im;
+    const R ay = y < R(0) ? -y : y;
+    const R pi_2 = R(1.5707963267948966192313216916397514);
+    cplx<R> w;
+    const R big = std::is_same_v<R, double> ? R(1e150) : R(1e18);
+    if (x > big || ay > big) {
+        // |z| huge: atanh z -> 1/z +- i pi/2, without squaring the parts
+        const R s = x > ay ? x : ay;
+        const R xs = x / s, ys = y / s;
+        w = {xs / ((xs * xs + ys * ys) * s), m_copysign(pi_2, y)};
+    }
+    else if (x == R(1) && y == R(0)) {
+        w = {(R)__builtin_inff(), y};
+    }
+    else {
+        const R d = (R(1) - x) * (R(1) - x) + y * y;
+        w = {R(0.25) * m_log1p(R(4) * x / d), R(0.5) * m_atan2(R(2) * y, (R(1) - x) * (R(1) + x) - y * y)};
+    }
+    return neg ? cplx<R>{-w.re, -w.im} : w;
+}
+// atan z = -i atanh(iz)
+template <class R> DPX_D cplx<R> c_atan(cplx<R> z) { const cplx<R> w = c_atanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
 
 template <class T> using V = value_of_t<T>;
 
@@ -483,12 +529,12 @@ DPX_FP_UNARY(CbrtOp, m_cbrt(x))
 DPX_FPC_UNARY(ReciprocalOp, T(1) / x, (T{real_of_t<T>(1), real_of_t<T>(0)} / x))
 DPX_FPC_UNARY(SinhOp, m_sinh(x), c_sinh(x))
 DPX_FPC_UNARY(CoshOp, m_cosh(x), c_cosh(x))
-DPX_FP_UNARY(AsinOp, m_asin(x))
-DPX_FP_UNARY(AcosOp, m_acos(x))
-DPX_FP_UNARY(AtanOp, m_atan(x))
-DPX_FP_UNARY(AsinhOp, m_asinh(x))
-DPX_FP_UNARY(AcoshOp, m_acosh(x))
-DPX_FP_UNARY(AtanhOp, m_atanh(x))
+DPX_FPC_UNARY(AsinOp, m_asin(x), c_asin(x))
+DPX_FPC_UNARY(AcosOp, m_acos(x), c_acos(x))
+DPX_FPC_UNARY(AtanOp, m_atan(x), c_atan(x))
+DPX_FPC_UNARY(AsinhOp, m_asinh(x), c_asinh(x))
+DPX_FPC_UNARY(AcoshOp, m_acosh(x), c_acosh(x))
+DPX_FPC_UNARY(AtanhOp, m_atanh(x), c_atanh(x))
 #undef DPX_FP_UNARY
 #undef DPX_FPC_UNARY
 struct ErfOp { // dpnp/backend/kernels/elementwise_functions/erf.hpp:52-95; f2 -> f4

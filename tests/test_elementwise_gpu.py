@@ -361,6 +361,30 @@ def test_complex_elementary_functions(op):
     np.testing.assert_allclose(host(dpt.pow(dev(z[1:]), dev(np.full(4, 2 + 0j)))), z[1:] ** 2, rtol=1e-14, atol=1e-15)
 
 
+@pytest.mark.parametrize("op", ["asin", "acos", "atan", "asinh", "acosh", "atanh"])
+def test_complex_inverse_functions(op):
+    rng = np.random.default_rng(131)
+    npf = getattr(np, "arc" + op[1:])
+    for dt, rtol in (("c8", 4e-6), ("c16", 2e-14)):
+        a = (rng.uniform(-3, 3, 4000) + 1j * rng.uniform(-3, 3, 4000)).astype(dt)
+        a[:6] = [0.5 + 0j, 2 + 0j, -2 + 0j, 0.25j, 3j, -3j]
+        got = host(getattr(dpt, op)(dev(a)))
+        want = npf(a.astype("c16" if dt == "c8" else np.clongdouble))
+        assert got.dtype == np.dtype(dt)
+        err = np.abs(got - want) / np.maximum(np.abs(want), 1e-2)
+        assert float(err.max()) <= rtol, (float(err.max()), a[int(np.argmax(err))])
+    # the side of a branch cut is chosen by the sign of the zero part, as in NumPy
+    cuts = np.array([complex(2, 0.0), complex(2, -0.0), complex(-2, 0.0), complex(-2, -0.0),
+                     complex(0.0, 2), complex(-0.0, 2), complex(0.0, -2), complex(-0.0, -2), complex(0.5, -0.0)],
+                    dtype="c16")
+    got, want = host(getattr(dpt, op)(dev(cuts))), npf(cuts)
+    np.testing.assert_allclose(got, want, rtol=1e-14, atol=1e-15)
+    assert np.array_equal(np.signbit(got.real), np.signbit(want.real))
+    assert np.array_equal(np.signbit(got.imag), np.signbit(want.imag))
+    big = np.array([1e200 + 1e200j, -1e200 + 3j, 5 - 1e300j], dtype="c16")
+    np.testing.assert_allclose(host(getattr(dpt, op)(dev(big))), npf(big), rtol=1e-13)
+
+
 def test_angle_logaddexp_nextafter():
     rng = np.random.default_rng(101)
     z = (rng.standard_normal(3000) + 1j * rng.standard_normal(3000)).astype("c8")
