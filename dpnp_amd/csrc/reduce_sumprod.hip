@@ -29,6 +29,13 @@ template <class F> static bool for_sum_pair(int in_dt, int out_dt, F &&f)
     DPX_PAIR(uint8_t, uint64_t) DPX_PAIR(uint16_t, uint64_t) DPX_PAIR(uint32_t, uint64_t)
     // wider floating accumulation (sum.cpp:130-241 lists these among others)
     DPX_PAIR(half_t, float) DPX_PAIR(half_t, double) DPX_PAIR(float, double) DPX_PAIR(c64, c128)
+    // integers and bool summed in floating point: what mean() of an integer array asks for
+    // (dpnp/tensor/_statistical_functions.py:166-270 sums with dtype float64), in one pass
+    DPX_PAIR(bool_t, double) DPX_PAIR(int8_t, double) DPX_PAIR(uint8_t, double) DPX_PAIR(int16_t, double)
+    DPX_PAIR(uint16_t, double) DPX_PAIR(int32_t, double) DPX_PAIR(uint32_t, double) DPX_PAIR(int64_t, double)
+    DPX_PAIR(uint64_t, double) DPX_PAIR(bool_t, float) DPX_PAIR(int8_t, float) DPX_PAIR(uint8_t, float)
+    DPX_PAIR(int16_t, float) DPX_PAIR(uint16_t, float) DPX_PAIR(int32_t, float) DPX_PAIR(uint32_t, float)
+    DPX_PAIR(int64_t, float) DPX_PAIR(uint64_t, float)
 #undef DPX_PAIR
     return hit;
 }
@@ -79,23 +86,37 @@ int sum_acc_size(int in_dt, int out_dt)
     });
     return sz;
 }
-// sum((x - aux)^2): real floating types only
+// sum((x - aux)^2): real floating types, and integers / bool accumulated in double (var of an
+// integer array)
+template <class F> static bool for_sqdev_pair(int in_dt, int out_dt, F &&f)
+{
+    bool hit = false;
+#define DPX_PAIR(I, O)                                         \
+    if (!hit && in_dt == id_of_v<I> && out_dt == id_of_v<O>) { \
+        f(tag<I>{}, tag<O>{});                                 \
+        hit = true;                                            \
+    }
+    DPX_PAIR(half_t, half_t) DPX_PAIR(half_t, float) DPX_PAIR(float, float) DPX_PAIR(float, double)
+    DPX_PAIR(double, double) DPX_PAIR(bool_t, double) DPX_PAIR(int8_t, double) DPX_PAIR(uint8_t, double)
+    DPX_PAIR(int16_t, double) DPX_PAIR(uint16_t, double) DPX_PAIR(int32_t, double) DPX_PAIR(uint32_t, double)
+    DPX_PAIR(int64_t, double) DPX_PAIR(uint64_t, double)
+#undef DPX_PAIR
+    return hit;
+}
 bool sqdev_pair_supported(int in_dt, int out_dt)
 {
-    return (in_dt == DPX_HALF && (out_dt == DPX_HALF || out_dt == DPX_FLOAT)) ||
-           (in_dt == DPX_FLOAT && (out_dt == DPX_FLOAT || out_dt == DPX_DOUBLE)) ||
-           (in_dt == DPX_DOUBLE && out_dt == DPX_DOUBLE);
+    return for_sqdev_pair(in_dt, out_dt, [](auto, auto) {});
 }
 int sqdev_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view *dst, const dpx_array_view *aux,
               hipStream_t stream)
 {
-    const int i = src->dtype, o = dst->dtype;
-    if (i == DPX_HALF && o == DPX_HALF) return red_run<K_SUMSQDEV, half_t, half_t>(pl, src, dst, aux, stream);
-    if (i == DPX_HALF && o == DPX_FLOAT) return red_run<K_SUMSQDEV, half_t, float>(pl, src, dst, aux, stream);
-    if (i == DPX_FLOAT && o == DPX_FLOAT) return red_run<K_SUMSQDEV, float, float>(pl, src, dst, aux, stream);
-    if (i == DPX_FLOAT && o == DPX_DOUBLE) return red_run<K_SUMSQDEV, float, double>(pl, src, dst, aux, stream);
-    if (i == DPX_DOUBLE && o == DPX_DOUBLE) return red_run<K_SUMSQDEV, double, double>(pl, src, dst, aux, stream);
-    return DPX_ERR_NOT_IMPLEMENTED;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    for_sqdev_pair(src->dtype, dst->dtype, [&](auto it, auto ot) {
+        using I = typename decltype(it)::type;
+        using O = typename decltype(ot)::type;
+        rc = red_run<K_SUMSQDEV, I, O>(pl, src, dst, aux, stream);
+    });
+    return rc;
 }
 #endif
 

@@ -101,7 +101,10 @@ def test_reduction_dtype_support():
     assert lib.dpx_reduce_dtype_supported(R["sum"], L.DOUBLE, L.FLOAT) == 0
     assert lib.dpx_reduce_dtype_supported(R["max"], L.FLOAT, L.DOUBLE) == 0
     assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.FLOAT, L.DOUBLE) == 1
-    assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.INT32, L.DOUBLE) == 0
+    assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.INT32, L.DOUBLE) == 1   # var of an integer array
+    assert lib.dpx_reduce_dtype_supported(R["sumsqdev"], L.INT32, L.FLOAT) == 0
+    assert lib.dpx_reduce_dtype_supported(R["sum"], L.INT32, L.DOUBLE) == 1        # mean of an integer array
+    assert lib.dpx_reduce_dtype_supported(R["sum"], L.DOUBLE, L.INT32) == 0
 
 
 def c_collapse(shape, strides_list, keep_order=False):

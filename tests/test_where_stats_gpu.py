@@ -115,3 +115,22 @@ def test_mean_var_random(dt, rtol):
     nanned[3, 17] = np.nan
     r = host(dpt.var(dev(nanned), axis=1))
     assert np.isnan(r[3]) and not np.isnan(np.delete(r, 3)).any()
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8"])
+def test_mean_var_of_integer_arrays_in_one_pass(dt):
+    """Integer input is summed straight into float64 (no cast copy): same values as the cast path."""
+    import dpnp_amd._lib as L
+    from dpnp_amd.tensor._dtypes import dtype_id
+
+    rng = np.random.default_rng(61)
+    a = random_array(rng, (37, 501), dt, -100, 100)
+    d = dev(a)
+    for axis in (None, 0, 1):
+        m, v = host(dpt.mean(d, axis=axis)), host(dpt.var(d, axis=axis))
+        assert m.dtype == np.dtype("f8") and v.dtype == np.dtype("f8")
+        np.testing.assert_allclose(m, np.mean(a.astype("f8"), axis=axis), rtol=1e-13)
+        np.testing.assert_allclose(v, np.var(a.astype("f8"), axis=axis), rtol=1e-12, atol=1e-12)
+    assert L.lib.dpx_reduce_dtype_supported(L.REDUCE_ID["sum"], dtype_id(np.dtype(dt)), dtype_id(np.dtype("f8"))) == 1
+    s = dpt.sum(d, dtype="f4")
+    np.testing.assert_allclose(float(s), float(np.sum(a.astype("f8"))), rtol=1e-5, atol=1e-2)
