@@ -98,6 +98,7 @@ SIGNATURES = {
     "dpx_unary_result_type": (_i, [_i, _i]),
     "dpx_binary_result_type": (_i, [_i, _i, _i]),
     "dpx_binary_inplace_supported": (_i, [_i, _i, _i]),
+    "dpx_binary_fused_cast_result_type": (_i, [_i, _i, _i]),
     "dpx_reduce_dtype_supported": (_i, [_i, _i, _i]),
     "dpx_search_dtype_supported": (_i, [_i, _i, _i]),
     "dpx_array_overlap": (_i, [_VP, _VP]),

@@ -21,12 +21,23 @@ static int unary_result_type(int op, int dt)
     return r;
 }
 static bool is_compare(int op) { return op >= DPX_B_EQUAL && op <= DPX_B_GREATER_EQUAL; }
-static int binary_result_type(int op, int dt1, int dt2)
+static int mixed_result_type(int op, int dt1, int dt2)
+{
+    int r = -1;
+    if (dt1 != dt2 && is_mixed_arith(op))
+        for_mixed_pair(dt1, dt2, [&](auto tt, auto, auto) { r = id_of_v<typename decltype(tt)::type>; });
+    return r;
+}
+// with_fused: also the pairs whose conversion is folded into the kernel.  The exported type table
+// leaves them out: the caller's promotion search must see the same table as the reference's.
+static int binary_result_type(int op, int dt1, int dt2, bool with_fused = false)
 {
     int r = -1;
     if (dt1 != dt2) {
         if (is_compare(op) && ((dt1 == DPX_INT64 && dt2 == DPX_UINT64) || (dt1 == DPX_UINT64 && dt2 == DPX_INT64)))
             r = DPX_BOOL;
+        else if (with_fused)
+            r = mixed_result_type(op, dt1, dt2);
         return r;
     }
     for_binary_op(op, [&](auto otag) {
@@ -65,7 +76,7 @@ static int binary_call(int op, const dpx_array_view *a, const dpx_array_view *b,
     if (!view_ok(a) || !view_ok(b) || !view_ok(dst))
         return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
     if (op < 0 || op >= DPX_B_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown binary op id");
-    const int rt = binary_result_type(op, a->dtype, b->dtype);
+    const int rt = binary_result_type(op, a->dtype, b->dtype, true);
     if (rt < 0 || rt != dst->dtype)
         return fail(DPX_ERR_BAD_DTYPE, "Output array of type " + std::string(dtype_name(dst->dtype)) +
                                            " does not match the result type of the operation.");
@@ -91,6 +102,7 @@ extern "C" {
 
 int dpx_unary_result_type(int op, int dt) { return unary_result_type(op, dt); }
 int dpx_binary_result_type(int op, int dt1, int dt2) { return binary_result_type(op, dt1, dt2); }
+int dpx_binary_fused_cast_result_type(int op, int dt1, int dt2) { return mixed_result_type(op, dt1, dt2); }
 int dpx_binary_inplace_supported(int op, int lhs_dt, int rhs_dt)
 {
     // lhs op= rhs needs a kernel whose result type is lhs's type
@@ -120,7 +132,8 @@ int dpx_binary_plan(int op, const dpx_array_view *src1, const dpx_array_view *sr
 int dpx_binary_inplace(int op, const dpx_array_view *lhs, const dpx_array_view *rhs, void *stream)
 {
     if (!view_ok(lhs) || !view_ok(rhs)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
-    if (!dpx_binary_inplace_supported(op, lhs->dtype, rhs->dtype))
+    if (!dpx_binary_inplace_supported(op, lhs->dtype, rhs->dtype) &&
+        mixed_result_type(op, lhs->dtype, rhs->dtype) != lhs->dtype)
         return fail(DPX_ERR_BAD_DTYPE, "Left-hand side array has unexpected elemental data type for the "
                                        "in-place operation.");
     return binary_call(op, lhs, rhs, lhs, stream, nullptr);

@@ -29,9 +29,19 @@ int DPX_CAT(binary_group_, DPX_GROUP)(int op, const dpx_array_view *const *views
     int rc = DPX_ERR_NOT_IMPLEMENTED;
     const int dt1 = views[0]->dtype, dt2 = views[1]->dtype;
     if (dt1 != dt2) {
-        // the only mixed pairs: int64 <-> uint64 comparisons (greater.hpp:62-146)
+        // mixed pairs: int64 <-> uint64 comparisons (greater.hpp:62-146) and arithmetic with the
+        // conversion of one operand folded in
         for_binary_op(op, [&](auto otag) {
             using Op = typename decltype(otag)::type;
+            if constexpr (std::is_same_v<Op, AddOp> || std::is_same_v<Op, SubOp> || std::is_same_v<Op, MulOp> ||
+                          std::is_same_v<Op, DivOp>) {
+                for_mixed_pair(dt1, dt2, [&](auto tt, auto at, auto bt) {
+                    using T = typename decltype(tt)::type;
+                    using A = typename decltype(at)::type;
+                    using B = typename decltype(bt)::type;
+                    rc = run_ew<MixedFn<Op, T, A, B>, T, A, B>({}, views, stream, plan_out);
+                });
+            }
             if constexpr (std::is_same_v<Op, CmpOp<0>> || std::is_same_v<Op, CmpOp<1>> ||
                           std::is_same_v<Op, CmpOp<2>> || std::is_same_v<Op, CmpOp<3>> ||
                           std::is_same_v<Op, CmpOp<4>> || std::is_same_v<Op, CmpOp<5>>) {

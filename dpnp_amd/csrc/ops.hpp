@@ -843,6 +843,39 @@ template <bool LCM> struct GcdOp { // gcd.hpp / lcm.hpp: integers; the result is
     }
 };
 
+// Arithmetic on operands of two different types with the conversion folded into the load:
+// (A, B) -> T where one operand already has the result type T.  The reference has same-type
+// kernels only and its Python layer casts the other operand into a temporary first
+// (_find_buf_dtype2, dpnp/tensor/_type_utils.py:389-485); converting while reading gives the same
+// values without the extra pass.  f(tag<T>, tag<A>, tag<B>) is called for a supported pair.
+inline bool is_mixed_arith(int op)
+{
+    return op == DPX_B_ADD || op == DPX_B_SUBTRACT || op == DPX_B_MULTIPLY || op == DPX_B_DIVIDE;
+}
+template <class F> inline bool for_mixed_pair(int dt1, int dt2, F &&f)
+{
+#define DPX_MIX(T, X)                                       \
+    if (dt1 == id_of_v<T> && dt2 == id_of_v<X>) {           \
+        f(tag<T>{}, tag<T>{}, tag<X>{});                    \
+        return true;                                        \
+    }                                                       \
+    if (dt1 == id_of_v<X> && dt2 == id_of_v<T>) {           \
+        f(tag<T>{}, tag<X>{}, tag<T>{});                    \
+        return true;                                        \
+    }
+    DPX_MIX(double, float) DPX_MIX(double, int32_t) DPX_MIX(double, int64_t) DPX_MIX(double, bool_t)
+    DPX_MIX(float, bool_t)
+#undef DPX_MIX
+    return false;
+}
+template <class Op, class T, class A, class B> struct MixedFn {
+    DPX_D V<T> operator()(V<A> a, V<B> b) const
+    {
+        return Op::template apply<T>(to_value(convert<T, A>(to_storage<A>(a))),
+                                     to_value(convert<T, B>(to_storage<B>(b))));
+    }
+};
+
 // op id -> op struct; f(tag<Op>{}) is called for a valid id.  A translation unit built with
 // -DDPX_GROUP=g -DDPX_NGROUPS=n instantiates f only for the ids with id % n == g (the others
 // still return true, without a call), so the kernels of an op are compiled exactly once.

@@ -237,6 +237,7 @@ class BinaryElementwiseFunc:
         self.__doc__ = docs
         self.acceptance_fn_ = acceptance_fn
         self.weak_type_resolver_ = weak_type_resolver
+        self._fused_cache = {}
 
     def __str__(self):
         return f"<{self.__name__} '{self.name_}'>"
@@ -298,6 +299,18 @@ class BinaryElementwiseFunc:
         d1, d2 = self.weak_type_resolver_(d1, d2, None)
         return res_shape, d1, d2
 
+    def _fused_cast(self, d1, d2):
+        """dtype the kernel gives for operands of dtypes d1 != d2 when it converts one of them
+        while reading (a few arithmetic pairs), else None.  Only consulted after the promotion
+        search has settled on casting that operand, so result dtypes stay the reference's."""
+        key = (d1, d2)
+        hit = self._fused_cache.get(key, False)
+        if hit is False:
+            from . import _tensor_elementwise_impl as tei
+
+            hit = self._fused_cache[key] = tei._fused_cast_result_type(self.name_, d1, d2)
+        return hit
+
     def __call__(self, o1, o2, /, *, out=None, order="K"):
         order = _norm_order(order)
         res_shape, d1, d2 = self._resolve(o1, o2)
@@ -308,6 +321,14 @@ class BinaryElementwiseFunc:
                 f"function '{self.name_}' does not support input types ({d1}, {d2}), "
                 "and the inputs could not be safely coerced to any supported types according to "
                 "the casting rule ''safe''.")
+        if (buf1_dt is None) != (buf2_dt is None):
+            # "cast one operand to the result type, then compute": one kernel does both for some pairs
+            # (a dtype compares equal to None when it is float64, hence the explicit tests)
+            fused = self._fused_cast(d1, d2)
+            if fused is not None and fused == res_dt and (
+                    (buf1_dt is not None and buf1_dt == res_dt and d2 == res_dt)
+                    or (buf2_dt is not None and buf2_dt == res_dt and d1 == res_dt)):
+                buf1_dt = buf2_dt = None
         orig_out = out
         if out is not None:
             _check_out(out, res_shape, res_dt)
@@ -396,6 +417,10 @@ class BinaryElementwiseFunc:
                 "the casting rule ''same_kind''.")
         if res_dt != d1:
             raise ValueError(f"Output array of type {res_dt} is needed, got {d1}")
+        if buf_dt is not None and buf_dt == d1:
+            fused = self._fused_cast(d1, d2)
+            if fused is not None and fused == d1:
+                buf_dt = None  # the kernel converts the right operand while reading it
         rhs = _as_device_array(o2, d2)
         if buf_dt is None and isinstance(o2, usm_ndarray) and ti._array_overlap(o2, o1) \
                 and not ti._same_logical_tensors(o2, o1):

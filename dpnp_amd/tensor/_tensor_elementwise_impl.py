@@ -62,6 +62,16 @@ def _divide_by_scalar(src, scalar, dst, sycl_queue=None, depends=()):
     return _events(sycl_queue)
 
 
+def _fused_cast_result_type(name, dt1, dt2):
+    """Result dtype of binary function `name` for two different operand dtypes when the library
+    converts one operand while reading it (no counterpart in the reference), else None."""
+    op = _lib.BINARY_ID.get(name)
+    if op is None:
+        return None
+    r = lib.dpx_binary_fused_cast_result_type(op, dtype_id(dt1), dtype_id(dt2))
+    return None if r < 0 else dtype_from_id(r)
+
+
 def _nan_to_num(src, nan, posinf, neginf, dst, sycl_queue=None, depends=()):
     """ufi._nan_to_num of the reference's ufunc extension
     (dpnp/backend/extensions/ufunc/elementwise_functions/nan_to_num.cpp): scalar replacements."""

@@ -63,6 +63,13 @@ def test_binary_result_types():
         assert lib.dpx_binary_result_type(B["maximum"], i, i) == i
     # only same-dtype pairs, except int64/uint64 comparisons
     assert lib.dpx_binary_result_type(B["add"], L.FLOAT, L.DOUBLE) == -1
+    # pairs whose conversion is folded into the kernel are reported separately
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.DOUBLE) == L.DOUBLE
+    assert lib.dpx_binary_fused_cast_result_type(B["divide"], L.INT32, L.DOUBLE) == L.DOUBLE
+    assert lib.dpx_binary_fused_cast_result_type(B["multiply"], L.FLOAT, L.BOOL) == L.FLOAT
+    assert lib.dpx_binary_fused_cast_result_type(B["maximum"], L.FLOAT, L.DOUBLE) == -1
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.INT32) == -1
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.FLOAT) == -1
     assert lib.dpx_binary_result_type(B["less"], L.INT64, L.UINT64) == L.BOOL
     assert lib.dpx_binary_result_type(B["less"], L.UINT64, L.INT64) == L.BOOL
     assert lib.dpx_binary_result_type(B["less"], L.INT32, L.UINT32) == -1

@@ -616,3 +616,35 @@ def test_extension_binary_misc():
         assert np.array_equal(np.isnan(got), np.isnan(want.astype(dt)))
     with pytest.raises((ValueError, TypeError)):
         dpt.gcd(dev(np.ones(3, dtype="f4")), dev(np.ones(3, dtype="f4")))
+
+
+# ---- mixed-dtype arithmetic: the cast of one operand is folded into the kernel -------------------
+@pytest.mark.parametrize("op", ["add", "subtract", "multiply", "divide"])
+@pytest.mark.parametrize("pair", [("f8", "f4"), ("f8", "i4"), ("f8", "i8"), ("f8", "?"), ("f4", "?")])
+def test_mixed_dtype_arithmetic_equals_cast_then_compute(op, pair):
+    import dpnp_amd._lib as L
+    from dpnp_amd.tensor._dtypes import dtype_id
+
+    rng = np.random.default_rng(151)
+    wide, narrow = pair
+    a = random_array(rng, (37, 130), wide, -9, 9)
+    b = random_array(rng, (37, 130), narrow, -9, 9)
+    if narrow != "?":
+        b[b == 0] = 1
+    assert L.lib.dpx_binary_fused_cast_result_type(L.BINARY_ID[op], dtype_id(np.dtype(wide)),
+                                                   dtype_id(np.dtype(narrow))) == dtype_id(np.dtype(wide))
+    for x, y in ((a, b), (b, a)):
+        with np.errstate(all="ignore"):
+            want = getattr(np, op if op != "divide" else "true_divide")(x.astype(wide), y.astype(wide))
+        assert_same(host(getattr(dpt, op)(dev(x), dev(y))), want)                       # contiguous
+        assert_same(host(getattr(dpt, op)(dev(x)[:, ::2], dev(y)[:, ::2])), want[:, ::2])  # strided
+        assert_same(host(getattr(dpt, op)(dev(x.T.copy()).T, dev(y))), want)            # transposed operand
+    # in place: the left operand has the result type
+    d = dev(a)
+    getattr(dpt, op)(d, dev(b), out=d)
+    with np.errstate(all="ignore"):
+        assert_same(host(d), getattr(np, op if op != "divide" else "true_divide")(a, b.astype(wide)))
+    d2 = dev(a)
+    if op == "add":
+        d2 += dev(b)
+        assert_same(host(d2), a + b.astype(wide))
