@@ -15,7 +15,8 @@
  *     caller keeps the device memory alive until the stream has passed the work;
  *   - `dst` is always allocated by the caller; the library allocates only
  *     scratch (partial results of multi-block reductions) from a grow-only,
- *     per-stream pool it owns;
+ *     per-stream pool it owns, and four 16 MiB pinned host buffers per device
+ *     for the host <-> device copies;
  *   - strides are in ELEMENTS (as usm_ndarray.strides), may be zero
  *     (broadcast) or negative; `data` points at the element with all indices 0;
  *   - a return value != DPX_OK leaves `dst` untouched (all validation happens
