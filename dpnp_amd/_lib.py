@@ -40,7 +40,8 @@ BINARY_OPS = [
     "fmax", "fmin", "fmod", "logaddexp2", "heaviside", "gcd", "lcm",
 ]
 REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot",
-              "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev"]
+              "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev",
+              "any", "all", "count_nonzero"]
 SEARCH_OPS = ["argmax", "argmin", "nanargmax", "nanargmin"]
 UNARY_ID = {n: i for i, n in enumerate(UNARY_OPS)}
 BINARY_ID = {n: i for i, n in enumerate(BINARY_OPS)}

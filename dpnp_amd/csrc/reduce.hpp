@@ -124,7 +124,9 @@ template <class In, class Out> DPX_D acc_of_t<Out> in_to_acc(In x)
 enum {
     K_SUM = 0, K_PROD = 1, K_MAX = 2, K_MIN = 3, K_SUMSQDEV = 4, K_LOGSUMEXP = 5, K_HYPOT = 6,
     // NaN-ignoring forms: a NaN element contributes the identity (0, 1, nothing, not counted)
-    K_NANSUM = 7, K_NANPROD = 8, K_NANMAX = 9, K_NANMIN = 10, K_NANCOUNT = 11, K_NANSUMSQDEV = 12
+    K_NANSUM = 7, K_NANPROD = 8, K_NANMAX = 9, K_NANMIN = 10, K_NANCOUNT = 11, K_NANSUMSQDEV = 12,
+    // truth-value reductions of any input type: an element counts as true when it is not zero
+    K_ANY = 13, K_ALL = 14, K_COUNT_NONZERO = 15
 };
 constexpr bool kind_is_minmax(int k) { return k == K_MAX || k == K_MIN || k == K_NANMAX || k == K_NANMIN; }
 
@@ -167,7 +169,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc identity()
     {
         if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
-        else if constexpr (is_bool_v<Out>) return KIND == K_PROD ? 1 : 0;
+        else if constexpr (is_bool_v<Out>) return (KIND == K_PROD || KIND == K_ALL) ? 1 : 0;
+        else if constexpr (KIND == K_COUNT_NONZERO) return Acc(0);
         else if constexpr (KIND == K_NANMAX || KIND == K_NANMIN) return (Acc)__builtin_nanf(""); // "nothing yet"
         else if constexpr (KIND == K_NANSUM || KIND == K_NANCOUNT || KIND == K_NANSUMSQDEV)
             return red_identity<K_SUM, Acc>();
@@ -187,6 +190,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         }
         else if constexpr (KIND == K_NANSUM || KIND == K_NANPROD) return isnan_(x) ? identity() : in_to_acc<In, Out>(x);
         else if constexpr (KIND == K_NANCOUNT) return isnan_(x) ? Acc(0) : Acc(1);
+        else if constexpr (KIND == K_ANY || KIND == K_ALL || KIND == K_COUNT_NONZERO)
+            return (Acc)convert<bool_t, In>(x).v;
         else if constexpr (kind_is_minmax(KIND)) {
             if constexpr (is_bool_v<Out>) return (int32_t)(x.v != 0);
             else return x; // In == Out
@@ -196,11 +201,11 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc combine(Acc a, Acc b)
     {
         if constexpr (is_bool_v<Out>) {
-            if constexpr (KIND == K_PROD || KIND == K_MIN) return a & b;
+            if constexpr (KIND == K_PROD || KIND == K_MIN || KIND == K_ALL) return a & b;
             else return a | b;
         }
         else if constexpr (KIND == K_SUM || KIND == K_SUMSQDEV || KIND == K_NANSUM || KIND == K_NANCOUNT ||
-                           KIND == K_NANSUMSQDEV)
+                           KIND == K_NANSUMSQDEV || KIND == K_COUNT_NONZERO)
             return a + b;
         else if constexpr (KIND == K_PROD || KIND == K_NANPROD) return a * b;
         else if constexpr (KIND == K_LOGSUMEXP) return LogaddexpOp::apply<Acc>(a, b);

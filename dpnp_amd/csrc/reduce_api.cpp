@@ -19,6 +19,9 @@ int nan_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, cons
 int nan_acc_size(int, const dpx_array_view *, const dpx_array_view *);
 int nanarg_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 
+bool truth_pair_supported(int, int, int);
+int truth_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
+static bool is_truth_op(int op) { return op == DPX_R_ANY || op == DPX_R_ALL || op == DPX_R_COUNT_NONZERO; }
 static bool is_nan_op(int op) { return op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV; }
 static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV; }
 
@@ -33,7 +36,9 @@ static bool reduce_supported(int op, int s, int d)
     case DPX_R_SUMSQDEV: return sqdev_pair_supported(s, d);
     case DPX_R_LOGSUMEXP:
     case DPX_R_HYPOT: return fpred_pair_supported(s, d);
-    default: return is_nan_op(op) && nan_pair_supported(op, s, d);
+    default:
+        if (is_truth_op(op)) return truth_pair_supported(op, s, d);
+        return is_nan_op(op) && nan_pair_supported(op, s, d);
     }
 }
 
@@ -57,11 +62,13 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
         if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
         if (is_nan_op(op)) acc = nan_acc_size(op, src, dst);
+        if (is_truth_op(op)) acc = op == DPX_R_COUNT_NONZERO ? 8 : 4;
         red_export_plan(pl, plan_out, acc);
         return DPX_OK;
     }
     hipStream_t s = (hipStream_t)stream;
     if (is_nan_op(op)) return nan_run(op, pl, src, dst, aux, s);
+    if (is_truth_op(op)) return truth_run(op, pl, src, dst, s);
     switch (op) {
     case DPX_R_SUM: return sum_run(pl, src, dst, s);
     case DPX_R_PROD: return prod_run(pl, src, dst, s);

@@ -169,40 +169,32 @@ def argmin(x, /, *, axis=None, keepdims=False, out=None):
 
 
 def _boolean_reduction(x, axis, keepdims, out, fn):
-    """all/any through max/min of the truth values (bool max is logical or, min is and)."""
-    from ._copy_utils import astype
+    """all / any of an array of any dtype in one pass (an element is true when it is not zero):
+    _boolean_reduction, dpnp/tensor/_utility_functions.py:31-85."""
     from ._dtypes import bool as _bool
 
     if not isinstance(x, usm_ndarray):
         raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
-    b = astype(x, _bool, copy=False)
-    nd = b.ndim
-    arr, axis, perm = _move_reduced_axes_last(b, axis)
+    nd = x.ndim
+    arr, axis, perm = _move_reduced_axes_last(x, axis)
     red_nd = len(axis)
     res_shape = arr.shape[: nd - red_nd]
-    n = 1
-    for i in range(nd - red_nd, nd):
-        n *= arr.shape[i]
-    out, user = _prepare_out(b, out, axis, keepdims, res_shape, _bool, guard_overlap=True)
+    out, user = _prepare_out(x, out, axis, keepdims, res_shape, _bool, guard_overlap=True)
     if red_nd == 0:
-        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=out)
+        ti._copy_usm_ndarray_into_usm_ndarray(src=arr, dst=out)  # a cast to bool
         return _finish(out, user, False, res_shape, red_nd, perm, nd)
-    if n == 0:
-        if out.size:
-            ti._full_usm_ndarray(fn is tri._min_over_axis, out)  # all([]) is True, any([]) is False
-    else:
-        fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)
+    fn(src=arr, trailing_dims_to_reduce=red_nd, dst=out)  # an empty run gives the identity
     return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
 
 
 def all(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
     """True where every element along `axis` is non-zero."""
-    return _boolean_reduction(x, axis, keepdims, out, tri._min_over_axis)
+    return _boolean_reduction(x, axis, keepdims, out, tri._all)
 
 
 def any(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
     """True where some element along `axis` is non-zero."""
-    return _boolean_reduction(x, axis, keepdims, out, tri._max_over_axis)
+    return _boolean_reduction(x, axis, keepdims, out, tri._any)
 
 
 def logsumexp(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
@@ -222,10 +214,7 @@ def reduce_hypot(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
 
 
 def count_nonzero(x, /, *, axis=None, keepdims=False, out=None):
-    """Number of non-zero elements over `axis` (int64)."""
-    from ._copy_utils import astype
-    from ._dtypes import bool as _bool
-
-    if not isinstance(x, usm_ndarray):
-        raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
-    return sum(astype(x, _bool, copy=False), axis=axis, dtype="i8", keepdims=keepdims, out=out)
+    """Number of non-zero elements over `axis` (int64), counted while reading `x` (the reference
+    casts to bool and sums, dpnp/tensor/_reduction.py:472-512)."""
+    return _reduction_over_axis(x, axis, "i8", keepdims, out, tri._count_nonzero_over_axis,
+                                tri._count_nonzero_over_axis_dtype_supported, lambda dt, q=None: dt)

@@ -38,6 +38,11 @@ _max_over_axis, _max_over_axis_dtype_supported = _make_reduction("max", _lib.RED
 _min_over_axis, _min_over_axis_dtype_supported = _make_reduction("min", _lib.REDUCE_ID["min"])
 _logsumexp_over_axis, _logsumexp_over_axis_dtype_supported = _make_reduction("logsumexp", _lib.REDUCE_ID["logsumexp"])
 _hypot_over_axis, _hypot_over_axis_dtype_supported = _make_reduction("hypot", _lib.REDUCE_ID["hypot"])
+# all / any of any dtype (tri._all, tri._any) and the one-pass count of non-zero elements
+_any, _any_dtype_supported = _make_reduction("any", _lib.REDUCE_ID["any"])
+_all, _all_dtype_supported = _make_reduction("all", _lib.REDUCE_ID["all"])
+_count_nonzero_over_axis, _count_nonzero_over_axis_dtype_supported = _make_reduction(
+    "count_nonzero", _lib.REDUCE_ID["count_nonzero"])
 _argmax_over_axis = _make_search("argmax", _lib.SEARCH_ID["argmax"])
 _argmin_over_axis = _make_search("argmin", _lib.SEARCH_ID["argmin"])
 

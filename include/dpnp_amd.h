@@ -216,6 +216,12 @@ typedef enum dpx_reduce_op {
     DPX_R_NANMIN,
     DPX_R_NANCOUNT,
     DPX_R_NANSUMSQDEV,
+    /* truth-value reductions of any input type (an element is true when it is not zero):
+     * ANY / ALL give bool (py_boolean_reduction, reduction_over_axis.hpp:1057-1303: tri._any,
+     * tri._all), COUNT_NONZERO gives int64 (dpnp/tensor/_reduction.py:472-512) */
+    DPX_R_ANY,
+    DPX_R_ALL,
+    DPX_R_COUNT_NONZERO,
     DPX_R_NUM_OPS
 } dpx_reduce_op;
 

@@ -440,3 +440,31 @@ def test_nan_functions_arguments_and_other_dtypes():
     assert_same(dpnp.nansum(e, axis=0).asnumpy(), np.zeros(3, dtype="f4"))
     with pytest.raises(ValueError):
         dpnp.nanmax(e, axis=0)
+
+
+@pytest.mark.parametrize("dt", [str(np.dtype(d)) for d in ALL])
+def test_all_any_count_nonzero_every_dtype_in_one_pass(dt):
+    rng = np.random.default_rng(241)
+    a = random_array(rng, (9, 70, 11), dt, -2, 2)
+    if np.dtype(dt).kind in "fc":
+        a[0, 0, 0] = np.nan                      # NaN is true
+    if np.dtype(dt).kind == "c":
+        a[1, 1, 1] = 1j                          # a non-zero imaginary part alone is true
+    a[:, 5, :] = 0                               # an all-false run along axis 1 ... not a full one
+    a[3] = 0
+    d = dev(a)
+    for axis in (None, 0, 1, 2, (0, 2), (1, 2)):
+        assert_same(host(dpt.all(d, axis=axis)), np.all(a, axis=axis))
+        assert_same(host(dpt.any(d, axis=axis)), np.any(a, axis=axis))
+        assert_same(host(dpt.count_nonzero(d, axis=axis)), np.asarray(np.count_nonzero(a, axis=axis), dtype="i8"))
+    v = d[::2, ::-3, 1:]
+    hv = a[::2, ::-3, 1:]
+    assert_same(host(dpt.any(v, axis=1, keepdims=True)), np.any(hv, axis=1, keepdims=True))
+    assert_same(host(dpt.count_nonzero(v, axis=(0, 1))), np.asarray(np.count_nonzero(hv, axis=(0, 1)), dtype="i8"))
+    e = dpt.empty((0, 4), dtype=dt)
+    assert_same(host(dpt.all(e, axis=0)), np.ones(4, dtype=bool))
+    assert_same(host(dpt.any(e, axis=0)), np.zeros(4, dtype=bool))
+    assert int(dpt.count_nonzero(e)) == 0
+    big = np.zeros(3_000_001, dtype=dt)
+    big[-1] = 1
+    assert bool(dpt.any(dev(big))) and not bool(dpt.all(dev(big))) and int(dpt.count_nonzero(dev(big))) == 1
