@@ -47,7 +47,13 @@ template <int N> struct InPtrs {
 
 template <class Out, class... Ins> struct ew_traits {
     static constexpr int width = max_sizeof<Out, Ins...>();
-    static constexpr int E = 16 / width; // elements per thread
+    static constexpr int E = 16 / width; // elements per pack: the widest operand moves 16 bytes
+    // Contiguous kernels: packs per thread.  A thread that moves 20 bytes or less per pack (a cast
+    // from a wide to a narrow type, a predicate) takes two.  Measured on MI355X over 1 GiB of
+    // input: f8 -> i1 0.224 -> 0.193 ms, isnan(f4) 0.227 -> 0.198 ms; at 24 bytes per pack
+    // (f4 -> f8) two packs are slower than one, 0.476 -> 0.521 ms.
+    static constexpr int pack_bytes = E * (int)(sizeof(Out) + (size_t(0) + ... + sizeof(Ins)));
+    static constexpr int U = pack_bytes <= 20 ? 2 : 1;
 };
 
 template <class T, int E> DPX_D pack<T, E> splat(T v)
@@ -59,50 +65,66 @@ template <class T, int E> DPX_D pack<T, E> splat(T v)
 }
 
 // ---- contiguous ---------------------------------------------------------------
-// grid.x * blockDim.x * E >= n.  bcast bit i set: input i is a single element.
-template <bool VEC, class Fn, class Out, class... Ins, size_t... I>
-DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
-                          const InPtrs<sizeof...(Ins)> &in, std::index_sequence<I...>)
+// grid.x * blockDim.x * E * U >= n.  bcast bit i set: input i is a single element.
+// Pack u of thread t in block b covers elements ((b * U + u) * blockDim.x + t) * E ... + E.
+template <class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_contig_pack(const Fn &fn, uint32_t bcast, Out *out, const InPtrs<sizeof...(Ins)> &in,
+                          int64_t base, std::tuple<pack<Ins, ew_traits<Out, Ins...>::E>...> &v,
+                          std::index_sequence<I...>)
 {
     constexpr int E = ew_traits<Out, Ins...>::E;
-    const int64_t block_base = (int64_t)blockIdx.x * ((int)blockDim.x * E);
-    if constexpr (VEC) {
-        const int64_t base = block_base + (int64_t)threadIdx.x * E;
+    (keep_whole(std::get<I>(v)), ...);
+    pack<Out, E> r;
+#pragma unroll
+    for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+    store_pack<Out, E>(out + base, r);
+}
+
+template <class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
+                          const InPtrs<sizeof...(Ins)> &in, std::index_sequence<I...> seq)
+{
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    constexpr int U = ew_traits<Out, Ins...>::U;
+    const int64_t block_base = (int64_t)blockIdx.x * ((int)blockDim.x * E * U);
+    auto load = [&](int64_t base, std::tuple<pack<Ins, E>...> &v) {
+        ((std::get<I>(v) = ((bcast >> I) & 1u)
+                               ? splat<Ins, E>(load_one((const Ins *)in.p[I]))
+                               : load_pack<Ins, E>((const Ins *)in.p[I] + base)),
+         ...);
+    };
+    if (block_base + (int64_t)blockDim.x * E * U <= n) { // the usual case: every load first
+        std::tuple<pack<Ins, E>...> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            load(block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E, v[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            ew_contig_pack<Fn, Out, Ins...>(fn, bcast, out, in,
+                                            block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E,
+                                            v[u], seq);
+        return;
+    }
+    for (int u = 0; u < U; ++u) { // the block that holds the end of the array
+        const int64_t base = block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E;
         if (base + E <= n) {
             std::tuple<pack<Ins, E>...> v;
-            ((std::get<I>(v) = ((bcast >> I) & 1u)
-                                   ? splat<Ins, E>(load_one((const Ins *)in.p[I]))
-                                   : load_pack<Ins, E>((const Ins *)in.p[I] + base)),
-             ...);
-            pack<Out, E> r;
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
-            store_pack<Out, E>(out + base, r);
+            load(base, v);
+            ew_contig_pack<Fn, Out, Ins...>(fn, bcast, out, in, base, v, seq);
         }
-        else {
+        else
             for (int64_t i = base; i < n; ++i)
                 out[i] = to_storage<Out>(fn(to_value(
                     load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
-        }
-    }
-    else {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            const int64_t i = block_base + e * (int)blockDim.x + threadIdx.x;
-            if (i < n)
-                out[i] = to_storage<Out>(fn(to_value(
-                    load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
-        }
     }
 }
 
-template <bool VEC, class Fn, class Out, class... Ins>
+template <class Fn, class Out, class... Ins>
 __global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, uint32_t bcast,
                                                             Out *out,
                                                             InPtrs<sizeof...(Ins)> in)
 {
-    ew_contig_body<VEC, Fn, Out, Ins...>(fn, n, bcast, out, in,
+    ew_contig_body<Fn, Out, Ins...>(fn, n, bcast, out, in,
                                          std::index_sequence_for<Ins...>{});
 }
 
@@ -230,6 +252,7 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     ((std::get<I>(v) = load_operand((const Ins *)in.p[I], off[I], ix.strides[I][inner],
                                     (modes >> (2 * I)) & 3u, (modes >> (MODE_KEEP_SHIFT + I)) & 1u)),
      ...);
+    (keep_whole(std::get<I>(v)), ...);
     pack<Out, E> r;
 #pragma unroll
     for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
@@ -337,12 +360,20 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         const T *base = p + off[k] + i0 + j0 * sj;
         if (((modes >> (2 * k)) & 3u) == MODE_VEC) {
             const int lv = threadIdx.x % VPR, lr = threadIdx.x / VPR;
-            const bool col_ok = lv * VE < ci; // shape[dT] is a multiple of VE: a pack is inside or outside
+            const bool col_ok = lv * VE < ci;
+            const bool whole = lv * VE + VE <= ci; // else: the pack that holds the end of dim dT
             pack<T, VE> m[PASSES];
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
                 const int r = q * RPP + lr;
-                if (col_ok && r < cj) m[q] = load_pack<T, VE>(base + r * sj + lv * VE);
+                if (col_ok && r < cj) {
+                    const T *src = base + r * sj + lv * VE;
+                    if (whole) m[q] = load_pack<T, VE>(src);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < VE; ++e) m[q].v[e] = load_one(src + ((lv * VE + e < ci) ? e : 0));
+                    }
+                }
             }
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
@@ -445,7 +476,8 @@ struct EwPlan {
 void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views);
 // fills the launch parameters for E elements per thread and the operands' item sizes
 // and (displaced) base pointers
-void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs);
+// (U: packs per thread of the contiguous kernel)
+void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *const *ptrs);
 
 // dry != 0: only fill the launch parameters of pl
 template <class Fn, class Out, class... Ins>
@@ -466,19 +498,14 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
             if (pl.tmask == 0) pl.path = DPX_PATH_EW_ROWS;
         }
     }
-    ew_finish_plan(pl, E, sizes, ptrs);
+    ew_finish_plan(pl, E, ew_traits<Out, Ins...>::U, sizes, ptrs);
     if (pl.path == DPX_PATH_NOOP || dry) return hipSuccess;
     InPtrs<N> in;
     for (int k = 0; k < N; ++k) in.p[k] = ptrs[k];
     Out *out = (Out *)ptrs[N];
     if (pl.path == DPX_PATH_EW_CONTIG) {
-        if (pl.vec)
-            hipLaunchKernelGGL((ew_contig_kernel<true, Fn, Out, Ins...>), dim3((unsigned)pl.grid),
-                               dim3(pl.block), 0, stream, fn, pl.n, pl.bcast, out, in);
-        else
-            hipLaunchKernelGGL((ew_contig_kernel<false, Fn, Out, Ins...>),
-                               dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, fn, pl.n,
-                               pl.bcast, out, in);
+        hipLaunchKernelGGL((ew_contig_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(pl.block), 0,
+                           stream, fn, pl.n, pl.bcast, out, in);
     }
     else {
         NdIndex<N + 1> ix;

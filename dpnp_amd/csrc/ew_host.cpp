@@ -109,20 +109,19 @@ static uint32_t keep_bits(const EwPlan &pl)
     return bits;
 }
 
-void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *ptrs)
+void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *const *ptrs)
 {
     if (pl.path == DPX_PATH_NOOP) return;
     const int nops = pl.nops;
-    auto aligned = [&](int k) { return ((uintptr_t)ptrs[k] % (uintptr_t)(E * itemsize[k])) == 0; };
+    (void)ptrs, (void)itemsize; // packs need no alignment: any operand whose inner stride is 1 is read in packs
     if (pl.path == DPX_PATH_EW_CONTIG) {
         pl.vec = true;
         pl.bcast = 0;
         for (int k = 0; k < nops; ++k) {
             if (k + 1 < nops && pl.strides[k][0] == 0 && pl.n > 1) pl.bcast |= 1u << k;
-            else pl.vec = pl.vec && aligned(k);
         }
         pl.block = env_block("DPX_EW_CONTIG_BLOCK", EW_CONTIG_BLOCK);
-        pl.grid = (pl.n + (int64_t)pl.block * E - 1) / ((int64_t)pl.block * E);
+        pl.grid = (pl.n + (int64_t)pl.block * E * U - 1) / ((int64_t)pl.block * E * U);
         return;
     }
     const int inner = pl.nd - 1;
@@ -133,16 +132,10 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         for (int k = 0; k < nops; ++k) {
             uint32_t mode = MODE_STRIDED;
             const bool staged = k + 1 < nops && ((pl.tmask >> k) & 1u);
-            // elements per 16-byte access of this operand and the dim those accesses run along
-            const int64_t ve = staged ? 16 / itemsize[k] : E;
+            // the dim this operand's 16-byte accesses run along
             const int run = staged ? pl.dT : inner;
             if (pl.strides[k][run] == 0 && !staged && k + 1 < nops) mode = MODE_BCAST;
-            else if (pl.strides[k][run] == 1 && ((uintptr_t)ptrs[k] % (uintptr_t)(ve * itemsize[k])) == 0 &&
-                     (!staged || pl.shape[run] % ve == 0)) {
-                mode = MODE_VEC;
-                for (int d = 0; d < pl.nd; ++d)
-                    if (d != run && pl.strides[k][d] % ve != 0) mode = MODE_STRIDED;
-            }
+            else if (pl.strides[k][run] == 1) mode = MODE_VEC;
             pl.modes |= mode << (2 * k);
         }
         pl.modes |= keep_bits(pl);
@@ -162,11 +155,8 @@ void ew_finish_plan(EwPlan &pl, int E, const int *itemsize, const void *const *p
         uint32_t mode = MODE_STRIDED;
         const int64_t s = pl.strides[k][inner];
         if (s == 0 && k + 1 < nops) mode = MODE_BCAST;
-        else if ((s == 1 || (s == 2 && E >= 2 && k + 1 < nops)) && aligned(k)) {
-            mode = s == 1 ? MODE_VEC : MODE_VEC2;
-            for (int d = 0; d < inner; ++d)
-                if (pl.strides[k][d] % E != 0) mode = MODE_STRIDED;
-        }
+        else if (s == 1) mode = MODE_VEC;
+        else if (s == 2 && E >= 2 && k + 1 < nops) mode = MODE_VEC2;
         pl.modes |= mode << (2 * k);
     }
     pl.modes |= keep_bits(pl);

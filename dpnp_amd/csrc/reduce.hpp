@@ -531,27 +531,43 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         if constexpr (P::has_aux) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (e < ecnt) a[e] = P::load_aux(aux + ao + (col0 + e) * ix.aux_str[last]);
+                if (e < ecnt && col0 + e < L.inner) a[e] = P::load_aux(aux + ao + (col0 + e) * ix.aux_str[last]);
         }
         const In *p = src + so + col0;
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         int64_t r = beg + ty;
         if (L.vec) {
-            for (; r + (U - 1) * TY < end; r += U * TY) {
-                pack<In, E> v[U];
+            // the pack that holds the end of a row is read element by element: its own copy of the
+            // loops, so the loads of the usual case stay free of branches
+            auto walk = [&](auto whole_tag) {
+                constexpr bool WHOLE = decltype(whole_tag)::value;
+                auto load = [&](const In *q) {
+                    if constexpr (WHOLE) return load_pack<In, E>(q);
+                    else {
+                        pack<In, E> t;
 #pragma unroll
-                for (int u = 0; u < U; ++u) v[u] = load_pack<In, E>(p + (r + u * TY) * L.rstride);
+                        for (int e = 0; e < E; ++e) t.v[e] = load_one(q + ((col0 + e < L.inner) ? e : 0));
+                        return t;
+                    }
+                };
+                for (; r + (U - 1) * TY < end; r += U * TY) {
+                    pack<In, E> v[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
+                    for (int u = 0; u < U; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                    for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], P::pre(v[u].v[e], a[e]));
-            }
-            for (; r < end; r += TY) {
-                pack<In, E> v = load_pack<In, E>(p + r * L.rstride);
+                    for (int u = 0; u < U; ++u)
 #pragma unroll
-                for (int e = 0; e < E; ++e) acc[0][e] = P::combine(acc[0][e], P::pre(v.v[e], a[e]));
-            }
+                        for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], P::pre(v[u].v[e], a[e]));
+                }
+                for (; r < end; r += TY) {
+                    pack<In, E> v = load(p + r * L.rstride);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[0][e] = P::combine(acc[0][e], P::pre(v.v[e], a[e]));
+                }
+            };
+            if (col0 + E <= L.inner) walk(std::true_type{});
+            else walk(std::false_type{});
         }
         else {
             for (; r + (U - 1) * TY < end; r += U * TY) {

@@ -147,7 +147,6 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
 
     const int E = 16 / in_size;
     const int64_t target = red_target_blocks();
-    const uintptr_t base = (uintptr_t)src->data + (uintptr_t)(pl.src_off * in_size);
     const int last = nd_i - 1;
     const int64_t inner = ishape[last];
     const bool contig_red = nd_r == 1 && (rstr[0][0] == 1 || n == 1);
@@ -156,9 +155,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
 
     if (!cols_ok) {
         // ---- rows / generic -------------------------------------------------------
-        bool vec = contig_red && (base % 16 == 0);
-        for (int d = 0; d < nd_i && vec; ++d)
-            if (ishape[d] > 1 && istr[0][d] % E != 0) vec = false;
+        const bool vec = contig_red; // packs need no alignment
         const int e = vec ? E : 1;
         L.vec = vec ? 1 : 0;
         rows_geometry(n, e, L.g_log2, pl.block);
@@ -189,9 +186,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
-    bool vec = !arg && (base % 16 == 0) && (inner % E == 0) && (rstride % E == 0);
-    for (int d = 0; d < last && vec; ++d)
-        if (ishape[d] > 1 && istr[0][d] % E != 0) vec = false;
+    const bool vec = !arg; // packs need no alignment; the kernel reads a row's last pack by element
     const int e = vec ? E : 1;
     L.vec = vec ? 1 : 0;
     L.rstride = rstride;

@@ -1,0 +1,111 @@
+"""Layouts whose rows or base pointers are aligned to the element only: rows of odd length, views that
+start at x[k:], transposed operands with odd extents.  The kernels read them with 16-byte accesses that
+start at any element; results must equal the oracle bit for bit (integers, IEEE basic ops) and every
+element outside the written view must keep its value."""
+import numpy as np
+import pytest
+
+import dpnp_amd.tensor as dpt
+from oracle import oracle as orc
+from tests.helpers import assert_same, dev, host, random_array
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_sum(a, axis):
+    if axis is None:
+        return orc.reduce("sum", a.reshape(-1), 1)
+    return orc.reduce("sum", np.moveaxis(a, axis, -1), 1)
+
+DTYPES = ["?", "i1", "u2", "f2", "i4", "f4", "i8", "f8", "c8", "c16"]
+ODD_SHAPES = [(37, 1001), (5, 4099), (1000, 3), (129, 17), (64, 1023), (3, 5, 257)]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_contiguous_with_offsets_and_guard_elements(dt):
+    rng = np.random.default_rng(3)
+    n = 9001
+    a, b = random_array(rng, n, dt), random_array(rng, n, dt)
+    op = (lambda x, y: dpt.logical_xor(x, y)) if dt == "?" else (lambda x, y: dpt.add(x, y))
+    ref = (lambda x, y: np.logical_xor(x, y)) if dt == "?" else (lambda x, y: x + y)
+    for ka, kb, ko in [(1, 0, 0), (0, 1, 3), (3, 2, 1), (5, 5, 5), (7, 1, 2)]:
+        m = n - 8
+        fill = random_array(rng, n, dt)
+        o = dev(fill)
+        r = op(dev(a)[ka:ka + m], dev(b)[kb:kb + m])
+        assert_same(host(r), ref(a[ka:ka + m], b[kb:kb + m]))
+        if dt == "?":
+            dpt.logical_xor(dev(a)[ka:ka + m], dev(b)[kb:kb + m], out=o[ko:ko + m])
+        else:
+            dpt.add(dev(a)[ka:ka + m], dev(b)[kb:kb + m], out=o[ko:ko + m])
+        want = fill.copy()
+        want[ko:ko + m] = ref(a[ka:ka + m], b[kb:kb + m])
+        assert_same(host(o), want)
+
+
+@pytest.mark.parametrize("src", ["i1", "f2", "i4", "f8"])
+@pytest.mark.parametrize("dst", ["?", "u1", "i2", "f4", "f8", "c16"])
+def test_casts_between_widths_at_offsets(src, dst):
+    # the narrow side of a cast moves fewer than 16 bytes per pack; several packs per thread
+    rng = np.random.default_rng(5)
+    for n in (1, 63, 64, 127, 1000, 4096, 16384 + 3, 70001):
+        a = random_array(rng, n + 3, src, lo=0)
+        for k in (0, 1, 3):
+            v = dev(a)[k:k + n]
+            assert_same(host(dpt.astype(v, dst)), orc.cast(a[k:k + n], dst))
+    for n in (255, 8192, 50001):  # predicates: wide in, one byte out
+        a = random_array(rng, n, src)
+        assert_same(host(dpt.less(dev(a), dev(a[::-1].copy()))), a < a[::-1])
+
+
+@pytest.mark.parametrize("dt", ["i1", "f2", "f4", "f8", "c16"])
+@pytest.mark.parametrize("shape", ODD_SHAPES)
+def test_rows_of_odd_length(dt, shape):
+    rng = np.random.default_rng(7)
+    a, b = random_array(rng, shape, dt), random_array(rng, shape, dt)
+    da, db = dev(a), dev(b)
+    inner = shape[-1]
+    # slices along the last dim make every row start at another alignment
+    if inner > 4:
+        sl = (Ellipsis, slice(1, inner - 1))
+        assert_same(host(dpt.add(da[sl], db[sl])), a[sl] + b[sl])
+        fill = random_array(rng, shape, dt)
+        o = dev(fill)
+        dpt.subtract(da[sl], db[sl], out=o[sl])
+        want = fill.copy()
+        want[sl] = a[sl] - b[sl]
+        assert_same(host(o), want)
+        # stride 2 along the inner dim
+        s2 = (Ellipsis, slice(1, None, 2))
+        assert_same(host(dpt.add(da[s2], db[s2])), a[s2] + b[s2])
+    row = random_array(rng, (1,) * (len(shape) - 1) + (inner,), dt)
+    col = random_array(rng, shape[:-1] + (1,), dt)
+    assert_same(host(dpt.add(da, dev(row))), a + row)
+    assert_same(host(dpt.add(da, dev(col))), a + col)
+    if len(shape) == 2:
+        assert_same(host(dpt.add(da.mT, db.mT)), a.T + b.T)
+        assert_same(host(dpt.add(da.mT, dev(np.ascontiguousarray(b.T)))), a.T + b.T)
+        assert_same(host(dpt.copy(da.mT, order="C")), np.ascontiguousarray(a.T))
+        assert_same(host(dpt.where(da.mT != db.mT, da.mT, dev(np.ascontiguousarray(b.T)))), np.where(a.T != b.T, a.T, b.T))
+
+
+@pytest.mark.parametrize("dt", ["i1", "u2", "i4", "f4", "f8"])
+@pytest.mark.parametrize("shape", ODD_SHAPES + [(4097, 33), (2, 100003)])
+def test_reductions_over_odd_shapes_and_offsets(dt, shape):
+    rng = np.random.default_rng(11)
+    a = random_array(rng, shape, dt, lo=-5, hi=5)
+    da = dev(a)
+    for axis in list(range(len(shape))) + [None]:
+        assert_same(host(dpt.max(da, axis=axis)), np.max(a, axis=axis))
+        assert_same(host(dpt.argmin(da, axis=axis)), np.argmin(a, axis=axis))
+        got = host(dpt.sum(da, axis=axis))
+        if np.dtype(dt).kind == "f":
+            np.testing.assert_allclose(got, oracle_sum(a, axis), rtol=1e-5 if dt == "f4" else 1e-12, atol=1e-4 if dt == "f4" else 1e-10)
+        else:
+            assert_same(got, oracle_sum(a, axis))
+    if shape[-1] > 4:
+        sl = (Ellipsis, slice(1, shape[-1] - 2))
+        for axis in range(len(shape)):
+            assert_same(host(dpt.min(da[sl], axis=axis)), np.min(a[sl], axis=axis))
+            assert_same(host(dpt.argmax(da[sl], axis=axis)), np.argmax(a[sl], axis=axis))
+            assert_same(host(dpt.count_nonzero(da[sl], axis=axis)), np.count_nonzero(a[sl], axis=axis).astype(np.int64))
