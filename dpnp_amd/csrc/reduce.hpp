@@ -470,6 +470,7 @@ template <class In> struct cols_cfg {
 template <class P, int E> DPX_D void cols_block_combine(typename P::Acc (&v)[E], typename P::Acc *sm, int tx, int ty,
                                                         int TX, int TY)
 {
+    if (TY == 1) return;
     __syncthreads(); // sm may still be read by a previous call
 #pragma unroll
     for (int e = 0; e < E; ++e) sm[threadIdx.x * E + e] = v[e];
@@ -823,24 +824,29 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
     if (threadIdx.x == 0) dst[dof] = bidx;
 }
 
-// Column variant (reduced axis strided by L.rstride, outputs contiguous).  One column per
-// thread, 256 threads per block; partials laid out [split][output].
+// Column variant (reduced axis strided by L.rstride, outputs contiguous).  A thread owns the E
+// adjacent columns of one 16-byte pack and walks down the reduced axis, TY thread rows apart;
+// 256 threads per block; partials laid out [split][output].  Positions inside a chunk are kept
+// in 32 bits (the host keeps chunks below 2^32 rows).
 template <class T, bool IS_MAX>
 __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst,
                                                       Slot<T> *pval, Slot<int64_t> *pidx, unsigned *counters)
 {
     using VT = value_of_t<T>;
-    __shared__ VT smv[256];
-    __shared__ int64_t smi[256];
-    const int TX = 1 << L.g_log2, TY = 256 >> L.g_log2;
+    constexpr int E = 16 / (int)sizeof(T);
+    constexpr int U = E >= 8 ? 2 : 4; // rows in flight per thread
+    __shared__ VT smv[256 * E];
+    __shared__ int64_t smi[256 * E];
+    const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
     const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> L.g_log2;
     int64_t b = blockIdx.x;
     const int64_t cb = b % L.col_blocks;
     b /= L.col_blocks;
     const int split = (int)(b % L.splits);
     const int64_t outer = b / L.splits;
-    const int64_t col = cb * TX + tx;
-    const bool active = col < L.inner;
+    const int64_t col0 = (cb * TX + tx) * E;
+    const bool active = col0 < L.inner;
+    const bool whole = col0 + E <= L.inner;
     int64_t so = 0, dof = 0;
     {
         int64_t o = outer;
@@ -852,63 +858,132 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
             o = q;
         }
     }
-    VT best{};
-    int64_t bidx = ARG_NONE;
+    VT best[E];
+    int64_t bidx[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        best[e] = VT{};
+        bidx[e] = ARG_NONE;
+    }
     if (active) {
-        const T *p = src + so + col;
+        const T *p = src + so + col0;
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         int64_t r = beg + ty;
-        for (; r + (RED_U - 1) * TY < end; r += RED_U * TY) {
-            T v[RED_U];
+        uint32_t bl[E];
+        const bool have = r < end;
+        // the pack that holds the end of a row is read element by element, in its own copy of the loops
+        auto walk = [&](auto whole_tag) {
+            constexpr bool WHOLE = decltype(whole_tag)::value;
+            auto load = [&](const T *q) {
+                if constexpr (WHOLE) return load_pack<T, E>(q);
+                else {
+                    pack<T, E> t;
 #pragma unroll
-            for (int u = 0; u < RED_U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
+                    for (int e = 0; e < E; ++e) t.v[e] = load_one(q + ((col0 + e < L.inner) ? e : 0));
+                    return t;
+                }
+            };
+            auto take = [&](const pack<T, E> &v, int64_t row) {
 #pragma unroll
-            for (int u = 0; u < RED_U; ++u) {
-                const VT x = to_value(v[u]);
-                if (bidx == ARG_NONE || arg_better<IS_MAX, VT>(x, best)) {
-                    best = x;
-                    bidx = r + u * TY;
+                for (int e = 0; e < E; ++e) {
+                    const VT x = to_value(v.v[e]);
+                    if (arg_better<IS_MAX, VT>(x, best[e])) {
+                        best[e] = x;
+                        bl[e] = (uint32_t)(row - beg);
+                    }
+                }
+            };
+            if (have) { // the first row seeds the running extremum (and is then visited once more)
+                const pack<T, E> v = load(p + r * L.rstride);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    best[e] = to_value(v.v[e]);
+                    bl[e] = (uint32_t)(r - beg);
                 }
             }
-        }
-        for (; r < end; r += TY) {
-            const VT x = to_value(load_one(p + r * L.rstride));
-            if (bidx == ARG_NONE || arg_better<IS_MAX, VT>(x, best)) {
-                best = x;
-                bidx = r;
+            for (; r + (U - 1) * TY < end; r += U * TY) {
+                pack<T, E> v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+#pragma unroll
+                for (int u = 0; u < U; ++u) take(v[u], r + u * TY);
             }
+            for (; r < end; r += TY) take(load(p + r * L.rstride), r);
+        };
+        if (whole) walk(std::true_type{});
+        else walk(std::false_type{});
+        if (have) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) bidx[e] = beg + bl[e];
         }
     }
     auto combine_rows = [&]() {
+        if (TY == 1) return;
         __syncthreads();
-        smv[threadIdx.x] = best;
-        smi[threadIdx.x] = bidx;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            smv[threadIdx.x * E + e] = best[e];
+            smi[threadIdx.x * E + e] = bidx[e];
+        }
         __syncthreads();
         if (ty == 0)
-            for (int y = 1; y < TY; ++y) arg_merge<IS_MAX, VT>(best, bidx, smv[y * TX + tx], smi[y * TX + tx]);
+            for (int y = 1; y < TY; ++y) {
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    arg_merge<IS_MAX, VT>(best[e], bidx[e], smv[(y * TX + tx) * E + e], smi[(y * TX + tx) * E + e]);
+            }
+    };
+    auto write_out = [&]() {
+        const int last = ix.nd_i - 1;
+        int64_t *q = dst + dof + col0 * ix.dst_str[last];
+        if constexpr (E >= 2) {
+            if (whole && ix.dst_str[last] == 1) {
+#pragma unroll
+                for (int e = 0; e < E; e += 2) {
+                    pack<int64_t, 2> t;
+                    t.v[0] = bidx[e];
+                    t.v[1] = bidx[e + 1];
+                    store_pack<int64_t, 2>(q + e, t);
+                }
+                return;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (col0 + e < L.inner) q[e * ix.dst_str[last]] = bidx[e];
     };
     combine_rows();
-    const int last = ix.nd_i - 1;
-    const int64_t out = outer * L.inner + col;
+    const int64_t out0 = outer * L.inner + col0;
     if (L.splits == 1) {
-        if (ty == 0 && active) dst[dof + col * ix.dst_str[last]] = bidx;
+        if (ty == 0 && active) write_out();
         return;
     }
     uint32_t zero = 0;
     if (ty == 0 && active) {
-        zero = slot_publish(pval + (int64_t)split * L.m + out, to_storage<T>(best));
-        zero |= slot_publish(pidx + (int64_t)split * L.m + out, bidx);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (col0 + e < L.inner) {
+                zero |= slot_publish(pval + (int64_t)split * L.m + out0 + e, to_storage<T>(best[e]));
+                zero |= slot_publish(pidx + (int64_t)split * L.m + out0 + e, bidx[e]);
+            }
     }
     if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
-    best = VT{};
-    bidx = ARG_NONE;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        best[e] = VT{};
+        bidx[e] = ARG_NONE;
+    }
     if (active)
-        for (int sidx = ty; sidx < L.splits; sidx += TY)
-            arg_merge<IS_MAX, VT>(best, bidx, to_value(slot_read(pval + (int64_t)sidx * L.m + out)),
-                                  slot_read(pidx + (int64_t)sidx * L.m + out));
+        for (int sidx = ty; sidx < L.splits; sidx += TY) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (col0 + e < L.inner)
+                    arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(slot_read(pval + (int64_t)sidx * L.m + out0 + e)),
+                                          slot_read(pidx + (int64_t)sidx * L.m + out0 + e));
+        }
     combine_rows();
-    if (ty == 0 && active) dst[dof + col * ix.dst_str[last]] = bidx;
+    if (ty == 0 && active) write_out();
 }
 
 } // namespace dpx

@@ -92,7 +92,7 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         pval = (Slot<T> *)(s + RED_COUNTER_BYTES + (size_t)pl.scratch_elems * sizeof(Slot<int64_t>));
     }
     if (red_is_cols(pl))
-        hipLaunchKernelGGL((arg_cols_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(256), 0, stream, pl.ix, pl.L,
+        hipLaunchKernelGGL((arg_cols_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.ix, pl.L,
                            sp, dp, pval, pidx, counters);
     else if (pl.path == DPX_PATH_RED_GENERIC)
         hipLaunchKernelGGL((arg_rows_kernel<T, IS_MAX, false>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,

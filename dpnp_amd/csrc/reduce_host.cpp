@@ -186,26 +186,27 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
-    const bool vec = !arg; // packs need no alignment; the kernel reads a row's last pack by element
-    const int e = vec ? E : 1;
+    const bool vec = true; // packs need no alignment; the kernels read a row's last pack by element
+    const int e = E;
     L.vec = vec ? 1 : 0;
     L.rstride = rstride;
     L.inner = inner;
     // TX threads side by side cover 512 contiguous bytes of a row (32 x 16 B); up to 16 thread
     // rows walk down the reduced axis: 512-thread blocks, one per CU when splitting
-    int lg = std::min(arg ? 6 : 5, ceil_log2(cdiv(inner, e)));
+    // thread rows wanted for n reduced rows (4 or more rows per thread)
+    const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
+    // with a single thread row a whole wave lies side by side and nothing is combined in LDS
+    int lg = std::min(ty == 1 ? 6 : 5, ceil_log2(cdiv(inner, e)));
     const int forced = env_int("DPX_COLS_TX_LOG2", -1); // experiment knob
     if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(inner, e)), forced);
     L.g_log2 = lg;
     const int64_t TX = (int64_t)1 << lg;
-    int block = 256;
+    int block = (int)std::min<int64_t>(arg ? 256 : 512, std::max<int64_t>(64, TX * ty));
     if (!arg) {
-        int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
-        block = (int)std::min<int64_t>(512, std::max<int64_t>(64, TX * ty));
         const int fb = env_int("DPX_COLS_BLOCK", 0); // experiment knob
         if (fb == 256 || fb == 512 || fb == 1024) block = fb;
-        if (block < TX) block = (int)TX;
     }
+    if (block < TX) block = (int)TX;
     const int64_t TY = block / TX;
     L.col_blocks = cdiv(inner, TX * e);
     const int64_t outer = m / inner;
@@ -214,6 +215,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     int64_t splits = 1;
     if (base_blocks < want && base_blocks <= RED_MAX_TICKETS && n >= 2 * TY * 8)
         splits = std::min(cdiv(want, base_blocks), cdiv(n, TY * 8));
+    if (arg) splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
     int64_t chunk = cdiv(n, splits);
     splits = cdiv(n, chunk);
     L.chunk = chunk;
