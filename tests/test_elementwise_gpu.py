@@ -173,6 +173,35 @@ def test_unary_transcendentals_within_4_ulp(op):
             np.testing.assert_array_equal(np.signbit(got), np.signbit(want(x)))
 
 
+def test_log_float64_every_binade_within_1_ulp():
+    # log of a double is evaluated by the library's own routine (argument reduction + polynomial):
+    # dense check against an 80-bit evaluation, all binades including subnormals, and around 1
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("needs an extended-precision long double")
+    rng = np.random.default_rng(17)
+    n = 1 << 20
+    mant = rng.uniform(0.5, 1.0, n)
+    a = np.concatenate([
+        np.ldexp(mant, rng.integers(-1073, 1025, n)),          # every binade
+        1.0 + rng.uniform(-1e-3, 1e-3, n),                      # cancellation around 1
+        1.0 + np.ldexp(rng.uniform(-1, 1, n), rng.integers(-52, -8, n)),
+        rng.uniform(0.5, 2.0, n),                               # both sides of the sqrt(1/2) split
+        np.array([np.finfo("f8").max, np.finfo("f8").tiny, 5e-324, 1.0, 0.70710678118654746, 0.70710678118654757]),
+    ])
+    a = a[a > 0]
+    got = host(dpt.log(dev(a)))
+    assert_ulp(got, np.log(a.astype(np.longdouble)), 1.0)
+    x = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, -1.0, -5e-324])
+    with np.errstate(all="ignore"):
+        want = np.log(x)
+    got = host(dpt.log(dev(x)))
+    np.testing.assert_array_equal(got, want)
+    # the same routine behind logaddexp, the complex logarithm and logsumexp
+    b = rng.uniform(-700, 700, 4096)
+    c = rng.uniform(-700, 700, 4096)
+    assert_ulp(host(dpt.logaddexp(dev(b), dev(c))), np.logaddexp(b.astype(np.longdouble), c.astype(np.longdouble)), 2.0)
+
+
 def test_exp_known_answers():
     # dpnp/tests/tensor/elementwise/test_exp.py:111-120
     for dt in ("f2", "f4", "f8"):
