@@ -73,6 +73,13 @@ def check_limitations(**kwargs):
                                       f"but got {v}.")
 
 
+def _check_creation_subok(subok):
+    """Array creation functions take `subok` only at its default (dpnp/dpnp_iface.py:196-236)."""
+    if subok is not False:
+        raise NotImplementedError(f"Keyword argument `subok` is supported only with default value ``False``, "
+                                  f"but got {subok}.")
+
+
 def get_result_array(a, out=None, casting="safe"):
     """`out` filled with `a` (cast by `casting`), or `a` wrapped when there is no `out`."""
     if out is None:
@@ -97,7 +104,7 @@ def _wrap(u):
 
 def array(a, dtype=None, *, copy=True, order="K", subok=False, ndmin=0, like=None, device=None,
           usm_type=None, sycl_queue=None):
-    check_limitations(subok=True if not subok else subok)
+    _check_creation_subok(subok)
     src = a.get_array() if isinstance(a, dpnp_array) else a
     r = dpt.asarray(src, dtype=dtype, copy=True if copy else None, order=order)
     if ndmin > r.ndim:
@@ -108,6 +115,34 @@ def array(a, dtype=None, *, copy=True, order="K", subok=False, ndmin=0, like=Non
 def asarray(a, dtype=None, order=None, *, device=None, usm_type=None, sycl_queue=None, copy=None, like=None):
     src = a.get_array() if isinstance(a, dpnp_array) else a
     return _wrap(dpt.asarray(src, dtype=dtype, copy=copy, order=order or "K"))
+
+
+def asanyarray(a, dtype=None, order=None, *, like=None, device=None, usm_type=None, sycl_queue=None):
+    # dpnp/dpnp_iface_arraycreation.py:422-520
+    check_limitations(like=like)
+    return asarray(a, dtype=dtype, order=order)
+
+
+def ascontiguousarray(a, dtype=None, *, like=None, device=None, usm_type=None, sycl_queue=None):
+    # dpnp/dpnp_iface_arraycreation.py:648-763: C order, at least one dimension
+    check_limitations(like=like)
+    r = asarray(a, dtype=dtype, order="C")
+    return reshape(r, (1,)) if r.ndim == 0 else r
+
+
+def asfortranarray(a, dtype=None, *, like=None, device=None, usm_type=None, sycl_queue=None):
+    # dpnp/dpnp_iface_arraycreation.py:766-880: Fortran order, at least one dimension
+    check_limitations(like=like)
+    r = asarray(a, dtype=dtype, order="F")
+    return reshape(r, (1,)) if r.ndim == 0 else r
+
+
+def copy(a, order="K", subok=False, device=None, usm_type=None, sycl_queue=None):
+    # dpnp/dpnp_iface_arraycreation.py:977-1070: always a new array
+    _check_creation_subok(subok)
+    if isinstance(a, (dpnp_array, usm_ndarray)):
+        return _wrap(dpt.copy(get_usm_ndarray(a), order=order or "K"))
+    return array(a, order=order, copy=True)
 
 
 def asnumpy(a, order="C"):
@@ -135,6 +170,7 @@ def full(shape, fill_value, *, dtype=None, order="C", like=None, device=None, us
 
 def empty_like(a, /, *, dtype=None, order="C", subok=False, shape=None, device=None, usm_type=None,
                sycl_queue=None):
+    _check_creation_subok(subok)
     u = get_usm_ndarray(a)
     if shape is not None:
         return _wrap(dpt.empty(shape, dtype=dtype or u.dtype, order="C" if order in ("K", "A") else order))
@@ -152,6 +188,29 @@ def ones_like(a, /, *, dtype=None, order="C", subok=False, shape=None, device=No
               sycl_queue=None):
     r = empty_like(a, dtype=dtype, order=order, shape=shape)
     r.fill(1)
+    return r
+
+
+def full_like(a, /, fill_value, *, dtype=None, order="K", subok=False, shape=None, device=None, usm_type=None,
+              sycl_queue=None):
+    _check_creation_subok(subok)
+    # dpnp/dpnp_iface_arraycreation.py:2426-2530
+    r = empty_like(a, dtype=dtype, order=order, shape=shape)
+    r.fill(fill_value.get_array() if isinstance(fill_value, dpnp_array) else fill_value)
+    return r
+
+
+def linspace(start, stop, /, num, *, dtype=None, device=None, usm_type=None, sycl_queue=None, endpoint=True,
+             retstep=False, axis=0):
+    # dpnp/dpnp_iface_arraycreation.py:2789-2900, scalar end points (the tensor-level constructor)
+    if not (isscalar(start) and isscalar(stop)):
+        raise NotImplementedError("linspace: only scalar start and stop are supported")
+    if axis != 0:
+        raise NotImplementedError("linspace: axis must be 0 for scalar end points")
+    r = _wrap(dpt.linspace(start, stop, num, dtype=dtype, endpoint=endpoint))
+    if retstep:
+        div = (num - 1) if endpoint else num
+        return r, ((stop - start) / div if div > 0 else float("nan"))
     return r
 
 

@@ -243,3 +243,39 @@ def test_transfer_entry_points_through_the_c_abi():
     assert L.lib.dpx_copy_to_host(out.ctypes.data, buf.data_ptr(), 0, stream) == 0
     assert L.lib.dpx_copy_from_host(None, h.ctypes.data, 8, stream) != 0  # null pointer: an error, no crash
     assert b"null" in L.lib.dpx_last_error()
+
+
+def test_copy_and_layout_constructors():
+    # dpnp/tests/test_arraycreation.py: copy / ascontiguousarray / asfortranarray / asanyarray / full_like / linspace
+    rng = np.random.default_rng(5)
+    a = rng.normal(size=(37, 53)).astype("f4")
+    d = dpnp.asarray(a)
+    for order in ("C", "F", "K", "A"):
+        c = dpnp.copy(d.T, order=order)
+        want = np.copy(a.T, order=order)
+        np.testing.assert_array_equal(c.asnumpy(), want)
+        assert c.flags.c_contiguous == want.flags.c_contiguous and c.flags.f_contiguous == want.flags.f_contiguous
+        assert c.get_array()._buf is not d.get_array()._buf
+    c = dpnp.copy([[1, 2], [3, 4]])
+    np.testing.assert_array_equal(c.asnumpy(), [[1, 2], [3, 4]])
+    cc = dpnp.ascontiguousarray(d.T)
+    assert cc.flags.c_contiguous and cc.shape == (53, 37)
+    np.testing.assert_array_equal(cc.asnumpy(), a.T)
+    assert dpnp.ascontiguousarray(d).get_array()._buf is d.get_array()._buf  # already C: no copy
+    ff = dpnp.asfortranarray(d, dtype="f8")
+    assert ff.flags.f_contiguous and ff.dtype == np.float64
+    np.testing.assert_array_equal(ff.asnumpy(), a.astype("f8"))
+    assert dpnp.ascontiguousarray(3.5).shape == (1,) and dpnp.asfortranarray(2).shape == (1,)
+    assert dpnp.asanyarray(d) is d or dpnp.asanyarray(d).get_array()._buf is d.get_array()._buf
+    np.testing.assert_array_equal(dpnp.asanyarray([1, 2, 3], dtype="i2").asnumpy(), np.array([1, 2, 3], "i2"))
+    f = dpnp.full_like(d, 7, dtype="i4")
+    assert f.shape == d.shape and f.dtype == np.int32 and (f.asnumpy() == 7).all()
+    f = dpnp.full_like(d, 2.5, shape=(3, 2))
+    assert f.shape == (3, 2) and f.dtype == np.float32 and (f.asnumpy() == 2.5).all()
+    for num, endpoint in ((11, True), (10, False), (1, True)):
+        r = dpnp.linspace(0, 5, num, endpoint=endpoint)
+        np.testing.assert_allclose(r.asnumpy(), np.linspace(0, 5, num, endpoint=endpoint), rtol=1e-15)
+    r, step = dpnp.linspace(1, 2, 5, dtype="f4", retstep=True)
+    assert r.dtype == np.float32 and step == 0.25
+    with pytest.raises(NotImplementedError):
+        dpnp.copy(d, subok=True)
