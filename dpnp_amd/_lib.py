@@ -111,6 +111,9 @@ SIGNATURES = {
     "dpx_divide_by_scalar": (_i, [_VP, _d, _VP, _vp]),
     "dpx_nan_to_num": (_i, [_VP, _d, _d, _d, _VP, _vp]),
     "dpx_isclose": (_i, [_VP, _VP, _d, _d, _i, _VP, _vp]),
+    "dpx_ldexp_result_type": (_i, [_i, _i]),
+    "dpx_ldexp": (_i, [_VP, _VP, _VP, _vp]),
+    "dpx_frexp": (_i, [_VP, _VP, _VP, _vp]),
     "dpx_copy_cast": (_i, [_VP, _VP, _vp]),
     "dpx_copy_from_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
     "dpx_copy_to_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),

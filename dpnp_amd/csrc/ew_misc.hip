@@ -213,6 +213,98 @@ static int isclose_call(const dpx_array_view *a, const dpx_array_view *b, double
     }
 }
 
+// ---- ldexp: dpnp/backend/kernels/elementwise_functions/ldexp.hpp:39-58 -------------------------------
+// x1 * 2^x2; an exponent outside the int range gives +inf when positive and 0 otherwise, whatever x1 is
+// (as the reference's functor does).
+template <class T, class I> struct LdexpFn {
+    DPX_D V<T> operator()(V<T> x, I n) const
+    {
+        if ((I)(int)n == n) {
+            if constexpr (std::is_same_v<V<T>, double>) return ::ldexp(x, (int)n);
+            else return ::ldexpf(x, (int)n);
+        }
+        if (n > 0) return (V<T>)__builtin_inff();
+        return V<T>(0);
+    }
+};
+
+static int ldexp_call(const dpx_array_view *a, const dpx_array_view *b, const dpx_array_view *dst, void *stream)
+{
+    if (!view_ok(a) || !view_ok(b) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (dpx_ldexp_result_type(a->dtype, b->dtype) < 0)
+        return fail(DPX_ERR_BAD_DTYPE, "ldexp: needs a floating first and a signed integer second operand");
+    if (dst->dtype != a->dtype) return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    const dpx_array_view *views[3] = {a, b, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(3, views, n)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    auto with_int = [&](auto ft) {
+        using T = typename decltype(ft)::type;
+        switch (b->dtype) {
+        case DPX_INT8: rc = run_ew<LdexpFn<T, int8_t>, T, T, int8_t>({}, views, s, nullptr); break;
+        case DPX_INT16: rc = run_ew<LdexpFn<T, int16_t>, T, T, int16_t>({}, views, s, nullptr); break;
+        case DPX_INT32: rc = run_ew<LdexpFn<T, int32_t>, T, T, int32_t>({}, views, s, nullptr); break;
+        case DPX_INT64: rc = run_ew<LdexpFn<T, int64_t>, T, T, int64_t>({}, views, s, nullptr); break;
+        default: break;
+        }
+    };
+    switch (a->dtype) {
+    case DPX_HALF: with_int(tag<half_t>{}); break;
+    case DPX_FLOAT: with_int(tag<float>{}); break;
+    case DPX_DOUBLE: with_int(tag<double>{}); break;
+    default: break;
+    }
+    return rc;
+}
+
+// ---- frexp: dpnp/backend/kernels/elementwise_functions/frexp.hpp:36-56 ------------------------------
+// x = mantissa * 2^exponent with |mantissa| in [0.5, 1); zeros, infinities and NaN come back
+// unchanged with exponent 0.  PART 0: the mantissa (type of x), PART 1: the exponent (int32).
+template <class T, int PART> struct FrexpFn {
+    DPX_D auto operator()(V<T> x) const
+    {
+        constexpr bool dbl = std::is_same_v<V<T>, double>;
+        if constexpr (PART == 0) {
+            if constexpr (dbl) return __builtin_amdgcn_frexp_mant(x);
+            else return __builtin_amdgcn_frexp_mantf(x);
+        }
+        else {
+            const bool special = !(x == x) || m_isinf(x) || x == V<T>(0);
+            int32_t e;
+            if constexpr (dbl) e = __builtin_amdgcn_frexp_exp(x);
+            else e = __builtin_amdgcn_frexp_expf(x);
+            return special ? (int32_t)0 : e;
+        }
+    }
+};
+
+static int frexp_call(const dpx_array_view *x, const dpx_array_view *mant, const dpx_array_view *ex, void *stream)
+{
+    if (!view_ok(x) || !view_ok(mant) || !view_ok(ex)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (x->dtype != DPX_HALF && x->dtype != DPX_FLOAT && x->dtype != DPX_DOUBLE)
+        return fail(DPX_ERR_BAD_DTYPE, "frexp: only floating types");
+    if (mant->dtype != x->dtype || ex->dtype != DPX_INT32)
+        return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    if (views_overlap(mant, ex)) return fail(DPX_ERR_OVERLAP, "frexp: the two outputs overlap");
+    const dpx_array_view *v1[2] = {x, mant}, *v2[2] = {x, ex};
+    int64_t n = 0;
+    if (int rc = ew_validate(2, v2, n)) return rc; // before anything is written
+    if (int rc = ew_validate(2, v1, n)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    auto both = [&](auto ft) {
+        using T = typename decltype(ft)::type;
+        // the exponent first: x may be the mantissa's destination
+        if (int rc = run_ew<FrexpFn<T, 1>, int32_t, T>({}, v2, s, nullptr)) return rc;
+        return run_ew<FrexpFn<T, 0>, T, T>({}, v1, s, nullptr);
+    };
+    switch (x->dtype) {
+    case DPX_HALF: return both(tag<half_t>{});
+    case DPX_FLOAT: return both(tag<float>{});
+    default: return both(tag<double>{});
+    }
+}
+
 // ---- fill ----------------------------------------------------------------------------------------------
 template <class T> struct FillFn {
     T v;
@@ -330,6 +422,20 @@ int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol, d
                 const dpx_array_view *dst, void *stream)
 {
     return isclose_call(a, b, rtol, atol, equal_nan, dst, stream);
+}
+int dpx_ldexp_result_type(int dt1, int dt2)
+{
+    const bool fp = dt1 == DPX_HALF || dt1 == DPX_FLOAT || dt1 == DPX_DOUBLE;
+    const bool in = dt2 == DPX_INT8 || dt2 == DPX_INT16 || dt2 == DPX_INT32 || dt2 == DPX_INT64;
+    return (fp && in) ? dt1 : -1;
+}
+int dpx_ldexp(const dpx_array_view *x1, const dpx_array_view *x2, const dpx_array_view *dst, void *stream)
+{
+    return ldexp_call(x1, x2, dst, stream);
+}
+int dpx_frexp(const dpx_array_view *x, const dpx_array_view *mantissa, const dpx_array_view *exponent, void *stream)
+{
+    return frexp_call(x, mantissa, exponent, stream);
 }
 int dpx_fill(const dpx_array_view *dst, double value_re, double value_im, int64_t value_int, int use_int,
              void *stream)

@@ -426,6 +426,96 @@ def modf(x, /, out1=None, out2=None, *, out=(None, None), where=True, order="K",
     return frac, whole
 
 
+def _checked_out(out, shape, dt, name):
+    """The usm_ndarray behind a user-supplied `out`, validated as the ufunc wrappers do."""
+    u = get_usm_ndarray(out)
+    if tuple(u.shape) != tuple(shape):
+        raise ValueError(f"The shape of input and output arrays are inconsistent. Expected output shape is "
+                         f"{tuple(shape)}, got {tuple(u.shape)}")
+    if u.dtype != dt:
+        raise ValueError(f"Output array of type {dt} is needed, got {u.dtype}")
+    if not u.flags.writable:
+        raise ValueError(f"{name}: output array is read-only")
+    return u
+
+
+def ldexp(x1, x2, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+    """x1 * 2**x2 for a floating x1 and an integer x2: dpnp.ldexp
+    (dpnp/dpnp_iface_mathematical.py:3150-3220).  Integer x1 converts to the smallest float type that
+    holds it, unsigned x2 to the next signed type; a Python int as x2 is the default integer type."""
+    _check_ufunc_kwargs("ldexp", where, subok, dtype, out, kwargs)
+    check_supported_arrays_type(x1, x2, scalar_type=True)
+
+    def bad(d1, d2):
+        return ValueError(f"function 'ldexp' does not support input types ({d1}, {d2}), and the inputs could not "
+                          "be safely coerced to any supported types according to the casting rule ''safe''.")
+
+    d1 = get_usm_ndarray(x1).dtype if is_supported_array_type(x1) else np.result_type(x1)
+    d2 = get_usm_ndarray(x2).dtype if is_supported_array_type(x2) else np.result_type(x2)
+    if d1.kind in "biu":
+        f1 = np.dtype("f2" if d1.itemsize == 1 else ("f4" if d1.itemsize == 2 else "f8"))
+        if not is_supported_array_type(x1):
+            f1 = np.dtype("f8")
+    elif d1.kind == "f":
+        f1 = d1 if is_supported_array_type(x1) else np.dtype("f8")
+    else:
+        raise bad(d1, d2)
+    if not is_supported_array_type(x2):
+        if d2.kind not in "biu":
+            raise bad(d1, d2)
+        i2 = np.dtype("i8")
+    elif d2.kind == "i":
+        i2 = d2
+    elif d2.kind in "bu" and d2.itemsize < 8:
+        i2 = np.dtype("i1" if d2.kind == "b" else "i" + str(2 * d2.itemsize))
+    else:
+        raise bad(d1, d2)
+    u1 = dpt.astype(get_usm_ndarray(x1), f1, copy=False) if is_supported_array_type(x1) else dpt.asarray(x1, dtype=f1)
+    u2 = dpt.astype(get_usm_ndarray(x2), i2, copy=False) if is_supported_array_type(x2) else dpt.asarray(x2, dtype=i2)
+    shape = np.broadcast_shapes(u1.shape, u2.shape)
+    u1, u2 = dpt.broadcast_to(u1, shape), dpt.broadcast_to(u2, shape)
+    res = None
+    if out is not None:
+        ou = get_usm_ndarray(_unpack_out(out))
+        if tuple(ou.shape) == tuple(shape) and ou.dtype == f1 and ou.flags.writable and not (
+                ti._array_overlap(ou, u1) and not ti._same_logical_tensors(ou, u1)) and not ti._array_overlap(ou, u2):
+            res = ou
+    if res is None:
+        res = dpt.empty(shape, dtype=f1, order="F" if order == "F" else "C")
+    if res.size:
+        tei._ldexp(u1, u2, res)
+    if dtype is not None and np.dtype(dtype) != f1:
+        if not np.can_cast(f1, np.dtype(dtype), "same_kind"):
+            raise TypeError(f"Cannot cast ufunc 'ldexp' output from dtype({f1}) to dtype({np.dtype(dtype)})")
+        res = dpt.astype(res, dtype)
+    if out is not None:
+        return get_result_array(_wrap(res), _unpack_out(out), casting="same_kind")
+    return _wrap(res)
+
+
+def frexp(x, out1=None, out2=None, /, *, out=(None, None), where=True, order="K", dtype=None, subok=True,
+          **kwargs):
+    """(mantissa, exponent) with x = mantissa * 2**exponent and |mantissa| in [0.5, 1): dpnp.frexp
+    (dpnp/dpnp_iface_mathematical.py:2395-2457); the exponent is int32."""
+    _check_ufunc_kwargs("frexp", where, subok, None, None, kwargs)
+    if dtype is not None:
+        raise NotImplementedError("frexp: the `dtype` keyword is not supported")
+    check_supported_arrays_type(x)
+    o1, o2 = (out1, out2) if (out1 is not None or out2 is not None) else tuple(out)
+    u = get_usm_ndarray(x)
+    if u.dtype.kind == "c":
+        raise ValueError(f"function 'frexp' does not support input type ({u.dtype}), and the input could not be "
+                         "safely coerced to any supported types according to the casting rule ''safe''.")
+    if u.dtype.kind != "f":
+        u = dpt.astype(u, "f2" if u.dtype.itemsize == 1 else ("f4" if u.dtype.itemsize == 2 else "f8"))
+    mant = _checked_out(o1, u.shape, u.dtype, "frexp") if o1 is not None else dpt.empty_like(u, order=order or "K")
+    expo = _checked_out(o2, u.shape, np.dtype("i4"), "frexp") if o2 is not None else dpt.empty_like(
+        u, dtype="i4", order=order or "K")
+    if u.size:
+        tei._frexp(u, mant, expo)
+    return (o1 if isinstance(o1, dpnp_array) else _wrap(mant)), (o2 if isinstance(o2, dpnp_array) else _wrap(expo))
+
+
 def nan_to_num(x, copy=True, nan=0.0, posinf=None, neginf=None):
     """NaN -> `nan`, +inf -> `posinf` (largest finite value by default), -inf -> `neginf`:
     dpnp.nan_to_num (dpnp/dpnp_iface_mathematical.py:3584-3760), scalar replacement values."""

@@ -87,6 +87,32 @@ def _isclose_scalar(a, b, rtol, atol, equal_nan, dst, sycl_queue=None, depends=(
     return _events(sycl_queue)
 
 
+def _ldexp_result_type(dt1, dt2):
+    """ufi._ldexp_result_type (dpnp/backend/extensions/ufunc/elementwise_functions/ldexp.cpp:62-93)."""
+    r = lib.dpx_ldexp_result_type(dtype_id(dt1), dtype_id(dt2))
+    return None if r < 0 else dtype_from_id(r)
+
+
+def _ldexp(x1, x2, dst, sycl_queue=None, depends=()):
+    """ufi._ldexp: dst = x1 * 2**x2, operands already broadcast to dst's shape."""
+    _lib.check(lib.dpx_ldexp(x1._as_view(), x2._as_view(), dst._as_view(), _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
+def _frexp_result_type(dt):
+    """ufi._frexp_result_type (frexp.cpp:70-86): (mantissa dtype, exponent dtype) or None."""
+    import numpy as np
+
+    dt = np.dtype(dt)
+    return (dt, np.dtype("i4")) if dt.kind == "f" else None
+
+
+def _frexp(x, mantissa, exponent, sycl_queue=None, depends=()):
+    """ufi._frexp: x = mantissa * 2**exponent."""
+    _lib.check(lib.dpx_frexp(x._as_view(), mantissa._as_view(), exponent._as_view(), _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
 def _black_scholes(price, strike, t, rate, vol, call, put, sycl_queue=None, depends=()):
     """Fused Black-Scholes pricing over 1-D contiguous arrays (no counterpart in the reference)."""
     arrs = (price, strike, t, call, put)

@@ -338,6 +338,21 @@ int dpx_nan_to_num(const dpx_array_view *src, double nan, double posinf,
 int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol,
                 double atol, int equal_nan, const dpx_array_view *dst,
                 void *stream);
+/* dst = x1 * 2^x2: x1 float16/32/64, x2 int8/16/32/64, dst of x1's dtype; an exponent outside the
+ * int range gives +inf (positive) or 0.  Replaces the ldexp calls of
+ * dpnp/backend/extensions/ufunc/elementwise_functions/ldexp.cpp:62-180 (kernel:
+ * dpnp/backend/kernels/elementwise_functions/ldexp.hpp:39-58).  dpx_ldexp_result_type: the dtype of
+ * the result for an operand pair, -1 if the pair is not supported (ufi._ldexp_result_type). */
+int dpx_ldexp_result_type(int dtype1, int dtype2);
+int dpx_ldexp(const dpx_array_view *x1, const dpx_array_view *x2, const dpx_array_view *dst,
+              void *stream);
+/* x = mantissa * 2^exponent, |mantissa| in [0.5, 1): x and mantissa of one dtype (float16/32/64),
+ * exponent int32; the outputs must not overlap each other, the mantissa may be written over x.
+ * Replaces dpnp/backend/extensions/ufunc/elementwise_functions/frexp.cpp:70-200 (kernel:
+ * dpnp/backend/kernels/elementwise_functions/frexp.hpp:36-56; the reference runs one kernel with
+ * two outputs, here the exponent and the mantissa are written by one launch each). */
+int dpx_frexp(const dpx_array_view *x, const dpx_array_view *mantissa,
+              const dpx_array_view *exponent, void *stream);
 /* ti._copy_usm_ndarray_into_usm_ndarray,
  * libtensor/source/copy_and_cast_usm_to_usm.cpp:137-216: dst = cast(src), any
  * dtype pair, equal shapes */

@@ -279,3 +279,92 @@ def test_copy_and_layout_constructors():
     assert r.dtype == np.float32 and step == 0.25
     with pytest.raises(NotImplementedError):
         dpnp.copy(d, subok=True)
+
+
+@pytest.mark.parametrize("fdt", ["f2", "f4", "f8"])
+@pytest.mark.parametrize("idt", ["i1", "i2", "i4", "i8"])
+def test_ldexp_matrix(fdt, idt):
+    # dpnp/tests/test_mathematical.py (TestLdexp): float x int -> float, result bit-exact (ldexp is exact)
+    rng = np.random.default_rng(21)
+    a = rng.uniform(-8, 8, 4099).astype(fdt)
+    a[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1.0]
+    lim = 20 if fdt == "f2" else 100
+    b = rng.integers(-lim, lim, 4099).astype(idt)
+    with np.errstate(all="ignore"):
+        want = np.ldexp(a, b)
+    got = dpnp.ldexp(dpnp.asarray(a), dpnp.asarray(b))
+    assert_same(got.asnumpy(), want)
+    # broadcast, strided views and a scalar exponent
+    m = rng.uniform(-2, 2, (17, 33)).astype(fdt)
+    e = rng.integers(-5, 6, (33,)).astype(idt)
+    assert_same(dpnp.ldexp(dpnp.asarray(m), dpnp.asarray(e)).asnumpy(), np.ldexp(m, e))
+    assert_same(dpnp.ldexp(dpnp.asarray(m).T, dpnp.asarray(e)[:17]).asnumpy(), np.ldexp(m.T, e[:17]))
+    assert_same(dpnp.ldexp(dpnp.asarray(m)[::2, 1::2], 3).asnumpy(), np.ldexp(m[::2, 1::2], 3))
+    o = dpnp.empty(m.shape, dtype=fdt)
+    r = dpnp.ldexp(dpnp.asarray(m), dpnp.asarray(e), out=o)
+    assert r is o
+    assert_same(o.asnumpy(), np.ldexp(m, e))
+
+
+def test_ldexp_promotions_and_limits():
+    x = dpnp.asarray(np.array([1, 2, 3], "i4"))
+    r = dpnp.ldexp(x, dpnp.asarray(np.array([1, 2, 3], "u2")))
+    assert r.dtype == np.float64
+    assert_same(r.asnumpy(), np.array([2.0, 8.0, 24.0]))
+    assert dpnp.ldexp(dpnp.asarray(np.array([1, 2], "i1")), 2).dtype == np.float16
+    assert dpnp.ldexp(dpnp.asarray(np.array([1, 2], "u2")), 2).dtype == np.float32
+    r = dpnp.ldexp(2.0, dpnp.asarray(np.array([1, -1], "i8")))
+    assert_same(r.asnumpy(), np.array([4.0, 1.0]))
+    # exponents beyond the int range: +inf for positive ones, 0 otherwise (ldexp.hpp:45-57)
+    big = dpnp.asarray(np.array([2**40, -(2**40), 2**31, -(2**31) - 1], "i8"))
+    r = dpnp.ldexp(dpnp.asarray(np.array([1.5, 1.5, -1.5, -1.5])), big)
+    assert_same(r.asnumpy(), np.array([np.inf, 0.0, np.inf, 0.0]))
+    assert_same(dpnp.ldexp(dpnp.asarray(np.array([1.0], "f4")), dpnp.asarray(np.array([2], "i4")), dtype="f8").asnumpy(),
+                np.array([4.0]))
+    with pytest.raises(ValueError):
+        dpnp.ldexp(dpnp.asarray(np.array([1.0])), dpnp.asarray(np.array([1.0])))
+    with pytest.raises(ValueError):
+        dpnp.ldexp(dpnp.asarray(np.array([1.0])), dpnp.asarray(np.array([1], "u8")))
+    with pytest.raises(ValueError):
+        dpnp.ldexp(dpnp.asarray(np.array([1j])), 2)
+    with pytest.raises(NotImplementedError):
+        dpnp.ldexp(x, 1, where=False)
+
+
+@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
+def test_frexp_every_binade_and_special_values(dt):
+    # dpnp/tests/test_mathematical.py (TestFrexp)
+    rng = np.random.default_rng(23)
+    info = np.finfo(dt)
+    a = np.ldexp(rng.uniform(0.5, 1.0, 6000), rng.integers(info.minexp - info.nmant, info.maxexp + 1, 6000)).astype(dt)
+    a[::2] *= -1
+    a[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, info.tiny, info.max, info.smallest_subnormal]
+    want_m, want_e = np.frexp(a)
+    m, e = dpnp.frexp(dpnp.asarray(a))
+    assert e.dtype == np.int32 and m.dtype == np.dtype(dt)
+    assert_same(m.asnumpy(), want_m)
+    assert_same(e.asnumpy(), want_e.astype("i4"))
+    np.testing.assert_array_equal(np.signbit(m.asnumpy()), np.signbit(want_m))
+    # views, out arguments, in-place mantissa
+    a2 = rng.normal(size=(33, 65)).astype(dt)
+    d2 = dpnp.asarray(a2)
+    wm, we = np.frexp(a2.T[::2])
+    m, e = dpnp.frexp(d2.T[::2])
+    assert_same(m.asnumpy(), wm)
+    assert_same(e.asnumpy(), we.astype("i4"))
+    om, oe = dpnp.empty(a2.shape, dtype=dt), dpnp.empty(a2.shape, dtype="i4")
+    rm, re_ = dpnp.frexp(d2, out=(om, oe))
+    assert rm is om and re_ is oe
+    assert_same(om.asnumpy(), np.frexp(a2)[0])
+    assert_same(oe.asnumpy(), np.frexp(a2)[1].astype("i4"))
+    rm, re_ = dpnp.frexp(d2, d2, None)
+    assert_same(d2.asnumpy(), np.frexp(a2)[0])
+    assert_same(re_.asnumpy(), np.frexp(a2)[1].astype("i4"))
+    with pytest.raises(ValueError):
+        dpnp.frexp(d2, out=(dpnp.empty((3,), dtype=dt), None))
+    with pytest.raises(ValueError):
+        dpnp.frexp(dpnp.asarray(np.array([1j])))
+    mi, ei = dpnp.frexp(dpnp.asarray(np.array([8, 3], "i4")))
+    assert mi.dtype == np.float64
+    assert_same(mi.asnumpy(), np.array([0.5, 0.75]))
+    assert_same(ei.asnumpy(), np.array([4, 2], "i4"))
