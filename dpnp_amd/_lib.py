@@ -111,6 +111,7 @@ SIGNATURES = {
     "dpx_divide_by_scalar": (_i, [_VP, _d, _VP, _vp]),
     "dpx_nan_to_num": (_i, [_VP, _d, _d, _d, _VP, _vp]),
     "dpx_isclose": (_i, [_VP, _VP, _d, _d, _i, _VP, _vp]),
+    "dpx_clip": (_i, [_VP, _VP, _VP, _VP, _vp]),
     "dpx_ldexp_result_type": (_i, [_i, _i]),
     "dpx_ldexp": (_i, [_VP, _VP, _VP, _vp]),
     "dpx_frexp": (_i, [_VP, _VP, _VP, _vp]),

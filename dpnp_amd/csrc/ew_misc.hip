@@ -213,6 +213,43 @@ static int isclose_call(const dpx_array_view *a, const dpx_array_view *b, double
     }
 }
 
+// ---- clip: libtensor/include/kernels/clip.hpp:66-86 (contiguous 89-200, strided 232-290) ------------
+// max(x, lo) then min(.., hi); a NaN in x stays, a NaN bound wins; bool: (x || lo) && hi; complex
+// through the NaN-propagating lexicographic extrema.
+template <class T> struct ClipFn {
+    DPX_D V<T> operator()(V<T> x, V<T> lo, V<T> hi) const
+    {
+        if constexpr (is_cplx_v<T>) return min_nan(max_nan(x, lo), hi);
+        else if constexpr (is_bool_v<T>) return (x || lo) && hi;
+        else if constexpr (is_fp_v<V<T>>) {
+            const V<T> t = (x != x || x > lo) ? x : lo;
+            return (t != t || t < hi) ? t : hi;
+        }
+        else {
+            const V<T> t = (x > lo) ? x : lo;
+            return (t < hi) ? t : hi;
+        }
+    }
+};
+
+static int clip_call(const dpx_array_view *x, const dpx_array_view *lo, const dpx_array_view *hi,
+                     const dpx_array_view *dst, void *stream)
+{
+    if (!view_ok(x) || !view_ok(lo) || !view_ok(hi) || !view_ok(dst))
+        return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
+    if (x->dtype != lo->dtype || x->dtype != hi->dtype) return fail(DPX_ERR_BAD_DTYPE, "Input arrays must have the same data type");
+    if (x->dtype != dst->dtype) return fail(DPX_ERR_BAD_DTYPE, "Destination array has unexpected elemental data type.");
+    const dpx_array_view *views[4] = {x, lo, hi, dst};
+    int64_t n = 0;
+    if (int rc = ew_validate(4, views, n)) return rc;
+    int rc = DPX_ERR_NOT_IMPLEMENTED;
+    for_dtype(x->dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        rc = run_ew<ClipFn<T>, T, T, T, T>({}, views, (hipStream_t)stream, nullptr);
+    });
+    return rc;
+}
+
 // ---- ldexp: dpnp/backend/kernels/elementwise_functions/ldexp.hpp:39-58 -------------------------------
 // x1 * 2^x2; an exponent outside the int range gives +inf when positive and 0 otherwise, whatever x1 is
 // (as the reference's functor does).
@@ -422,6 +459,11 @@ int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol, d
                 const dpx_array_view *dst, void *stream)
 {
     return isclose_call(a, b, rtol, atol, equal_nan, dst, stream);
+}
+int dpx_clip(const dpx_array_view *x, const dpx_array_view *lo, const dpx_array_view *hi, const dpx_array_view *dst,
+             void *stream)
+{
+    return clip_call(x, lo, hi, dst, stream);
 }
 int dpx_ldexp_result_type(int dt1, int dt2)
 {

@@ -97,6 +97,11 @@ class dpnp_array:
         return dpnp_array._create_from_usm_ndarray(
             dpt.astype(self._array_obj, dtype, order=order, casting=casting, copy=copy))
 
+    def clip(self, /, min=None, max=None, out=None, **kwargs):  # noqa: A002
+        from . import dpnp_iface
+
+        return dpnp_iface.clip(self, min, max, out=out, **kwargs)
+
     def copy(self, order="C"):
         return dpnp_array._create_from_usm_ndarray(dpt.copy(self._array_obj, order=order))
 

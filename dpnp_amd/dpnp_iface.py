@@ -516,6 +516,20 @@ def frexp(x, out1=None, out2=None, /, *, out=(None, None), where=True, order="K"
     return (o1 if isinstance(o1, dpnp_array) else _wrap(mant)), (o2 if isinstance(o2, dpnp_array) else _wrap(expo))
 
 
+def clip(a, /, min=None, max=None, *, out=None, order="K", **kwargs):  # noqa: A002
+    """Values of `a` limited to [min, max]: dpnp.clip (dpnp/dpnp_iface_mathematical.py:722-830)."""
+    if kwargs:
+        raise NotImplementedError(f"kwargs={kwargs} is currently not supported")
+    order = order if order is not None else "K"
+    usm_min = None if min is None else get_usm_ndarray_or_scalar(min)
+    usm_max = None if max is None else get_usm_ndarray_or_scalar(max)
+    usm_out = None if out is None else get_usm_ndarray(out)
+    res = dpt.clip(get_usm_ndarray(a), usm_min, usm_max, out=usm_out, order=order)
+    if out is not None and isinstance(out, dpnp_array):
+        return out
+    return _wrap(res)
+
+
 def nan_to_num(x, copy=True, nan=0.0, posinf=None, neginf=None):
     """NaN -> `nan`, +inf -> `posinf` (largest finite value by default), -inf -> `neginf`:
     dpnp.nan_to_num (dpnp/dpnp_iface_mathematical.py:3584-3760), scalar replacement values."""

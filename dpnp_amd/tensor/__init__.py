@@ -59,6 +59,7 @@ from ._reduction import (  # noqa: A004
     sum,
 )
 from ._search_functions import where
+from ._clip import clip
 from ._statistical_functions import mean, std, var
 from ._type_utils import can_cast, result_type
 from ._usmarray import usm_ndarray

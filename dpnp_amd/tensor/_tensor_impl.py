@@ -29,6 +29,14 @@ def _where(condition, x1, x2, dst, sycl_queue=None, depends=()):
     return _events(sycl_queue)
 
 
+def _clip(src, min, max, dst, sycl_queue=None, depends=()):  # noqa: A002
+    """ti._clip (libtensor/source/clip.cpp:69-263): dst = min(max(src, min), max), operands of dst's
+    dtype and shape."""
+    views = [a._as_view() for a in (src, min, max, dst)]
+    _lib.check(lib.dpx_clip(*views, _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
 def _where_compare(cmp_name, lhs, rhs, x1, x2, dst, sycl_queue=None, depends=()):
     """dst = (lhs CMP rhs) ? x1 : x2 in one pass (no counterpart in the reference)."""
     views = [a._as_view() for a in (lhs, rhs, x1, x2, dst)]

@@ -338,6 +338,12 @@ int dpx_nan_to_num(const dpx_array_view *src, double nan, double posinf,
 int dpx_isclose(const dpx_array_view *a, const dpx_array_view *b, double rtol,
                 double atol, int equal_nan, const dpx_array_view *dst,
                 void *stream);
+/* dst = min(max(x, lo), hi) elementwise: four arrays of one dtype (any of the 14) and one shape
+ * (broadcast operands carry zero strides); a NaN element stays NaN, a NaN bound gives NaN; bool:
+ * (x || lo) && hi.  Replaces ti._clip, libtensor/source/clip.cpp:69-263 (kernels:
+ * libtensor/include/kernels/clip.hpp:66-86 the functor, 89-225 contiguous, 232-330 strided). */
+int dpx_clip(const dpx_array_view *x, const dpx_array_view *lo, const dpx_array_view *hi,
+             const dpx_array_view *dst, void *stream);
 /* dst = x1 * 2^x2: x1 float16/32/64, x2 int8/16/32/64, dst of x1's dtype; an exponent outside the
  * int range gives +inf (positive) or 0.  Replaces the ldexp calls of
  * dpnp/backend/extensions/ufunc/elementwise_functions/ldexp.cpp:62-180 (kernel:

@@ -368,6 +368,27 @@ def ulp_error(result, exact_hi):
     return err
 
 
+def clip(x, lo, hi):
+    """libtensor/include/kernels/clip.hpp:66-86: max(x, lo) then min(.., hi).  Floats: a NaN in x
+    stays, a NaN bound wins; bool: (x or lo) and hi; complex through max_complex / min_complex
+    (math_utils.hpp:99-129), i.e. the first operand unless the second is lexicographically beyond
+    it, NaN first operands kept."""
+    x, lo, hi = np.broadcast_arrays(np.asarray(x), np.asarray(lo), np.asarray(hi))
+    dt = x.dtype
+    assert lo.dtype == dt and hi.dtype == dt
+    if dt.kind == "b":
+        return (x | lo) & hi
+    if dt.kind == "c":
+        t = np.where(_cplx_pick(x, lo, True), x, lo)
+        return np.where(_cplx_pick(t, hi, False), t, hi).astype(dt)
+    if dt.kind == "f":
+        with np.errstate(invalid="ignore"):
+            t = np.where(np.isnan(x) | (x > lo), x, lo)
+            return np.where(np.isnan(t) | (t < hi), t, hi).astype(dt)
+    t = np.where(x > lo, x, lo)
+    return np.where(t < hi, t, hi).astype(dt)
+
+
 def where(cond, x1, x2):
     """where.hpp:72-161: cond is true when non-zero (any dtype); x1, x2 of one dtype."""
     x1, x2 = _same(x1, x2)

@@ -398,3 +398,30 @@ def test_oracle_extension_functions_known_values():
                           np.array([1.0, 2.0, nan]), equal_nan=True)
     assert orc.binary("heaviside", np.array([-1.0, 0.0, 2.0]), np.array([0.5, 0.5, 0.5])).tolist() == [0.0, 0.5, 1.0]
     assert orc.binary("logaddexp2", np.array([3.0]), np.array([3.0]))[0] == 4.0
+
+
+def test_clip_matches_numpy_and_the_reference_special_cases():
+    # pins oracle.clip: np.clip wherever lo <= hi and nothing is NaN; hi wins when lo > hi
+    # (dpnp/tests/tensor/test_tensor_clip.py:638-644); a NaN bound gives NaN, a NaN element stays
+    # (test_tensor_clip.py:178-187); bool: (x or lo) and hi by truth table
+    rng = np.random.default_rng(3)
+    for dt in ("i1", "u2", "i4", "i8", "f2", "f4", "f8"):
+        x = (rng.uniform(-100, 100, 500)).astype(dt)
+        lo = (rng.uniform(-100, 0, 500)).astype(dt)
+        hi = (rng.uniform(0, 100, 500)).astype(dt)
+        np.testing.assert_array_equal(orc.clip(x, lo, hi), np.clip(x, lo, hi))
+        got = orc.clip(x, hi, lo)  # lo > hi: the upper bound is applied last
+        np.testing.assert_array_equal(got[hi > lo], lo[hi > lo])
+    x = np.arange(10, dtype="f4")
+    assert np.isnan(orc.clip(x, np.float32(np.nan), np.float32(np.inf))).all()
+    assert np.isnan(orc.clip(x, np.float32(-np.inf), np.float32(np.nan))).all()
+    xn = np.array([np.nan, 1.0, 5.0], "f8")
+    np.testing.assert_array_equal(orc.clip(xn, np.float64(2), np.float64(3)), np.array([np.nan, 2.0, 3.0]))
+    for xv in (False, True):
+        for lv in (False, True):
+            for hv in (False, True):
+                assert bool(orc.clip(np.array(xv), np.array(lv), np.array(hv))) == ((xv or lv) and hv)
+    # complex: lexicographic order on (real, imag)
+    z = np.array([1 + 1j, 1 + 5j, 3 + 0j, 0 + 9j], "c8")
+    got = orc.clip(z, np.complex64(1 + 2j), np.complex64(2 + 0j))
+    np.testing.assert_array_equal(got, np.array([1 + 2j, 1 + 5j, 2 + 0j, 1 + 2j], "c8"))
