@@ -609,7 +609,25 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = P::identity();
     if (active) {
-        for (int sidx = ty; sidx < L.splits; sidx += TY) {
+        // FU partials per column in flight: with few columns and many splits this loop is the tail
+        // of the kernel (512 splits over 16 thread rows: 32 dependent L2 round trips without it)
+        constexpr int FU = E >= 16 ? 2 : (E >= 8 ? 4 : 8);
+        int sidx = ty;
+        for (; sidx + (FU - 1) * TY < L.splits; sidx += FU * TY) {
+            Acc t[FU][E];
+#pragma unroll
+            for (int u = 0; u < FU; ++u)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if (e < ecnt && col0 + e < L.inner)
+                        t[u][e] = slot_read(partial + (int64_t)(sidx + u * TY) * L.m + out0 + e);
+#pragma unroll
+            for (int u = 0; u < FU; ++u)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if (e < ecnt && col0 + e < L.inner) v[e] = P::combine(v[e], t[u][e]);
+        }
+        for (; sidx < L.splits; sidx += TY) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
                 if (e < ecnt && col0 + e < L.inner)
@@ -622,6 +640,128 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         for (int e = 0; e < E; ++e)
             if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e]);
     }
+}
+
+// ================================ flat columns kernel =========================================
+// A row-major matrix with short rows (a row shorter than 512 bytes), reduced over its rows: the
+// column kernel would leave most lanes of a wave without a pack.  Here the matrix is one flat
+// stream of 16-byte packs and element i belongs to column i mod inner.  A block has T threads with
+// T * E a multiple of inner, thread t takes packs t, t + T, t + 2T, ... of the block's rows, so the
+// columns of its E accumulators never change.  Block b owns rows [b * chunk, (b + 1) * chunk).
+// LDS holds T * E accumulators, entry k of column k mod inner; a tree over k folds them to one
+// entry per column.  With several blocks the last one (ticket) folds the per-block partials,
+// laid out [block][column], the same way.  L.m = L.inner = columns, L.n = rows, L.splits = blocks.
+template <class P> DPX_D void flat_fold_columns(typename P::Acc *sm, int count, int inner)
+{
+    const int J = (count + inner - 1) / inner;
+    int s = 1;
+    while (2 * s < J) s *= 2; // the largest power of two below J (1 when J <= 2)
+    if (J < 2) s = 0;
+    for (; s >= 1; s >>= 1) {
+        __syncthreads();
+        const int lim = (count - s * inner < s * inner) ? count - s * inner : s * inner;
+        for (int k = threadIdx.x; k < lim; k += (int)blockDim.x) sm[k] = P::combine(sm[k], sm[k + s * inner]);
+    }
+    __syncthreads();
+}
+
+template <class P>
+__global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
+                                                      typename P::Out *dst, Slot<typename P::Acc> *partial,
+                                                      const typename P::Aux *aux, unsigned *counters)
+{
+    using In = typename P::In;
+    using Acc = typename P::Acc;
+    constexpr int E = cols_cfg<In>::E;
+    constexpr int U = E >= 8 ? 2 : (E >= 4 ? 4 : 8); // packs in flight per thread
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    Acc *sm = reinterpret_cast<Acc *>(smem_raw);
+    const int T = (int)blockDim.x, t = (int)threadIdx.x;
+    const int inner = (int)L.inner;
+    const int split = (int)blockIdx.x;
+    const int64_t row0 = (int64_t)split * L.chunk;
+    const int64_t rows = (row0 + L.chunk < L.n) ? L.chunk : L.n - row0;
+    const int64_t elems = rows * inner;
+    const int64_t packs = elems / E;
+    const In *p = src + row0 * inner;
+
+    Acc a[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) a[e] = P::identity();
+    if constexpr (P::has_aux) {
+        int c = (int)(((int64_t)t * E) % inner);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            a[e] = P::load_aux(aux + (int64_t)c * ix.aux_str[0]);
+            c = (c + 1 == inner) ? 0 : c + 1;
+        }
+    }
+    Acc acc[U][E];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[u][e] = P::identity();
+    int64_t q = t;
+    for (; q + (int64_t)(U - 1) * T < packs; q += (int64_t)U * T) {
+        pack<In, E> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = load_pack<In, E>(p + (q + (int64_t)u * T) * E);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], P::pre(v[u].v[e], a[e]));
+    }
+    for (; q < packs; q += T) {
+        const pack<In, E> v = load_pack<In, E>(p + q * E);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[0][e] = P::combine(acc[0][e], P::pre(v.v[e], a[e]));
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        Acc r = acc[0][e];
+#pragma unroll
+        for (int u = 1; u < U; ++u) r = P::combine(r, acc[u][e]);
+        sm[t * E + e] = r;
+    }
+    __syncthreads();
+    // the elements after the last whole pack of the block (fewer than E): entry k of the table has
+    // the column of every flat position congruent to k modulo T * E
+    const int tail = (int)(elems - packs * E);
+    if (t < tail) {
+        const int64_t i = packs * E + t;
+        const int k = (int)(i % ((int64_t)T * E));
+        Acc ax = P::identity();
+        if constexpr (P::has_aux) ax = P::load_aux(aux + (int64_t)(k % inner) * ix.aux_str[0]);
+        sm[k] = P::combine(sm[k], P::pre(load_one(p + i), ax));
+    }
+    flat_fold_columns<P>(sm, T * E, inner);
+    if (L.splits == 1) {
+        for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c]);
+        return;
+    }
+    uint32_t zero = 0;
+    for (int c = t; c < inner; c += T) zero |= slot_publish(partial + (int64_t)split * inner + c, sm[c]);
+    if (!last_block_of(counters, L.splits, zero)) return;
+    // the last block: thread t < parts * inner folds blocks part, part + parts, ... of column t mod inner
+    const int parts = T / inner;
+    Acc v = P::identity();
+    if (t < parts * inner) {
+        constexpr int FU = 8;
+        const int c = t % inner, part = t / inner;
+        int g = part;
+        for (; g + (FU - 1) * parts < L.splits; g += FU * parts) {
+            Acc w[FU];
+#pragma unroll
+            for (int u = 0; u < FU; ++u) w[u] = slot_read(partial + (int64_t)(g + u * parts) * inner + c);
+#pragma unroll
+            for (int u = 0; u < FU; ++u) v = P::combine(v, w[u]);
+        }
+        for (; g < L.splits; g += parts) v = P::combine(v, slot_read(partial + (int64_t)g * inner + c));
+    }
+    __syncthreads(); // every thread has read its column results of the first fold
+    if (t < parts * inner) sm[t] = v;
+    flat_fold_columns<P>(sm, parts * inner, inner);
+    for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c]);
 }
 
 // identity fill for an empty reduced run (reductions.hpp:1417-1422)
@@ -974,14 +1114,34 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
         best[e] = VT{};
         bidx[e] = ARG_NONE;
     }
-    if (active)
-        for (int sidx = ty; sidx < L.splits; sidx += TY) {
+    if (active) {
+        constexpr int FU = E >= 16 ? 1 : (E >= 8 ? 2 : 4); // partial pairs per column in flight
+        int sidx = ty;
+        for (; sidx + (FU - 1) * TY < L.splits; sidx += FU * TY) {
+            T tv[FU][E];
+            int64_t ti[FU][E];
+#pragma unroll
+            for (int u = 0; u < FU; ++u)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if (col0 + e < L.inner) {
+                        tv[u][e] = slot_read(pval + (int64_t)(sidx + u * TY) * L.m + out0 + e);
+                        ti[u][e] = slot_read(pidx + (int64_t)(sidx + u * TY) * L.m + out0 + e);
+                    }
+#pragma unroll
+            for (int u = 0; u < FU; ++u)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if (col0 + e < L.inner) arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(tv[u][e]), ti[u][e]);
+        }
+        for (; sidx < L.splits; sidx += TY) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
                 if (col0 + e < L.inner)
                     arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(slot_read(pval + (int64_t)sidx * L.m + out0 + e)),
                                           slot_read(pidx + (int64_t)sidx * L.m + out0 + e));
         }
+    }
     combine_rows();
     if (ty == 0 && active) write_out();
 }

@@ -186,6 +186,40 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
+    if (!arg && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
+        env_int("DPX_RED_FLAT", 1) != 0) { // (experiment knob: 0 keeps the column kernel)
+        // a row-major matrix with rows shorter than 512 bytes: one flat stream of packs, a block of
+        // T threads with T * E a multiple of the row length (see red_flat_kernel)
+        int64_t g = inner, b = E;
+        while (b) {
+            const int64_t r = g % b;
+            g = b;
+            b = r;
+        }
+        const int64_t period = inner / g; // threads after which the columns of a pack repeat
+        if (period <= 256) {
+            const int64_t T = period * (256 / period);
+            const int64_t per_block = T * E * 8; // at least 8 packs per thread
+            int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(target, (n * inner) / per_block));
+            {
+                const int64_t chunk = cdiv(n, blocks);
+                blocks = cdiv(n, chunk);
+                L.vec = 1;
+                L.g_log2 = 0;
+                L.rstride = rstride;
+                L.inner = inner;
+                L.col_blocks = 1;
+                L.chunk = chunk;
+                L.splits = (int32_t)blocks;
+                L.tgroup = 0;
+                pl.block = (int)T;
+                pl.grid = blocks;
+                pl.path = DPX_PATH_RED_FLAT;
+                if (blocks > 1) pl.scratch_elems = blocks * inner;
+                return;
+            }
+        }
+    }
     const bool vec = true; // packs need no alignment; the kernels read a row's last pack by element
     const int e = E;
     L.vec = vec ? 1 : 0;

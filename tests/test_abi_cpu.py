@@ -202,6 +202,17 @@ def test_reduction_plans():
     pa = L.Plan()
     L.check(lib.dpx_argreduce_plan(0, view([1 << 28]), 1, view([], dt=L.INT64, ptr=P1), pa))
     assert L.PATH_NAMES[pa.path] == "red_rows_split"
+    # axis=0 of a row-major matrix with short rows: flat stream, block size a multiple of the column period
+    for cols, threads in ((17, 255), (64, 256), (3, 255), (10, 255), (100, 250), (127, 254)):
+        p = plan_reduce("sum", view([cols, 1 << 20], [1, cols]), 1, view([cols], ptr=P1))
+        assert L.PATH_NAMES[p.path] == "red_flat" and p.block == threads and p.splits == p.grid[0] > 1, (cols, p.block)
+        assert p.scratch_bytes == 131072 + 4 * p.splits * cols
+    p = plan_reduce("sum", view([17, 100], [1, 17]), 1, view([17], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_flat" and p.splits == 1 and p.scratch_bytes == 0
+    p = plan_reduce("sum", view([128, 1 << 20], [1, 128]), 1, view([128], ptr=P1))  # 512-byte rows: column kernel
+    assert L.PATH_NAMES[p.path] == "red_cols_split"
+    p = plan_reduce("sum", view([17, 1 << 20], [1, 18]), 1, view([17], ptr=P1))  # padded rows: column kernel
+    assert L.PATH_NAMES[p.path] == "red_cols_split"
 
 
 def test_validation_errors_are_raised_before_any_launch():

@@ -468,3 +468,65 @@ def test_all_any_count_nonzero_every_dtype_in_one_pass(dt):
     big = np.zeros(3_000_001, dtype=dt)
     big[-1] = 1
     assert bool(dpt.any(dev(big))) and not bool(dpt.all(dev(big))) and int(dpt.count_nonzero(dev(big))) == 1
+
+
+FLAT_COLS = [2, 3, 5, 7, 10, 16, 17, 31, 33, 60, 64, 100, 127]
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "f2", "f4", "f8", "c8", "c16"])
+def test_axis0_of_matrices_with_short_rows(dt):
+    # a row shorter than 512 bytes: the reduction over rows reads the matrix as one flat stream
+    rng = np.random.default_rng(41)
+    itemsize = np.dtype(dt).itemsize
+    for cols in FLAT_COLS:
+        if cols * itemsize >= 512:
+            continue
+        for rows in (16, 17, 255, 4099, 60013):
+            a = random_array(rng, (rows, cols), dt, lo=-3, hi=3)
+            da = dev(a)
+            check_sum(host(dpt.sum(da, axis=0)), a, 0)
+            assert_same(host(dpt.max(da, axis=0)), orc.reduce("max", a.T, 1))
+            assert_same(host(dpt.min(da, axis=0)), orc.reduce("min", a.T, 1))
+            assert_same(host(dpt.any(da, axis=0)), a.astype(bool).any(axis=0))
+            assert_same(host(dpt.all(da, axis=0)), a.astype(bool).all(axis=0))
+            assert_same(host(dpt.count_nonzero(da, axis=0)), np.count_nonzero(a, axis=0).astype("i8"))
+    # a view that starts at a later row, and a strided destination
+    a = random_array(rng, (5000, 17), dt, lo=-3, hi=3)
+    da = dev(a)
+    check_sum(host(dpt.sum(da[3:], axis=0)), a[3:], 0)
+    assert_same(host(dpt.max(da[1:4001], axis=0)), orc.reduce("max", a[1:4001].T, 1))
+    out = dpt.zeros(34, dtype=dpt.max(da, axis=0).dtype)
+    dpt.max(da, axis=0, out=out[::2])
+    assert_same(host(out)[::2], orc.reduce("max", a.T, 1))
+    assert (host(out)[1::2] == 0).all()
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+def test_statistics_over_samples_of_few_features(dt):
+    # (samples, features) with few features: mean / var / std / logsumexp / hypot / nan forms over axis 0
+    rng = np.random.default_rng(43)
+    for cols in (3, 8, 17, 64 if dt == "f8" else 100):
+        if cols * np.dtype(dt).itemsize >= 512:
+            continue
+        a = rng.normal(2.0, 3.0, (100003, cols)).astype(dt)
+        da = dev(a)
+        tol = dict(rtol=2e-5, atol=1e-5) if dt == "f4" else dict(rtol=1e-12, atol=1e-12)
+        a64 = a.astype("f8") if dt == "f4" else a.astype(np.longdouble)
+        np.testing.assert_allclose(host(dpt.mean(da, axis=0)), a64.mean(axis=0).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.var(da, axis=0)), a64.var(axis=0).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.std(da, axis=0, correction=1)), a64.std(axis=0, ddof=1).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.reduce_hypot(da, axis=0)), np.sqrt((a64 * a64).sum(axis=0)).astype(dt), **tol)
+        m = a64.max(axis=0)
+        np.testing.assert_allclose(host(dpt.logsumexp(da, axis=0)), (m + np.log(np.exp(a64 - m).sum(axis=0))).astype(dt), **tol)
+        b = a.copy()
+        b[rng.random(b.shape) < 0.1] = np.nan
+        b64 = b.astype("f8") if dt == "f4" else b.astype(np.longdouble)
+        db = dpnp.asarray(b)
+        np.testing.assert_allclose(dpnp.nansum(db, axis=0).asnumpy(), np.nansum(b64, axis=0).astype(dt), **tol)
+        np.testing.assert_allclose(dpnp.nanmean(db, axis=0).asnumpy(), np.nanmean(b64, axis=0).astype(dt), **tol)
+        np.testing.assert_allclose(dpnp.nanvar(db, axis=0).asnumpy(), np.nanvar(b64, axis=0).astype(dt), **tol)
+        assert_same(dpnp.nanmax(db, axis=0).asnumpy(), np.nanmax(b, axis=0))
+    # results are reproducible bit for bit
+    a = rng.normal(size=(200003, 17)).astype(dt)
+    r1, r2 = host(dpt.sum(dev(a), axis=0)), host(dpt.sum(dev(a), axis=0))
+    assert_same(r1, r2)
