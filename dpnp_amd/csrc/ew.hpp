@@ -65,12 +65,44 @@ template <class T, int E> DPX_D pack<T, E> splat(T v)
 }
 
 // ---- contiguous ---------------------------------------------------------------
-// grid.x * blockDim.x * E * U >= n.  bcast bit i set: input i is a single element.
-// Pack u of thread t in block b covers elements ((b * U + u) * blockDim.x + t) * E ... + E.
+// grid.x * blockDim.x * E * U >= n.  Pack u of thread t in block b covers elements
+// ((b * U + u) * blockDim.x + t) * E ... + E of the output.  `bcast` holds 2 bits per input:
+// BC_FULL the input has an element per output element; BC_SCALAR it is a single element;
+// BC_PERIODIC it has `period` elements and output element i takes element i mod period (a row
+// added to every row of a row-major matrix with short rows); BC_REPEAT output element i takes
+// element i / period (a column, one element per row).  The last two need n < 2^32.
+enum : uint32_t { BC_FULL = 0, BC_SCALAR = 1, BC_PERIODIC = 2, BC_REPEAT = 3 };
+
+template <class T> DPX_D T load_bcast_one(const T *p, uint32_t mode, int64_t i, uint32_t period)
+{
+    switch (mode) {
+    case BC_FULL: return load_one(p + i);
+    case BC_SCALAR: return load_one(p);
+    case BC_PERIODIC: return load_one(p + (uint32_t)i % period);
+    default: return load_one(p + (uint32_t)i / period);
+    }
+}
+template <class T, int E> DPX_D pack<T, E> load_bcast_pack(const T *p, uint32_t mode, int64_t base, uint32_t period)
+{
+    if (mode == BC_FULL) return load_pack<T, E>(p + base);
+    if (mode == BC_SCALAR) return splat<T, E>(load_one(p));
+    // a small vector that stays in cache: element-wise reads, one division per pack
+    uint32_t r = (uint32_t)base / period, c = (uint32_t)base - r * period;
+    pack<T, E> v;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        v.v[e] = load_one(p + (mode == BC_PERIODIC ? c : r));
+        if (++c == period) {
+            c = 0;
+            ++r;
+        }
+    }
+    return v;
+}
+
 template <class Fn, class Out, class... Ins, size_t... I>
-DPX_D void ew_contig_pack(const Fn &fn, uint32_t bcast, Out *out, const InPtrs<sizeof...(Ins)> &in,
-                          int64_t base, std::tuple<pack<Ins, ew_traits<Out, Ins...>::E>...> &v,
-                          std::index_sequence<I...>)
+DPX_D void ew_contig_pack(const Fn &fn, Out *out, int64_t base,
+                          std::tuple<pack<Ins, ew_traits<Out, Ins...>::E>...> &v, std::index_sequence<I...>)
 {
     constexpr int E = ew_traits<Out, Ins...>::E;
     (keep_whole(std::get<I>(v)), ...);
@@ -81,17 +113,14 @@ DPX_D void ew_contig_pack(const Fn &fn, uint32_t bcast, Out *out, const InPtrs<s
 }
 
 template <class Fn, class Out, class... Ins, size_t... I>
-DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
+DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, uint32_t period, Out *out,
                           const InPtrs<sizeof...(Ins)> &in, std::index_sequence<I...> seq)
 {
     constexpr int E = ew_traits<Out, Ins...>::E;
     constexpr int U = ew_traits<Out, Ins...>::U;
     const int64_t block_base = (int64_t)blockIdx.x * ((int)blockDim.x * E * U);
     auto load = [&](int64_t base, std::tuple<pack<Ins, E>...> &v) {
-        ((std::get<I>(v) = ((bcast >> I) & 1u)
-                               ? splat<Ins, E>(load_one((const Ins *)in.p[I]))
-                               : load_pack<Ins, E>((const Ins *)in.p[I] + base)),
-         ...);
+        ((std::get<I>(v) = load_bcast_pack<Ins, E>((const Ins *)in.p[I], (bcast >> (2 * I)) & 3u, base, period)), ...);
     };
     if (block_base + (int64_t)blockDim.x * E * U <= n) { // the usual case: every load first
         std::tuple<pack<Ins, E>...> v[U];
@@ -100,8 +129,7 @@ DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
             load(block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E, v[u]);
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            ew_contig_pack<Fn, Out, Ins...>(fn, bcast, out, in,
-                                            block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E,
+            ew_contig_pack<Fn, Out, Ins...>(fn, out, block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E,
                                             v[u], seq);
         return;
     }
@@ -110,22 +138,20 @@ DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, Out *out,
         if (base + E <= n) {
             std::tuple<pack<Ins, E>...> v;
             load(base, v);
-            ew_contig_pack<Fn, Out, Ins...>(fn, bcast, out, in, base, v, seq);
+            ew_contig_pack<Fn, Out, Ins...>(fn, out, base, v, seq);
         }
         else
             for (int64_t i = base; i < n; ++i)
                 out[i] = to_storage<Out>(fn(to_value(
-                    load_one((const Ins *)in.p[I] + (((bcast >> I) & 1u) ? 0 : i)))...));
+                    load_bcast_one((const Ins *)in.p[I], (bcast >> (2 * I)) & 3u, i, period))...));
     }
 }
 
 template <class Fn, class Out, class... Ins>
-__global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, uint32_t bcast,
-                                                            Out *out,
-                                                            InPtrs<sizeof...(Ins)> in)
+__global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, uint32_t bcast, uint32_t period,
+                                                            Out *out, InPtrs<sizeof...(Ins)> in)
 {
-    ew_contig_body<Fn, Out, Ins...>(fn, n, bcast, out, in,
-                                         std::index_sequence_for<Ins...>{});
+    ew_contig_body<Fn, Out, Ins...>(fn, n, bcast, period, out, in, std::index_sequence_for<Ins...>{});
 }
 
 // Stride-2 operand (x[:, ::2], real or imaginary parts) read by a whole wave: the lane's E
@@ -461,7 +487,9 @@ struct EwPlan {
     int64_t n;                      // total elements
     // launch parameters, filled by ew_finish_plan for a given E / item sizes
     bool vec;
-    uint32_t bcast;
+    bool flat2d;     // contiguous path over a row-major matrix with short rows (nd == 2 kept in shape/strides)
+    uint32_t bcast;  // contiguous path: 2 bits per input (BC_*)
+    uint32_t period; // ... row length for BC_PERIODIC / BC_REPEAT inputs
     uint32_t modes;
     int tx_log2;
     int block; // threads per block
@@ -505,7 +533,7 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
     Out *out = (Out *)ptrs[N];
     if (pl.path == DPX_PATH_EW_CONTIG) {
         hipLaunchKernelGGL((ew_contig_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(pl.block), 0,
-                           stream, fn, pl.n, pl.bcast, out, in);
+                           stream, fn, pl.n, pl.bcast, pl.period, out, in);
     }
     else {
         NdIndex<N + 1> ix;

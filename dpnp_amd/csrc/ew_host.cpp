@@ -47,6 +47,8 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     pl.nops = nops;
     pl.n = view_size(dst);
     pl.vec = false;
+    pl.flat2d = false;
+    pl.period = 1;
     pl.bcast = pl.modes = 0;
     pl.tx_log2 = 0;
     pl.block = EW_CONTIG_BLOCK;
@@ -74,6 +76,29 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     pl.tmask = 0;
     pl.dT = -1;
     if (contig || pl.nd < 2 || nops < 2) return;
+    // A row-major matrix with rows shorter than 512 bytes combined with a row and/or a column
+    // (x - mean(x, axis=0), x / norm(x, axis=1)[:, None]): the row kernel would leave most lanes of a
+    // wave without a pack; the contiguous kernel walks the matrix flat and indexes the small
+    // operands by position modulo / divided by the row length.
+    if (pl.nd == 2 && pl.n < ((int64_t)1 << 32) && pl.strides[nops - 1][1] == 1 &&
+        pl.strides[nops - 1][0] == pl.shape[1] && pl.shape[1] * itemsize_of(dst->dtype) < 512) {
+        bool ok = true;
+        for (int k = 0; k + 1 < nops && ok; ++k) {
+            const int64_t s0 = pl.strides[k][0], s1 = pl.strides[k][1];
+            ok = (s0 == pl.shape[1] && s1 == 1) || (s0 == 0 && s1 == 1) || (s0 == 1 && s1 == 0) || (s0 == 0 && s1 == 0);
+        }
+        // rows of 8, 16 or 32 whole packs fill the lanes of the row kernel, which then is a little
+        // faster (fp32, 10^6 x 64 minus a row: 76 % against 72 % of peak)
+        int widest = 1;
+        for (int k = 0; k < nops; ++k) widest = std::max(widest, itemsize_of(views[k]->dtype));
+        const int64_t row_bytes = pl.shape[1] * widest;
+        if (row_bytes == 128 || row_bytes == 256 || row_bytes == 512) ok = false;
+        if (ok) {
+            pl.path = DPX_PATH_EW_CONTIG;
+            pl.flat2d = true;
+            return;
+        }
+    }
     // Transposed operands: the output runs along the inner dim, some input runs along another
     // dim dT (stride 1 there, a long stride along the inner dim).  All such inputs must agree
     // on dT; the others are read in output orientation.
@@ -117,9 +142,16 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     if (pl.path == DPX_PATH_EW_CONTIG) {
         pl.vec = true;
         pl.bcast = 0;
-        for (int k = 0; k < nops; ++k) {
-            if (k + 1 < nops && pl.strides[k][0] == 0 && pl.n > 1) pl.bcast |= 1u << k;
+        for (int k = 0; k + 1 < nops; ++k) {
+            uint32_t mode = BC_FULL;
+            if (pl.flat2d) {
+                const int64_t s0 = pl.strides[k][0], s1 = pl.strides[k][1];
+                mode = (s0 == 0 && s1 == 0) ? BC_SCALAR : (s0 == 0 ? BC_PERIODIC : (s1 == 0 ? BC_REPEAT : BC_FULL));
+            }
+            else if (pl.strides[k][0] == 0 && pl.n > 1) mode = BC_SCALAR;
+            pl.bcast |= mode << (2 * k);
         }
+        pl.period = pl.flat2d ? (uint32_t)pl.shape[1] : 1u;
         pl.block = env_block("DPX_EW_CONTIG_BLOCK", EW_CONTIG_BLOCK);
         pl.grid = (pl.n + (int64_t)pl.block * E * U - 1) / ((int64_t)pl.block * E * U);
         return;

@@ -172,6 +172,15 @@ def test_elementwise_plans():
     p = plan_binary("multiply", view([8192, 4096], [8192, 2]), view([8192, 4096], [0, 1], ptr=P1),
                     view([8192, 4096], ptr=P2))
     assert L.PATH_NAMES[p.path] == "ew_rows" and p.nd == 2 and list(p.shape[:2]) == [8192, 4096]
+    # a matrix with short rows and a row / a column: the contiguous kernel walks it flat
+    p = plan_binary("subtract", view([100000, 17]), view([100000, 17], [0, 1], ptr=P1), view([100000, 17], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_contig" and p.nd == 2 and p.grid[0] == -(-100000 * 17 // 256)
+    p = plan_binary("divide", view([100000, 17]), view([100000, 17], [1, 0], ptr=P1), view([100000, 17], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_contig"
+    p = plan_binary("subtract", view([100000, 128]), view([100000, 128], [0, 1], ptr=P1), view([100000, 128], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"  # 512-byte rows
+    p = plan_binary("subtract", view([100000, 17], [34, 2]), view([100000, 17], [0, 1], ptr=P1), view([100000, 17], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"  # strided matrix
     # empty
     p = plan_binary("add", view([0, 3]), view([0, 3]), view([0, 3]))
     assert L.PATH_NAMES[p.path] == "noop"

@@ -109,3 +109,37 @@ def test_reductions_over_odd_shapes_and_offsets(dt, shape):
             assert_same(host(dpt.min(da[sl], axis=axis)), np.min(a[sl], axis=axis))
             assert_same(host(dpt.argmax(da[sl], axis=axis)), np.argmax(a[sl], axis=axis))
             assert_same(host(dpt.count_nonzero(da[sl], axis=axis)), np.count_nonzero(a[sl], axis=axis).astype(np.int64))
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "f2", "i4", "f4", "f8", "c16"])
+def test_short_rows_with_row_and_column_operands(dt):
+    # x - mean(x, axis=0), x / norm(x, axis=1)[:, None]: rows shorter than 512 bytes are walked flat,
+    # the small operands indexed by position modulo / divided by the row length
+    rng = np.random.default_rng(13)
+    itemsize = np.dtype(dt).itemsize
+    for cols in (2, 3, 7, 16, 17, 33, 100, 127):
+        if cols * itemsize >= 512:
+            continue
+        for rows in (1, 5, 1000, 20011):
+            x = random_array(rng, (rows, cols), dt, lo=1, hi=9)
+            row = random_array(rng, (cols,), dt, lo=1, hi=9)
+            col = random_array(rng, (rows, 1), dt, lo=1, hi=9)
+            dx, drow, dcol = dev(x), dev(row), dev(col)
+            if dt == "?":
+                assert_same(host(dpt.logical_xor(dx, drow)), np.logical_xor(x, row))
+                assert_same(host(dpt.logical_and(dcol, dx)), np.logical_and(col, x))
+                continue
+            assert_same(host(dpt.subtract(dx, drow)), x - row)
+            assert_same(host(dpt.subtract(drow, dx)), row - x)
+            assert_same(host(dpt.add(dx, dcol)), x + col)
+            assert_same(host(dpt.add(dcol, drow)), col + row)
+            assert_same(host(dpt.less(dx, drow)), x < row)
+            assert_same(host(dpt.where(dx > drow, dx, dcol)), np.where(x > row, x, np.broadcast_to(col, x.shape)))
+            assert_same(host(dpt.clip(dx, drow, dcol)), orc.clip(x, np.broadcast_to(row, x.shape).copy(), np.broadcast_to(col, x.shape).copy()))
+            fill = random_array(rng, (rows, cols), dt)
+            o = dev(fill)
+            dpt.multiply(dx, drow, out=o)
+            if np.dtype(dt).kind != "c":
+                assert_same(host(o), x * row)
+            dpt.add(dx, drow, out=dx)  # in place
+            assert_same(host(dx), x + row)
