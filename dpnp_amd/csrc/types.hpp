@@ -244,6 +244,14 @@ template <class T, int N, bool NT = true> DPX_D void store_pack(T *p, const pack
         *reinterpret_cast<raw_t *>(p) = u.r;
 }
 
+// 16 bytes as four words (for code that works on words whatever the element type)
+template <bool NT = true> DPX_D u32x4 load_words16(const void *p)
+{
+    using raw_t = typename raw_of<16>::type;
+    if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(p));
+    else return *reinterpret_cast<const raw_t *>(p);
+}
+
 // Called on a loaded pack where its elements are first used, after every load of the thread has
 // been issued: the compiler then sees a use of all its bytes.  Without it, where only parts of
 // the elements are used (int16 -> int8 needs the low bytes), the 16-byte load is split into one

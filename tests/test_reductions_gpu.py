@@ -530,3 +530,34 @@ def test_statistics_over_samples_of_few_features(dt):
     a = rng.normal(size=(200003, 17)).astype(dt)
     r1, r2 = host(dpt.sum(dev(a), axis=0)), host(dpt.sum(dev(a), axis=0))
     assert_same(r1, r2)
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u1"])
+def test_one_byte_counting_reductions_word_arithmetic(dt):
+    # sum / any / all / count_nonzero of one-byte types fold 16 elements at a time with word arithmetic:
+    # every byte value, lengths around the pack and wave sizes, offsets, rows and full reductions
+    rng = np.random.default_rng(47)
+    every = np.arange(256, dtype="u1").view(dt) if dt != "?" else (np.arange(256) % 2).astype(bool)
+    for n in (1, 15, 16, 17, 255, 1024, 4099, 65536 + 5, 3000017):
+        a = np.resize(every, n).copy()
+        rng.shuffle(a)
+        for k in (0, 1, 3):
+            v, dv = a[k:], dev(a)[k:]
+            assert_same(host(dpt.sum(dv)), orc.reduce("sum", v, 1))
+            assert_same(host(dpt.count_nonzero(dv)), np.array(np.count_nonzero(v), "i8"))
+            assert bool(dpt.any(dv)) == bool(v.any()) and bool(dpt.all(dv)) == bool(v.all())
+    z = np.zeros(100003, dtype=dt)
+    assert not bool(dpt.any(dev(z))) and int(dpt.count_nonzero(dev(z))) == 0
+    z[77777] = True if dt == "?" else (-128 if dt == "i1" else 128)
+    assert bool(dpt.any(dev(z))) and int(dpt.count_nonzero(dev(z))) == 1 and not bool(dpt.all(dev(z)))
+    o = np.full(100003, 1 if dt != "i1" else -1, dtype=dt)
+    assert bool(dpt.all(dev(o)))
+    o[3] = 0
+    assert not bool(dpt.all(dev(o)))
+    m = np.resize(every, (257, 1031)).copy()
+    dm = dev(m)
+    assert_same(host(dpt.sum(dm, axis=1)), orc.reduce("sum", m, 1))
+    assert_same(host(dpt.count_nonzero(dm, axis=1)), np.count_nonzero(m, axis=1).astype("i8"))
+    assert_same(host(dpt.all(dm, axis=1)), m.astype(bool).all(axis=1))
+    assert_same(host(dpt.any(dm[:, :5], axis=1)), m[:, :5].astype(bool).any(axis=1))
+    assert_same(host(dpt.sum(dm, axis=1, dtype="i4")), orc.reduce("sum", m, 1, out_dtype="i4"))
