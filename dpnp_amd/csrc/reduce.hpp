@@ -817,6 +817,84 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c]);
 }
 
+// ================================ short rows kernel ===========================================
+// A row-major matrix with rows of at most 256 bytes, reduced along its rows (one result per row:
+// row norms of points, softmax statistics over a few classes).  With a lane or two per row the
+// rows kernel issues 16-byte loads a row pitch apart, which the memory pipeline serves badly, and
+// keeps few bytes in flight.  Here a block takes R consecutive rows, i.e. R * n contiguous
+// elements, reads them as one flat stream of packs (all loads of a thread issued before the
+// first use, up to 8 per thread), spreads the elements into LDS rows of an odd word pitch, and
+// thread r then folds rows r, r + 256, ... from LDS (conflict-free across r) in element order.
+// L.chunk = R, at most 2048.
+constexpr int SROW_LDS_BYTES = 32768;
+// elements per LDS row for an element size: the row padded to a whole and odd number of words
+// (8- and 16-byte elements: an odd number of elements)
+DPX_HD constexpr int srow_pitch_for(int n, int size)
+{
+    if (size >= 4) return n | 1;
+    const int per_word = 4 / size;
+    return (((n + per_word - 1) / per_word) | 1) * per_word;
+}
+template <class In> DPX_HD constexpr int srow_pitch(int n) { return srow_pitch_for(n, (int)sizeof(In)); }
+
+template <class P>
+__global__ __launch_bounds__(256) void red_short_rows_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
+                                                            typename P::Out *dst, const typename P::Aux *aux)
+{
+    using In = typename P::In;
+    using Acc = typename P::Acc;
+    constexpr int E = 16 / (int)sizeof(In);
+    constexpr int MAXP = SROW_LDS_BYTES / 16 / 256; // packs per thread: 8
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    In *sm = reinterpret_cast<In *>(smem_raw);
+    const int t = (int)threadIdx.x;
+    const uint32_t n = (uint32_t)L.n;
+    const int pitch = srow_pitch<In>((int)n);
+    const int64_t row0 = (int64_t)blockIdx.x * L.chunk;
+    const int R = (int)((row0 + L.chunk < L.m) ? L.chunk : L.m - row0);
+    const uint32_t elems = (uint32_t)R * n;
+    const uint32_t packs = elems / E;
+    const In *p = src + row0 * n;
+    pack<In, E> v[MAXP];
+#pragma unroll
+    for (int k = 0; k < MAXP; ++k) {
+        const uint32_t q = (uint32_t)t + (uint32_t)k * 256u;
+        if (q < packs) v[k] = load_pack<In, E>(p + (int64_t)q * E);
+    }
+#pragma unroll
+    for (int k = 0; k < MAXP; ++k) {
+        const uint32_t q = (uint32_t)t + (uint32_t)k * 256u;
+        if (q < packs) {
+            uint32_t r = (q * E) / n, c = q * E - r * n;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                sm[r * pitch + c] = v[k].v[e];
+                if (++c == n) {
+                    c = 0;
+                    ++r;
+                }
+            }
+        }
+    }
+    { // the elements after the last whole pack (fewer than E)
+        const uint32_t i = packs * E + (uint32_t)t;
+        if (i < elems) {
+            const uint32_t r = i / n;
+            sm[r * pitch + (i - r * n)] = load_one(p + i);
+        }
+    }
+    __syncthreads();
+    for (int r = t; r < R; r += 256) { // very short rows: several rows per thread
+        const int64_t o = row0 + r;
+        Acc a = P::identity();
+        if constexpr (P::has_aux) a = P::load_aux(aux + o * ix.aux_str[0]);
+        const In *row = sm + r * pitch;
+        Acc acc = P::identity();
+        for (uint32_t j = 0; j < n; ++j) acc = P::combine(acc, P::pre(row[j], a));
+        dst[o * ix.dst_str[0]] = P::post(acc);
+    }
+}
+
 // identity fill for an empty reduced run (reductions.hpp:1417-1422)
 template <class P>
 __global__ __launch_bounds__(256) void red_fill_kernel(RedIndex ix, int64_t m, typename P::Out *dst)

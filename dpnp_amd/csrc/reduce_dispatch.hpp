@@ -63,6 +63,11 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         hipLaunchKernelGGL((red_cols_kernel<P>), dim3((unsigned)pl.grid), dim3(block), smem, stream, pl.ix, pl.L, sp,
                            dp, partial, ap, counters);
     }
+    else if (pl.path == DPX_PATH_RED_SHORT_ROWS) {
+        const size_t smem = (size_t)pl.L.chunk * srow_pitch<In>((int)pl.L.n) * sizeof(In); // at most 32 KiB
+        hipLaunchKernelGGL((red_short_rows_kernel<P>), dim3((unsigned)pl.grid), dim3(256), smem, stream, pl.ix, pl.L,
+                           sp, dp, ap);
+    }
     else if (pl.path == DPX_PATH_RED_FLAT) {
         const size_t smem = (size_t)pl.block * cols_cfg<In>::E * sizeof(Acc); // at most 32 KiB
         hipLaunchKernelGGL((red_flat_kernel<P>), dim3((unsigned)pl.grid), dim3(pl.block), smem, stream, pl.ix, pl.L,

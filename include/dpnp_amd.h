@@ -247,8 +247,9 @@ typedef enum dpx_path {
     DPX_PATH_RED_COLS_SPLIT = 13, /* ... reduced run split over blocks, folded by the last one */
     DPX_PATH_RED_GENERIC = 14,  /* fully strided */
     DPX_PATH_RED_SMALL = 15,    /* tiny reduced run: one thread per output */
-    DPX_PATH_RED_FLAT = 16      /* row-major matrix with short rows reduced over its rows: a flat
+    DPX_PATH_RED_FLAT = 16,     /* row-major matrix with short rows reduced over its rows: a flat
                                    stream of 16-byte packs, column = position modulo row length */
+    DPX_PATH_RED_SHORT_ROWS = 17 /* ... reduced along its rows: a block stages whole rows in LDS */
 } dpx_path;
 
 typedef struct dpx_plan {

@@ -201,7 +201,14 @@ def test_reduction_plans():
     # axis=0 of a C-contiguous matrix: the caller passes the transposed view
     p = plan_reduce("sum", view([16384, 16384], [1, 16384]), 1, view([16384], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_cols_split" and p.vec == 1
+    # rows of at most 256 bytes, one result per row: whole rows staged in LDS (32 KiB of padded rows per block)
     p = plan_reduce("sum", view([1 << 20, 4]), 1, view([1 << 20], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_short_rows" and p.block == 256 and p.grid[0] == -(-(1 << 20) // (32768 // 20))
+    p = plan_reduce("max", view([1 << 20, 64]), 1, view([1 << 20], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_short_rows" and p.grid[0] == -(-(1 << 20) // (32768 // (65 * 4)))
+    p = plan_reduce("sum", view([1 << 20, 65]), 1, view([1 << 20], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_small", "red_rows")
+    p = plan_reduce("sum", view([1 << 20, 4], [8, 1]), 1, view([1 << 20], ptr=P1))  # padded rows
     assert L.PATH_NAMES[p.path] in ("red_small", "red_rows")
     # reduce a middle axis of (a, r, c): outputs contiguous along c
     p = plan_reduce("max", view([8, 64, 1000], [64000, 1, 64]), 1, view([8, 64], ptr=P1))

@@ -561,3 +561,59 @@ def test_one_byte_counting_reductions_word_arithmetic(dt):
     assert_same(host(dpt.all(dm, axis=1)), m.astype(bool).all(axis=1))
     assert_same(host(dpt.any(dm[:, :5], axis=1)), m[:, :5].astype(bool).any(axis=1))
     assert_same(host(dpt.sum(dm, axis=1, dtype="i4")), orc.reduce("sum", m, 1, out_dtype="i4"))
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "f2", "f4", "f8", "c8", "c16"])
+def test_last_axis_of_matrices_with_short_rows(dt):
+    # rows of at most 256 bytes reduced along the row: a block stages whole rows in LDS
+    rng = np.random.default_rng(53)
+    itemsize = np.dtype(dt).itemsize
+    for cols in (2, 3, 4, 5, 8, 10, 16, 17, 31, 32, 33, 63, 64, 128, 256):
+        if cols * itemsize > 256:
+            continue
+        for rows in (64, 65, 255, 256, 257, 1000, 40009):
+            a = random_array(rng, (rows, cols), dt, lo=-3, hi=3)
+            da = dev(a)
+            check_sum(host(dpt.sum(da, axis=1)), a, 1)
+            assert_same(host(dpt.max(da, axis=-1)), orc.reduce("max", a, 1))
+            assert_same(host(dpt.min(da, axis=-1)), orc.reduce("min", a, 1))
+            assert_same(host(dpt.all(da, axis=1)), a.astype(bool).all(axis=1))
+            assert_same(host(dpt.count_nonzero(da, axis=1)), np.count_nonzero(a, axis=1).astype("i8"))
+    a = random_array(rng, (5000, 3, 7), dt, lo=-3, hi=3)  # outer dims collapse into the rows
+    da = dev(a)
+    assert_same(host(dpt.max(da, axis=2)), orc.reduce("max", a, 1))
+    check_sum(host(dpt.sum(da, axis=(1, 2))), a.reshape(5000, 21), 1)
+    b = random_array(rng, (5000, 10), dt, lo=-3, hi=3)
+    db = dev(b)
+    assert_same(host(dpt.max(db[7:], axis=1)), orc.reduce("max", b[7:], 1))  # view that starts at a later row
+    out = dpt.zeros(10000, dtype=dt)
+    dpt.max(db, axis=1, out=out[::2])
+    assert_same(host(out)[::2], orc.reduce("max", b, 1))
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+def test_per_row_statistics_of_short_rows(dt):
+    # (points, 3) norms, (samples, classes) softmax statistics: mean / var / logsumexp / hypot / nan forms
+    rng = np.random.default_rng(59)
+    tol = dict(rtol=2e-5, atol=1e-5) if dt == "f4" else dict(rtol=1e-12, atol=1e-12)
+    for cols in (3, 10, 17, 32 if dt == "f8" else 64):
+        a = rng.normal(1.0, 2.0, (30011, cols)).astype(dt)
+        da = dev(a)
+        a64 = a.astype("f8") if dt == "f4" else a.astype(np.longdouble)
+        np.testing.assert_allclose(host(dpt.mean(da, axis=1)), a64.mean(axis=1).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.var(da, axis=1)), a64.var(axis=1).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.std(da, axis=1, correction=1)), a64.std(axis=1, ddof=1).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.reduce_hypot(da, axis=1)), np.sqrt((a64 * a64).sum(axis=1)).astype(dt), **tol)
+        mx = a64.max(axis=1, keepdims=True)
+        np.testing.assert_allclose(host(dpt.logsumexp(da, axis=1)),
+                                   (mx[:, 0] + np.log(np.exp(a64 - mx).sum(axis=1))).astype(dt), **tol)
+        np.testing.assert_allclose(host(dpt.prod(dev(a[:, :5]), axis=1)), a64[:, :5].prod(axis=1).astype(dt), **tol)
+        b = a.copy()
+        b[rng.random(b.shape) < 0.2] = np.nan
+        b[:, 0] = 1.0
+        b64 = b.astype("f8") if dt == "f4" else b.astype(np.longdouble)
+        db = dpnp.asarray(b)
+        np.testing.assert_allclose(dpnp.nansum(db, axis=1).asnumpy(), np.nansum(b64, axis=1).astype(dt), **tol)
+        np.testing.assert_allclose(dpnp.nanmean(db, axis=1).asnumpy(), np.nanmean(b64, axis=1).astype(dt), **tol)
+        np.testing.assert_allclose(dpnp.nanvar(db, axis=1).asnumpy(), np.nanvar(b64, axis=1).astype(dt), **tol)
+        assert_same(dpnp.nanmin(db, axis=1).asnumpy(), np.nanmin(b, axis=1))
