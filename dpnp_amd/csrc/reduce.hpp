@@ -1277,4 +1277,66 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     if (ty == 0 && active) write_out();
 }
 
+// Short rows variant (see red_short_rows_kernel): position of the extremum of each row of a
+// row-major matrix with rows of at most 256 bytes (the predicted class of each sample).
+template <class T, bool IS_MAX>
+__global__ __launch_bounds__(256) void arg_short_rows_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst)
+{
+    using VT = value_of_t<T>;
+    constexpr int E = 16 / (int)sizeof(T);
+    constexpr int MAXP = SROW_LDS_BYTES / 16 / 256;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *sm = reinterpret_cast<T *>(smem_raw);
+    const int t = (int)threadIdx.x;
+    const uint32_t n = (uint32_t)L.n;
+    const int pitch = srow_pitch<T>((int)n);
+    const int64_t row0 = (int64_t)blockIdx.x * L.chunk;
+    const int R = (int)((row0 + L.chunk < L.m) ? L.chunk : L.m - row0);
+    const uint32_t elems = (uint32_t)R * n;
+    const uint32_t packs = elems / E;
+    const T *p = src + row0 * n;
+    pack<T, E> v[MAXP];
+#pragma unroll
+    for (int k = 0; k < MAXP; ++k) {
+        const uint32_t q = (uint32_t)t + (uint32_t)k * 256u;
+        if (q < packs) v[k] = load_pack<T, E>(p + (int64_t)q * E);
+    }
+#pragma unroll
+    for (int k = 0; k < MAXP; ++k) {
+        const uint32_t q = (uint32_t)t + (uint32_t)k * 256u;
+        if (q < packs) {
+            uint32_t r = (q * E) / n, c = q * E - r * n;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                sm[r * pitch + c] = v[k].v[e];
+                if (++c == n) {
+                    c = 0;
+                    ++r;
+                }
+            }
+        }
+    }
+    {
+        const uint32_t i = packs * E + (uint32_t)t;
+        if (i < elems) {
+            const uint32_t r = i / n;
+            sm[r * pitch + (i - r * n)] = load_one(p + i);
+        }
+    }
+    __syncthreads();
+    for (int r = t; r < R; r += 256) {
+        const T *row = sm + r * pitch;
+        VT best = to_value(row[0]);
+        uint32_t bj = 0;
+        for (uint32_t j = 1; j < n; ++j) {
+            const VT x = to_value(row[j]);
+            if (arg_better<IS_MAX, VT>(x, best)) {
+                best = x;
+                bj = j;
+            }
+        }
+        dst[(row0 + r) * ix.dst_str[0]] = (int64_t)bj;
+    }
+}
+
 } // namespace dpx

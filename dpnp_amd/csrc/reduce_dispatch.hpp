@@ -101,7 +101,12 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         pidx = (Slot<int64_t> *)(s + RED_COUNTER_BYTES);
         pval = (Slot<T> *)(s + RED_COUNTER_BYTES + (size_t)pl.scratch_elems * sizeof(Slot<int64_t>));
     }
-    if (red_is_cols(pl))
+    if (pl.path == DPX_PATH_RED_SHORT_ROWS) {
+        const size_t smem = (size_t)pl.L.chunk * srow_pitch<T>((int)pl.L.n) * sizeof(T);
+        hipLaunchKernelGGL((arg_short_rows_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(256), smem, stream, pl.ix,
+                           pl.L, sp, dp);
+    }
+    else if (red_is_cols(pl))
         hipLaunchKernelGGL((arg_cols_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.ix, pl.L,
                            sp, dp, pval, pidx, counters);
     else if (pl.path == DPX_PATH_RED_GENERIC)

@@ -153,7 +153,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const bool cols_ok = !contig_red && nd_r == 1 && istr[0][last] == 1 && inner > 1;
     RedLaunch &L = pl.L;
 
-    if (contig_red && !arg && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
+    if (contig_red && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
         env_int("DPX_RED_SHORT_ROWS", 1) != 0) { // (experiment knob: 0 keeps the rows kernel)
         // ---- short rows: a block stages R whole rows in LDS (see red_short_rows_kernel) ----
         const int64_t pitch_bytes = (int64_t)srow_pitch_for((int)n, in_size) * in_size;

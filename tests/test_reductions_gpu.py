@@ -617,3 +617,32 @@ def test_per_row_statistics_of_short_rows(dt):
         np.testing.assert_allclose(dpnp.nanmean(db, axis=1).asnumpy(), np.nanmean(b64, axis=1).astype(dt), **tol)
         np.testing.assert_allclose(dpnp.nanvar(db, axis=1).asnumpy(), np.nanvar(b64, axis=1).astype(dt), **tol)
         assert_same(dpnp.nanmin(db, axis=1).asnumpy(), np.nanmin(b, axis=1))
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "f2", "f4", "f8", "c8"])
+def test_argmax_argmin_along_short_rows(dt):
+    # the predicted class of each sample: first position of the extremum, the first NaN wins
+    rng = np.random.default_rng(61)
+    itemsize = np.dtype(dt).itemsize
+    for cols in (2, 3, 5, 10, 17, 32, 33, 64, 100):
+        if cols * itemsize > 256:
+            continue
+        for rows in (64, 257, 3001, 50021):
+            a = random_array(rng, (rows, cols), dt, lo=-4, hi=4)  # many ties
+            if np.dtype(dt).kind == "f":
+                a[rng.random(a.shape) < 0.02] = np.nan
+                a[1, :] = np.nan
+            da = dev(a)
+            assert_same(host(dpt.argmax(da, axis=1)), orc.argreduce("argmax", a, 1))
+            assert_same(host(dpt.argmin(da, axis=-1)), orc.argreduce("argmin", a, 1))
+    a = rng.normal(size=(4001, 3, 7)).astype("f4") if dt == "f4" else None
+    if a is not None:
+        a[rng.random(a.shape) < 0.1] = np.nan
+        a[:, 0, 0] = 0.0
+        da = dpnp.asarray(a)
+        assert_same(host(dpt.argmax(dev(a), axis=2)), orc.argreduce("argmax", a, 1))
+        assert_same(dpnp.nanargmax(da, axis=2).asnumpy(), np.nanargmax(a, axis=2))
+        assert_same(dpnp.nanargmin(da[:, 0, :], axis=1).asnumpy(), np.nanargmin(a[:, 0, :], axis=1))
+        out = dpt.zeros(2 * 4001, dtype="i8")
+        dpt.argmax(dev(a[:, 1, :]), axis=1, out=out[::2])
+        assert_same(host(out)[::2], orc.argreduce("argmax", a[:, 1, :], 1))
