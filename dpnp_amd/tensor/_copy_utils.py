@@ -29,8 +29,10 @@ def _like_strides(shape, stride_lists, dt):
     return permute_dims(r, inv)
 
 
-def _empty_like_orderK(x, dt):
+def _empty_like_orderK(x, dt, usm_type=None, dev=None):
     """Same shape as `x`, dtype `dt`, strides ordered like x's (C stays C, F stays F)."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray, got {type(x)}")
     fl = x.flags
     if fl.c_contiguous or x.size <= 1:
         return _empty(x.shape, dt, "C")
@@ -39,7 +41,10 @@ def _empty_like_orderK(x, dt):
     return _like_strides(x.shape, [x.strides], dt)
 
 
-def _empty_like_pair_orderK(x1, x2, dt, res_shape):
+def _empty_like_pair_orderK(x1, x2, dt, res_shape, usm_type=None, dev=None):
+    for x in (x1, x2):
+        if not isinstance(x, usm_ndarray):
+            raise TypeError(f"Expected usm_ndarray, got {type(x)}")
     nd1, nd2 = x1.ndim, x2.ndim
     if nd1 > nd2 and x1.shape == res_shape:
         return _empty_like_orderK(x1, dt)
@@ -119,10 +124,18 @@ def from_numpy(np_ary, /, *, dtype=None, order="K"):
     """New device array with the contents of a NumPy array."""
     a = np.asarray(np_ary)
     src_dt = _as_dtype(a.dtype)
+    keep_nesting = order == "K" and a.ndim > 1 and a.size > 1 and not (a.flags.c_contiguous or a.flags.f_contiguous)
     if order == "K":
         order = "F" if (a.flags.f_contiguous and not a.flags.c_contiguous) else "C"
     elif order == "A":
         order = "F" if (a.flags.f_contiguous and not a.flags.c_contiguous) else "C"
+    if keep_nesting:
+        # order "K" of an array that is neither C- nor F-contiguous: keep the nesting of its axes
+        # (a permuted contiguous array gets the same strides: dpnp/tensor/_copy_utils.py:837-856)
+        perm = sorted(range(a.ndim), key=lambda d: (-abs(a.strides[d]) if a.shape[d] > 1 else 0, d))
+        inv = sorted(range(a.ndim), key=lambda i: perm[i])
+        r = from_numpy(np.ascontiguousarray(a.transpose(perm)), dtype=dtype, order="C")
+        return permute_dims(r, inv)
     host = np.asarray(a, dtype=src_dt, order=order)
     if not (host.flags.c_contiguous or host.flags.f_contiguous):
         host = np.ascontiguousarray(host)
@@ -164,13 +177,15 @@ def _assign(dst_view, value):
         return
     else:
         src = from_numpy(np.asarray(value))
-    if dst_view.size == 0:
-        return
+    if src.ndim > dst_view.ndim and all(s == 1 for s in src.shape[: src.ndim - dst_view.ndim]):
+        src = src._view(src.shape[src.ndim - dst_view.ndim:], src.strides[src.ndim - dst_view.ndim:], src._offset)
     if src.shape != dst_view.shape:
         try:
             src = broadcast_to(src, dst_view.shape)
         except ValueError:
             raise ValueError(f"Shape of the value {src.shape} can not be broadcast to {dst_view.shape}")
+    if dst_view.size == 0:
+        return
     if ti._array_overlap(src, dst_view) and not ti._same_logical_tensors(src, dst_view):
         src = copy(src)
         if src.shape != dst_view.shape:

@@ -3,7 +3,7 @@ ones, full, asarray, arange, linspace-free minimal set and their *_like forms.""
 import numpy as np
 
 from . import _tensor_impl as ti
-from ._copy_utils import _empty_like_orderK, astype, copy, from_numpy
+from ._copy_utils import _empty_like_orderK, asnumpy, astype, copy, from_numpy
 from ._dtypes import dtype as _as_dtype
 from ._usmarray import usm_ndarray
 
@@ -85,10 +85,35 @@ def ones_like(x, /, *, dtype=None, order="K", device=None, usm_type=None, sycl_q
     return full_like(x, 1, dtype=dtype, order=order)
 
 
-def asarray(obj, /, *, dtype=None, device=None, copy=None, usm_type=None, sycl_queue=None, order="K"):
-    """Convert `obj` (device array, NumPy array, nested sequence or scalar) to a device array."""
+def _host_image(obj):
+    """Nested sequences with device arrays replaced by their host copies (for np.asarray)."""
     if isinstance(obj, usm_ndarray):
-        tgt = obj.dtype if dtype is None else _as_dtype(dtype)
+        return asnumpy(obj)
+    if hasattr(obj, "get_array") and isinstance(obj.get_array(), usm_ndarray):
+        return asnumpy(obj.get_array())
+    if isinstance(obj, (list, tuple)):
+        return [_host_image(o) for o in obj]
+    return obj
+
+
+def asarray(obj, /, *, dtype=None, device=None, copy=None, usm_type=None, sycl_queue=None, order="K"):
+    """Convert `obj` (device array, NumPy array, nested sequence or scalar) to a device array
+    (dpnp/tensor/_ctors.py:560-760)."""
+    if copy is not None and not isinstance(copy, bool):
+        raise TypeError(f"Argument 'copy' is expected to be a boolean or None, got {type(copy)}")
+    if not isinstance(order, str):
+        raise TypeError(f"Expected order keyword to be of type str, got {type(order)}")
+    if order.upper() not in ("K", "C", "F", "A"):
+        raise ValueError("Unrecognized order keyword value, expecting 'K', 'A', 'F', or 'C'.")
+    if usm_type is not None:
+        if not isinstance(usm_type, str):
+            raise TypeError(f"Expected usm_type to be a str or None, got {type(usm_type)}")
+        if usm_type not in ("device", "shared", "host"):
+            raise ValueError(f"Unrecognized value of usm_type={usm_type}, expected 'device', 'shared', 'host'")
+    if dtype is not None:
+        dtype = _as_dtype(dtype)
+    if isinstance(obj, usm_ndarray):
+        tgt = obj.dtype if dtype is None else dtype
         c, f = obj.flags.c_contiguous, obj.flags.f_contiguous
         layout_ok = order in ("K", "k") or (order in ("A", "a") and (c or f)) or \
             (order in ("C", "c") and c) or (order in ("F", "f") and f)
@@ -101,8 +126,15 @@ def asarray(obj, /, *, dtype=None, device=None, copy=None, usm_type=None, sycl_q
         return asarray(obj.get_array(), dtype=dtype, copy=copy, order=order)
     if copy is False:
         raise ValueError("Converting a host object to a device array requires a copy")
-    a = np.asarray(obj)
+    if isinstance(obj, (list, tuple)):
+        obj = _host_image(obj)
+    if isinstance(obj, int) and not isinstance(obj, bool) and dtype is not None:
+        a = np.asarray(obj, dtype=dtype)  # raises OverflowError for values outside the dtype
+    else:
+        a = np.asarray(obj)
     if a.dtype == object:
+        if isinstance(obj, int):
+            raise OverflowError("Python int too large to convert to a device integer")
         raise TypeError("object arrays are not supported")
     if dtype is None:
         # Python scalars and sequences: NumPy's defaults (int64, float64, complex128)

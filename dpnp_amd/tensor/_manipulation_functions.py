@@ -3,13 +3,15 @@ squeeze, expand_dims (behaviour of dpnp/tensor/_manipulation_functions.py and
 dpnp/tensor/_reshape.py for these five)."""
 import operator
 
+import numpy as np
+
 from ._usmarray import usm_ndarray
 
 
 def normalize_axis_index(axis, ndim, name="axis"):
     axis = operator.index(axis)
     if axis < -ndim or axis >= ndim:
-        raise IndexError(f"{name} {axis} is out of bounds for array of dimension {ndim}")
+        raise np.exceptions.AxisError(f"{name} {axis} is out of bounds for array of dimension {ndim}")
     return axis + ndim if axis < 0 else axis
 
 
@@ -136,8 +138,17 @@ def _reshape_strides(shape, strides, new_shape):
 def reshape(x, shape, /, *, order="C", copy=None):
     if not isinstance(x, usm_ndarray):
         raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    if order in ("F", "f"):
+        # column-major reshape: the row-major reshape of the array with its axes reversed, reversed again
+        # (dpnp/tensor/_reshape.py:98-190)
+        if isinstance(shape, (tuple, list)):
+            rshape = tuple(shape)[::-1]
+        else:
+            rshape = (shape,)
+        r = reshape(permute_dims(x, tuple(range(x.ndim - 1, -1, -1))), rshape, order="C", copy=copy)
+        return permute_dims(r, tuple(range(r.ndim - 1, -1, -1)))
     if order not in ("C", "c"):
-        raise ValueError("only order='C' reshapes are supported")
+        raise ValueError(f"Keyword 'order' not recognized. Expecting 'C' or 'F', got {order}")
     shape = [operator.index(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,))]
     if shape.count(-1) > 1:
         raise ValueError("Only one dimension of the new shape may be -1")

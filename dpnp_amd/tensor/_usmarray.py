@@ -254,6 +254,11 @@ class usm_ndarray:
         return _device.default_queue().sycl_device
 
     @property
+    def usm_data(self):
+        """The allocation this array lives in (one object for an array and all of its views)."""
+        return self._buf
+
+    @property
     def _pointer(self):
         return self._buf.data_ptr() + self._offset * self._dtype.itemsize
 
