@@ -34,7 +34,7 @@ def full(shape, fill_value, *, dtype=None, order="C", device=None, usm_type=None
             dtype = "i8"
         elif isinstance(fill_value, complex):
             dtype = "c16"
-        elif isinstance(fill_value, np.generic):
+        elif isinstance(fill_value, (np.generic, np.ndarray)):
             dtype = fill_value.dtype
         else:
             dtype = "f8"

@@ -282,3 +282,150 @@ def test_setitem_broadcasting_scalars_and_errors():
     d = dpt.empty(4, dtype="int32")
     d[:] = np.arange(4, dtype="intc")
     assert_same(host(d), np.arange(4, dtype="i4"))
+
+
+# ---- zeros / ones / full / arange / linspace / *_like: test_usm_ndarray_ctor.py:1278-1720, 2100-2215 ----
+@pytest.mark.parametrize("dt", ALL, ids=str)
+def test_filled_constructors_every_dtype(dt):
+    assert_same(host(dpt.zeros(10, dtype=dt)), np.zeros(10, dtype=dt))
+    assert_same(host(dpt.ones(10, dtype=dt)), np.ones(10, dtype=dt))
+    assert_same(host(dpt.full(10, 4, dtype=dt)), np.full(10, 4, dtype=dt))
+    np.testing.assert_allclose(host(dpt.linspace(0, 1, num=2, dtype=dt)), np.linspace(0, 1, num=2, dtype=dt))
+    for shape in ((4, 5), ()):
+        x = dpt.empty(shape, dtype=dt)
+        e = dpt.empty_like(x)
+        assert e.shape == x.shape and e.dtype == x.dtype
+        assert_same(host(dpt.zeros_like(x)), np.zeros(shape, dtype=dt))
+        assert_same(host(dpt.ones_like(x)), np.ones(shape, dtype=dt))
+        assert_same(host(dpt.full_like(x, np.dtype(dt).type(1))), np.ones(shape, dtype=dt))
+    if dt != np.dtype("?"):
+        x = dpt.arange(0, 123, dtype=dt)
+        assert complex(x[47]) == 47
+        assert dpt.arange(128, dtype=dt).shape == (128,) and dpt.arange(127, 0, -1, dtype=dt).shape == (127,)
+
+
+def test_full_inference_special_values_and_array_fill():
+    for v in (1 + 1j, 0 + 1j, 0 + 0j):
+        assert_same(host(dpt.full((), fill_value=v, dtype="c16")), np.full((), v, dtype="c16"))
+    assert np.issubdtype(dpt.full(10, 4).dtype, np.integer)
+    assert dpt.full(10, True).dtype == np.dtype(bool)
+    assert np.issubdtype(dpt.full(10, 12.3).dtype, np.floating)
+    assert np.issubdtype(dpt.full(10, 0.3 - 2j).dtype, np.complexfloating)
+    assert np.issubdtype(dpt.full(10, 12.3, dtype=int).dtype, np.integer)
+    assert np.issubdtype(dpt.full(10, 0.3 - 2j, dtype=int).dtype, np.integer)
+    assert np.issubdtype(dpt.full(10, 0.3 - 2j, dtype="f8").dtype, np.floating)
+    for dt in ("f2", "f4", "f8"):
+        assert bool(dpt.isnan(dpt.full(10, fill_value=dpt.nan, dtype=dt)[0]))
+        hi, lo = dpt.full(10, fill_value=dpt.inf, dtype=dt)[0], dpt.full(10, fill_value=-dpt.inf, dtype=dt)[0]
+        assert bool(dpt.isinf(hi)) and bool(dpt.greater(hi, 0)) and bool(dpt.isinf(lo)) and bool(dpt.less(lo, 0))
+        ar = dpt.full(10, fill_value=dpt.pi, dtype=dt)
+        assert abs(float(ar[0]) - dpt.pi) < 16 * dpt.finfo(ar.dtype).eps
+    xnp = np.array([1, 2, 3], dtype="i4")
+    y = dpt.full((3, 3), dpt.asarray(xnp))
+    assert y.dtype == np.int32
+    assert_same(host(y), np.full((3, 3), xnp))
+    x = dpt.arange(10, dtype="i4")
+    y = dpt.full(10, x[3])
+    assert y.dtype == x.dtype
+    assert_same(host(y), np.full(10, 3, dtype="i4"))
+    assert_same(host(dpt.full(10, x[3], dtype="f4")), np.full(10, 3, dtype="f4"))
+    for o1 in "FC":
+        for o2 in "FC":
+            src = np.array([1, 2, 3], order=o1)
+            want = np.full((3, 3), src, order=o2)
+            got = dpt.full((3, 3), src, order=o2)
+            assert got.flags.c_contiguous == want.flags.c_contiguous and got.flags.f_contiguous == want.flags.f_contiguous
+            assert_same(host(got), want)
+    for fill in (dpt.arange(3, dtype="i4"), dpt.arange(6, dtype="i4")[::2]):
+        got = dpt.full((3, 3), fill)
+        assert got.strides == (3, 1)
+        assert_same(host(got), np.full((3, 3), host(fill)))
+    for dt in ("i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8"):
+        with pytest.raises(OverflowError):
+            dpt.full(1, int(np.iinfo(dt).max) + 1, dtype=dt)
+    with pytest.raises(TypeError):
+        dpt.empty(1, dtype=np.object_)
+
+
+def test_arange_and_linspace_rules():
+    assert dpt.arange(7, 0, -2, dtype="f4").shape == (4,) and dpt.arange(0, 1, 0.25, dtype="f4").shape == (4,)
+    assert dpt.arange(7, 0, -2, dtype="f8").shape == (4,)
+    x = dpt.arange(9.7, stop=10)
+    assert x.shape == (1,) and x.dtype == np.float64
+    assert dpt.arange(0, stop=10, step=None, dtype="int32").shape == (10,)
+    b = dpt.arange(0, stop=2, dtype="bool")
+    assert b.shape == (2,) and b.dtype == np.dtype(bool)
+    x = dpt.arange(-2.5, stop=200, step=100, dtype="int32")
+    assert x.shape[0] == 3 and int(x[1]) == 99 + int(x[0])
+    x = dpt.arange(+2.5, stop=200, step=100, dtype="int32")
+    assert x.shape[0] == 2 and int(x[1]) == 100 + int(x[0])
+    assert dpt.arange(0, stop=np.float32(504), step=100, dtype="f4").shape == (6,)
+    assert dpt.arange(-5, stop=10**2, step=2.7, dtype="int64").shape == (39,)  # length from the uncast arguments
+    x = dpt.linspace(0, 15, num=16)
+    assert x.dtype == np.float64 and x.shape == (16,) and x.strides == (1,)
+    for dt in ("f2", "f4", "f8"):
+        mx = np.finfo(dt).max
+        x = dpt.linspace(mx, mx, endpoint=True, num=16, dtype=dt)
+        assert x.shape == (16,)
+        np.testing.assert_allclose(host(x), np.linspace(mx, mx, endpoint=True, num=16, dtype=dt))
+    assert_same(host(dpt.linspace(0.1, 9.1, 11, endpoint=True, dtype=int)), np.linspace(0.1, 9.1, 11, endpoint=True, dtype=int))
+
+
+def test_like_constructors_layout():
+    sh = (10, 10)
+    likes = (lambda x, o: dpt.full_like(x, 2, order=o), lambda x, o: dpt.empty_like(x, order=o),
+             lambda x, o: dpt.ones_like(x, order=o), lambda x, o: dpt.zeros_like(x, order=o))
+    values = (2, None, 1, 0)
+    for order in "KA":
+        for src_order, flag in (("C", "c_contiguous"), ("F", "f_contiguous")):
+            x = dpt.zeros(sh, dtype="i4", order=src_order)
+            for mk, v in zip(likes, values):
+                r = mk(x, order)
+                assert getattr(r.flags, flag)
+                assert v is None or (host(r) == v).all()
+        x3 = dpt.zeros(sh, dtype="i4", order="C")[::-2, :5]
+        for mk, v in zip(likes, values):
+            r = mk(x3, order)
+            if order == "K":
+                assert r.strides == (-5, 1) and not r.flags.forc
+            else:
+                assert r.flags.c_contiguous
+            assert v is None or (host(r) == v).all()
+    x = dpt.zeros(sh, dtype="i4")
+    assert (host(dpt.full_like(x, dpt.asarray(2, dtype="i4"), order="K")) == 2).all()
+    col = dpt.arange(10, dtype="i4")[:, dpt.newaxis]
+    assert_same(host(dpt.full_like(x, col, order="K")), np.tile(np.arange(10, dtype="i4")[:, None], (1, 10)))
+
+
+# ---- dtype routines: test_tensor_dtype_routines.py:73-172 ---------------------------------------------
+def test_isdtype_finfo_iinfo():
+    names = ["bool", "int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64",
+             "float16", "float32", "float64", "complex64", "complex128"]
+    cats = {
+        "bool": ["bool"],
+        "signed integer": ["int8", "int16", "int32", "int64"],
+        "unsigned integer": ["uint8", "uint16", "uint32", "uint64"],
+        "integral": ["int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64"],
+        "real floating": ["float16", "float32", "float64"],
+        "complex floating": ["complex64", "complex128"],
+        "numeric": [d for d in names if d != "bool"],
+    }
+    for name in names:
+        dt = dpt.dtype(name)
+        for kind, members in cats.items():
+            assert dpt.isdtype(dt, kind) == (name in members)
+    assert dpt.isdtype(dpt.bool, ("real floating", "bool")) and not dpt.isdtype(dpt.bool, ("integral", "real floating"))
+    assert dpt.isdtype(dpt.int16, ("real floating", "signed integer"))
+    assert not dpt.isdtype(dpt.int16, ("bool", "unsigned integer", "real floating"))
+    assert dpt.isdtype(dpt.uint8, (dpt.uint8, dpt.uint16)) and not dpt.isdtype(dpt.uint8, (dpt.bool, dpt.int32, dpt.float32))
+    assert dpt.isdtype(dpt.float32, (dpt.float16, dpt.float32, dpt.float64))
+    assert dpt.isdtype(dpt.complex64, ("integral", "complex floating"))
+    for bad in ([dpt.int32, dpt.bool], "f4", float, 123, "complex"):
+        with pytest.raises((TypeError, ValueError)):
+            dpt.isdtype(dpt.int32, bad)
+    assert dpt.finfo(dpt.empty((), dtype="f4")).dtype == np.float32
+    assert dpt.iinfo(dpt.empty((), dtype="i4")).dtype == np.int32
+    with pytest.raises(ValueError):
+        dpt.iinfo("O")
+    with pytest.raises(ValueError):
+        dpt.finfo("O")
