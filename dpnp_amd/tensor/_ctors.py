@@ -38,7 +38,12 @@ def full(shape, fill_value, *, dtype=None, order="C", device=None, usm_type=None
             dtype = fill_value.dtype
         else:
             dtype = "f8"
-    r = usm_ndarray(shape, dtype=_as_dtype(dtype), order=_norm_order(order))
+    dt = _as_dtype(dtype)
+    if dt.kind in "iu" and isinstance(fill_value, int) and not isinstance(fill_value, bool):
+        info = np.iinfo(dt)
+        if not (info.min <= fill_value <= info.max):
+            raise OverflowError(f"Python integer {fill_value} out of bounds for {dt}")
+    r = usm_ndarray(shape, dtype=dt, order=_norm_order(order))
     if r.size:
         if isinstance(fill_value, (usm_ndarray, np.ndarray)):
             r[...] = fill_value
