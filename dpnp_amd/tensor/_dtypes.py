@@ -25,11 +25,16 @@ _TO_ID = {dt: i for i, dt in enumerate(ALL_DTYPES)}
 assert _TO_ID[float32] == _lib.FLOAT and _TO_ID[complex128] == _lib.CDOUBLE
 
 
+class UnsupportedDtypeError(TypeError, ValueError):
+    """A valid NumPy dtype that device arrays do not have (object, strings, datetimes...).  The
+    reference raises TypeError from its array constructor and ValueError from finfo / iinfo."""
+
+
 def dtype(obj):
     """Normalise `obj` to one of the 14 supported dtype objects."""
     dt = np.dtype(obj)
     if dt not in _TO_ID:
-        raise ValueError(f"Data type '{dt}' is not supported")
+        raise UnsupportedDtypeError(f"Data type '{dt}' is not supported")
     return ALL_DTYPES[_TO_ID[dt]]
 
 
