@@ -184,13 +184,78 @@ template <class T> DPX_D bool m_isinf(T x)
 // ---- complex elementary functions (textbook formulas on the real functions above; the
 // reference gets these from the SYCL complex library, results agree to rounding error for
 // finite arguments of moderate size) -----------------------------------------------------------
+template <class R> DPX_D bool m_finite(R v) { return v == v && !m_isinf(v); }
+// exp with the non-finite cases of libtensor/include/kernels/elementwise_functions/exp.hpp:75-132
 template <class R> DPX_D cplx<R> c_exp(cplx<R> z)
 {
-    const R e = m_exp(z.re);
-    if (z.im == R(0)) return {e, z.im};
-    return {e * m_cos(z.im), e * m_sin(z.im)};
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    if (m_finite(x)) {
+        if (!m_finite(y)) return {q_nan, q_nan};
+        const R e = m_exp(x);
+        if (y == R(0)) return {e, y};
+        return {e * m_cos(y), e * m_sin(y)};
+    }
+    if (x != x) return (y == R(0)) ? z : cplx<R>{x, q_nan};
+    if (!m_signbit(x)) { // +inf
+        if (y == R(0)) return {x, y};
+        if (m_finite(y)) return {x * m_cos(y), x * m_sin(y)};
+        return {x, q_nan};
+    }
+    if (m_finite(y)) return {R(0) * m_cos(y), R(0) * m_sin(y)}; // exp(-inf) = 0
+    return {R(0), R(0)};
+}
+// 2^z = exp(z ln 2) (exp2.hpp:75-133)
+template <class R> DPX_D cplx<R> c_exp2(cplx<R> z)
+{
+    const R ln2 = R(0.69314718055994530941723212145817657);
+    const cplx<R> t{z.re * ln2, z.im * ln2};
+    if (t.re != t.re && t.im == R(0)) return z; // the reference hands back its argument here
+    return c_exp(t);
+}
+// expm1(x + iy) = expm1(x) cos y - 2 sin^2(y/2) + i exp(x) sin y (expm1.hpp:75-138)
+template <class R> DPX_D cplx<R> c_expm1(cplx<R> z)
+{
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    if (m_isinf(x)) {
+        if (x > R(0)) {
+            if (!m_finite(y)) return {x, q_nan};
+            if (y == R(0)) return z;
+            return {m_copysign(x, m_cos(y)), m_copysign(x, m_sin(y))};
+        }
+        if (!m_finite(y)) return {R(-1), m_copysign(R(0), y)};
+        return {R(-1), m_copysign(R(0), m_sin(y))};
+    }
+    if (x != x) return (y == R(0)) ? z : cplx<R>{q_nan, q_nan};
+    if (x == R(0) && y == R(0)) return {R(0), y};
+    const R cy = m_cos(y);
+    const R sy = (y == R(0)) ? y : m_sin(y);
+    const R sh = (y == R(0)) ? y : m_sin(y / R(2));
+    return {m_expm1(x) * cy - R(2) * sh * sh, m_exp(x) * sy};
 }
 template <class R> DPX_D cplx<R> c_log(cplx<R> z) { return {m_log(m_hypot(z.re, z.im)), m_atan2(z.im, z.re)}; }
+// log1p.hpp:75-100, log2.hpp:75-83, log10.hpp:75-84
+template <class R> DPX_D cplx<R> c_log1p(cplx<R> z)
+{
+    const R x = z.re, y = z.im;
+    const R im = m_atan2(y, x + R(1));
+    const R ax = x < R(0) ? -x : x, ay = y < R(0) ? -y : y;
+    if ((ax > ay ? ax : ay) < R(0.1)) return {m_log1p(x * (R(2) + x) + y * y) / R(2), im};
+    return {m_log(m_hypot(x + R(1), y)), im};
+}
+template <class R> DPX_D cplx<R> c_log2(cplx<R> z)
+{
+    const cplx<R> l = c_log(z);
+    const R ln2 = m_log(R(2));
+    return {l.re / ln2, l.im / ln2};
+}
+template <class R> DPX_D cplx<R> c_log10(cplx<R> z)
+{
+    const cplx<R> l = c_log(z);
+    const R ln10 = m_log(R(10));
+    return {l.re / ln10, l.im / ln10};
+}
 template <class R> DPX_D cplx<R> c_sqrt(cplx<R> z)
 {
     if (z.re == R(0) && z.im == R(0)) return {R(0), z.im};
@@ -201,31 +266,71 @@ template <class R> DPX_D cplx<R> c_sqrt(cplx<R> z)
     const R ai = m_copysign(z.im, R(1)); // |im| also for -0.0: the real part of a root is never -0.0
     return {ai / (t + t), m_copysign(t, z.im)};
 }
+// sinh, cosh, tanh: finite arguments by the textbook formulas, the others case by case as in
+// libtensor/include/kernels/elementwise_functions/{sinh.hpp:75-160, cosh.hpp:75-150, tanh.hpp:75-135}
 template <class R> DPX_D cplx<R> c_sinh(cplx<R> z)
 {
-    if (z.im == R(0)) return {m_sinh(z.re), z.im};
-    return {m_sinh(z.re) * m_cos(z.im), m_cosh(z.re) * m_sin(z.im)};
+    const R x = z.re, y = z.im;
+    const bool xf = m_finite(x), yf = m_finite(y);
+    if (xf && yf) {
+        if (y == R(0)) return {m_sinh(x), y};
+        return {m_sinh(x) * m_cos(y), m_cosh(x) * m_sin(y)};
+    }
+    if (x == R(0) && !yf) return {m_copysign(R(0), x * (y - y)), y - y};
+    if (y == R(0) && !xf) return (x != x) ? cplx<R>{x, y} : cplx<R>{x, m_copysign(R(0), y)};
+    if (xf && !yf) return {y - y, x * (y - y)};
+    if (x == x) { // +-inf
+        if (!yf) return {x * x, x * (y - y)};
+        return {x * m_cos(y), (R)__builtin_inff() * m_sin(y)};
+    }
+    return {(x * x) * (y - y), (x + x) * (y - y)};
 }
 template <class R> DPX_D cplx<R> c_cosh(cplx<R> z)
 {
-    if (z.im == R(0)) return {m_cosh(z.re), z.re * z.im};
-    return {m_cosh(z.re) * m_cos(z.im), m_sinh(z.re) * m_sin(z.im)};
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    const bool xf = m_finite(x), yf = m_finite(y);
+    if (xf && yf) {
+        if (y == R(0)) return {m_cosh(x), x * y};
+        return {m_cosh(x) * m_cos(y), m_sinh(x) * m_sin(y)};
+    }
+    if (x == R(0) && !yf) return {q_nan, m_copysign(R(0), x * q_nan)};
+    if (y == R(0) && !xf) return {x * x, m_copysign(R(0), x) * y};
+    if (xf && !yf) return {q_nan, x * q_nan};
+    if (m_isinf(x)) {
+        if (!yf) return {x * x, x * q_nan};
+        return {(x * x) * m_cos(y), x * m_sin(y)};
+    }
+    return {(x * x) * (y - y), (x + x) * (y - y)};
 }
 template <class R> DPX_D cplx<R> c_tanh(cplx<R> z)
 {
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    if (!m_finite(x)) {
+        if (x != x) return {q_nan, (y == R(0)) ? y : q_nan};
+        return {m_copysign(R(1), x), m_copysign(R(0), m_isinf(y) ? y : m_sin(y) * m_cos(y))};
+    }
+    if (!m_finite(y)) return (x == R(0)) ? cplx<R>{x, q_nan} : cplx<R>{q_nan, q_nan};
     // Kahan's formulation: no cancellation near the poles at x = 0, y = pi/2 + k pi
-    const R ax = z.re < R(0) ? -z.re : z.re;
-    if (ax > R(20)) return {m_copysign(R(1), z.re), m_copysign(R(0), m_sin(z.im + z.im))};
-    const R t = m_tan(z.im);
+    const R ax = x < R(0) ? -x : x;
+    if (ax > R(20)) return {m_copysign(R(1), x), m_copysign(R(0), m_sin(y + y))};
+    const R t = m_tan(y);
     const R beta = R(1) + t * t;
-    const R s = m_sinh(z.re);
-    const R rho = m_sqrt(R(1) + s * s);
-    if (m_isinf(t)) return {rho / s, R(1) / t};
-    const R d = R(1) + beta * s * s;
-    return {beta * rho * s / d, t / d};
+    const R sh = m_sinh(x);
+    const R rho = m_sqrt(R(1) + sh * sh);
+    if (m_isinf(t)) return {rho / sh, R(1) / t};
+    const R d = R(1) + beta * sh * sh;
+    return {beta * rho * sh / d, t / d};
 }
 // sin z = -i sinh(iz), cos z = cosh(iz), tan z = -i tanh(iz)
-template <class R> DPX_D cplx<R> c_sin(cplx<R> z) { const cplx<R> w = c_sinh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+template <class R> DPX_D cplx<R> c_sin(cplx<R> z)
+{
+    const cplx<R> w = c_sinh(cplx<R>{-z.im, z.re});
+    // a zero real part of a finite argument keeps its sign (sin.hpp:84-92)
+    if (z.re == R(0) && m_finite(z.im)) return {m_copysign(R(0), z.re), -w.re};
+    return {w.im, -w.re};
+}
 template <class R> DPX_D cplx<R> c_cos(cplx<R> z) { return c_cosh(cplx<R>{-z.im, z.re}); }
 template <class R> DPX_D cplx<R> c_tan(cplx<R> z) { const cplx<R> w = c_tanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
 
@@ -551,15 +656,15 @@ struct SquareOp { // square.hpp:64-90; bool -> int8
 DPX_FPC_UNARY(SqrtOp, m_sqrt(x), c_sqrt(x))
 DPX_FPC_UNARY(ExpOp, m_exp(x), c_exp(x))
 DPX_FPC_UNARY(LogOp, m_log(x), c_log(x))
-DPX_FPC_UNARY(SinOp, m_sin(x), c_sin(x))
+DPX_FPC_UNARY(SinOp, (x == T(0)) ? x : m_sin(x), c_sin(x)) // sin.hpp:186-194: a zero comes back as it is
 DPX_FPC_UNARY(CosOp, m_cos(x), c_cos(x))
 DPX_FPC_UNARY(TanOp, m_tan(x), c_tan(x))
 DPX_FPC_UNARY(TanhOp, m_tanh(x), c_tanh(x))
-DPX_FP_UNARY(Exp2Op, m_exp2(x))
-DPX_FP_UNARY(Expm1Op, m_expm1(x))
-DPX_FP_UNARY(Log2Op, m_log2(x))
-DPX_FP_UNARY(Log10Op, m_log10(x))
-DPX_FP_UNARY(Log1pOp, m_log1p(x))
+DPX_FPC_UNARY(Exp2Op, m_exp2(x), c_exp2(x))
+DPX_FPC_UNARY(Expm1Op, (x == T(0)) ? x : m_expm1(x), c_expm1(x)) // expm1.hpp:139-146
+DPX_FPC_UNARY(Log2Op, m_log2(x), c_log2(x))
+DPX_FPC_UNARY(Log10Op, m_log10(x), c_log10(x))
+DPX_FPC_UNARY(Log1pOp, (x == T(0)) ? x : m_log1p(x), c_log1p(x))
 DPX_FP_UNARY(RsqrtOp, T(1) / m_sqrt(x))
 DPX_FP_UNARY(CbrtOp, m_cbrt(x))
 DPX_FPC_UNARY(ReciprocalOp, T(1) / x, (T{real_of_t<T>(1), real_of_t<T>(0)} / x))
