@@ -334,41 +334,86 @@ template <class R> DPX_D cplx<R> c_sin(cplx<R> z)
 template <class R> DPX_D cplx<R> c_cos(cplx<R> z) { return c_cosh(cplx<R>{-z.im, z.re}); }
 template <class R> DPX_D cplx<R> c_tan(cplx<R> z) { const cplx<R> w = c_tanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
 
-// Inverse functions after W. Kahan, "Branch cuts for complex elementary functions" (1987): the
-// square roots of 1 -/+ z (or z -/+ 1) carry the branch cuts, signed zeros pick the side.
-template <class R> DPX_D cplx<R> c_asin(cplx<R> z)
+// Inverse functions.  Ordinary arguments after W. Kahan, "Branch cuts for complex elementary
+// functions" (1987): the square roots of 1 -/+ z (or z -/+ 1) carry the branch cuts, signed zeros
+// pick the side.  NaN parts and large arguments are handled around them as the reference does
+// (libtensor/include/kernels/elementwise_functions/complex_math.hpp:57-262, acosh.hpp:76-105).
+template <class R> DPX_D cplx<R> c_asin_ordinary(cplx<R> z)
 {
     const cplx<R> s1 = c_sqrt(cplx<R>{R(1) - z.re, -z.im}), s2 = c_sqrt(cplx<R>{R(1) + z.re, z.im});
     return {m_atan2(z.re, s1.re * s2.re - s1.im * s2.im), m_asinh(s1.re * s2.im - s1.im * s2.re)};
 }
+// beyond sqrt(1/eps)/2 the functions are log(2z) to working precision
+template <class R> inline constexpr R inv_big = std::is_same_v<R, double> ? R(33554432.0) : R(1448.15466);
+template <class R> DPX_D R m_abs(R v) { return m_copysign(v, R(1)); }
 template <class R> DPX_D cplx<R> c_acos(cplx<R> z)
 {
-    const cplx<R> s1 = c_sqrt(cplx<R>{R(1) - z.re, -z.im}), s2 = c_sqrt(cplx<R>{R(1) + z.re, z.im});
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    const R ln2 = R(0.6931471805599453094172321214581765);
+    if (x != x) return m_isinf(y) ? cplx<R>{q_nan, -y} : cplx<R>{q_nan, q_nan};
+    if (y != y) {
+        if (m_isinf(x)) return {q_nan, -(R)__builtin_inff()};
+        if (x == R(0)) return {R(1.5707963267948966192313216916397514), q_nan};
+        return {q_nan, q_nan};
+    }
+    if (m_abs(x) > inv_big<R> || m_abs(y) > inv_big<R>) {
+        const cplx<R> l = c_log(z);
+        const R ry = l.re + ln2;
+        return {m_abs(l.im), m_signbit(y) ? ry : -ry};
+    }
+    const cplx<R> s1 = c_sqrt(cplx<R>{R(1) - x, -y}), s2 = c_sqrt(cplx<R>{R(1) + x, y});
     return {R(2) * m_atan2(s1.re, s2.re), m_asinh(s2.re * s1.im - s2.im * s1.re)};
 }
 template <class R> DPX_D cplx<R> c_acosh(cplx<R> z)
 {
-    const cplx<R> t1 = c_sqrt(cplx<R>{z.re - R(1), z.im}), t2 = c_sqrt(cplx<R>{z.re + R(1), z.im});
-    return {m_asinh(t1.re * t2.re + t1.im * t2.im), R(2) * m_atan2(t1.im, t2.re)};
+    // from acos: acosh z = +-i acos z, with the sign that makes the real part positive
+    const cplx<R> a = c_acos(z);
+    if (a.re != a.re && a.im != a.im) return {a.im, a.re};
+    if (a.re != a.re) return {m_abs(a.im), a.re};
+    return {m_abs(a.im), m_copysign(a.re, z.im)};
 }
-// asinh z = -i asin(iz)
-template <class R> DPX_D cplx<R> c_asinh(cplx<R> z) { const cplx<R> w = c_asin(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+template <class R> DPX_D cplx<R> c_asinh(cplx<R> z)
+{
+    const R x = z.re, y = z.im;
+    const R q_nan = (R)__builtin_nanf("");
+    const R ln2 = R(0.6931471805599453094172321214581765);
+    if (x != x) {
+        if (m_isinf(y)) return {y, q_nan};
+        if (y == R(0)) return {q_nan, y};
+        return {q_nan, q_nan};
+    }
+    if (y != y) return m_isinf(x) ? cplx<R>{x, q_nan} : cplx<R>{q_nan, q_nan};
+    if (m_abs(x) > inv_big<R> || m_abs(y) > inv_big<R>) {
+        const cplx<R> l = m_signbit(x) ? c_log(cplx<R>{-x, -y}) : c_log(z);
+        return {m_copysign(l.re + ln2, x), m_copysign(l.im, y)};
+    }
+    // asinh z = -i asin(iz)
+    const cplx<R> w = c_asin_ordinary(cplx<R>{-y, x});
+    return {w.im, -w.re};
+}
+// asin(x + iy) = swap(asinh(y + ix))
+template <class R> DPX_D cplx<R> c_asin(cplx<R> z) { const cplx<R> w = c_asinh(cplx<R>{z.im, z.re}); return {w.im, w.re}; }
 template <class R> DPX_D cplx<R> c_atanh(cplx<R> z)
 {
+    const R pi_2 = R(1.5707963267948966192313216916397514);
+    const R q_nan = (R)__builtin_nanf("");
+    if (z.re != z.re) {
+        if (m_isinf(z.im)) return {m_copysign(R(0), z.re), m_copysign(pi_2, z.im)};
+        return {q_nan, q_nan};
+    }
+    if (z.im != z.im) {
+        if (m_isinf(z.re)) return {m_copysign(R(0), z.re), q_nan};
+        if (z.re == R(0)) return {z.re, q_nan};
+        return {q_nan, q_nan};
+    }
+    const R huge = std::is_same_v<R, double> ? R(4503599627370496.0) : R(8388608.0); // 1/eps
+    if (m_abs(z.re) > huge || m_abs(z.im) > huge) return {R(0), m_copysign(pi_2, z.im)};
     // odd function: work in the right half plane
     const bool neg = m_signbit(z.re);
     const R x = neg ? -z.re : z.re, y = neg ? -z.im : z.im;
-    const R ay = y < R(0) ? -y : y;
-    const R pi_2 = R(1.5707963267948966192313216916397514);
     cplx<R> w;
-    const R big = std::is_same_v<R, double> ? R(1e150) : R(1e18);
-    if (x > big || ay > big) {
-        // |z| huge: atanh z -> 1/z +- i pi/2, without squaring the parts
-        const R s = x > ay ? x : ay;
-        const R xs = x / s, ys = y / s;
-        w = {xs / ((xs * xs + ys * ys) * s), m_copysign(pi_2, y)};
-    }
-    else if (x == R(1) && y == R(0)) {
+    if (x == R(1) && y == R(0)) {
         w = {(R)__builtin_inff(), y};
     }
     else {
@@ -377,8 +422,8 @@ template <class R> DPX_D cplx<R> c_atanh(cplx<R> z)
     }
     return neg ? cplx<R>{-w.re, -w.im} : w;
 }
-// atan z = -i atanh(iz)
-template <class R> DPX_D cplx<R> c_atan(cplx<R> z) { const cplx<R> w = c_atanh(cplx<R>{-z.im, z.re}); return {w.im, -w.re}; }
+// atan(x + iy) = swap(atanh(y + ix))
+template <class R> DPX_D cplx<R> c_atan(cplx<R> z) { const cplx<R> w = c_atanh(cplx<R>{z.im, z.re}); return {w.im, w.re}; }
 
 template <class T> using V = value_of_t<T>;
 

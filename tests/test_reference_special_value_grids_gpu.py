@@ -248,6 +248,68 @@ def test_complex_exponentials_and_logarithms_on_finite_arguments(name, dt):
     np.testing.assert_allclose(got, want.astype(dt), atol=tol, rtol=tol)
 
 
+INVERSE = {"asin": "arcsin", "acos": "arccos", "atan": "arctan", "asinh": "arcsinh", "acosh": "arccosh",
+           "atanh": "arctanh"}
+
+
+@pytest.mark.parametrize("dt", ["c8", "c16"])
+@pytest.mark.parametrize("name", sorted(INVERSE))
+def test_complex_inverse_functions_with_nan_and_infinite_parts(name, dt):
+    # complex_math.hpp:57-262 and acosh.hpp:76-105 spell out the Annex G results for NaN and infinite parts; NumPy's
+    # loops give the same table.  Signs that the standard leaves open ("opt(+-)") are not compared.
+    z = np.array(CPLX_GRID, dtype=dt)
+    got = host(getattr(dpt, name)(dev(z)))
+    with np.errstate(all="ignore"), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        want = getattr(np, INVERSE[name])(z)
+    if name == "acosh":
+        # acosh(+-0 + NaN j) = NaN +- pi/2 j in the reference (cacos gives pi/2 + NaN j there, test_hyperbolic.py:207-221);
+        # NumPy has NaN in both parts
+        at = (z.real == 0) & np.isnan(z.imag)
+        want.imag[at] = np.pi / 2
+    tol = 8 * np.finfo(dt).resolution
+    for g, w in ((got.real, want.real), (got.imag, want.imag)):
+        np.testing.assert_array_equal(np.isnan(g), np.isnan(w))
+        ok = ~np.isnan(w)
+        np.testing.assert_allclose(np.abs(g[ok]), np.abs(w[ok]), atol=tol, rtol=tol)
+    signed = ~(np.isnan(z.real) | np.isnan(z.imag))
+    if name in ("atan", "atanh"):
+        # beyond 1/eps the reference returns 0 + i copysign(pi/2, y) for atanh whatever the sign of x
+        # (complex_math.hpp:222-227), and the mirrored value for atan
+        big = np.isinf(z.real) | np.isinf(z.imag)
+        zero_part = got.real if name == "atanh" else got.imag
+        assert not np.signbit(zero_part[signed & big]).any() and (zero_part[signed & big] == 0).all()
+        signed &= ~big
+    np.testing.assert_array_equal(np.signbit(got.real[signed]), np.signbit(want.real[signed]))
+    np.testing.assert_array_equal(np.signbit(got.imag[signed]), np.signbit(want.imag[signed]))
+
+
+@pytest.mark.parametrize("dt", ["c8", "c16"])
+def test_acosh_of_zero_plus_nan(dt):
+    # test_hyperbolic.py:207-221: acosh(+-0 + NaN j) = NaN +- pi/2 j
+    y = host(dpt.acosh(dev(np.array([complex(+0.0, np.nan), complex(-0.0, np.nan)], dtype=dt))))
+    assert np.isnan(y.real).all()
+    np.testing.assert_allclose(np.abs(y.imag), np.pi / 2, atol=1e-6)
+
+
+@pytest.mark.parametrize("dt", ["c8", "c16"])
+@pytest.mark.parametrize("name", sorted(INVERSE))
+def test_complex_inverse_functions_of_large_arguments(name, dt):
+    # test_hyperbolic.py:222-305, test_trigonometric.py:240-320: arguments around the switch to the logarithmic form,
+    # in all four quadrants
+    thr1 = 1 / np.finfo(dt).eps
+    thr2 = np.sqrt(thr1) / 2
+    base = [complex(4e7, 1.0), complex(9e7, 1.0), complex(1e8, 1.0), complex(4.45712982e8, 1.0), complex(thr1, 1.0),
+            complex(thr2, 1.0), complex(np.nextafter(thr1, np.inf), 1.0), complex(np.nextafter(thr2, np.inf), 1.0),
+            complex(1.0, 4e7), complex(1.0, thr2 * 1.01), complex(3e4, 4e4), complex(2e30, 1e30)]
+    x = np.array([complex(sr * v.real, si * v.imag) for v in base for sr in (1, -1) for si in (1, -1)], dtype=dt)
+    got = host(getattr(dpt, name)(dev(x)))
+    want = getattr(np, INVERSE[name])(x)
+    tol = 8 * np.finfo(dt).resolution
+    assert not np.isinf(got.real).any() and not np.isinf(got.imag).any()
+    np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
+
+
 def test_comparisons_with_python_ints_beyond_the_dtype():
     # test_greater.py:172-200, test_less.py:172-200 (and _equal forms)
     x = dpt.zeros(10, dtype="i4")
