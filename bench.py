@@ -142,8 +142,8 @@ def build_workload(name, dpnp, torch):
                ("var_f32_acc64", lambda: dpnp.var(clean, dtype="f8", out=m[1]), 2 * 4 * n + 8, n),  # two passes
                ("mean_f64", lambda: dpnp.mean(clean64, out=m[2]), 8 * n + 8, n),
                ("var_f64", lambda: dpnp.var(clean64, out=m[3]), 2 * 8 * n + 8, n),
-               # NaN-ignoring forms on the NaN variant: count + search, and count + sum (two passes each)
-               ("nanargmax_nan", lambda: dpnp.nanargmax(x, out=i0), 2 * 4 * n + 16, n),
+               # NaN-ignoring forms on the NaN variant: one search pass; count + sum (two passes)
+               ("nanargmax_nan", lambda: dpnp.nanargmax(x, out=i0), 4 * n + 8, n),
                ("nanmean_nan", lambda: dpnp.nanmean(x, out=m32), 2 * 4 * n + 12, n)]
         return ops, "f32 (fp64 accumulation)", "synthetic (seeded normal(0,1) with planted extrema / NaN, resident in HBM)"
     if name == "cfg4":

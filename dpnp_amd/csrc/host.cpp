@@ -154,6 +154,14 @@ struct Block {
 };
 std::mutex g_pool_mu;
 std::map<std::pair<int, hipStream_t>, Block> g_pool;
+
+// Clears a fresh block.  A kernel rather than a memset call: memset nodes recorded into a stream
+// capture have replayed wrongly on these machines.
+__global__ void scratch_zero_kernel(uint4 *p, size_t n16)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = uint4{0u, 0u, 0u, 0u};
+}
 } // namespace
 
 void *scratch_get(hipStream_t stream, size_t bytes)
@@ -177,7 +185,10 @@ void *scratch_get(hipStream_t stream, size_t bytes)
         return nullptr;
     }
     // callers rely on fresh blocks being zero (ticket counters) and keep them zero
-    if (hipMemsetAsync(b.p, 0, want, stream) != hipSuccess) {
+    const size_t n16 = want / 16; // want is a multiple of 4096
+    const unsigned blocks = (unsigned)std::min<size_t>((n16 + 255) / 256, 1024);
+    scratch_zero_kernel<<<blocks, 256, 0, stream>>>(static_cast<uint4 *>(b.p), n16);
+    if (hipGetLastError() != hipSuccess) {
         (void)hipFree(b.p);
         b.p = nullptr;
         return nullptr;

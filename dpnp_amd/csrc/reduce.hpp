@@ -50,6 +50,7 @@ struct RedLaunch {
     int64_t rstride;  // cols: stride of the reduced axis
     int64_t inner;    // cols: length of the inner (contiguous) iteration dim
     int64_t col_blocks;
+    int32_t mark_fill; // NaN-ignoring searches: report "extreme equals the value NaNs count as" as -1 - index
 };
 
 template <class T> DPX_D T shfl_down_any(T v, int off)
@@ -969,6 +970,20 @@ template <bool IS_MAX, class VT> DPX_D void arg_group_reduce(VT &best, int64_t &
     }
 }
 
+// Result of a search as it is stored.  A NaN-ignoring search reads NaN as the infinity that loses, so
+// an all-NaN run and a run whose extreme is that infinity look alike; when the caller asks for it
+// (L.mark_fill) both are reported as -1 - index, and the caller tells them apart.
+template <class T> DPX_D int64_t arg_result(const RedLaunch &L, int64_t idx, value_of_t<T> best)
+{
+    if constexpr (is_nanskip<T>::value) {
+        using V = value_of_t<T>;
+        const V inf = (V)__builtin_inff();
+        const V fill = is_nanskip<T>::is_max ? -inf : inf;
+        if (L.mark_fill && best == fill) return -1 - idx;
+    }
+    return idx;
+}
+
 // Position = index along the reduced run.  Linear block id = oblock * splits + split, lanes
 // per output as in red_rows_kernel; partial (value, position) pairs laid out [output][split].
 template <class T, bool IS_MAX, bool CONTIG>
@@ -1077,7 +1092,7 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
     }
     arg_group_reduce<IS_MAX, VT>(best, bidx, whole_block, G);
     if (L.splits == 1) {
-        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = bidx;
+        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = arg_result<T>(L, bidx, best);
         return;
     }
     uint32_t zero = 0;
@@ -1092,7 +1107,7 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
         arg_merge<IS_MAX, VT>(best, bidx, to_value(slot_read(pval + o * L.splits + i)),
                               slot_read(pidx + o * L.splits + i));
     arg_group_reduce<IS_MAX, VT>(best, bidx, true, G);
-    if (threadIdx.x == 0) dst[dof] = bidx;
+    if (threadIdx.x == 0) dst[dof] = arg_result<T>(L, bidx, best);
 }
 
 // Column variant (reduced axis strided by L.rstride, outputs contiguous).  A thread owns the E
@@ -1213,8 +1228,8 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
 #pragma unroll
                 for (int e = 0; e < E; e += 2) {
                     pack<int64_t, 2> t;
-                    t.v[0] = bidx[e];
-                    t.v[1] = bidx[e + 1];
+                    t.v[0] = arg_result<T>(L, bidx[e], best[e]);
+                    t.v[1] = arg_result<T>(L, bidx[e + 1], best[e + 1]);
                     store_pack<int64_t, 2>(q + e, t);
                 }
                 return;
@@ -1222,7 +1237,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
         }
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (col0 + e < L.inner) q[e * ix.dst_str[last]] = bidx[e];
+            if (col0 + e < L.inner) q[e * ix.dst_str[last]] = arg_result<T>(L, bidx[e], best[e]);
     };
     combine_rows();
     const int64_t out0 = outer * L.inner + col0;
@@ -1335,7 +1350,7 @@ __global__ __launch_bounds__(256) void arg_short_rows_kernel(RedIndex ix, RedLau
                 bj = j;
             }
         }
-        dst[(row0 + r) * ix.dst_str[0]] = (int64_t)bj;
+        dst[(row0 + r) * ix.dst_str[0]] = arg_result<T>(L, (int64_t)bj, best);
     }
 }
 

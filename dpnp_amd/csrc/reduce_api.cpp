@@ -84,14 +84,14 @@ static bool search_supported(int op, int s, int d)
 {
     if (s < 0 || s >= DPX_NUM_DTYPES || d != DPX_INT64) return false;
     if (op == DPX_S_ARGMAX || op == DPX_S_ARGMIN) return true;
-    if (op == DPX_S_NANARGMAX || op == DPX_S_NANARGMIN) return s == DPX_HALF || s == DPX_FLOAT || s == DPX_DOUBLE;
+    if (op >= DPX_S_NANARGMAX && op <= DPX_S_NANARGMIN_MARKED) return s == DPX_HALF || s == DPX_FLOAT || s == DPX_DOUBLE;
     return false;
 }
 
 static int argreduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
                           void *stream, dpx_plan *plan_out)
 {
-    if (op < 0 || op > DPX_S_NANARGMIN) return fail(DPX_ERR_BAD_ARGUMENT, "unknown search op id");
+    if (op < 0 || op > DPX_S_NANARGMIN_MARKED) return fail(DPX_ERR_BAD_ARGUMENT, "unknown search op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
     if (!search_supported(op, src->dtype, dst->dtype)) return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
     if (int rc = red_validate(src, trailing, dst, nullptr, false)) return rc;
@@ -101,8 +101,10 @@ static int argreduce_call(int op, const dpx_array_view *src, int trailing, const
         red_export_plan(pl, plan_out, itemsize_of(src->dtype) + 8);
         return DPX_OK;
     }
-    if (op == DPX_S_NANARGMAX || op == DPX_S_NANARGMIN)
-        return nanarg_run(op == DPX_S_NANARGMAX, pl, src, dst, (hipStream_t)stream);
+    if (op >= DPX_S_NANARGMAX) {
+        pl.L.mark_fill = (op == DPX_S_NANARGMAX_MARKED || op == DPX_S_NANARGMIN_MARKED) ? 1 : 0;
+        return nanarg_run(op == DPX_S_NANARGMAX || op == DPX_S_NANARGMAX_MARKED, pl, src, dst, (hipStream_t)stream);
+    }
     return arg_run_any(op == DPX_S_ARGMAX, pl, src, dst, (hipStream_t)stream);
 }
 

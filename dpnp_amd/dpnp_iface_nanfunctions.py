@@ -18,6 +18,7 @@ from .dpnp_iface import (
     argmax,
     argmin,
     check_limitations,
+    check_supported_arrays_type,
     get_result_array,
     get_usm_ndarray,
     max,  # noqa: A004
@@ -57,9 +58,21 @@ def _nanarg(a, axis, out, keepdims, fused, plain):
             raise ValueError("All-NaN slice encountered")
         return plain(_wrap(dpt.where(nan, dpt.asarray(fill, dtype=u.dtype), u)), axis=axis, out=out,
                      keepdims=keepdims)
-    if u.size and _any_true(dpt.equal(nr.nancount(u, axis=axis), 0)):
-        raise ValueError("All-NaN slice encountered")
-    return _wrap_reduction_call(u, out, fused, _search_res_dt(out), axis=axis, keepdims=keepdims)
+    if u.size == 0:
+        return _wrap_reduction_call(u, out, fused, _search_res_dt(out), axis=axis, keepdims=keepdims)
+    if out is not None:
+        check_supported_arrays_type(out)
+        _search_res_dt(out)  # rejects an `out` that cannot hold indices before anything is computed
+    # one pass: the search marks the runs that may be all NaN (their extreme is the infinity NaNs are
+    # read as) with negative results; only then is the input read again to tell which they are
+    marked = nr.nanargmax_marked if fused is nr.nanargmax else nr.nanargmin_marked
+    res = marked(u, axis=axis, keepdims=keepdims)
+    doubtful = dpt.less(res, 0)
+    if _any_true(doubtful):
+        if _any_true(dpt.equal(nr.nancount(u, axis=axis), 0)):
+            raise ValueError("All-NaN slice encountered")
+        res = dpt.where(doubtful, dpt.subtract(-1, res), res)
+    return get_result_array(_wrap(res), out, casting="unsafe")
 
 
 def nanargmax(a, axis=None, out=None, *, keepdims=False):

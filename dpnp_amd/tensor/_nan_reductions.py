@@ -50,3 +50,14 @@ def nanargmax(x, /, *, axis=None, keepdims=False, out=None):
 def nanargmin(x, /, *, axis=None, keepdims=False, out=None):
     """Index of the minimum along `axis` with NaN read as +inf (first occurrence)."""
     return _search_over_axis(x, axis, keepdims, out, tri._nanargmin_over_axis)
+
+
+def nanargmax_marked(x, /, *, axis=None, keepdims=False):
+    """nanargmax in which a run that is all NaN, or whose maximum is -inf, reports -1 - index: a
+    caller that must raise on all-NaN runs looks at the input again only when a result is negative."""
+    return _search_over_axis(x, axis, keepdims, None, tri._nanargmax_marked_over_axis)
+
+
+def nanargmin_marked(x, /, *, axis=None, keepdims=False):
+    """nanargmin in which a run that is all NaN, or whose minimum is +inf, reports -1 - index."""
+    return _search_over_axis(x, axis, keepdims, None, tri._nanargmin_marked_over_axis)

@@ -57,6 +57,9 @@ _nanmin_over_axis, _nanmin_over_axis_dtype_supported = _make_reduction("nanmin",
 _nancount_over_axis, _nancount_over_axis_dtype_supported = _make_reduction("nancount", _lib.REDUCE_ID["nancount"])
 _nanargmax_over_axis = _make_search("nanargmax", _lib.SEARCH_ID["nanargmax"])
 _nanargmin_over_axis = _make_search("nanargmin", _lib.SEARCH_ID["nanargmin"])
+# the same, with results of runs whose extreme is the infinity NaNs are read as stored as -1 - index
+_nanargmax_marked_over_axis = _make_search("nanargmax_marked", _lib.SEARCH_ID["nanargmax_marked"])
+_nanargmin_marked_over_axis = _make_search("nanargmin_marked", _lib.SEARCH_ID["nanargmin_marked"])
 
 
 def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None, depends=(), nan=False):

@@ -231,7 +231,14 @@ typedef enum dpx_search_op {
     /* NaN elements never win (real floating inputs): dpnp.nanargmax / nanargmin,
      * dpnp/dpnp_iface_nanfunctions.py:119-284 */
     DPX_S_NANARGMAX = 2,
-    DPX_S_NANARGMIN = 3
+    DPX_S_NANARGMIN = 3,
+    /* the same searches, for callers that must raise on an all-NaN run as dpnp.nanargmax does
+     * (dpnp/dpnp_iface_nanfunctions.py:195-200) without a pass of their own over the input: a run
+     * whose extreme equals the infinity that NaNs are read as (-inf for the maximum, +inf for the
+     * minimum) is all-NaN or really has that extreme, and its result is stored as -1 - index.
+     * No negative result: no all-NaN run, and every index is final. */
+    DPX_S_NANARGMAX_MARKED = 4,
+    DPX_S_NANARGMIN_MARKED = 5
 } dpx_search_op;
 
 /* which kernel family a call resolves to (reported by the dpx_*_plan queries;

@@ -367,6 +367,37 @@ def test_nanarg_ties_infinities_and_large():
     assert_same(dpnp.nanmin(dm, axis=0).asnumpy(), np.nanmin(m, axis=0))
 
 
+@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
+@pytest.mark.parametrize("shape, axis", [((5000,), None), ((3_000_003,), None), ((300, 700), 1), ((300, 700), 0),
+                                         ((40_000, 24), 0), ((40_000, 12), 1), ((70_000, 1500), 0)])
+def test_nanarg_runs_whose_extreme_is_the_infinity_nan_counts_as(dt, shape, axis):
+    """nanargmax reads NaN as -inf (dpnp/dpnp_iface_nanfunctions.py:195-200): a run with a NaN before a real -inf
+    gives the position of the NaN, an all-NaN run raises, and the search kernel alone tells which runs need a
+    second look."""
+    if shape == (70_000, 1500) and dt != "f4":
+        pytest.skip("one dtype is enough for the large matrix")
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(shape).astype(dt)
+    a[rng.random(shape) < 0.05] = np.nan
+    runs = a.reshape(1, -1) if axis is None else (a if axis == 1 else a.T)  # views: one run per row
+    assert np.shares_memory(runs, a)
+    # some runs hold nothing but NaN and -inf, with the NaNs first
+    for r in range(0, runs.shape[0], max(1, runs.shape[0] // 7)):
+        runs[r] = -np.inf
+        runs[r, : max(1, runs.shape[1] // 3)] = np.nan
+    assert_same(dpnp.nanargmax(dpnp.array(a), axis=axis).asnumpy(), np.asarray(np.nanargmax(a, axis=axis), dtype="i8"))
+    assert_same(dpnp.nanargmin(dpnp.array(-a), axis=axis).asnumpy(), np.asarray(np.nanargmin(-a, axis=axis), dtype="i8"))
+    # an all-NaN run raises and leaves `out` as it was
+    runs[runs.shape[0] // 2] = np.nan
+    d = dpnp.array(a)
+    out = dpnp.full(() if axis is None else (runs.shape[0],), -7, dtype="i8")
+    with pytest.raises(ValueError, match="All-NaN slice"):
+        dpnp.nanargmax(d, axis=axis, out=out)
+    with pytest.raises(ValueError, match="All-NaN slice"):
+        dpnp.nanargmin(d, axis=axis, out=out)
+    assert (out.asnumpy() == -7).all()
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 @pytest.mark.parametrize("axis", [None, 0, 1, (0, 1)])
 @pytest.mark.parametrize("keepdims", [False, True])
