@@ -142,9 +142,9 @@ def build_workload(name, dpnp, torch):
                ("var_f32_acc64", lambda: dpnp.var(clean, dtype="f8", out=m[1]), 2 * 4 * n + 8, n),  # two passes
                ("mean_f64", lambda: dpnp.mean(clean64, out=m[2]), 8 * n + 8, n),
                ("var_f64", lambda: dpnp.var(clean64, out=m[3]), 2 * 8 * n + 8, n),
-               # NaN-ignoring forms on the NaN variant: one search pass; count + sum (two passes)
+               # NaN-ignoring forms on the NaN variant, one pass each
                ("nanargmax_nan", lambda: dpnp.nanargmax(x, out=i0), 4 * n + 8, n),
-               ("nanmean_nan", lambda: dpnp.nanmean(x, out=m32), 2 * 4 * n + 12, n)]
+               ("nanmean_nan", lambda: dpnp.nanmean(x, out=m32), 4 * n + 4, n)]
         return ops, "f32 (fp64 accumulation)", "synthetic (seeded normal(0,1) with planted extrema / NaN, resident in HBM)"
     if name == "cfg4":
         side = 8192

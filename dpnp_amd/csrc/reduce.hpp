@@ -127,7 +127,14 @@ enum {
     // NaN-ignoring forms: a NaN element contributes the identity (0, 1, nothing, not counted)
     K_NANSUM = 7, K_NANPROD = 8, K_NANMAX = 9, K_NANMIN = 10, K_NANCOUNT = 11, K_NANSUMSQDEV = 12,
     // truth-value reductions of any input type: an element counts as true when it is not zero
-    K_ANY = 13, K_ALL = 14, K_COUNT_NONZERO = 15
+    K_ANY = 13, K_ALL = 14, K_COUNT_NONZERO = 15,
+    // mean of the elements that are not NaN: sum and count travel together, divided at the end
+    K_NANMEAN = 16
+};
+// accumulator of K_NANMEAN
+template <class A> struct mean_acc {
+    A s;
+    int64_t c;
 };
 constexpr bool kind_is_minmax(int k) { return k == K_MAX || k == K_MIN || k == K_NANMAX || k == K_NANMIN; }
 
@@ -162,14 +169,16 @@ template <int KIND, class T> DPX_D T red_identity()
 template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy {
     using In = In_;
     using Out = Out_;
-    using Acc = std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>,
-                                   acc_of_t<Out_>>;
+    using Acc = std::conditional_t<
+        KIND == K_NANMEAN, mean_acc<acc_of_t<Out_>>,
+        std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>;
     using Aux = Out_;
     static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV) && !FINAL;
     static constexpr int kind = KIND;
     DPX_D static Acc identity()
     {
-        if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
+        if constexpr (KIND == K_NANMEAN) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
+        else if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
         else if constexpr (is_bool_v<Out>) return (KIND == K_PROD || KIND == K_ALL) ? 1 : 0;
         else if constexpr (KIND == K_COUNT_NONZERO) return Acc(0);
         else if constexpr (KIND == K_NANMAX || KIND == K_NANMIN) return (Acc)__builtin_nanf(""); // "nothing yet"
@@ -181,6 +190,10 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc pre(In x, Acc aux)
     {
         if constexpr (FINAL) return x; // In == Acc
+        else if constexpr (KIND == K_NANMEAN) {
+            const bool skip = isnan_(x);
+            return Acc{skip ? red_identity<K_SUM, acc_of_t<Out>>() : in_to_acc<In, Out>(x), skip ? 0 : 1};
+        }
         else if constexpr (KIND == K_SUMSQDEV) {
             const Acc d = in_to_acc<In, Out>(x) - aux;
             return d * d;
@@ -201,7 +214,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     }
     DPX_D static Acc combine(Acc a, Acc b)
     {
-        if constexpr (is_bool_v<Out>) {
+        if constexpr (KIND == K_NANMEAN) return Acc{a.s + b.s, a.c + b.c};
+        else if constexpr (is_bool_v<Out>) {
             if constexpr (KIND == K_PROD || KIND == K_MIN || KIND == K_ALL) return a & b;
             else return a | b;
         }
@@ -257,7 +271,19 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
             return acc + (Acc)((int32_t)t - 16 * 128);
         }
     }
-    DPX_D static Out post(Acc a) { return acc_to_out<Acc, Out>(a); }
+    DPX_D static Out post(Acc a)
+    {
+        if constexpr (KIND == K_NANMEAN) {
+            // sum / count in the accumulator's type: 0 / 0 = NaN for a run without a number
+            using A = acc_of_t<Out>;
+            if constexpr (is_cplx_v<A>) {
+                using R = real_of_t<A>;
+                return acc_to_out<A, Out>(A{a.s.re / (R)a.c, a.s.im / (R)a.c});
+            }
+            else return acc_to_out<A, Out>(a.s / (A)a.c);
+        }
+        else return acc_to_out<Acc, Out>(a);
+    }
     DPX_D static Acc load_aux(const Aux *p)
     {
         if constexpr (std::is_same_v<Aux, half_t>) return (float)*p;

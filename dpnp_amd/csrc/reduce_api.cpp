@@ -22,7 +22,7 @@ int nanarg_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, 
 bool truth_pair_supported(int, int, int);
 int truth_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 static bool is_truth_op(int op) { return op == DPX_R_ANY || op == DPX_R_ALL || op == DPX_R_COUNT_NONZERO; }
-static bool is_nan_op(int op) { return op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV; }
+static bool is_nan_op(int op) { return (op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV) || op == DPX_R_NANMEAN; }
 static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV; }
 
 static bool reduce_supported(int op, int s, int d)

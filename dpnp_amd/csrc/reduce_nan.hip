@@ -15,7 +15,7 @@ template <class F> static bool for_nan_pair(int op, int in_dt, int out_dt, F &&f
         f(tag<I>{}, tag<O>{});                                 \
         hit = true;                                            \
     }
-    if (op == DPX_R_NANSUM || op == DPX_R_NANPROD) {
+    if (op == DPX_R_NANSUM || op == DPX_R_NANPROD || op == DPX_R_NANMEAN) {
         DPX_PAIR(half_t, half_t) DPX_PAIR(float, float) DPX_PAIR(double, double) DPX_PAIR(c64, c64)
         DPX_PAIR(c128, c128) DPX_PAIR(half_t, float) DPX_PAIR(float, double) DPX_PAIR(c64, c128)
     }
@@ -70,6 +70,7 @@ static int nan_dispatch(int op, RedPlan &pl, const dpx_array_view *src, const dp
     case DPX_R_NANMIN: return nan_run_kind<K_NANMIN>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANCOUNT: return nan_run_kind<K_NANCOUNT>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANSUMSQDEV: return nan_run_kind<K_NANSUMSQDEV>(op, pl, src, dst, aux, stream, acc_size);
+    case DPX_R_NANMEAN: return nan_run_kind<K_NANMEAN>(op, pl, src, dst, aux, stream, acc_size);
     default: return DPX_ERR_NOT_IMPLEMENTED;
     }
 }

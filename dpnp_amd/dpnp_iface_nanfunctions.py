@@ -163,13 +163,10 @@ def nanmean(a, axis=None, dtype=None, out=None, keepdims=False, *, where=True):
         return mean(a, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
     dtype = _check_inexact_targets(dtype, out)
     res_dt = u.dtype if dtype is None else dtype
-    cnt = nr.nancount(u, axis=axis, keepdims=keepdims)
     usm_out = None if out is None else get_usm_ndarray(out)
     direct = usm_out is not None and usm_out.dtype == res_dt
-    avg = nr.nansum(u, axis=axis, dtype=res_dt, keepdims=keepdims, out=usm_out if direct else None)
-    real_dt = dpt.dtype("f" + str(res_dt.itemsize // 2)) if res_dt.kind == "c" else res_dt
-    if avg.size:
-        dpt.divide(avg, dpt.astype(cnt, real_dt), out=avg)  # 0 / 0 -> NaN for an all-NaN slice
+    # sum and count of the numbers in one pass; 0 / 0 -> NaN for an all-NaN slice
+    avg = nr.nanmean(u, axis=axis, dtype=res_dt, keepdims=keepdims, out=usm_out if direct else None)
     return get_result_array(avg, out, casting="unsafe")
 
 
@@ -199,9 +196,7 @@ def nanvar(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=
         if avg.shape != cnt.shape:
             avg = dpt.broadcast_to(avg, cnt.shape)
     else:
-        avg = nr.nansum(u, axis=axis, dtype=res_dt, keepdims=True)
-        if avg.size:
-            dpt.divide(avg, dpt.astype(cnt, res_dt), out=avg)
+        avg = nr.nanmean(u, axis=axis, dtype=res_dt, keepdims=True)
     # sum of squared deviations of the non-NaN elements, one pass
     nd = u.ndim
     axes = tuple(range(nd)) if axis is None else normalize_axis_tuple(

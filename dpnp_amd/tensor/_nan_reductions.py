@@ -42,6 +42,13 @@ def nancount(x, /, *, axis=None, keepdims=False, out=None):
                                 tri._nancount_over_axis_dtype_supported, _same_dtype)
 
 
+def nanmean(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
+    """Mean over `axis` of the elements that are not NaN, NaN where there is none: sum and count in
+    one pass, divided in the accumulation type."""
+    return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._nanmean_over_axis,
+                                tri._nanmean_over_axis_dtype_supported, _same_dtype)
+
+
 def nanargmax(x, /, *, axis=None, keepdims=False, out=None):
     """Index of the maximum along `axis` with NaN read as -inf (first occurrence)."""
     return _search_over_axis(x, axis, keepdims, out, tri._nanargmax_over_axis)

@@ -55,6 +55,7 @@ _nanprod_over_axis, _nanprod_over_axis_dtype_supported = _make_reduction("nanpro
 _nanmax_over_axis, _nanmax_over_axis_dtype_supported = _make_reduction("nanmax", _lib.REDUCE_ID["nanmax"])
 _nanmin_over_axis, _nanmin_over_axis_dtype_supported = _make_reduction("nanmin", _lib.REDUCE_ID["nanmin"])
 _nancount_over_axis, _nancount_over_axis_dtype_supported = _make_reduction("nancount", _lib.REDUCE_ID["nancount"])
+_nanmean_over_axis, _nanmean_over_axis_dtype_supported = _make_reduction("nanmean", _lib.REDUCE_ID["nanmean"])
 _nanargmax_over_axis = _make_search("nanargmax", _lib.SEARCH_ID["nanargmax"])
 _nanargmin_over_axis = _make_search("nanargmin", _lib.SEARCH_ID["nanargmin"])
 # the same, with results of runs whose extreme is the infinity NaNs are read as stored as -1 - index

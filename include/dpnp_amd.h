@@ -222,6 +222,9 @@ typedef enum dpx_reduce_op {
     DPX_R_ANY,
     DPX_R_ALL,
     DPX_R_COUNT_NONZERO,
+    /* mean of the elements that are not NaN in one pass (sum and count travel together; NaN
+     * for a run without a number): dpnp.nanmean, dpnp/dpnp_iface_nanfunctions.py:521-635 */
+    DPX_R_NANMEAN,
     DPX_R_NUM_OPS
 } dpx_reduce_op;
 

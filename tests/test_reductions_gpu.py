@@ -10,6 +10,7 @@ import pytest
 
 import dpnp_amd as dpnp
 import dpnp_amd.tensor as dpt
+from dpnp_amd.tensor import _nan_reductions as nr
 from oracle import oracle as orc
 from tests.helpers import ALL, assert_same, dev, dev_view_like, host, random_array
 
@@ -396,6 +397,40 @@ def test_nanarg_runs_whose_extreme_is_the_infinity_nan_counts_as(dt, shape, axis
     with pytest.raises(ValueError, match="All-NaN slice"):
         dpnp.nanargmin(d, axis=axis, out=out)
     assert (out.asnumpy() == -7).all()
+
+
+@pytest.mark.parametrize("dt, res", [("f2", None), ("f4", None), ("f8", None), ("c8", None), ("c16", None), ("f2", "f4"),
+                                     ("f4", "f8"), ("c8", "c16")])
+@pytest.mark.parametrize("shape, axis", [((4099,), None), ((2_000_003,), None), ((300, 700), 1), ((300, 700), 0),
+                                         ((40_000, 24), 0), ((40_000, 12), 1), ((60_000, 40), 0), ((9, 50, 11), (0, 2))])
+def test_nanmean_one_pass_over_every_kernel_family(dt, res, shape, axis):
+    """Sum and count of the numbers travel together through the reduction kernels; the quotient equals the one of
+    the reference's composition nansum / count (dpnp/dpnp_iface_nanfunctions.py:600-636) to rounding."""
+    rng = np.random.default_rng(31)
+    a = rng.uniform(0.5, 1.5, shape).astype(dt)
+    if a.dtype.kind == "c":
+        a = a + 1j * rng.uniform(0.5, 1.5, shape).astype(a.real.dtype)
+        a.imag[rng.random(shape) < 0.1] = np.nan
+    a[rng.random(shape) < 0.2] = np.nan
+    # a run without any number
+    if axis == 1:
+        a[0, :] = np.nan
+    elif axis == 0:
+        a[:, 0] = np.nan
+    elif axis == (0, 2):
+        a[:, 0, :] = np.nan
+    out_dt = np.dtype(res or dt)
+    got = nr.nanmean(dev(a), axis=axis, dtype=res)
+    assert got.dtype == out_dt
+    wide = a.astype("c16" if a.dtype.kind == "c" else "f8")
+    good = ~np.isnan(wide)
+    with np.errstate(all="ignore"):
+        want = (np.where(good, wide, 0).sum(axis=axis) / good.sum(axis=axis)).astype(out_dt)
+    eps = float(np.finfo(out_dt).eps)
+    rtol = 2e-3 if eps > 1e-4 else (2e-5 if eps > 1e-10 else 1e-12)
+    np.testing.assert_allclose(host(got), want, rtol=rtol, equal_nan=True)
+    if axis is not None:
+        assert np.isnan(host(got)).any()
 
 
 @pytest.mark.parametrize("dt", ["f4", "f8"])
