@@ -169,6 +169,38 @@ class dpnp_array:
 
         return dpnp.std(self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims, where=where)
 
+    def all(self, axis=None, out=None, keepdims=False, *, where=True):
+        from . import dpnp_iface as dpnp
+
+        return dpnp.all(self, axis=axis, out=out, keepdims=keepdims, where=where)
+
+    def any(self, axis=None, out=None, keepdims=False, *, where=True):
+        from . import dpnp_iface as dpnp
+
+        return dpnp.any(self, axis=axis, out=out, keepdims=keepdims, where=where)
+
+    def round(self, decimals=0, out=None):
+        from . import dpnp_iface_compositions as comp
+
+        return comp.round(self, decimals, out)
+
+    def conj(self):
+        """Complex conjugate; an array of a real dtype comes back as it is (dpnp_array.conj)."""
+        from . import dpnp_iface as dpnp
+
+        return dpnp.conj(self) if self.dtype.kind == "c" else self
+
+    conjugate = conj
+
+    def __copy__(self):
+        return self.copy(order="K")
+
+    def __array_namespace__(self, /, *, api_version=None):
+        return self._array_obj.__array_namespace__(api_version=api_version)
+
+    def tolist(self):
+        return self.asnumpy().tolist()
+
     # -- operators ------------------------------------------------------------------------------------
     def _b(self, name, other, reflected=False):
         from . import dpnp_iface as dpnp
@@ -210,7 +242,16 @@ class dpnp_array:
     def __rxor__(self, o): return self._b("bitwise_xor", o, True)
     def __ixor__(self, o): return self._ib("bitwise_xor", o)
     def __lshift__(self, o): return self._b("left_shift", o)
+    def __rlshift__(self, o): return self._b("left_shift", o, True)
+    def __ilshift__(self, o): return self._ib("left_shift", o)
     def __rshift__(self, o): return self._b("right_shift", o)
+    def __rrshift__(self, o): return self._b("right_shift", o, True)
+    def __irshift__(self, o): return self._ib("right_shift", o)
+    def __ifloordiv__(self, o): return self._ib("floor_divide", o)
+    def __imod__(self, o): return self._ib("remainder", o)
+    def __ipow__(self, o): return self._ib("power", o)
+    def __divmod__(self, o): return self._b("divmod", o)
+    def __rdivmod__(self, o): return self._b("divmod", o, True)
     def __eq__(self, o): return self._b("equal", o)
     def __ne__(self, o): return self._b("not_equal", o)
     def __lt__(self, o): return self._b("less", o)
