@@ -15,7 +15,9 @@ from .dpnp_iface_compositions import *  # noqa: F401,F403
 from .dpnp_iface_compositions import __all__ as _comp_all
 from .dpnp_iface_types import *  # noqa: F401,F403
 from .dpnp_iface_types import __all__ as _types_all
+from .dpnp_iface_manipulation import *  # noqa: F401,F403
+from .dpnp_iface_manipulation import __all__ as _manip_all
 from .dpnp_array import dpnp_array as ndarray
 
-__all__ = list(_iface_all) + list(_nan_all) + list(_comp_all) + list(_types_all) + ["ndarray", "tensor"]
+__all__ = list(_iface_all) + list(_nan_all) + list(_comp_all) + list(_types_all) + list(_manip_all) + ["ndarray", "tensor"]
 __version__ = "0.1.0"

@@ -198,6 +198,18 @@ class dpnp_array:
     def __array_namespace__(self, /, *, api_version=None):
         return self._array_obj.__array_namespace__(api_version=api_version)
 
+    def swapaxes(self, axis1, axis2):
+        return dpnp_array._create_from_usm_ndarray(dpt.swapaxes(self._array_obj, axis1, axis2))
+
+    def ravel(self, order="C"):
+        from . import dpnp_iface_manipulation as manip
+
+        return manip.ravel(self, order=order)
+
+    def flatten(self, order="C"):
+        """A 1-D copy of the elements in the given order."""
+        return self.reshape(-1, order=order, copy=True)
+
     def tolist(self):
         return self.asnumpy().tolist()
 

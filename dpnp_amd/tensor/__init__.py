@@ -38,12 +38,16 @@ from ._dtypes import (
 from ._elementwise_funcs import *  # noqa: F401,F403
 from ._elementwise_funcs import abs, pow, round  # noqa: A004
 from ._manipulation_functions import (
+    broadcast_arrays,
     broadcast_to,
     expand_dims,
     flip,
+    matrix_transpose,
+    moveaxis,
     permute_dims,
     reshape,
     squeeze,
+    swapaxes,
 )
 from ._reduction import (  # noqa: A004
     all,

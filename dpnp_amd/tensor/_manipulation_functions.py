@@ -192,3 +192,47 @@ def flip(x, /, *, axis=None):
     axes = range(x.ndim) if axis is None else normalize_axis_tuple(axis, x.ndim)
     key = tuple(slice(None, None, -1) if d in axes else slice(None) for d in range(x.ndim))
     return x[key]
+
+
+def moveaxis(x, source, destination, /):
+    """View with the axes `source` moved to the positions `destination`; the other axes keep their
+    order (dpnp/tensor/_manipulation_functions.py, `moveaxis`)."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    source = normalize_axis_tuple(source, x.ndim, "source")
+    destination = normalize_axis_tuple(destination, x.ndim, "destination")
+    if len(source) != len(destination):
+        raise ValueError("`source` and `destination` arguments must have the same number of elements")
+    order = [n for n in range(x.ndim) if n not in source]
+    for dest, src in sorted(zip(destination, source)):
+        order.insert(dest, src)
+    return permute_dims(x, tuple(order))
+
+
+def swapaxes(x, axis1, axis2):
+    """View with two axes exchanged (dpnp/tensor/_manipulation_functions.py, `swapaxes`)."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    axis1 = normalize_axis_index(axis1, x.ndim, "axis1")
+    axis2 = normalize_axis_index(axis2, x.ndim, "axis2")
+    order = list(range(x.ndim))
+    order[axis1], order[axis2] = order[axis2], order[axis1]
+    return permute_dims(x, tuple(order))
+
+
+def matrix_transpose(x):
+    """View with the last two axes exchanged; needs at least two dimensions."""
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expected usm_ndarray type; got {type(x)}.")
+    return x.mT
+
+
+def broadcast_arrays(*args):
+    """Views of the arrays stretched to their common shape."""
+    if len(args) == 0:
+        raise ValueError("`broadcast_arrays` requires at least one argument")
+    for a in args:
+        if not isinstance(a, usm_ndarray):
+            raise TypeError(f"Expected usm_ndarray type; got {type(a)}.")
+    shape = _broadcast_shape_impl([a.shape for a in args])
+    return [a if a.shape == shape else broadcast_to(a, shape) for a in args]
