@@ -41,7 +41,7 @@ BINARY_OPS = [
 ]
 REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot",
               "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev",
-              "any", "all", "count_nonzero", "nanmean"]
+              "any", "all", "count_nonzero", "nanmean", "nanvar"]
 SEARCH_OPS = ["argmax", "argmin", "nanargmax", "nanargmin", "nanargmax_marked", "nanargmin_marked"]
 UNARY_ID = {n: i for i, n in enumerate(UNARY_OPS)}
 BINARY_ID = {n: i for i, n in enumerate(BINARY_OPS)}
@@ -125,6 +125,7 @@ SIGNATURES = {
     "dpx_where_compare": (_i, [_i, _VP, _VP, _VP, _VP, _VP, _vp]),
     "dpx_black_scholes": (_i, [_vp, _vp, _vp, _d, _d, _vp, _vp, _i64, _i, _vp]),
     "dpx_reduce": (_i, [_i, _VP, _i, _VP, _VP, _vp]),
+    "dpx_nan_variance": (_i, [_VP, _i, _VP, _d, _VP, _vp]),
     "dpx_argreduce": (_i, [_i, _VP, _i, _VP, _vp]),
     "dpx_reduce_plan": (_i, [_i, _VP, _i, _VP, _PP]),
     "dpx_argreduce_plan": (_i, [_i, _VP, _i, _VP, _PP]),

@@ -51,6 +51,7 @@ struct RedLaunch {
     int64_t inner;    // cols: length of the inner (contiguous) iteration dim
     int64_t col_blocks;
     int32_t mark_fill; // NaN-ignoring searches: report "extreme equals the value NaNs count as" as -1 - index
+    double param;      // K_NANVAR: delta degrees of freedom
 };
 
 template <class T> DPX_D T shfl_down_any(T v, int off)
@@ -129,8 +130,12 @@ enum {
     // truth-value reductions of any input type: an element counts as true when it is not zero
     K_ANY = 13, K_ALL = 14, K_COUNT_NONZERO = 15,
     // mean of the elements that are not NaN: sum and count travel together, divided at the end
-    K_NANMEAN = 16
+    K_NANMEAN = 16,
+    // variance of the elements that are not NaN around a given mean: squared deviations and count travel
+    // together, divided by count - ddof at the end
+    K_NANVAR = 17
 };
+constexpr bool kind_has_count(int k) { return k == K_NANMEAN || k == K_NANVAR; }
 // accumulator of K_NANMEAN
 template <class A> struct mean_acc {
     A s;
@@ -170,14 +175,14 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     using In = In_;
     using Out = Out_;
     using Acc = std::conditional_t<
-        KIND == K_NANMEAN, mean_acc<acc_of_t<Out_>>,
+        kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
         std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>;
     using Aux = Out_;
-    static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV) && !FINAL;
+    static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV || KIND == K_NANVAR) && !FINAL;
     static constexpr int kind = KIND;
     DPX_D static Acc identity()
     {
-        if constexpr (KIND == K_NANMEAN) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
+        if constexpr (kind_has_count(KIND)) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
         else if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
         else if constexpr (is_bool_v<Out>) return (KIND == K_PROD || KIND == K_ALL) ? 1 : 0;
         else if constexpr (KIND == K_COUNT_NONZERO) return Acc(0);
@@ -193,6 +198,11 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         else if constexpr (KIND == K_NANMEAN) {
             const bool skip = isnan_(x);
             return Acc{skip ? red_identity<K_SUM, acc_of_t<Out>>() : in_to_acc<In, Out>(x), skip ? 0 : 1};
+        }
+        else if constexpr (KIND == K_NANVAR) { // aux.s holds the mean
+            const acc_of_t<Out> d = in_to_acc<In, Out>(x) - aux.s;
+            const bool skip = isnan_(x);
+            return Acc{skip ? acc_of_t<Out>(0) : d * d, skip ? 0 : 1};
         }
         else if constexpr (KIND == K_SUMSQDEV) {
             const Acc d = in_to_acc<In, Out>(x) - aux;
@@ -214,7 +224,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     }
     DPX_D static Acc combine(Acc a, Acc b)
     {
-        if constexpr (KIND == K_NANMEAN) return Acc{a.s + b.s, a.c + b.c};
+        if constexpr (kind_has_count(KIND)) return Acc{a.s + b.s, a.c + b.c};
         else if constexpr (is_bool_v<Out>) {
             if constexpr (KIND == K_PROD || KIND == K_MIN || KIND == K_ALL) return a & b;
             else return a | b;
@@ -273,7 +283,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     }
     DPX_D static Out post(Acc a)
     {
-        if constexpr (KIND == K_NANMEAN) {
+        if constexpr (KIND == K_NANVAR) return post(a, 0.0);
+        else if constexpr (KIND == K_NANMEAN) {
             // sum / count in the accumulator's type: 0 / 0 = NaN for a run without a number
             using A = acc_of_t<Out>;
             if constexpr (is_cplx_v<A>) {
@@ -284,9 +295,20 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         }
         else return acc_to_out<Acc, Out>(a);
     }
+    // result of a run given the launch's scalar parameter
+    DPX_D static Out post(Acc a, double param)
+    {
+        if constexpr (KIND == K_NANVAR) {
+            using A = acc_of_t<Out>;
+            const A dof = (A)a.c - (A)param;
+            return acc_to_out<A, Out>(dof > A(0) ? a.s / dof : (A)__builtin_nanf(""));
+        }
+        else return post(a);
+    }
     DPX_D static Acc load_aux(const Aux *p)
     {
-        if constexpr (std::is_same_v<Aux, half_t>) return (float)*p;
+        if constexpr (KIND == K_NANVAR) return Acc{(acc_of_t<Out>)*p, 0};
+        else if constexpr (std::is_same_v<Aux, half_t>) return (float)*p;
         else if constexpr (is_bool_v<Aux>) return (int32_t)p->v;
         else return (Acc)*p;
     }
@@ -518,7 +540,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L
     static_assert(RED_U == 4);
     r = group_reduce<P>(r, whole_block, G);
     if (L.splits == 1) {
-        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = P::post(r);
+        if (active && lane == 0 && (!whole_block || threadIdx.x == 0)) dst[dof] = P::post(r, L.param);
         return;
     }
     // split mode (always a whole block per output): pass two by the last block to finish
@@ -528,7 +550,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L
     Acc v = P::identity();
     for (int i = threadIdx.x; i < L.splits; i += blockDim.x) v = P::combine(v, slot_read(partial + o * L.splits + i));
     v = group_reduce<P>(v, true, G);
-    if (threadIdx.x == 0) dst[dof] = P::post(v);
+    if (threadIdx.x == 0) dst[dof] = P::post(v, L.param);
 }
 
 // ================================ cols kernel ================================================
@@ -674,7 +696,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         if (ty == 0 && active) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e]);
+                if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e], L.param);
         }
         return;
     }
@@ -718,7 +740,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     if (ty == 0 && active) {
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e]);
+            if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e], L.param);
     }
 }
 
@@ -816,7 +838,7 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     }
     flat_fold_columns<P>(sm, T * E, inner);
     if (L.splits == 1) {
-        for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c]);
+        for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c], L.param);
         return;
     }
     uint32_t zero = 0;
@@ -841,7 +863,7 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     __syncthreads(); // every thread has read its column results of the first fold
     if (t < parts * inner) sm[t] = v;
     flat_fold_columns<P>(sm, parts * inner, inner);
-    for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c]);
+    for (int c = t; c < inner; c += T) dst[(int64_t)c * ix.dst_str[0]] = P::post(sm[c], L.param);
 }
 
 // ================================ short rows kernel ===========================================
@@ -918,7 +940,7 @@ __global__ __launch_bounds__(256) void red_short_rows_kernel(RedIndex ix, RedLau
         const In *row = sm + r * pitch;
         Acc acc = P::identity();
         for (uint32_t j = 0; j < n; ++j) acc = P::combine(acc, P::pre(row[j], a));
-        dst[o * ix.dst_str[0]] = P::post(acc);
+        dst[o * ix.dst_str[0]] = P::post(acc, L.param);
     }
 }
 

@@ -22,8 +22,11 @@ int nanarg_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, 
 bool truth_pair_supported(int, int, int);
 int truth_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 static bool is_truth_op(int op) { return op == DPX_R_ANY || op == DPX_R_ALL || op == DPX_R_COUNT_NONZERO; }
-static bool is_nan_op(int op) { return (op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV) || op == DPX_R_NANMEAN; }
-static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV; }
+static bool is_nan_op(int op)
+{
+    return (op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV) || op == DPX_R_NANMEAN || op == DPX_R_NANVAR;
+}
+static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV || op == DPX_R_NANVAR; }
 
 static bool reduce_supported(int op, int s, int d)
 {
@@ -43,7 +46,7 @@ static bool reduce_supported(int op, int s, int d)
 }
 
 static int reduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
-                       const dpx_array_view *aux, void *stream, dpx_plan *plan_out)
+                       const dpx_array_view *aux, void *stream, dpx_plan *plan_out, double param = 0.0)
 {
     if (op < 0 || op >= DPX_R_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown reduction op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
@@ -67,6 +70,7 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         return DPX_OK;
     }
     hipStream_t s = (hipStream_t)stream;
+    pl.L.param = param;
     if (is_nan_op(op)) return nan_run(op, pl, src, dst, aux, s);
     if (is_truth_op(op)) return truth_run(op, pl, src, dst, s);
     switch (op) {
@@ -126,7 +130,13 @@ int dpx_reduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_redu
     // a plan for a squared-deviation op is that of the matching sum with the same dtypes
     if (op == DPX_R_SUMSQDEV) op = DPX_R_SUM;
     if (op == DPX_R_NANSUMSQDEV) op = DPX_R_NANSUM;
+    if (op == DPX_R_NANVAR) op = DPX_R_NANMEAN;
     return reduce_call(op, src, trailing_dims_to_reduce, dst, nullptr, nullptr, plan);
+}
+int dpx_nan_variance(const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *mean, double ddof,
+                     const dpx_array_view *dst, void *stream)
+{
+    return reduce_call(DPX_R_NANVAR, src, trailing_dims_to_reduce, dst, mean, stream, nullptr, ddof);
 }
 int dpx_argreduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
                   void *stream)

@@ -26,7 +26,7 @@ template <class F> static bool for_nan_pair(int op, int in_dt, int out_dt, F &&f
         DPX_PAIR(half_t, int64_t) DPX_PAIR(float, int64_t) DPX_PAIR(double, int64_t) DPX_PAIR(c64, int64_t)
         DPX_PAIR(c128, int64_t)
     }
-    else if (op == DPX_R_NANSUMSQDEV) {
+    else if (op == DPX_R_NANSUMSQDEV || op == DPX_R_NANVAR) {
         DPX_PAIR(half_t, half_t) DPX_PAIR(float, float) DPX_PAIR(double, double) DPX_PAIR(half_t, float)
         DPX_PAIR(float, double)
     }
@@ -47,7 +47,7 @@ template <int KIND> static int nan_run_kind(int op, RedPlan &pl, const dpx_array
         using I = typename decltype(it)::type;
         using O = typename decltype(ot)::type;
         // the pair lists above keep complex inputs away from the ordered and the squared-deviation kinds
-        constexpr bool ok = !(is_cplx_v<I> && (kind_is_minmax(KIND) || KIND == K_NANSUMSQDEV)) &&
+        constexpr bool ok = !(is_cplx_v<I> && (kind_is_minmax(KIND) || KIND == K_NANSUMSQDEV || KIND == K_NANVAR)) &&
                             (KIND == K_NANCOUNT) == std::is_same_v<O, int64_t>;
         if constexpr (ok) {
             if (acc_size) {
@@ -71,6 +71,7 @@ static int nan_dispatch(int op, RedPlan &pl, const dpx_array_view *src, const dp
     case DPX_R_NANCOUNT: return nan_run_kind<K_NANCOUNT>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANSUMSQDEV: return nan_run_kind<K_NANSUMSQDEV>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANMEAN: return nan_run_kind<K_NANMEAN>(op, pl, src, dst, aux, stream, acc_size);
+    case DPX_R_NANVAR: return nan_run_kind<K_NANVAR>(op, pl, src, dst, aux, stream, acc_size);
     default: return DPX_ERR_NOT_IMPLEMENTED;
     }
 }

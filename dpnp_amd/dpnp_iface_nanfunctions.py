@@ -190,17 +190,18 @@ def nanvar(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=
     res_dt = u.dtype if dtype is None else dtype
     if res_dt.kind == "c":
         raise NotImplementedError("nanvar with a complex dtype is outside this library's scope")
-    cnt = nr.nancount(u, axis=axis, keepdims=True)
-    if mean is not None:
-        avg = dpt.astype(get_usm_ndarray(mean), res_dt, copy=False)
-        if avg.shape != cnt.shape:
-            avg = dpt.broadcast_to(avg, cnt.shape)
-    else:
-        avg = nr.nanmean(u, axis=axis, dtype=res_dt, keepdims=True)
-    # sum of squared deviations of the non-NaN elements, one pass
     nd = u.ndim
     axes = tuple(range(nd)) if axis is None else normalize_axis_tuple(
         axis if isinstance(axis, (tuple, list)) else (axis,), nd, "axis")
+    kept_shape = tuple(1 if d in axes else u.shape[d] for d in range(nd))
+    if mean is not None:
+        avg = dpt.astype(get_usm_ndarray(mean), res_dt, copy=False)
+        if avg.shape != kept_shape:
+            avg = dpt.broadcast_to(avg, kept_shape)
+    else:
+        avg = nr.nanmean(u, axis=axis, dtype=res_dt, keepdims=True)
+    # squared deviations and count of the non-NaN elements travel together: one pass gives
+    # sum / (count - ddof), NaN where count <= ddof
     perm = [i for i in range(nd) if i not in axes] + list(axes)
     red_nd = len(axes)
     src = u
@@ -210,19 +211,10 @@ def nanvar(a, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=
     res_shape = arr.shape[: nd - red_nd]
     ssq = dpt.empty(res_shape, dtype=res_dt)
     avg_flat = dpt.reshape(dpt.permute_dims(avg, perm), res_shape)
-    if not avg_flat.flags.writable or avg_flat.dtype != res_dt:
+    if avg_flat.dtype != res_dt:
         avg_flat = dpt.astype(avg_flat, res_dt)
-    cnt_flat = dpt.reshape(dpt.permute_dims(cnt, perm), res_shape)
     if ssq.size:
-        if red_nd:
-            tri._sumsqdev_over_axis(src=arr, mean=avg_flat, trailing_dims_to_reduce=red_nd, dst=ssq, nan=True)
-        else:
-            ti._full_usm_ndarray(0, ssq)
-        dof = dpt.subtract(dpt.astype(cnt_flat, res_dt), dpt.asarray(ddof, dtype=res_dt))
-        tei._divide(src1=ssq, src2=dof, dst=ssq)
-        bad = dpt.less_equal(dof, 0)
-        if _any_true(bad):
-            ssq = dpt.where(bad, dpt.asarray(math.nan, dtype=res_dt), ssq)
+        tri._nanvar_over_axis(src=arr, mean=avg_flat, trailing_dims_to_reduce=red_nd, ddof=ddof, dst=ssq)
     if keepdims:
         inv = sorted(range(nd), key=lambda d: perm[d])
         ssq = dpt.permute_dims(dpt.reshape(ssq, tuple(res_shape) + (1,) * red_nd), inv)

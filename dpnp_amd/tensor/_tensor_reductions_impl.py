@@ -76,3 +76,12 @@ def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None
 def _sumsqdev_over_axis_dtype_supported(arg_dtype, out_dtype, dst_usm_type=None, sycl_queue=None):
     return bool(lib.dpx_reduce_dtype_supported(_lib.REDUCE_ID["sumsqdev"], dtype_id(arg_dtype),
                                                dtype_id(out_dtype)))
+
+
+def _nanvar_over_axis(src, mean, trailing_dims_to_reduce, ddof, dst, sycl_queue=None, depends=()):
+    """dst[i] = sum_j (src[i, j] - mean[i])**2 / (count_i - ddof) over the elements that are not NaN, NaN where
+    count_i <= ddof: the second pass of nanvar in one kernel (dpnp/dpnp_iface_nanfunctions.py:1318-1390 runs
+    count, subtract, square, sum and divide as separate calls)."""
+    vs, vm, vd = src._as_view(), mean._as_view(), dst._as_view()
+    _lib.check(lib.dpx_nan_variance(vs, int(trailing_dims_to_reduce), vm, float(ddof), vd, _stream(sycl_queue)))
+    return _events(sycl_queue)

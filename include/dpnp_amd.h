@@ -225,6 +225,11 @@ typedef enum dpx_reduce_op {
     /* mean of the elements that are not NaN in one pass (sum and count travel together; NaN
      * for a run without a number): dpnp.nanmean, dpnp/dpnp_iface_nanfunctions.py:521-635 */
     DPX_R_NANMEAN,
+    /* variance of the elements that are not NaN around the mean given in `aux`, in one pass:
+     * sum of squared deviations / (count - ddof), NaN where count <= ddof (dpnp.nanvar,
+     * dpnp/dpnp_iface_nanfunctions.py:1188-1391).  ddof is 0 through dpx_reduce; dpx_nan_variance
+     * takes it as an argument. */
+    DPX_R_NANVAR,
     DPX_R_NUM_OPS
 } dpx_reduce_op;
 
@@ -432,6 +437,13 @@ int dpx_black_scholes(const void *price, const void *strike, const void *t,
 int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
                const dpx_array_view *dst, const dpx_array_view *aux,
                void *stream);
+/* DPX_R_NANVAR with a delta degrees of freedom: dst[i] = sum_j (src[i,j] - mean[i])^2 /
+ * (count_i - ddof) over the elements that are not NaN, NaN where count_i <= ddof.  The second pass
+ * of dpnp.nanvar / nanstd (dpnp/dpnp_iface_nanfunctions.py:1318-1390: count, mean, subtract,
+ * square, sum and divide as separate calls there). */
+int dpx_nan_variance(const dpx_array_view *src, int trailing_dims_to_reduce,
+                     const dpx_array_view *mean, double ddof,
+                     const dpx_array_view *dst, void *stream);
 /* py_search_over_axis, reduction_over_axis.hpp:781-1047 (tri._argmax_over_axis,
  * tri._argmin_over_axis): int64 C-order flat index over the reduced axes,
  * smallest index among equal extrema, NaN counts as the extremum (first NaN) */

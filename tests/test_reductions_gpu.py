@@ -433,6 +433,44 @@ def test_nanmean_one_pass_over_every_kernel_family(dt, res, shape, axis):
         assert np.isnan(host(got)).any()
 
 
+@pytest.mark.parametrize("dt, res", [("f2", None), ("f4", None), ("f8", None), ("f2", "f4"), ("f4", "f8")])
+@pytest.mark.parametrize("shape, axis", [((4099,), None), ((2_000_003,), None), ((300, 700), 1), ((300, 700), 0),
+                                         ((40_000, 24), 0), ((40_000, 12), 1), ((60_000, 40), 0), ((9, 50, 11), (0, 2))])
+@pytest.mark.parametrize("ddof", [0, 1, 2.5])
+def test_nanvar_second_pass_over_every_kernel_family(dt, res, shape, axis, ddof):
+    """Squared deviations and count of the numbers travel together through the reduction kernels and are divided by
+    count - ddof at the end; slices with count <= ddof give NaN (dpnp/dpnp_iface_nanfunctions.py:1318-1390)."""
+    rng = np.random.default_rng(37)
+    a = rng.uniform(0.5, 1.5, shape).astype(dt)
+    a[rng.random(shape) < 0.2] = np.nan
+    if axis == 1:
+        a[0, :] = np.nan          # no number at all
+        a[1, 2:] = np.nan         # two numbers: NaN for ddof 2.5
+    elif axis == 0:
+        a[:, 0] = np.nan
+        a[2:, 1] = np.nan
+    elif axis == (0, 2):
+        a[:, 0, :] = np.nan
+        a[:, 1, :] = np.nan
+        a[0, 1, :2] = 1.0
+    out_dt = np.dtype(res or dt)
+    got = dpnp.nanvar(dpnp.array(a), axis=axis, dtype=res, ddof=ddof)
+    assert got.dtype == out_dt
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        want = np.nanvar(a.astype("f8"), axis=axis, ddof=ddof)
+    want = np.where(np.isfinite(want) & (want >= 0), want, np.nan)  # NumPy divides by a negative count - ddof
+    eps = float(np.finfo(out_dt).eps)
+    rtol = 4e-3 if eps > 1e-4 else (4e-5 if eps > 1e-10 else 1e-11)
+    np.testing.assert_allclose(got.asnumpy().astype("f8"), want, rtol=rtol, atol=rtol * 1e-2, equal_nan=True)
+    if axis is not None:
+        assert np.isnan(got.asnumpy()).any()
+    # a mean handed in by the caller is taken as it is
+    mu = dpnp.nanmean(dpnp.array(a), axis=axis, dtype=res, keepdims=True)
+    again = dpnp.nanvar(dpnp.array(a), axis=axis, dtype=res, ddof=ddof, mean=mu)
+    np.testing.assert_array_equal(again.asnumpy(), got.asnumpy())
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 @pytest.mark.parametrize("axis", [None, 0, 1, (0, 1)])
 @pytest.mark.parametrize("keepdims", [False, True])
