@@ -85,9 +85,9 @@ template <class T> DPX_HD T min_nan(T x, T y)
 // its last bits do not reach the result.  Measured on MI355X against a long double reference
 // over 4 M arguments (all binades, dense around 1): error below 0.82 ULP (the device
 // library's: 0.63 ULP); 2^27 elements take 0.37 ms instead of 0.57 ms.
-DPX_D double log_f64(double x)
+// k and log(m) = hi + lo for x = 2^k m, sqrt(1/2) <= m < sqrt(2) (x > 0 and finite)
+DPX_D void log_f64_parts(double x, double &dk, double &f, double &hfsq, double &tail)
 {
-    constexpr double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
     constexpr double Lg1 = 6.666666666666735130e-01, Lg2 = 3.999999999940941908e-01,
                      Lg3 = 2.857142874366239149e-01, Lg4 = 2.222219843214978396e-01,
                      Lg5 = 1.818357216161805012e-01, Lg6 = 1.531383769920937332e-01,
@@ -97,7 +97,8 @@ DPX_D double log_f64(double x)
     const bool low = m < 0.70710678118654752440;
     m = low ? m * 2.0 : m;
     e = low ? e - 1 : e;
-    const double f = m - 1.0, dk = (double)e;
+    f = m - 1.0;
+    dk = (double)e;
     const double d = 2.0 + f;
     double rc = __builtin_amdgcn_rcp(d);
     rc = __builtin_fma(__builtin_fma(-d, rc, 1.0), rc, rc);
@@ -105,13 +106,192 @@ DPX_D double log_f64(double x)
     const double s = f * rc, z = s * s, w = z * z;
     const double t1 = w * __builtin_fma(w, __builtin_fma(w, Lg6, Lg4), Lg2);
     const double p2 = __builtin_fma(w, __builtin_fma(w, __builtin_fma(w, Lg7, Lg5), Lg3), Lg1);
-    const double R = __builtin_fma(z, p2, t1), hfsq = (0.5 * f) * f;
-    const double in = __builtin_fma(s, hfsq + R, dk * ln2_lo);
-    double r = __builtin_fma(dk, ln2_hi, -((hfsq - in) - f));
+    const double R = __builtin_fma(z, p2, t1);
+    hfsq = (0.5 * f) * f;
+    tail = s * (hfsq + R); // log(m) = f - hfsq + tail
+}
+DPX_D double log_special(double x, double r)
+{
     r = (x == 0.0) ? -__builtin_inf() : r;
     r = (x < 0.0) ? __builtin_nan("") : r;
     return !(x < __builtin_inf()) ? x : r; // +inf and NaN
 }
+DPX_D double log_f64(double x)
+{
+    constexpr double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
+    double dk, f, hfsq, tail;
+    log_f64_parts(x, dk, f, hfsq, tail);
+    const double in = __builtin_fma(dk, ln2_lo, tail);
+    const double r = __builtin_fma(dk, ln2_hi, -((hfsq - in) - f));
+    return log_special(x, r);
+}
+// log2 and log10 of a double from the same parts: log(m) as an unevaluated sum hi + lo, times
+// the constant split in two, plus k (log2) or k log10(2).  Exact for powers of two (log2) and within
+// about 1 ULP elsewhere; the device library's routines run at half the speed of its log.
+DPX_D double log_scaled_f64(double x, double c_hi, double c_lo, double k_hi, double k_lo)
+{
+    double dk, f, hfsq, tail;
+    log_f64_parts(x, dk, f, hfsq, tail);
+    const double hi = f - hfsq;
+    const double lo = ((f - hi) - hfsq) + tail;
+    const double p = hi * c_hi;
+    double v_lo = __builtin_fma(hi, c_hi, -p) + __builtin_fma(hi, c_lo, lo * c_hi);
+    const double y = dk * k_hi; // exact: k_hi has few significant bits
+    v_lo = __builtin_fma(dk, k_lo, v_lo);
+    const double w = y + p;
+    v_lo += (y - w) + p;
+    return log_special(x, w + v_lo);
+}
+DPX_D double log2_f64(double x)
+{
+    return log_scaled_f64(x, 1.44269504088896338700e+00, 2.03552737409310331e-17, 1.0, 0.0);
+}
+DPX_D double log10_f64(double x)
+{
+    // log10(2) split: the high part has its low 32 bits clear
+    return log_scaled_f64(x, 4.34294481903251816668e-01, 1.09831965021676510e-17, 3.01029995663611771306e-01,
+                          3.69423907715893078616e-13);
+}
+// log1p: log(u) for u = 1 + x rounded, plus the rounding error of that sum over u
+// (log(1 + x) = log(u) + log(1 + c/u), c = (1 + x) - u).
+template <class R, class LOG> DPX_D R log1p_via(R x, LOG log_fn)
+{
+    const R u = R(1) + x;
+    const R c = (x < R(1) && x > R(-1)) ? x - (u - R(1)) : R(1) - (u - x);
+    // c / u through the hardware reciprocal (about 25 bits for a double: two Newton steps; for tiny x
+    // the quotient is the whole result)
+    R rcp;
+    if constexpr (std::is_same_v<R, double>) {
+        rcp = __builtin_amdgcn_rcp(u);
+        rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
+        rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
+    }
+    else rcp = __builtin_amdgcn_rcpf(u);
+    R r = log_fn(u) + c * rcp;
+    r = (u == R(0)) ? -(R)__builtin_inff() : r; // x = -1
+    r = (x == (R)__builtin_inff()) ? x : r;
+    const R ax = x < R(0) ? -x : x;
+    return (ax < (std::is_same_v<R, double> ? R(1e-17) : R(1e-8))) ? x : r; // also keeps -0.0
+}
+DPX_D double log1p_f64(double x) { return log1p_via<double>(x, [](double u) { return log_f64(u); }); }
+DPX_D float log1p_f32(float x) { return log1p_via<float>(x, [](float u) { return ::logf(u); }); }
+
+// Inverse hyperbolic functions through log1p (the formulas of fdlibm's s_asinh.c, e_acosh.c, e_atanh.c
+// with log(y) written log1p(y - 1), exact there since y >= 2, so that one logarithm serves every range):
+//   asinh a = log1p(a + a^2/(1 + sqrt(1 + a^2)))            a <= 2
+//           = log1p((2a - 1) + 1/(a + sqrt(a^2 + 1)))       a > 2
+//   acosh x = log1p(t + sqrt(t (2 + t))), t = x - 1         x <= 2
+//           = log1p((2x - 1) - 1/(x + sqrt(x^2 - 1)))       x > 2
+//   atanh a = log1p(2a + 2a^2/(1 - a))/2                    a < 1/2
+//           = log1p(2a/(1 - a))/2                           a >= 1/2
+// and log1p(a - 1) + ln 2 where a^2 + 1 = a^2 to working precision.
+template <class R> inline constexpr R asinh_big = std::is_same_v<R, double> ? R(268435456.0) : R(16384.0);
+template <class R, class LOG1P, class SQRT> DPX_D R asinh_via(R x, LOG1P log1p_fn, SQRT sqrt_fn)
+{
+    const R ln2 = R(0.69314718055994530941723212145817657);
+    const R a = x < R(0) ? -x : x;
+    const bool big = a > asinh_big<R>, mid = a > R(2);
+    const R t = a * a;
+    const R s = sqrt_fn(t + R(1));
+    const R q = (mid ? R(1) : t) / (mid ? s + a : R(1) + s);
+    R w = (mid ? (a + a) - R(1) : a) + q;
+    w = big ? a - R(1) : w;
+    R r = log1p_fn(w);
+    r = big ? r + ln2 : r;
+    return (x != x) ? x : __builtin_copysign(r, x);
+}
+template <class R, class LOG1P, class SQRT> DPX_D R acosh_via(R x, LOG1P log1p_fn, SQRT sqrt_fn)
+{
+    const R ln2 = R(0.69314718055994530941723212145817657);
+    const bool big = x > asinh_big<R>, mid = x > R(2);
+    const R t = x - R(1);
+    const R s = sqrt_fn(mid ? x * x - R(1) : t * (R(2) + t));
+    R w = mid ? ((x + x) - R(1)) - R(1) / (x + s) : t + s;
+    w = big ? t : w;
+    R r = log1p_fn(w);
+    r = big ? r + ln2 : r;
+    return (x < R(1)) ? (R)__builtin_nanf("") : r; // NaN goes through
+}
+template <class R, class LOG1P> DPX_D R atanh_via(R x, LOG1P log1p_fn)
+{
+    const R a = x < R(0) ? -x : x;
+    const R t = a + a;
+    const bool small = a < R(0.5);
+    const R q = (small ? t * a : t) / (R(1) - a);
+    const R w = small ? t + q : q;
+    const R r = R(0.5) * log1p_fn(w);
+    return (x != x) ? x : __builtin_copysign(r, x);
+}
+DPX_D double asinh_f64(double x)
+{
+    return asinh_via<double>(x, [](double v) { return log1p_f64(v); }, [](double v) { return __builtin_sqrt(v); });
+}
+DPX_D double acosh_f64(double x)
+{
+    return acosh_via<double>(x, [](double v) { return log1p_f64(v); }, [](double v) { return __builtin_sqrt(v); });
+}
+DPX_D double atanh_f64(double x) { return atanh_via<double>(x, [](double v) { return log1p_f64(v); }); }
+DPX_D float asinh_f32(float x)
+{
+    return asinh_via<float>(x, [](float v) { return log1p_f32(v); }, [](float v) { return __builtin_sqrtf(v); });
+}
+DPX_D float acosh_f32(float x)
+{
+    return acosh_via<float>(x, [](float v) { return log1p_f32(v); }, [](float v) { return __builtin_sqrtf(v); });
+}
+DPX_D float atanh_f32(float x) { return atanh_via<float>(x, [](float v) { return log1p_f32(v); }); }
+
+// Hyperbolic functions from exp and expm1 (the forms of fdlibm's s_tanh.c, e_sinh.c, e_cosh.c):
+//   tanh a = t / (t + 2), t = expm1(2a);   sinh a = (t + t/(t+1))/2, t = expm1(a);
+//   cosh a = (e + 1/e)/2, e = exp(a), for a = |x|; where exp(a) would overflow and the function does
+// not yet, (exp(a/2)/2) exp(a/2).
+template <class R, class EXPM1> DPX_D R tanh_via(R x, EXPM1 expm1_fn)
+{
+    const R a = x < R(0) ? -x : x;
+    const R big = std::is_same_v<R, double> ? R(22) : R(10);
+    const R t = expm1_fn(a + a);
+    R r = t / (t + R(2));
+    r = (a > big) ? R(1) : r;
+    r = (a == R(0)) ? a : r;
+    return (x != x) ? x : __builtin_copysign(r, x);
+}
+template <class R, class EXP, class EXPM1> DPX_D R sinh_via(R x, EXP exp_fn, EXPM1 expm1_fn)
+{
+    const R a = x < R(0) ? -x : x;
+    const R over = std::is_same_v<R, double> ? R(709) : R(88); // exp(a) and expm1(a) are finite up to here
+    const R t = expm1_fn(a);
+    const R q = t / (t + R(1));
+    R r = R(0.5) * ((a < R(1)) ? R(2) * t - t * q : t + q);
+    if (a > over) { // rare: the band where sinh is finite and exp is not, and beyond
+        const R w = exp_fn(R(0.5) * a);
+        r = (R(0.5) * w) * w;
+    }
+    r = (a == R(0)) ? a : r;
+    return (x != x) ? x : __builtin_copysign(r, x);
+}
+template <class R, class EXP> DPX_D R cosh_via(R x, EXP exp_fn)
+{
+    const R a = x < R(0) ? -x : x;
+    const R over = std::is_same_v<R, double> ? R(709) : R(88);
+    const R e = exp_fn(a);
+    R r = R(0.5) * e + R(0.5) / e; // NaN goes through exp
+    if (a > over) {
+        const R w = exp_fn(R(0.5) * a);
+        r = (R(0.5) * w) * w;
+    }
+    return r;
+}
+DPX_D double tanh_f64(double x) { return tanh_via<double>(x, [](double v) { return ::expm1(v); }); }
+DPX_D double sinh_f64(double x)
+{
+    return sinh_via<double>(x, [](double v) { return ::exp(v); }, [](double v) { return ::expm1(v); });
+}
+DPX_D double cosh_f64(double x) { return cosh_via<double>(x, [](double v) { return ::exp(v); }); }
+DPX_D float sinh_f32(float x)
+{
+    return sinh_via<float>(x, [](float v) { return ::expf(v); }, [](float v) { return ::expm1f(v); });
+}
+DPX_D float cosh_f32(float x) { return cosh_via<float>(x, [](float v) { return ::expf(v); }); }
 
 // fp64 erf from a table of erf(r) and erf'(r) at r = i/128 and the Taylor series of erf about r:
 //   erf(r + d) = erf(r) + erf'(r) (d - r d^2 + (2r^2-1)/3 d^3 - r(2r^2-3)/6 d^4 + (4r^4-12r^2+3)/30 d^5
@@ -161,12 +341,12 @@ DPX_FP_FN1(m_erf, ::erff, erf_f64)
 DPX_FP_FN1(m_sin, ::sinf, ::sin)
 DPX_FP_FN1(m_cos, ::cosf, ::cos)
 DPX_FP_FN1(m_tan, ::tanf, ::tan)
-DPX_FP_FN1(m_tanh, ::tanhf, ::tanh)
+DPX_FP_FN1(m_tanh, ::tanhf, tanh_f64)
 DPX_FP_FN1(m_exp2, ::exp2f, ::exp2)
 DPX_FP_FN1(m_expm1, ::expm1f, ::expm1)
-DPX_FP_FN1(m_log2, ::log2f, ::log2)
-DPX_FP_FN1(m_log10, ::log10f, ::log10)
-DPX_FP_FN1(m_log1p, ::log1pf, ::log1p)
+DPX_FP_FN1(m_log2, ::log2f, log2_f64)
+DPX_FP_FN1(m_log10, ::log10f, log10_f64)
+DPX_FP_FN1(m_log1p, log1p_f32, log1p_f64)
 DPX_FP_FN1(m_cbrt, ::cbrtf, ::cbrt)
 DPX_FP_FN1(m_floor, ::floorf, ::floor)
 DPX_FP_FN1(m_ceil, ::ceilf, ::ceil)
@@ -175,11 +355,11 @@ DPX_FP_FN1(m_rint, ::rintf, ::rint)
 DPX_FP_FN1(m_asin, ::asinf, ::asin)
 DPX_FP_FN1(m_acos, ::acosf, ::acos)
 DPX_FP_FN1(m_atan, ::atanf, ::atan)
-DPX_FP_FN1(m_sinh, ::sinhf, ::sinh)
-DPX_FP_FN1(m_cosh, ::coshf, ::cosh)
-DPX_FP_FN1(m_asinh, ::asinhf, ::asinh)
-DPX_FP_FN1(m_acosh, ::acoshf, ::acosh)
-DPX_FP_FN1(m_atanh, ::atanhf, ::atanh)
+DPX_FP_FN1(m_sinh, sinh_f32, sinh_f64)
+DPX_FP_FN1(m_cosh, cosh_f32, cosh_f64)
+DPX_FP_FN1(m_asinh, asinh_f32, asinh_f64)
+DPX_FP_FN1(m_acosh, acosh_f32, acosh_f64)
+DPX_FP_FN1(m_atanh, atanh_f32, atanh_f64)
 DPX_FP_FN1(m_erfc, ::erfcf, ::erfc)
 DPX_FP_FN1(m_erfcx, ::erfcxf, ::erfcx)
 DPX_FP_FN1(m_erfinv, ::erfinvf, ::erfinv)

@@ -173,6 +173,44 @@ def test_unary_transcendentals_within_4_ulp(op):
             np.testing.assert_array_equal(np.signbit(got), np.signbit(want(x)))
 
 
+@pytest.mark.parametrize("op", ["log1p", "expm1", "sinh", "tanh", "asinh", "atanh", "acosh", "erf", "cosh", "log2", "log10"])
+def test_own_math_routines_keep_relative_accuracy_at_every_magnitude(op):
+    """The library's own fp32 / fp64 routines (log2, log10, log1p, erf, sinh, cosh, tanh, asinh, acosh, atanh) against
+    the high-precision evaluation on arguments spread over every binade: near zero the result is as small as the
+    argument and the error bound is relative to it.  Signed zeros, infinities and NaN as NumPy has them."""
+    rng = np.random.default_rng(29)
+    for dt in (np.dtype("f4"), np.dtype("f8")):
+        fi = np.finfo(dt)
+        lo, hi = float(fi.tiny) * 4, {"log1p": 1e30, "expm1": 80.0, "sinh": 80.0, "cosh": 80.0, "tanh": 30.0, "asinh": 1e30,
+                                      "atanh": 0.9999, "acosh": 1e30, "erf": 6.0, "log2": 1e30, "log10": 1e30}[op]
+        mag = np.exp(rng.uniform(np.log(lo), np.log(hi), 40000))
+        if op == "acosh":
+            a = 1.0 + mag
+        elif op in ("log2", "log10"):
+            a = np.concatenate([mag, 1.0 / mag[:20000], rng.uniform(0.5, 2.0, 20000)])
+        elif op == "log1p":
+            a = np.concatenate([mag, -mag[mag < 0.999]])
+        else:
+            a = mag * rng.choice([-1.0, 1.0], mag.size)
+        a = a.astype(dt)
+        got = host(getattr(dpt, op)(dev(a)))
+        assert_ulp(got, orc.hi_precision(op, a), 4.0)
+        special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 0.5, -2.0], dtype=dt)
+        with np.errstate(all="ignore"):
+            want = getattr(np, {"asinh": "arcsinh", "acosh": "arccosh", "atanh": "arctanh"}.get(op, op), None)
+            want = want(special) if want is not None else np.array([0.0, -0.0, 1.0, -1.0, np.nan] + [np.nan] * 4, dtype=dt)
+        got = host(getattr(dpt, op)(dev(special)))
+        n = 5 if op == "erf" else special.size
+        np.testing.assert_array_equal(np.isnan(got[:n]), np.isnan(want[:n]))
+        np.testing.assert_array_equal(np.isinf(got[:n]), np.isinf(want[:n]))
+        sel = np.isinf(want[:n]) | (want[:n] == 0)
+        np.testing.assert_array_equal(got[:n][sel], want[:n][sel])
+        np.testing.assert_array_equal(np.signbit(got[:n][sel]), np.signbit(want[:n][sel]))
+        if op == "log2":  # powers of two are exact
+            k = np.arange(-100, 101)
+            np.testing.assert_array_equal(host(dpt.log2(dev((2.0 ** k).astype(dt)))), k.astype(dt))
+
+
 def test_log_float64_every_binade_within_1_ulp():
     # log of a double is evaluated by the library's own routine (argument reduction + polynomial):
     # dense check against an 80-bit evaluation, all binades including subnormals, and around 1
