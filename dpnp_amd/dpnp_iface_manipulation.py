@@ -7,7 +7,6 @@ import math
 import numpy as np
 
 from . import tensor as dpt
-from .dpnp_array import dpnp_array
 from .dpnp_iface import (
     _wrap,
     ascontiguousarray,

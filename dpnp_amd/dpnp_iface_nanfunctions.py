@@ -31,7 +31,6 @@ from .dpnp_iface import (
 )
 from .tensor import _nan_reductions as nr
 from .tensor import _tensor_elementwise_impl as tei
-from .tensor import _tensor_impl as ti
 from .tensor import _tensor_reductions_impl as tri
 from .tensor._manipulation_functions import normalize_axis_tuple
 

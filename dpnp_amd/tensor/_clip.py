@@ -2,7 +2,6 @@
 
 The result always has the dtype of `x`; a bound must cast safely to it.  With both bounds one native
 call computes min(max(x, lo), hi); with one bound the call is maximum / minimum; with none a copy."""
-import numpy as np
 
 from . import _tensor_impl as ti
 from ._copy_utils import _empty_like_orderK, _empty_like_pair_orderK, _empty_like_triple_orderK

@@ -4,7 +4,6 @@ op `X` it exposes `_X(src[, src2], dst, sycl_queue, depends)`, `_X_result_type(d
 and, for binary ops, `_X_inplace(lhs, rhs, sycl_queue, depends)`, all backed by the C ABI.
 """
 from .. import _lib
-from ._device import Event
 from ._dtypes import dtype_from_id, dtype_id
 from ._tensor_impl import _events, _stream
 

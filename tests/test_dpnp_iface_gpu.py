@@ -225,7 +225,6 @@ def test_staged_transfers_round_trip(nbytes):
 
 
 def test_transfer_entry_points_through_the_c_abi():
-    import ctypes
 
     import torch
 

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import dpnp_amd.tensor as dpt
-from tests.helpers import assert_same, dev, host
+from tests.helpers import dev, host
 
 pytestmark = pytest.mark.gpu
 
