@@ -149,6 +149,23 @@ DPX_D double log10_f64(double x)
     return log_scaled_f64(x, 4.34294481903251816668e-01, 1.09831965021676510e-17, 3.01029995663611771306e-01,
                           3.69423907715893078616e-13);
 }
+// n / d for doubles of moderate size through the hardware reciprocal: two Newton steps on it and one
+// correction of the quotient (8 instructions, about 1 ULP; the IEEE division sequence takes 25).
+// Not for results or divisors near the ends of the exponent range.
+DPX_D double div_f64_fast(double n, double d)
+{
+    double r = __builtin_amdgcn_rcp(d);
+    r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
+    r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
+    const double q = n * r;
+    return __builtin_fma(__builtin_fma(-d, q, n), r, q);
+}
+template <class R> DPX_D R div_moderate(R n, R d)
+{
+    if constexpr (std::is_same_v<R, double>) return div_f64_fast(n, d);
+    else return n / d;
+}
+
 // log1p: log(u) for u = 1 + x rounded, plus the rounding error of that sum over u
 // (log(1 + x) = log(u) + log(1 + c/u), c = (1 + x) - u).
 template <class R, class LOG> DPX_D R log1p_via(R x, LOG log_fn)
@@ -190,7 +207,7 @@ template <class R, class LOG1P, class SQRT> DPX_D R asinh_via(R x, LOG1P log1p_f
     const bool big = a > asinh_big<R>, mid = a > R(2);
     const R t = a * a;
     const R s = sqrt_fn(t + R(1));
-    const R q = (mid ? R(1) : t) / (mid ? s + a : R(1) + s);
+    const R q = div_moderate<R>(mid ? R(1) : t, mid ? s + a : R(1) + s);
     R w = (mid ? (a + a) - R(1) : a) + q;
     w = big ? a - R(1) : w;
     R r = log1p_fn(w);
@@ -203,7 +220,7 @@ template <class R, class LOG1P, class SQRT> DPX_D R acosh_via(R x, LOG1P log1p_f
     const bool big = x > asinh_big<R>, mid = x > R(2);
     const R t = x - R(1);
     const R s = sqrt_fn(mid ? x * x - R(1) : t * (R(2) + t));
-    R w = mid ? ((x + x) - R(1)) - R(1) / (x + s) : t + s;
+    R w = mid ? ((x + x) - R(1)) - div_moderate<R>(R(1), x + s) : t + s;
     w = big ? t : w;
     R r = log1p_fn(w);
     r = big ? r + ln2 : r;
@@ -214,7 +231,7 @@ template <class R, class LOG1P> DPX_D R atanh_via(R x, LOG1P log1p_fn)
     const R a = x < R(0) ? -x : x;
     const R t = a + a;
     const bool small = a < R(0.5);
-    const R q = (small ? t * a : t) / (R(1) - a);
+    const R q = (small ? t * a : t) / (R(1) - a); // the divisor reaches 0 and below: IEEE division
     const R w = small ? t + q : q;
     const R r = R(0.5) * log1p_fn(w);
     return (x != x) ? x : __builtin_copysign(r, x);
@@ -247,7 +264,7 @@ template <class R, class EXPM1> DPX_D R tanh_via(R x, EXPM1 expm1_fn)
     const R a = x < R(0) ? -x : x;
     const R big = std::is_same_v<R, double> ? R(22) : R(10);
     const R t = expm1_fn(a + a);
-    R r = t / (t + R(2));
+    R r = div_moderate<R>(t, t + R(2));
     r = (a > big) ? R(1) : r;
     r = (a == R(0)) ? a : r;
     return (x != x) ? x : __builtin_copysign(r, x);
@@ -257,7 +274,7 @@ template <class R, class EXP, class EXPM1> DPX_D R sinh_via(R x, EXP exp_fn, EXP
     const R a = x < R(0) ? -x : x;
     const R over = std::is_same_v<R, double> ? R(709) : R(88); // exp(a) and expm1(a) are finite up to here
     const R t = expm1_fn(a);
-    const R q = t / (t + R(1));
+    const R q = div_moderate<R>(t, t + R(1));
     R r = R(0.5) * ((a < R(1)) ? R(2) * t - t * q : t + q);
     if (a > over) { // rare: the band where sinh is finite and exp is not, and beyond
         const R w = exp_fn(R(0.5) * a);
