@@ -181,6 +181,14 @@ def test_elementwise_plans():
     assert L.PATH_NAMES[p.path] == "ew_rows"  # 512-byte rows
     p = plan_binary("subtract", view([100000, 17], [34, 2]), view([100000, 17], [0, 1], ptr=P1), view([100000, 17], ptr=P2))
     assert L.PATH_NAMES[p.path] == "ew_rows"  # strided matrix
+    # rows of 2 MiB and more plus a row: flat as well; plus a column: the row kernel (one value per row there)
+    n = 600001
+    p = plan_binary("add", view([5, n]), view([5, n], [0, 1], ptr=P1), view([5, n], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_contig" and p.nd == 2
+    p = plan_binary("add", view([5, n]), view([5, n], [1, 0], ptr=P1), view([5, n], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"
+    p = plan_binary("add", view([5, 100000]), view([5, 100000], [0, 1], ptr=P1), view([5, 100000], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"  # 400 KB rows
     # empty
     p = plan_binary("add", view([0, 3]), view([0, 3]), view([0, 3]))
     assert L.PATH_NAMES[p.path] == "noop"

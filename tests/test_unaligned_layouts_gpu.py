@@ -143,3 +143,20 @@ def test_short_rows_with_row_and_column_operands(dt):
                 assert_same(host(o), x * row)
             dpt.add(dx, drow, out=dx)  # in place
             assert_same(host(dx), x + row)
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8", "i2", "c8"])
+def test_matrix_with_rows_of_megabytes_plus_a_row(dt):
+    """Rows of 2 MiB and more combined with a broadcast row take the flat contiguous kernel, the row indexed by
+    position modulo the (odd) row length; the same operands with a column stay with the row kernel."""
+    rng = np.random.default_rng(41)
+    ncols = (2 << 20) // np.dtype(dt).itemsize + 3
+    a = rng.integers(-50, 50, (3, ncols)).astype(dt)
+    row = rng.integers(-50, 50, (1, ncols)).astype(dt)
+    col = rng.integers(-50, 50, (3, 1)).astype(dt)
+    da, drow, dcol = dev(a), dev(row), dev(col)
+    np.testing.assert_array_equal(host(dpt.add(da, drow)), a + row)
+    np.testing.assert_array_equal(host(dpt.subtract(drow, da)), row - a)
+    np.testing.assert_array_equal(host(dpt.multiply(da, dcol)), a * col)
+    np.testing.assert_array_equal(host(dpt.where(dpt.greater(dpt.real(da) if dt == "c8" else da, 0), da, drow)),
+                                  np.where(a.real > 0, a, row))
