@@ -25,7 +25,14 @@ inline int run_ew(const Fn &fn, const dpx_array_view *const *views, hipStream_t 
     return e == hipSuccess ? DPX_OK : fail_hip(e, "elementwise kernel launch");
 }
 
+// unary functions of doubles that cost enough vector instructions to pay for two packs per thread
+template <class Op> struct op_two_packs : std::false_type {};
+#define DPX_TWO_PACKS(OP) \
+    template <> struct op_two_packs<OP> : std::true_type {};
+DPX_TWO_PACKS(Expm1Op) DPX_TWO_PACKS(Log2Op) DPX_TWO_PACKS(SinhOp) DPX_TWO_PACKS(TanhOp)
+#undef DPX_TWO_PACKS
 template <class Op, class T> struct UnaryFn {
+    static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
     DPX_D auto operator()(V<T> x) const { return Op::template apply<T>(x); }
 };
 template <class Op, class T> struct BinaryFn {
