@@ -1,7 +1,8 @@
-"""Views and shape queries of the dpnp surface that callers put around the elementwise and reduction
-calls (dpnp/dpnp_iface_manipulation.py): nothing here moves data except `ravel` of an array that
-cannot be flattened in place.  Joining, splitting, repeating and the other functions of that file
-that need kernels of their own are outside this library."""
+"""Views, shape queries and joins of the dpnp surface that callers put around the elementwise and reduction
+calls (dpnp/dpnp_iface_manipulation.py).  The views move no data; `ravel` of an array that cannot be flattened
+in place, `concatenate` / `stack` / `hstack` / `vstack` and `diff` / `trapezoid` (dpnp/dpnp_iface_mathematical.py)
+run on the copy / cast and elementwise kernels.  Splitting, repeating and the other functions of that file that
+need kernels of their own are outside this library."""
 import math
 
 import numpy as np
@@ -17,9 +18,9 @@ from .dpnp_iface import (
 )
 from .tensor._manipulation_functions import normalize_axis_index, normalize_axis_tuple
 
-__all__ = ["atleast_1d", "atleast_2d", "atleast_3d", "broadcast_arrays", "broadcast_shapes", "expand_dims", "flip",
-           "fliplr", "flipud", "matrix_transpose", "moveaxis", "ndim", "permute_dims", "ravel", "rollaxis", "shape",
-           "size", "squeeze", "swapaxes"]
+__all__ = ["atleast_1d", "atleast_2d", "atleast_3d", "broadcast_arrays", "broadcast_shapes", "concat", "concatenate",
+           "diff", "expand_dims", "flip", "fliplr", "flipud", "hstack", "matrix_transpose", "moveaxis", "ndim",
+           "permute_dims", "ravel", "rollaxis", "shape", "size", "squeeze", "stack", "swapaxes", "trapezoid", "vstack"]
 
 
 def _atleast(arys, fn):
@@ -150,3 +151,86 @@ def size(a, axis=None):
             return a.size
         return math.prod(a.shape[ax] for ax in normalize_axis_tuple(axis, a.ndim))
     return np.size(a, axis)
+
+
+# -- joining (copies through the cast / copy kernel into slices of the result) ---------------------------
+def _check_stack_arrays(arrays):
+    if not hasattr(arrays, "__getitem__"):
+        raise TypeError('arrays to stack must be passed as a "sequence" type such as list or tuple.')
+
+
+def _joined(res, out, dtype, casting):
+    from .dpnp_iface import copyto
+
+    if dtype is not None:
+        return res.astype(dtype, casting=casting, copy=False)
+    if out is not None:
+        copyto(out, res, casting=casting)
+        return out
+    return res
+
+
+def concatenate(arrays, /, *, axis=0, out=None, dtype=None, casting="same_kind"):
+    """Join arrays along an existing axis (dpnp/dpnp_iface_manipulation.py, `concatenate`)."""
+    if dtype is not None and out is not None:
+        raise TypeError("concatenate() only takes `out` or `dtype` as an argument, but both were provided.")
+    return _joined(_wrap(dpt.concat([get_usm_ndarray(x) for x in arrays], axis=axis)), out, dtype, casting)
+
+
+concat = concatenate
+
+
+def stack(arrays, /, *, axis=0, out=None, dtype=None, casting="same_kind"):
+    """Join arrays of one shape along a new axis."""
+    _check_stack_arrays(arrays)
+    if dtype is not None and out is not None:
+        raise TypeError("stack() only takes `out` or `dtype` as an argument, but both were provided.")
+    return _joined(_wrap(dpt.stack([get_usm_ndarray(x) for x in arrays], axis=axis)), out, dtype, casting)
+
+
+def hstack(tup, *, dtype=None, casting="same_kind"):
+    _check_stack_arrays(tup)
+    arrs = atleast_1d(*tup)
+    if not isinstance(arrs, tuple):
+        arrs = (arrs,)
+    if arrs and arrs[0].ndim == 1:
+        return concatenate(arrs, axis=0, dtype=dtype, casting=casting)
+    return concatenate(arrs, axis=1, dtype=dtype, casting=casting)
+
+
+def vstack(tup, *, dtype=None, casting="same_kind"):
+    _check_stack_arrays(tup)
+    arrs = atleast_2d(*tup)
+    if not isinstance(arrs, tuple):
+        arrs = (arrs,)
+    return concatenate(arrs, axis=0, dtype=dtype, casting=casting)
+
+
+# -- differences and the trapezoid rule (dpnp/dpnp_iface_mathematical.py, `diff`, `trapezoid`) ----------
+def diff(a, n=1, axis=-1, prepend=None, append=None):
+    from .dpnp_iface import get_usm_ndarray_or_scalar
+
+    pre = None if prepend is None else get_usm_ndarray_or_scalar(prepend)
+    app = None if append is None else get_usm_ndarray_or_scalar(append)
+    return _wrap(dpt.diff(get_usm_ndarray(a), axis=axis, n=n, prepend=pre, append=app))
+
+
+def trapezoid(y, x=None, dx=1.0, axis=-1):
+    """Integral along `axis` by the trapezoid rule: sum(d * (y[1:] + y[:-1]) / 2)."""
+    check_supported_arrays_type(y)
+    nd = y.ndim
+    if x is None:
+        d = dx
+    else:
+        check_supported_arrays_type(x)
+        if x.ndim == 1:
+            d = diff(x)
+            shape = [1] * nd
+            shape[axis] = d.shape[0]
+            d = d.reshape(shape)
+        else:
+            d = diff(x, axis=axis)
+    slice1, slice2 = [slice(None)] * nd, [slice(None)] * nd
+    slice1[axis] = slice(1, None)
+    slice2[axis] = slice(None, -1)
+    return (d * (y[tuple(slice1)] + y[tuple(slice2)]) / 2.0).sum(axis)

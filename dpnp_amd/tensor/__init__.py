@@ -38,6 +38,9 @@ from ._dtypes import (
 from ._elementwise_funcs import *  # noqa: F401,F403
 from ._elementwise_funcs import abs, pow, round  # noqa: A004
 from ._manipulation_functions import (
+    concat,
+    diff,
+    stack,
     broadcast_arrays,
     broadcast_to,
     expand_dims,

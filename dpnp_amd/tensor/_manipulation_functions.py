@@ -236,3 +236,124 @@ def broadcast_arrays(*args):
             raise TypeError(f"Expected usm_ndarray type; got {type(a)}.")
     shape = _broadcast_shape_impl([a.shape for a in args])
     return [a if a.shape == shape else broadcast_to(a, shape) for a in args]
+
+
+# -- joining: copies into slices of the result through the copy / cast kernel ---------------------------
+def _arrays_validation(arrays, check_ndim=True):
+    """Result dtype of a join; the checks of dpnp/tensor/_manipulation_functions.py:47-88."""
+    if not isinstance(arrays, (list, tuple)):
+        raise TypeError(f"Expected tuple or list type, got {type(arrays)}.")
+    if len(arrays) == 0:
+        raise TypeError("Missing 1 required positional argument: 'arrays'.")
+    for x in arrays:
+        if not isinstance(x, usm_ndarray):
+            raise TypeError(f"Expected usm_ndarray type, got {type(x)}.")
+    res_dtype = arrays[0].dtype
+    for x in arrays[1:]:
+        res_dtype = np.promote_types(res_dtype, x.dtype)
+    if check_ndim:
+        for x in arrays[1:]:
+            if x.ndim != arrays[0].ndim:
+                raise ValueError(
+                    "All the input arrays must have same number of dimensions, but the array at index 0 has "
+                    f"{arrays[0].ndim} dimension(s) and the array at index {arrays.index(x)} has {x.ndim} dimension(s).")
+    return res_dtype
+
+
+def concat(arrays, /, *, axis=0):
+    """Joins arrays along an existing axis (all of them flattened for axis=None); the result dtype follows
+    the promotion rules (dpnp/tensor/_manipulation_functions.py:314-392)."""
+    from ._copy_utils import _copy_into
+    from ._ctors import empty
+
+    if axis is None:
+        res_dtype = _arrays_validation(arrays, check_ndim=False)
+        res = empty(sum(x.size for x in arrays), dtype=res_dtype)
+        start = 0
+        for x in arrays:
+            if x.size:
+                _copy_into(reshape(x, (-1,)), res[start:start + x.size])
+            start += x.size
+        return res
+    res_dtype = _arrays_validation(arrays)
+    x0 = arrays[0]
+    if x0.ndim == 0:
+        raise ValueError("Zero-dimensional arrays cannot be concatenated")
+    axis = normalize_axis_index(axis, x0.ndim)
+    for i, x in enumerate(arrays[1:], 1):
+        for j, ext in enumerate(x0.shape):
+            if ext != x.shape[j] and j != axis:
+                raise ValueError(
+                    "All the input array dimensions for the concatenation axis must match exactly, but along "
+                    f"dimension {j}, the array at index 0 has size {ext} and the array at index {i} has size "
+                    f"{x.shape[j]}.")
+    shape = list(x0.shape)
+    shape[axis] = sum(x.shape[axis] for x in arrays)
+    res = empty(tuple(shape), dtype=res_dtype)
+    start = 0
+    for x in arrays:
+        stop = start + x.shape[axis]
+        if x.size:
+            _copy_into(x, res[(slice(None),) * axis + (slice(start, stop),)])
+        start = stop
+    return res
+
+
+def stack(arrays, /, *, axis=0):
+    """Joins arrays of one shape along a new axis (dpnp/tensor/_manipulation_functions.py, `stack`)."""
+    from ._copy_utils import _copy_into
+    from ._ctors import empty
+
+    res_dtype = _arrays_validation(arrays)
+    x0 = arrays[0]
+    axis = normalize_axis_index(axis, x0.ndim + 1)
+    for x in arrays[1:]:
+        if x.shape != x0.shape:
+            raise ValueError("All input arrays must have the same shape")
+    res = empty(x0.shape[:axis] + (len(arrays),) + x0.shape[axis:], dtype=res_dtype)
+    for i, x in enumerate(arrays):
+        if x.size:
+            _copy_into(x, res[(slice(None),) * axis + (i,)])
+    return res
+
+
+def diff(x, /, *, axis=-1, n=1, prepend=None, append=None):
+    """n-th forward difference along `axis`; `prepend` / `append` (arrays or scalars) are joined to `x`
+    first (dpnp/tensor/_utility_functions.py, `diff`).  Booleans difference with not_equal, as in NumPy."""
+    from ._ctors import asarray
+    from ._elementwise_funcs import not_equal, subtract
+
+    if not isinstance(x, usm_ndarray):
+        raise TypeError(f"Expecting dpnp.tensor.usm_ndarray type, got {type(x)}")
+    axis = normalize_axis_index(axis, x.ndim)
+    n = int(n)
+    if n < 0:
+        raise ValueError(f"`n` must be positive, got {n}")
+
+    def side(v):
+        if isinstance(v, usm_ndarray):
+            return v
+        from ._type_utils import result_type  # a Python scalar takes the array's kind where it can
+
+        shape = list(x.shape)
+        shape[axis] = 1
+        return broadcast_to(asarray(v, dtype=result_type(x, v)), tuple(shape))
+
+    parts = []
+    if prepend is not None:
+        parts.append(side(prepend))
+    parts.append(x)
+    if append is not None:
+        parts.append(side(append))
+    if len(parts) > 1:
+        for p in parts:
+            if p.ndim != x.ndim:
+                raise ValueError("`prepend` and `append` must have the same number of dimensions as `x`")
+        x = concat(parts, axis=axis)
+    op = not_equal if x.dtype == np.dtype("?") else subtract
+    for _ in range(n):
+        if x.shape[axis] == 0:
+            break
+        lead = (slice(None),) * axis
+        x = op(x[lead + (slice(1, None),)], x[lead + (slice(None, -1),)])
+    return x
