@@ -262,8 +262,10 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const int64_t base_blocks = L.col_blocks * outer;
     const int64_t want = std::max<int64_t>(target * 256 / block, 1); // same number of threads in flight
     int64_t splits = 1;
-    if (base_blocks < want && base_blocks <= RED_MAX_TICKETS && n >= 2 * TY * 8)
-        splits = std::min(cdiv(want, base_blocks), cdiv(n, TY * 8));
+    // the largest split count that still gives every block a CU of its own at once: a grid a little
+    // above a multiple of the CU count runs up to a third slower than one a little below it
+    if (2 * base_blocks <= want && base_blocks <= RED_MAX_TICKETS && n >= 2 * TY * 8)
+        splits = std::min(want / base_blocks, cdiv(n, TY * 8));
     if (arg) splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
     int64_t chunk = cdiv(n, splits);
     splits = cdiv(n, chunk);
