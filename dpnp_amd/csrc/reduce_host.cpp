@@ -180,8 +180,10 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         int64_t splits = 1;
         const int64_t per_pass = G * e * 8; // elements one group covers with 8 accesses per lane
         // splitting needs a whole block per output (G > 64) and one ticket counter per output
-        if (G > 64 && oblocks < target && oblocks <= RED_MAX_TICKETS && n >= 2 * per_pass)
-            splits = std::min(cdiv(target, oblocks), cdiv(n, per_pass));
+        // (the largest split count whose grid stays within the target: a grid a little above it
+        // runs a second, nearly empty round of blocks and loses 10-15 points of bandwidth)
+        if (G > 64 && 2 * oblocks <= target && oblocks <= RED_MAX_TICKETS && n >= 2 * per_pass)
+            splits = std::min(target / oblocks, cdiv(n, per_pass));
         if (arg && G > 64 && oblocks <= RED_MAX_TICKETS)
             splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
         int64_t chunk = cdiv(n, splits);
