@@ -819,12 +819,14 @@ struct PowOp { // pow.hpp: ints by repeated squaring (negative exponent -> 0), f
         if constexpr (is_cplx_v<T>) {
             using R = real_of_t<T>;
             if (b.re == R(0) && b.im == R(0)) return T{R(1), R(0)};
-            if (a.re == R(0) && a.im == R(0)) return T{R(0), R(0)};
+            // a zero base is zero only under a positive real exponent; every other exponent goes
+            // through exp(b log 0) like any base (0 ** -1 = inf + nan j, 0 ** 1j = nan + nan j)
+            if (a.re == R(0) && a.im == R(0) && b.re > R(0) && b.im == R(0)) return T{R(0), R(0)};
             return c_exp(b * c_log(a));
         }
         else if constexpr (is_int_v<T>) {
             if constexpr (std::is_signed_v<T>) {
-                if (b < 0) return (a == 1) ? T(1) : ((a == -1) ? ((b & 1) ? T(-1) : T(1)) : T(0));
+                if (b < 0) return T(0); // pow.hpp:72-78: invalid, 0 for every base
             }
             using U = std::make_unsigned_t<T>;
             U r = 1, base = (U)a;
@@ -859,15 +861,17 @@ template <bool LEFT> struct ShiftOp { // bitwise_left_shift.hpp / bitwise_right_
     template <class T> using out = T;
     template <class T> DPX_D static T apply(T a, T b)
     {
+        // bitwise_left_shift.hpp:88-103, bitwise_right_shift.hpp:88-105: a negative count gives 0
+        // in both directions; a count of the width or more gives 0, except that a right shift of
+        // a negative value gives -1
         constexpr int bits = 8 * sizeof(T);
-        bool big;
-        if constexpr (std::is_signed_v<T>) big = (b < 0) || (b >= bits);
-        else big = b >= (T)bits;
-        if constexpr (LEFT) return big ? T(0) : (T)((std::make_unsigned_t<T>)a << b);
-        else {
-            if constexpr (std::is_signed_v<T>) return big ? (a < 0 ? T(-1) : T(0)) : (T)(a >> b);
-            else return big ? T(0) : (T)(a >> b);
+        if constexpr (std::is_signed_v<T>) {
+            if (b < 0) return T(0);
+            if (b >= bits) return (!LEFT && a < 0) ? T(-1) : T(0);
         }
+        else if (b >= (T)bits) return T(0);
+        if constexpr (LEFT) return (T)((std::make_unsigned_t<T>)a << b);
+        else return (T)(a >> b);
     }
 };
 

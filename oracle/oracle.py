@@ -79,22 +79,83 @@ def _floor_divide(a, b):
 
 
 def _remainder(a, b):
+    # remainder.hpp:66-97.  ints: x % 0 == 0; C remainder (sign of the dividend), then `+= y` when
+    # it is non-zero and the operands' signs differ.  floats: fmod, then `+= y` when the
+    # remainder is non-zero and its sign differs from y's; a zero remainder takes y's sign.
     if a.dtype.kind in "iu":
+        shape = np.broadcast(a, b).shape
+        a, b = np.broadcast_to(a, shape), np.broadcast_to(b, shape)
+        zero = b == 0
         with np.errstate(all="ignore"):
-            r = np.remainder(a, np.where(b == 0, 1, b))
-        return np.where(b == 0, 0, r).astype(a.dtype)
+            r = np.fmod(a, np.where(zero, 1, b)).astype(a.dtype)      # C `%`, pinned by brute force
+            if a.dtype.kind == "i":
+                fix = (r != 0) & ((a < 0) != (b < 0))
+                r = np.where(fix, r + b, r).astype(a.dtype)
+        return np.where(zero, 0, r).astype(a.dtype)
     with np.errstate(all="ignore"):
-        return np.remainder(a, b)
+        r = np.fmod(a, b)
+        fix = (r != 0) & ((b < 0) != (r < 0))
+        r = np.where(fix, r + b, r)
+        r = np.where(r == 0, np.copysign(0, b), r)  # NaN != 0: NaNs pass through
+        return r.astype(a.dtype)
 
 
 def _shift(a, b, left):
+    # bitwise_left_shift.hpp:88-103, bitwise_right_shift.hpp:88-105: a negative count gives 0 in
+    # both directions; a count >= the width gives 0, except -1 for a right shift of a negative value
     bits = a.dtype.itemsize * 8
-    big = (b < 0) | (b >= bits) if a.dtype.kind == "i" else (b >= bits)
-    sb = np.where(big, 0, b).astype(a.dtype)
+    shape = np.broadcast(a, b).shape
+    a, b = np.broadcast_to(a, shape), np.broadcast_to(b, shape)
+    signed = a.dtype.kind == "i"
+    neg = (b < 0) if signed else np.zeros(shape, dtype=bool)
+    wide = (b >= bits) & ~neg
+    sb = np.where(neg | wide, 0, b).astype(a.dtype)
     if left:
-        return np.where(big, 0, np.left_shift(a, sb)).astype(a.dtype)
-    fill = np.where(a < 0, -1, 0) if a.dtype.kind == "i" else 0
-    return np.where(big, fill, np.right_shift(a, sb)).astype(a.dtype)
+        val = np.left_shift(a, sb)
+        over = np.zeros(shape, dtype=a.dtype)
+    else:
+        val = np.right_shift(a, sb)
+        over = np.where(a < 0, -1, 0).astype(a.dtype) if signed else np.zeros(shape, dtype=a.dtype)
+    return np.where(neg, 0, np.where(wide, over, val)).astype(a.dtype)
+
+
+def _int_pow(a, b):
+    # pow.hpp:72-92: a negative exponent gives 0 for every base; otherwise repeated squaring in
+    # the operand type (wraps), with 1 for base 1 or exponent 0
+    shape = np.broadcast(a, b).shape
+    dt = a.dtype
+    base = np.broadcast_to(a, shape).copy()
+    e = np.broadcast_to(b, shape).copy()
+    neg = (e < 0) if dt.kind == "i" else np.zeros(shape, dtype=bool)
+    e = np.where(neg, 0, e).astype(dt)
+    res = np.ones(shape, dtype=dt)
+    with np.errstate(over="ignore"):
+        while (e > 0).any():
+            odd = (e & 1).astype(bool)
+            res = np.where(odd, res * base, res).astype(dt)
+            e = (e >> 1).astype(dt)
+            base = (base * base).astype(dt)
+    return np.where(neg, 0, res).astype(dt)
+
+
+def _sign(a):
+    # sign.hpp:73-110: unsigned 0 < x; signed and floats (0 < x) - (x < 0), NaN stays NaN;
+    # complex z / |z| with sign(0) = 0
+    k = a.dtype.kind
+    if k == "b":
+        return a.copy()
+    if k == "u":
+        return (a > 0).astype(a.dtype)
+    if k == "c":
+        mag = np.where(a == 0, 1, np.abs(a))
+        with np.errstate(all="ignore"):
+            out = np.empty(a.shape, dtype=a.dtype)   # complex / real: each part divided once
+            out.real, out.imag = a.real / mag, a.imag / mag
+        return np.where(a == 0, 0, out).astype(a.dtype)
+    out = ((a > 0).astype(np.int8) - (a < 0).astype(np.int8)).astype(a.dtype)
+    if k == "f":
+        out[np.isnan(a)] = np.nan
+    return out
 
 
 def _maximum(a, b):
@@ -182,7 +243,7 @@ def binary(op, a, b):
         if op == "remainder":
             return _remainder(a, b)
         if op == "pow":
-            return np.power(a, b)
+            return _int_pow(a, b) if k in "iu" else np.power(a, b)
         if op == "atan2":
             return np.arctan2(a, b)
         if op == "hypot":
@@ -265,7 +326,7 @@ def unary(op, a):
         if op in ("floor", "ceil", "trunc"):
             return getattr(np, op)(a).astype(a.dtype) if k == "f" else a.copy()
         if op == "sign":
-            return np.sign(a).astype(a.dtype)
+            return _sign(a)
         if op == "isnan":
             return np.isnan(a)
         if op == "isinf":
@@ -676,9 +737,19 @@ def collapse(shape, strides_list, keep_order=False):
 # ---------------------------------------------------------------------------------------------
 # type promotion: dpnp/tensor/_type_utils.py:197-251 (a device with fp16 and fp64)
 # ---------------------------------------------------------------------------------------------
-def promote_binary(supported, dt1, dt2):
+def accept_divide(dt1, dt2, c1, c2, r):
+    """_acceptance_fn_divide, _type_utils.py:89-107: when BOTH operands change kind, only the
+    default dtype of the result's kind is taken (int8 / uint8 is float64, not float16)."""
+    if c1.kind != dt1.kind and c2.kind != dt2.kind:
+        return r == np.dtype({"f": "f8", "c": "c16"}.get(r.kind, r))
+    return True
+
+
+def promote_binary(supported, dt1, dt2, accept=None):
     """(cast1 or None, cast2 or None, result) where supported(d1, d2) -> result dtype or None:
-    first pair, in the fixed dtype order, that both inputs cast to safely."""
+    first pair, in the fixed dtype order, that both inputs cast to safely and that the op's
+    acceptance hook `accept(dt1, dt2, cast1, cast2, result)` takes (_find_buf_dtype2,
+    _type_utils.py:219-251)."""
     dt1, dt2 = np.dtype(dt1), np.dtype(dt2)
     r = supported(dt1, dt2)
     if r is not None:
@@ -687,6 +758,6 @@ def promote_binary(supported, dt1, dt2):
         for c2 in ALL_DTYPES:
             if np.can_cast(dt1, c1) and np.can_cast(dt2, c2):
                 r = supported(c1, c2)
-                if r is not None:
+                if r is not None and (accept is None or accept(dt1, dt2, c1, c2, r)):
                     return (None if c1 == dt1 else c1), (None if c2 == dt2 else c2), r
     return None, None, None

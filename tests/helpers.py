@@ -36,6 +36,9 @@ def assert_same(got, want):
     assert got.dtype == want.dtype, (got.dtype, want.dtype)
     assert got.shape == want.shape, (got.shape, want.shape)
     np.testing.assert_array_equal(got, want)
+    if got.dtype.kind == "f":  # -0.0 and +0.0 compare equal: check the sign bit as well
+        ok = ~np.isnan(want)
+        np.testing.assert_array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
 
 
 def assert_ulp(got, exact_hi, max_ulp=4.0):

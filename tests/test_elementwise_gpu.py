@@ -1,5 +1,7 @@
 """Elementwise kernels against the oracle, through the Python layer and the C ABI.
 Bar: bit-exact for integer/bool results and IEEE basic ops; <= 4 ULP for transcendentals."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -61,7 +63,7 @@ def test_add_dtype_matrix(d1):
 
 @pytest.mark.parametrize("op", EXACT_BINARY)
 def test_binary_exact_all_dtypes_and_sizes(op):
-    rng = np.random.default_rng(hash(op) % 2**32)
+    rng = np.random.default_rng(zlib.crc32(op.encode()))  # fixed per op: a failure can be replayed
     for dt in ALL:
         if not supported_binary(op, dt):
             continue
@@ -72,8 +74,12 @@ def test_binary_exact_all_dtypes_and_sizes(op):
                 b[rng.integers(0, n)] = np.inf
                 if n > 3:
                     b[rng.integers(0, n)] = 0.0
-            if "shift" in op:
-                b = np.abs(b).astype(dt) if dt.kind == "i" else b
+            if "shift" in op and n > 8:
+                # counts on both sides of every boundary: negative, 0, width - 1, width, beyond
+                bits = 8 * dt.itemsize
+                edge = [0, 1, bits - 1, bits, bits + 1, 127] + ([-1, -bits, -128] if dt.kind == "i" else [])
+                b[: len(edge)] = np.array(edge).astype(dt)
+                a[: len(edge)] = np.array([-8, 8] * 5)[: len(edge)].astype(dt) if dt.kind == "i" else 200
             got = host(getattr(dpt, op)(dev(a), dev(b)))
             want = orc.binary(op, a, b)
             if op in ("divide", "multiply") and dt.kind == "c":
@@ -95,11 +101,14 @@ def test_binary_ulp(op):
         f = {"pow": np.power, "atan2": np.arctan2, "hypot": np.hypot}[op]
         assert_ulp(got, f(a.astype(wide), b.astype(wide)), 4.0)
     for dt in INTS:
+        # negative exponents give 0 for every base, 1 and -1 included (pow.hpp:72-78)
         a = random_array(rng, 500, dt, -5, 5)
-        b = random_array(rng, 500, dt, 0, 7)
+        b = random_array(rng, 500, dt, -4, 7)
         if op == "pow":
+            assert_same(host(dpt.pow(dev(a), dev(b))), orc.binary("pow", a, b))
+            nonneg = b >= 0
             with np.errstate(over="ignore"):
-                assert_same(host(dpt.pow(dev(a), dev(b))), np.power(a, b))
+                assert_same(host(dpt.pow(dev(a[nonneg]), dev(b[nonneg]))), np.power(a[nonneg], b[nonneg]))
 
 
 @pytest.mark.parametrize("op", EXACT_UNARY)
@@ -475,7 +484,11 @@ def test_angle_logaddexp_nextafter():
         x, y = random_array(rng, 3000, dt, -5, 5), random_array(rng, 3000, dt, -5, 5)
         x[:6] = [0.0, 0.0, -0.0, 1.0, np.inf, np.nan]
         y[:6] = [1.0, -1.0, 0.0, 1.0, 0.0, 0.0]
-        assert_same(host(dpt.nextafter(dev(x), dev(y))), np.nextafter(x, y))
+        want = np.nextafter(x, y)
+        # C's rule for equal operands (the second one comes back, so -0.0 -> +0.0 gives +0.0), which NumPy
+        # follows for float32/64 but not for float16, where it hands back the first operand
+        want = np.where(x == y, y, want).astype(dt)
+        assert_same(host(dpt.nextafter(dev(x), dev(y))), want)
 
 
 # ---- transposed operands (LDS tile kernel) ----------------------------------------------------

@@ -1,5 +1,25 @@
 """Pins the CPU oracle: reference known answers, closed forms, brute force, mpmath.
-Runs without a GPU."""
+Runs without a GPU.
+
+Oracle function -> what pins it here (none of the pins calls NumPy for the rule under test):
+  binary add/subtract/multiply/bitwise_*  test_integer_ops_wrap_like_python_ints, test_add_ones_is_two
+  binary floor_divide, remainder (ints)   test_integer_functors_brute_force_int8 (scalar C-semantics
+                                          transcription of floor_divide.hpp:69-86, remainder.hpp:66-83)
+  binary floor_divide, remainder (floats) test_float_floor_divide_and_remainder_rules (Fractions; the
+                                          special cases of test_floor_divide.py:109-147, test_remainder.py:138-152)
+  binary bitwise_left/right_shift         test_integer_functors_brute_force_int8 (+ uint8),
+                                          test_shift_range_known_answer (test_bitwise_*_shift.py:107-117)
+  binary pow (ints)                       test_integer_functors_brute_force_int8 (pow.hpp:72-92)
+  binary fmod (ints)                      test_integer_functors_brute_force_int8 (fmod.hpp:52-62)
+  unary sign                              test_sign_rules (sign.hpp:73-110, test_sign.py:61-101)
+  unary round                             test_round_conj_parts_proj_rules (test_round.py:107-122)
+  comparisons (incl. int64/uint64)        test_mixed_int64_uint64_comparisons_are_exact
+  maximum / minimum                       test_maximum_minimum_nan_rule
+  promote_binary                          test_promotion_matches_numpy_result_type,
+                                          test_promotion_with_acceptance_hooks
+  cast, where, reductions, collapse       the tests of those names below
+"""
+from fractions import Fraction
 import itertools
 import json
 import math
@@ -58,6 +78,177 @@ def test_floor_divide_and_remainder_integer_rules():
             assert qq == 0 and rr == 0
         else:
             assert qq == int(x) // int(y) and rr == int(x) % int(y)
+
+
+# Scalar transcriptions of the reference's integer functors in C semantics (division truncates
+# towards zero, `%` takes the dividend's sign, results wrap to the operand width).  They are
+# written from the functor text, branch by branch, and share no code with the oracle.
+def _wrap(v, bits, signed):
+    v &= (1 << bits) - 1
+    return v - (1 << bits) if signed and v >= (1 << (bits - 1)) else v
+
+
+def _c_div(a, b):
+    q = abs(a) // abs(b)
+    return q if (a < 0) == (b < 0) else -q
+
+
+def _c_mod(a, b):
+    return a - _c_div(a, b) * b
+
+
+def _functor_right_shift(a, b, bits, signed):  # bitwise_right_shift.hpp:88-105
+    if not signed:
+        return (a >> b) if b < bits else 0
+    return 0 if b < 0 else ((a >> b) if b < bits else (-1 if a < 0 else 0))
+
+
+def _functor_left_shift(a, b, bits, signed):   # bitwise_left_shift.hpp:88-103
+    if not signed:
+        return _wrap(a << b, bits, False) if b < bits else 0
+    return 0 if b < 0 else (_wrap(a << b, bits, True) if b < bits else 0)
+
+
+def _functor_pow(a, b, bits, signed):          # pow.hpp:72-92
+    if signed and b < 0:
+        return 0
+    res = 1
+    if a == 1 or b == 0:
+        return res
+    while b > 0:
+        if b & 1:
+            res = _wrap(res * a, bits, signed)
+        b >>= 1
+        a = _wrap(a * a, bits, signed)
+    return res
+
+
+def _functor_floor_divide(a, b, bits, signed):  # floor_divide.hpp:69-86
+    if b == 0:
+        return 0
+    if not signed:
+        return a // b
+    div, mod = _c_div(a, b), _c_mod(a, b)
+    return _wrap(div - int(mod != 0 and ((mod < 0) != (b < 0))), bits, True)
+
+
+def _functor_remainder(a, b, bits, signed):     # remainder.hpp:66-83
+    if b == 0:
+        return 0
+    out = _c_mod(a, b)
+    if signed and out != 0 and ((a < 0) != (b < 0)):
+        out += b
+    return _wrap(out, bits, signed)
+
+
+def _functor_fmod(a, b, bits, signed):          # dpnp/backend/kernels/elementwise_functions/fmod.hpp:52-62
+    return 0 if b == 0 else _c_mod(a, b)
+
+
+@pytest.mark.parametrize("dt", ["i1", "u1"])
+def test_integer_functors_brute_force_int8(dt):
+    info = np.iinfo(dt)
+    signed = info.min < 0
+    vals = np.arange(info.min, info.max + 1).astype(dt)
+    a, b = np.meshgrid(vals, vals, indexing="ij")
+    for op, fn in (("bitwise_right_shift", _functor_right_shift), ("bitwise_left_shift", _functor_left_shift),
+                   ("pow", _functor_pow), ("floor_divide", _functor_floor_divide),
+                   ("remainder", _functor_remainder), ("fmod", _functor_fmod)):
+        got = orc.binary(op, a, b)
+        assert got.dtype == np.dtype(dt)
+        want = np.array([[fn(int(x), int(y), 8, signed) for y in vals] for x in vals], dtype=dt)
+        bad = np.argwhere(got != want)
+        assert bad.size == 0, (op, dt, [(int(vals[i]), int(vals[j]), int(got[i, j]), int(want[i, j])) for i, j in bad[:5]])
+
+
+def test_integer_functors_wider_types_spot_checks():
+    # the same rules at 16, 32 and 64 bits on the values where width matters
+    for dt in ("i2", "u2", "i4", "u4", "i8", "u8"):
+        info = np.iinfo(dt)
+        bits, signed = 8 * np.dtype(dt).itemsize, info.min < 0
+        vals = [info.min, info.min + 1, -3 if signed else 3, -1 if signed else 1, 0, 1, 2, 3, 7, bits - 1, bits,
+                bits + 1, info.max - 1, info.max]
+        a, b = np.meshgrid(np.array(vals, dtype=dt), np.array(vals, dtype=dt), indexing="ij")
+        for op, fn in (("bitwise_right_shift", _functor_right_shift), ("bitwise_left_shift", _functor_left_shift),
+                       ("pow", _functor_pow), ("floor_divide", _functor_floor_divide),
+                       ("remainder", _functor_remainder), ("fmod", _functor_fmod)):
+            got = orc.binary(op, a, b)
+            for i, x in enumerate(vals):
+                for j, y in enumerate(vals):
+                    if signed and y == -1 and x == info.min and op in ("floor_divide", "remainder", "fmod"):
+                        continue  # INT_MIN / -1 overflows in C: undefined in the reference
+                    assert int(got[i, j]) == fn(x, y, bits, signed), (op, dt, x, y)
+
+
+@pytest.mark.parametrize("dt", ["i1", "u1", "i2", "u2", "i4", "u4", "i8", "u8"])
+def test_shift_range_known_answer(dt):
+    # test_bitwise_right_shift.py:107-117, test_bitwise_left_shift.py:107-117: ones shifted by 64 are 0
+    x, y = np.ones(255, dtype=dt), np.asarray(64, dtype=dt)
+    assert not orc.binary("bitwise_right_shift", x, y).any()
+    assert not orc.binary("bitwise_left_shift", x, y).any()
+
+
+def test_float_floor_divide_and_remainder_rules():
+    # floor_divide.hpp:84-86: floor of the ROUNDED quotient (1.0 // 0.1 is 10, where Python's and
+    # NumPy's divmod-based rule give 9); remainder.hpp:84-96: fmod, `+= y` on a sign mismatch, a
+    # zero remainder takes y's sign.  Exact rational arithmetic is the independent evaluation.
+    rng = np.random.default_rng(21)
+    for dt in ("f4", "f8"):
+        a = rng.uniform(-50, 50, 400).astype(dt)
+        b = rng.uniform(-7, 7, 400).astype(dt)
+        a[:6] = [1.0, -1.0, 7.5, -7.5, 6.0, -6.0]
+        b[:6] = [0.1, 0.1, 2.5, 2.5, -3.0, 3.0]
+        q, r = orc.binary("floor_divide", a, b), orc.binary("remainder", a, b)
+        for x, y, qq, rr in zip(a, b, q, r):
+            assert float(qq) == float(math.floor(np.dtype(dt).type(x) / np.dtype(dt).type(y)))
+            fx, fy = Fraction(float(x)), Fraction(float(y))
+            t = fx - fy * int(fx / fy)              # C fmod: exact, truncated quotient
+            if t != 0 and ((fy < 0) != (t < 0)):
+                want = np.dtype(dt).type(float(t)) + np.dtype(dt).type(y)  # one rounded addition
+            else:
+                want = np.dtype(dt).type(float(t))
+            assert float(rr) == float(want), (x, y, rr, want)
+            if t == 0:
+                assert np.signbit(rr) == np.signbit(y)
+    assert orc.binary("floor_divide", np.array([1.0]), np.array([0.1]))[0] == 10.0
+    # special cases, test_floor_divide.py:109-147 and test_remainder.py:138-152
+    inf, nan = np.inf, np.nan
+    x = np.array([inf, 0.0, -1.0, -1.0, inf, 1.0], dtype="f4")
+    y = np.array([inf, -1.0, 0.0, inf, -1.0, nan], dtype="f4")
+    q = orc.binary("floor_divide", x, y)
+    assert np.isnan(q[0]) and q[1] == 0 and np.signbit(q[1]) and q[2] == -inf
+    assert q[3] == 0 and np.signbit(q[3]) and q[4] == -inf and np.isnan(q[5])
+    lhs = np.array([nan, inf, 0.0, -0.0, -0.0, 1.0, inf, -inf, 5.0, -5.0], dtype="f4")
+    rhs = np.array([nan, inf, -0.0, 1.0, -1.0, 0.0, 1.0, -1.0, inf, inf], dtype="f4")
+    r = orc.binary("remainder", lhs, rhs)
+    assert np.isnan(r[[0, 1, 2, 5, 6, 7]]).all()
+    assert r[3] == 0 and not np.signbit(r[3]) and r[4] == 0 and np.signbit(r[4])
+    assert r[8] == 5.0 and r[9] == inf  # fmod(-5, inf) = -5, sign differs from y: -5 + inf
+
+
+def test_sign_rules():
+    # sign.hpp:73-110; known answers of test_sign.py:61-101
+    for dt in ("i1", "i2", "i4", "i8", "f2", "f4", "f8"):
+        x = np.arange(-20, 20, 1).astype(dt)
+        want = [(0 < int(v)) - (int(v) < 0) for v in x]
+        assert orc.unary("sign", x).tolist() == want and orc.unary("sign", x).dtype == np.dtype(dt)
+    assert orc.unary("sign", np.array([0, 1, 200], dtype="u1")).tolist() == [0, 1, 1]
+    f = orc.unary("sign", np.array([np.nan, -np.inf, np.inf, -0.0, 0.0], dtype="f4"))
+    assert np.isnan(f[0]) and f[1:].tolist() == [-1, 1, 0, 0] and not np.signbit(f[3])
+    z = np.array([3 + 4j, -5j, 0], dtype="c16")
+    got = orc.unary("sign", z)
+    assert got[0] == complex(0.6, 0.8) and got[1] == -1j and got[2] == 0
+
+
+def test_promotion_with_acceptance_hooks():
+    # dpnp/tests/tensor/elementwise/test_divide.py dtype matrix: the result dtype of divide is
+    # NumPy's for every pair (int8 / uint8 is float64, not float16)
+    fp_only = lambda a, b: a if (a == b and a.kind in "fc") else None  # noqa: E731
+    for d1 in orc.ALL_DTYPES:
+        for d2 in orc.ALL_DTYPES:
+            _b1, _b2, r = orc.promote_binary(fp_only, d1, d2, accept=orc.accept_divide)
+            want = np.true_divide(np.ones(1, d1), np.ones(1, d2)).dtype
+            assert r == want, (d1, d2, r, want)
 
 
 def test_mixed_int64_uint64_comparisons_are_exact():
@@ -324,6 +515,13 @@ def test_round_conj_parts_proj_rules():
     # round.hpp:74-96 (rint: ties to even), conj.hpp / real.hpp / imag.hpp / proj.hpp type maps
     assert (orc.unary("round", np.array([0.5, 1.5, 2.5, -0.5, -1.5], dtype="f4")) == [0, 2, 2, -0.0, -2]).all()
     assert (orc.unary("round", np.array([3, -4], dtype="i2")) == [3, -4]).all()
+    for dt in ("f2", "f4", "f8"):  # test_round.py:107-122 (values spelled out: ties go to even)
+        x = np.array([np.nan, np.inf, -np.inf, 1.5, 2.5, -1.5, -2.5, 0.0, -0.0], dtype=dt)
+        y = orc.unary("round", x)
+        assert np.isnan(y[0]) and y[1:].tolist() == [np.inf, -np.inf, 2, 2, -2, -2, 0, 0]
+        assert np.signbit(y).tolist() == [False, False, True, False, False, True, True, False, True]
+        h = np.arange(-9, 10).astype(dt) + np.dtype(dt).type(0.5)
+        assert orc.unary("round", h).tolist() == [float(round(float(v))) for v in h]  # Python: half to even
     assert orc.unary("conj", np.array([True])).dtype == np.dtype("i1")
     assert orc.unary("conj", np.array([1 + 2j], dtype="c8"))[0] == 1 - 2j
     assert orc.unary("real", np.array([1 + 2j], dtype="c16")).dtype == np.dtype("f8")
