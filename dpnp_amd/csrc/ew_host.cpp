@@ -33,11 +33,11 @@ int ew_validate(int nops, const dpx_array_view *const *views, int64_t &n)
     return DPX_OK;
 }
 
-// block-size override for experiments: a power of two in [64, 256], else the default
+// block-size override for sweeps (a power of two in [64, 256], else the default); the product
+// build compiles tune_int() down to its default
 static int env_block(const char *name, int dflt)
 {
-    const char *s = std::getenv(name);
-    const int v = (s && *s) ? std::atoi(s) : dflt;
+    const int v = tune_int(name, dflt);
     return (v == 64 || v == 128 || v == 256) ? v : dflt;
 }
 

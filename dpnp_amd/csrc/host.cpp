@@ -1,5 +1,6 @@
 #include "host.hpp"
 #include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <numeric>
@@ -151,12 +152,12 @@ namespace {
 struct Block {
     void *p = nullptr;
     size_t bytes = 0;
+    bool dirty = false;
 };
 std::mutex g_pool_mu;
 std::map<std::pair<int, hipStream_t>, Block> g_pool;
+std::vector<void *> g_retired; // outgrown blocks: possibly still in use, freed by scratch_release_all()
 
-// Clears a fresh block.  A kernel rather than a memset call: memset nodes recorded into a stream
-// capture have replayed wrongly on these machines.
 __global__ void scratch_zero_kernel(uint4 *p, size_t n16)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
@@ -164,46 +165,75 @@ __global__ void scratch_zero_kernel(uint4 *p, size_t n16)
 }
 } // namespace
 
-void *scratch_get(hipStream_t stream, size_t bytes)
+hipError_t zero_fill_async(void *p, size_t n16, hipStream_t stream)
+{
+    if (n16 == 0) return hipSuccess;
+    const unsigned blocks = (unsigned)std::min<size_t>((n16 + 255) / 256, 1024);
+    scratch_zero_kernel<<<blocks, 256, 0, stream>>>(static_cast<uint4 *>(p), n16);
+    return hipGetLastError();
+}
+
+void *scratch_get(hipStream_t stream, size_t bytes, size_t counter_bytes)
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lk(g_pool_mu);
     Block &b = g_pool[{dev, stream}];
-    if (b.bytes >= bytes && b.p) return b.p;
-    if (b.p) {
-        // the old block may still be read by work queued on this stream
-        if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
-        (void)hipFree(b.p);
-        b.p = nullptr;
-        b.bytes = 0;
+    if (b.p && b.bytes >= bytes) {
+        if (b.dirty) {
+            if (zero_fill_async(b.p, std::min(counter_bytes, b.bytes) / 16, stream) != hipSuccess) return nullptr;
+            b.dirty = false;
+        }
+        return b.p;
     }
-    size_t want = std::max<size_t>(bytes, (size_t)1 << 20);
+    size_t want = std::max<size_t>(bytes, SCRATCH_BLOCK_BYTES);
     want = (want + 4095) & ~(size_t)4095;
-    if (hipMalloc(&b.p, want) != hipSuccess) {
-        b.p = nullptr;
-        return nullptr;
-    }
+    void *fresh = nullptr;
+    if (hipMalloc(&fresh, want) != hipSuccess) return nullptr;
     // callers rely on fresh blocks being zero (ticket counters) and keep them zero
-    const size_t n16 = want / 16; // want is a multiple of 4096
-    const unsigned blocks = (unsigned)std::min<size_t>((n16 + 255) / 256, 1024);
-    scratch_zero_kernel<<<blocks, 256, 0, stream>>>(static_cast<uint4 *>(b.p), n16);
-    if (hipGetLastError() != hipSuccess) {
-        (void)hipFree(b.p);
-        b.p = nullptr;
+    if (zero_fill_async(fresh, want / 16, stream) != hipSuccess) { // want is a multiple of 4096
+        (void)hipFree(fresh);
         return nullptr;
     }
+    if (b.p) g_retired.push_back(b.p);
+    b.p = fresh;
     b.bytes = want;
+    b.dirty = false;
     return b.p;
+}
+void scratch_mark_dirty(hipStream_t stream)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lk(g_pool_mu);
+    auto it = g_pool.find({dev, stream});
+    if (it != g_pool.end()) it->second.dirty = true;
 }
 int scratch_release_all()
 {
     std::lock_guard<std::mutex> lk(g_pool_mu);
     for (auto &kv : g_pool)
         if (kv.second.p) (void)hipFree(kv.second.p);
+    for (void *p : g_retired) (void)hipFree(p);
     g_pool.clear();
+    g_retired.clear();
     return DPX_OK;
 }
+
+#ifdef DPX_TUNING
+int tune_int(const char *name, int dflt)
+{
+    static std::mutex mu;
+    static std::map<std::string, int> seen;
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = seen.find(name);
+    if (it != seen.end()) return it->second;
+    const char *s = std::getenv(name);
+    const int v = (s && *s) ? std::atoi(s) : dflt;
+    seen[name] = v;
+    return v;
+}
+#endif
 
 int device_cus()
 {

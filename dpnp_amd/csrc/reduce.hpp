@@ -844,6 +844,16 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     uint32_t zero = 0;
     for (int c = t; c < inner; c += T) zero |= slot_publish(partial + (int64_t)split * inner + c, sm[c]);
     if (!last_block_of(counters, L.splits, zero)) return;
+    if (inner > T) {
+        // more columns than threads (1-byte elements, rows of 257 to 511 bytes): a thread folds whole
+        // columns, blocks in index order
+        for (int c = t; c < inner; c += T) {
+            Acc v = P::identity();
+            for (int g = 0; g < L.splits; ++g) v = P::combine(v, slot_read(partial + (int64_t)g * inner + c));
+            dst[(int64_t)c * ix.dst_str[0]] = P::post(v, L.param);
+        }
+        return;
+    }
     // the last block: thread t < parts * inner folds blocks part, part + parts, ... of column t mod inner
     const int parts = T / inner;
     Acc v = P::identity();

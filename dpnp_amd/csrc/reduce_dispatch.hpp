@@ -1,6 +1,7 @@
 // Host side of the reductions: plan (type independent) + templated launch sequence.
 #pragma once
 #include <algorithm>
+#include <string>
 #include "host.hpp"
 #include "reduce.hpp"
 
@@ -15,7 +16,36 @@ struct RedPlan {
     int block;                          // threads per block
     int64_t grid;
     int64_t scratch_elems; // partials: m * splits
+    // scratch block brought by the caller instead of the stream's pool block (the entry point that
+    // allocates nothing): [counters | partials], counters zero; nullptr: take the pool's
+    char *ext_scratch;
+    size_t ext_scratch_bytes;
 };
+
+// Scratch for a split launch: `need` bytes laid out [counters | partials].  DPX_OK and *out set, or
+// the failure recorded.
+inline int red_scratch(const RedPlan &pl, hipStream_t stream, size_t need, char **out)
+{
+    if (pl.ext_scratch) {
+        if (need > pl.ext_scratch_bytes)
+            return fail(DPX_ERR_BAD_ARGUMENT,
+                        "this reduction needs " + std::to_string(need) + " bytes of scratch for its partial results; "
+                        "the static scratch of the entry point that allocates nothing holds " +
+                        std::to_string(pl.ext_scratch_bytes) + ": use dpx_reduce");
+        *out = pl.ext_scratch;
+        return DPX_OK;
+    }
+    *out = (char *)scratch_get(stream, need, RED_COUNTER_BYTES);
+    return *out ? DPX_OK : fail(DPX_ERR_HIP, "cannot allocate reduction scratch");
+}
+// after a launch that used scratch: an error leaves the ticket counters in doubt
+inline int red_launch_status(const RedPlan &pl, hipStream_t stream, const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return DPX_OK;
+    if (pl.L.splits > 1 && !pl.ext_scratch) scratch_mark_dirty(stream);
+    return fail_hip(e, what);
+}
 
 // Validation shared by reductions and searches, in the order of py_reduction_over_axis
 // (libtensor/source/reductions/reduction_over_axis.hpp:188-238).
@@ -50,8 +80,9 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     Slot<Acc> *partial = nullptr;
     unsigned *counters = nullptr;
     if (pl.L.splits > 1) {
-        char *s = (char *)scratch_get(stream, RED_COUNTER_BYTES + (size_t)pl.scratch_elems * sizeof(Slot<Acc>));
-        if (!s) return fail(DPX_ERR_HIP, "cannot allocate reduction scratch");
+        char *s = nullptr;
+        if (int rc = red_scratch(pl, stream, RED_COUNTER_BYTES + (size_t)pl.scratch_elems * sizeof(Slot<Acc>), &s))
+            return rc;
         counters = (unsigned *)s;
         partial = (Slot<Acc> *)(s + RED_COUNTER_BYTES);
     }
@@ -59,6 +90,7 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         constexpr int E = cols_cfg<In>::E;
         int block = pl.block; // LDS: one accumulator pack per thread, at most 64 KiB
         while ((size_t)block * E * sizeof(Acc) > 65536) block /= 2;
+        if (block < (1 << pl.L.g_log2)) return fail(DPX_ERR_NOT_IMPLEMENTED, "column reduction: accumulator too wide");
         const size_t smem = (size_t)block * E * sizeof(Acc);
         hipLaunchKernelGGL((red_cols_kernel<P>), dim3((unsigned)pl.grid), dim3(block), smem, stream, pl.ix, pl.L, sp,
                            dp, partial, ap, counters);
@@ -79,8 +111,7 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     else
         hipLaunchKernelGGL((red_rows_kernel<P, true>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.ix,
                            pl.L, sp, dp, partial, ap, counters);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? DPX_OK : fail_hip(e, "reduction launch");
+    return red_launch_status(pl, stream, "reduction launch");
 }
 
 template <class T, bool IS_MAX>
@@ -94,9 +125,10 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     unsigned *counters = nullptr;
     if (pl.L.splits > 1) {
         // [counters | positions | values]
-        char *s = (char *)scratch_get(stream, RED_COUNTER_BYTES + (size_t)pl.scratch_elems *
-                                                                      (sizeof(Slot<int64_t>) + sizeof(Slot<T>)));
-        if (!s) return fail(DPX_ERR_HIP, "cannot allocate reduction scratch");
+        char *s = nullptr;
+        if (int rc = red_scratch(pl, stream,
+                                 RED_COUNTER_BYTES + (size_t)pl.scratch_elems * (sizeof(Slot<int64_t>) + sizeof(Slot<T>)), &s))
+            return rc;
         counters = (unsigned *)s;
         pidx = (Slot<int64_t> *)(s + RED_COUNTER_BYTES);
         pval = (Slot<T> *)(s + RED_COUNTER_BYTES + (size_t)pl.scratch_elems * sizeof(Slot<int64_t>));
@@ -115,8 +147,7 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     else
         hipLaunchKernelGGL((arg_rows_kernel<T, IS_MAX, true>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
                            pl.ix, pl.L, sp, dp, pval, pidx, counters);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? DPX_OK : fail_hip(e, "search launch");
+    return red_launch_status(pl, stream, "search launch");
 }
 
 } // namespace dpx

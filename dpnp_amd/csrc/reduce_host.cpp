@@ -40,11 +40,6 @@ int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *
     return DPX_OK;
 }
 
-static int env_int(const char *name, int dflt)
-{
-    const char *s = std::getenv(name);
-    return (s && *s) ? std::atoi(s) : dflt;
-}
 static int ceil_log2(int64_t v)
 {
     int lg = 0;
@@ -58,14 +53,18 @@ static int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // 1024-thread blocks, lose 5-10 points, and a grid that is not a multiple of the CU count
 // loses as much to the tail.  Hence: 256-thread blocks, two per CU when a reduction has to
 // be split.
-static int64_t red_target_blocks() { return env_int("DPX_RED_TARGET_BLOCKS", 2 * device_cus()); }
+// (the override is clamped so that outputs x splits stays within the ticket table)
+static int64_t red_target_blocks()
+{
+    return std::min<int64_t>(std::max(tune_int("DPX_RED_TARGET_BLOCKS", 2 * device_cus()), 1), RED_MAX_TICKETS);
+}
 
 // lanes cooperating on one output of `n` elements read `e` at a time: aim at ~8 accesses
 // per lane; more than a wave means a whole 256-thread block
 static void rows_geometry(int64_t n, int e, int &g_log2, int &block)
 {
     int64_t lanes = cdiv(n, (int64_t)e * 8);
-    const int forced = env_int("DPX_ROWS_G_LOG2", -1); // experiment knob
+    const int forced = tune_int("DPX_ROWS_G_LOG2", -1); // sweep override, product build: default
     if (forced >= 0) lanes = (int64_t)1 << forced;
     if (lanes <= 64) {
         g_log2 = ceil_log2(lanes);
@@ -154,7 +153,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     RedLaunch &L = pl.L;
 
     if (contig_red && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
-        env_int("DPX_RED_SHORT_ROWS", 1) != 0) { // (experiment knob: 0 keeps the rows kernel)
+        tune_int("DPX_RED_SHORT_ROWS", 1) != 0) { // (sweep override: 0 keeps the rows kernel)
         // ---- short rows: a block stages R whole rows in LDS (see red_short_rows_kernel) ----
         const int64_t pitch_bytes = (int64_t)srow_pitch_for((int)n, in_size) * in_size;
         const int64_t R = std::min<int64_t>(2048, SROW_LDS_BYTES / pitch_bytes);
@@ -204,7 +203,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
     if (!arg && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
-        env_int("DPX_RED_FLAT", 1) != 0) { // (experiment knob: 0 keeps the column kernel)
+        tune_int("DPX_RED_FLAT", 1) != 0) { // (sweep override: 0 keeps the column kernel)
         // a row-major matrix with rows shorter than 512 bytes: one flat stream of packs, a block of
         // T threads with T * E a multiple of the row length (see red_flat_kernel)
         int64_t g = inner, b = E;
@@ -248,13 +247,13 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
     // with a single thread row a whole wave lies side by side and nothing is combined in LDS
     int lg = std::min(ty == 1 ? 6 : 5, ceil_log2(cdiv(inner, e)));
-    const int forced = env_int("DPX_COLS_TX_LOG2", -1); // experiment knob
+    const int forced = tune_int("DPX_COLS_TX_LOG2", -1); // sweep override, product build: default
     if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(inner, e)), forced);
     L.g_log2 = lg;
     const int64_t TX = (int64_t)1 << lg;
     int block = (int)std::min<int64_t>(arg ? 256 : 512, std::max<int64_t>(64, TX * ty));
     if (!arg) {
-        const int fb = env_int("DPX_COLS_BLOCK", 0); // experiment knob
+        const int fb = tune_int("DPX_COLS_BLOCK", 0); // sweep override, product build: default
         if (fb == 256 || fb == 512 || fb == 1024) block = fb;
     }
     if (block < TX) block = (int)TX;
