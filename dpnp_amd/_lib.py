@@ -13,6 +13,7 @@ import os
 import torch  # noqa: F401,E402
 
 MAX_ND = 12
+NOALLOC_SCRATCH_BYTES = 2 << 20  # DPX_NOALLOC_SCRATCH_BYTES
 
 (BOOL, INT8, UINT8, INT16, UINT16, INT32, UINT32, INT64, UINT64, HALF, FLOAT,
  DOUBLE, CFLOAT, CDOUBLE) = range(14)
@@ -125,6 +126,7 @@ SIGNATURES = {
     "dpx_where_compare": (_i, [_i, _VP, _VP, _VP, _VP, _VP, _vp]),
     "dpx_black_scholes": (_i, [_vp, _vp, _vp, _d, _d, _vp, _vp, _i64, _i, _vp]),
     "dpx_reduce": (_i, [_i, _VP, _i, _VP, _VP, _vp]),
+    "dpx_reduce_noalloc": (_i, [_i, _VP, _i, _VP, _VP, _vp]),
     "dpx_nan_variance": (_i, [_VP, _i, _VP, _d, _VP, _vp]),
     "dpx_argreduce": (_i, [_i, _VP, _i, _VP, _vp]),
     "dpx_reduce_plan": (_i, [_i, _VP, _i, _VP, _PP]),

@@ -1,7 +1,38 @@
 // extern "C" reduction entry points.
+#include <mutex>
 #include "reduce_dispatch.hpp"
 
+// Scratch of dpx_reduce_noalloc: device memory that exists from the moment the library's code
+// object is loaded on a GPU, so the entry point never allocates.  Each GPU holds its own copy
+// until the process ends.  In host code the name below is only a handle for
+// hipGetSymbolAddress; kernels and fills get the per-device address it returns.
+static __device__ __align__(256) unsigned char scratch[DPX_NOALLOC_SCRATCH_BYTES];
+
 namespace dpx {
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+std::mutex g_noalloc_mu;
+char *g_noalloc_ptr[NOALLOC_MAX_DEVICES]; // address of `scratch` on each device, looked up once
+} // namespace
+
+// Address of the static scratch on the current device (first call on a device: one symbol lookup).
+static int noalloc_scratch(char **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail_hip(e, "hipGetDevice");
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fail(DPX_ERR_BAD_ARGUMENT, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    if (!g_noalloc_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail_hip(e, "hipGetSymbolAddress(static reduction scratch)");
+        g_noalloc_ptr[dev] = (char *)p;
+    }
+    *out = g_noalloc_ptr[dev];
+    return DPX_OK;
+}
+
 bool sum_pair_supported(int, int);
 bool prod_pair_supported(int, int);
 bool sqdev_pair_supported(int, int);
@@ -46,7 +77,8 @@ static bool reduce_supported(int op, int s, int d)
 }
 
 static int reduce_call(int op, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
-                       const dpx_array_view *aux, void *stream, dpx_plan *plan_out, double param = 0.0)
+                       const dpx_array_view *aux, void *stream, dpx_plan *plan_out, double param = 0.0,
+                       bool noalloc = false)
 {
     if (op < 0 || op >= DPX_R_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown reduction op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
@@ -58,7 +90,8 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false);
-    if (plan_out) {
+    // bytes of one partial result (the accumulator type of the typed kernel)
+    auto acc_bytes = [&]() {
         int acc = itemsize_of(dst->dtype);
         if (op == DPX_R_SUM || op == DPX_R_SUMSQDEV) acc = sum_acc_size(src->dtype, dst->dtype) ? sum_acc_size(src->dtype, dst->dtype) : acc;
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
@@ -66,11 +99,28 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
         if (is_nan_op(op)) acc = nan_acc_size(op, src, dst);
         if (is_truth_op(op)) acc = op == DPX_R_COUNT_NONZERO ? 8 : 4;
-        red_export_plan(pl, plan_out, acc);
+        return acc;
+    };
+    if (plan_out) {
+        red_export_plan(pl, plan_out, acc_bytes());
         return DPX_OK;
     }
     hipStream_t s = (hipStream_t)stream;
     pl.L.param = param;
+    if (noalloc && pl.L.splits > 1) {
+        const size_t need = RED_COUNTER_BYTES + (size_t)pl.scratch_elems * (size_t)((acc_bytes() + 3) / 4 * 4);
+        if (need > DPX_NOALLOC_SCRATCH_BYTES)
+            return fail(DPX_ERR_BAD_ARGUMENT,
+                        "dpx_reduce_noalloc: the partial results of this reduction need " + std::to_string(need) +
+                            " bytes of scratch, the static scratch holds " +
+                            std::to_string((size_t)DPX_NOALLOC_SCRATCH_BYTES) + "; use dpx_reduce");
+        // the static block instead of the pool's; its ticket counters must be zero when the kernel
+        // starts, whatever an earlier call left (a fill kernel: legal under stream capture)
+        if (int rc = noalloc_scratch(&pl.ext_scratch)) return rc;
+        pl.ext_scratch_bytes = DPX_NOALLOC_SCRATCH_BYTES;
+        const hipError_t e = zero_fill_async(pl.ext_scratch, RED_COUNTER_BYTES / 16, s);
+        if (e != hipSuccess) return fail_hip(e, "clearing the static scratch counters");
+    }
     if (is_nan_op(op)) return nan_run(op, pl, src, dst, aux, s);
     if (is_truth_op(op)) return truth_run(op, pl, src, dst, s);
     switch (op) {
@@ -122,6 +172,11 @@ int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce, c
                const dpx_array_view *aux, void *stream)
 {
     return reduce_call(op, src, trailing_dims_to_reduce, dst, aux, stream, nullptr);
+}
+int dpx_reduce_noalloc(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
+                       const dpx_array_view *aux, void *stream)
+{
+    return reduce_call(op, src, trailing_dims_to_reduce, dst, aux, stream, nullptr, 0.0, true);
 }
 int dpx_reduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *dst,
                     dpx_plan *plan)

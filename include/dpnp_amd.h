@@ -450,6 +450,23 @@ int dpx_nan_variance(const dpx_array_view *src, int trailing_dims_to_reduce,
 int dpx_argreduce(int op, const dpx_array_view *src,
                   int trailing_dims_to_reduce, const dpx_array_view *dst,
                   void *stream);
+/* dpx_reduce for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, validation and results as dpx_reduce (bit for bit: same kernels, same partition).
+ * A reduction that is split over several blocks per output keeps its partial results in a static
+ * device array of DPX_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the
+ * process ends, instead of the per-stream pool; the call clears the array's ticket counters with
+ * a fill kernel, launches the reduction, and calls no hipMalloc / hipFree.  A reduction whose
+ * partials do not fit fails with DPX_ERR_BAD_ARGUMENT before anything is launched
+ * (dpx_reduce_plan(...).scratch_bytes tells in advance: row and full reductions need at most
+ * 136 KiB, column reductions at most 1.2 MiB; only reductions over the rows of a row-major matrix
+ * of 1- and 2-byte elements with rows of 300 to 511 bytes exceed the limit).  All calls on one GPU share the array: two calls of this entry point that
+ * overlap in time on one GPU (different streams, or two host threads) race on it; calls on one
+ * stream, or calls ordered by events, are safe. */
+#define DPX_NOALLOC_SCRATCH_BYTES (2u << 20)
+int dpx_reduce_noalloc(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
+                       const dpx_array_view *dst, const dpx_array_view *aux,
+                       void *stream);
 int dpx_reduce_plan(int op, const dpx_array_view *src,
                     int trailing_dims_to_reduce, const dpx_array_view *dst,
                     dpx_plan *plan);
