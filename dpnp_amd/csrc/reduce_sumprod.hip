@@ -36,6 +36,18 @@ template <class F> static bool for_sum_pair(int in_dt, int out_dt, F &&f)
     DPX_PAIR(uint64_t, double) DPX_PAIR(bool_t, float) DPX_PAIR(int8_t, float) DPX_PAIR(uint8_t, float)
     DPX_PAIR(int16_t, float) DPX_PAIR(uint16_t, float) DPX_PAIR(int32_t, float) DPX_PAIR(uint32_t, float)
     DPX_PAIR(int64_t, float) DPX_PAIR(uint64_t, float)
+    // the remaining pairs of the reference's tables (sum.cpp:87-241, prod.cpp alike): narrower
+    // integer results (the input is converted to the result type, which then wraps), unsigned
+    // into signed, real into complex
+    DPX_PAIR(bool_t, int8_t) DPX_PAIR(bool_t, uint8_t) DPX_PAIR(bool_t, int16_t) DPX_PAIR(bool_t, uint16_t)
+    DPX_PAIR(bool_t, int32_t) DPX_PAIR(bool_t, uint32_t) DPX_PAIR(bool_t, uint64_t)
+    DPX_PAIR(int8_t, int16_t) DPX_PAIR(int8_t, int32_t)
+    DPX_PAIR(uint8_t, int16_t) DPX_PAIR(uint8_t, uint16_t) DPX_PAIR(uint8_t, int32_t) DPX_PAIR(uint8_t, uint32_t)
+    DPX_PAIR(uint8_t, int64_t)
+    DPX_PAIR(int16_t, int32_t)
+    DPX_PAIR(uint16_t, int32_t) DPX_PAIR(uint16_t, uint32_t) DPX_PAIR(uint16_t, int64_t)
+    DPX_PAIR(uint32_t, int64_t)
+    DPX_PAIR(half_t, c64) DPX_PAIR(half_t, c128) DPX_PAIR(float, c64) DPX_PAIR(float, c128) DPX_PAIR(double, c128)
 #undef DPX_PAIR
     return hit;
 }

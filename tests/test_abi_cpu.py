@@ -104,6 +104,18 @@ def test_reduction_dtype_support():
         assert lib.dpx_reduce_dtype_supported(R["max"], i, i) == 1
         assert lib.dpx_search_dtype_supported(0, i, L.INT64) == 1
         assert lib.dpx_search_dtype_supported(0, i, L.INT32) == 0
+    # every (input, result) pair of the reference's sum / prod tables has a kernel of its own
+    import json
+    import os
+
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+    names = [d.str[1:] if d.kind != "b" else "?" for d in NP]
+    pairs = gold["sum_prod_type_pairs"]["pairs"]
+    assert sorted(pairs) == sorted(names)
+    for src, outs in pairs.items():
+        for dst in outs:
+            assert lib.dpx_reduce_dtype_supported(R["sum"], names.index(src), names.index(dst)) == 1, (src, dst)
+            assert lib.dpx_reduce_dtype_supported(R["prod"], names.index(src), names.index(dst)) == 1, (src, dst)
     assert lib.dpx_reduce_dtype_supported(R["sum"], L.FLOAT, L.DOUBLE) == 1
     assert lib.dpx_reduce_dtype_supported(R["sum"], L.DOUBLE, L.FLOAT) == 0
     assert lib.dpx_reduce_dtype_supported(R["max"], L.FLOAT, L.DOUBLE) == 0

@@ -1,5 +1,7 @@
 """The five benchmark configurations at their full sizes: results checked through
 size-independent properties and through the oracle on samples / reduced problems."""
+import math
+
 import numpy as np
 import pytest
 
@@ -62,11 +64,15 @@ def test_config3_argmax_mean_var_2p28():
     want_v = float(np.mean((x64 - want_m) ** 2))
     assert abs(m - want_m) <= 1e-12 * max(abs(want_m), float(np.mean(np.abs(x64))))
     assert abs(v - want_v) <= 1e-12 * want_v
-    # float64 input (half the length to bound host memory): 1e-12
-    d64 = dev(x64[: n // 2])
-    want_m2 = float(np.mean(x64[: n // 2]))
-    want_v2 = float(np.mean((x64[: n // 2] - want_m2) ** 2))
-    assert abs(float(dpt.mean(d64)) - want_m2) <= 1e-12 * float(np.mean(np.abs(x64[: n // 2])))
+    # float64 input at the full 2^28 elements (the host check streams in chunks): 1e-12
+    d64 = dev(x64)
+    step = 1 << 24
+    want_m2 = math.fsum(float(np.sum(x64[i:i + step], dtype=np.longdouble)) for i in range(0, n, step)) / n
+    want_v2 = math.fsum(float(np.sum((x64[i:i + step] - want_m2) ** 2, dtype=np.longdouble))
+                        for i in range(0, n, step)) / n
+    mean_abs = math.fsum(float(np.sum(np.abs(x64[i:i + step]))) for i in range(0, n, step)) / n
+    assert d64.shape == (n,) and d64.dtype == np.dtype("f8")
+    assert abs(float(dpt.mean(d64)) - want_m2) <= 1e-12 * mean_abs
     assert abs(float(dpt.var(d64)) - want_v2) <= 1e-12 * want_v2
     del d64, x64
     # NaN variant: about 0.1 % NaNs -> index of the first NaN, NaN statistics

@@ -52,6 +52,35 @@ def test_sum_arg_out_dtype_matrix(arg):
         assert r.dtype == out and host(r) == 100
 
 
+@pytest.mark.parametrize("src", sorted(GOLD["sum_prod_type_pairs"]["pairs"]))
+def test_sum_prod_every_reference_pair_in_one_pass(src):
+    # sum.cpp:87-241, prod.cpp: each (input, result) pair of the reference's tables has a direct kernel;
+    # values chosen so that narrow results wrap: the element is converted to the result type, then added
+    import dpnp_amd._lib as L
+
+    rng = np.random.default_rng(59)
+    for dst in GOLD["sum_prod_type_pairs"]["pairs"][src]:
+        names = [d.str[1:] if d.kind != "b" else "?" for d in ALL]
+        for op in ("sum", "prod"):
+            assert L.lib.dpx_reduce_dtype_supported(L.REDUCE_ID[op], names.index(src), names.index(dst)) == 1
+        for shape, axis in (((5, 3001), 1), ((3001, 40), 0), ((1 << 20,), None)):
+            a = random_array(rng, shape, src, -100, 100)
+            got = host(dpt.sum(dev(a), axis=axis, dtype=dst))
+            want = orc.reduce("sum", a if axis != 0 else a.T, 1, out_dtype=dst)
+            if np.dtype(dst).kind in "fc":
+                scale = np.abs(a.astype("f8")).sum(axis=axis)
+                assert (np.abs(got - want) <= RTOL[np.dtype(dst)] * np.maximum(scale, 1)).all(), (src, dst, shape)
+            else:
+                assert_same(got, want)
+            small = random_array(rng, (7, 9), src, -3, 3)  # products that neither overflow floats nor vanish
+            gp = host(dpt.prod(dev(small), axis=1, dtype=dst))
+            wp = orc.reduce("prod", small, 1, out_dtype=dst)
+            if np.dtype(dst).kind in "fc":
+                np.testing.assert_allclose(gp, wp, rtol=1e-3 if dst == "f2" else 1e-5)
+            else:
+                assert_same(gp, wp)
+
+
 def test_sum_known_answers():
     g = GOLD["sum_gh1391"]
     a = dpt.reshape(dpt.arange(g["arange"], dtype="i4"), g["shape"])
@@ -368,15 +397,16 @@ def test_nanarg_ties_infinities_and_large():
     assert_same(dpnp.nanmin(dm, axis=0).asnumpy(), np.nanmin(m, axis=0))
 
 
-@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
-@pytest.mark.parametrize("shape, axis", [((5000,), None), ((3_000_003,), None), ((300, 700), 1), ((300, 700), 0),
-                                         ((40_000, 24), 0), ((40_000, 12), 1), ((70_000, 1500), 0)])
+_NANARG_SHAPES = [((5000,), None), ((3_000_003,), None), ((300, 700), 1), ((300, 700), 0), ((40_000, 24), 0),
+                  ((40_000, 12), 1)]
+
+
+@pytest.mark.parametrize("dt, shape, axis", [(dt, sh, ax) for dt in ("f2", "f4", "f8") for sh, ax in _NANARG_SHAPES] +
+                         [("f4", (70_000, 1500), 0)])  # one dtype is enough for the large matrix
 def test_nanarg_runs_whose_extreme_is_the_infinity_nan_counts_as(dt, shape, axis):
     """nanargmax reads NaN as -inf (dpnp/dpnp_iface_nanfunctions.py:195-200): a run with a NaN before a real -inf
     gives the position of the NaN, an all-NaN run raises, and the search kernel alone tells which runs need a
     second look."""
-    if shape == (70_000, 1500) and dt != "f4":
-        pytest.skip("one dtype is enough for the large matrix")
     rng = np.random.default_rng(5)
     a = rng.standard_normal(shape).astype(dt)
     a[rng.random(shape) < 0.05] = np.nan
