@@ -46,12 +46,16 @@ struct RedLaunch {
     int32_t splits;   // blocks cooperating on one output
     int32_t g_log2;   // rows: log2(lanes per output); cols: log2(threads along columns)
     int32_t vec;      // 16-byte packs allowed
-    int32_t tgroup;   // rows: blocks per first-level ticket group (0: one ticket counter per output)
+    int32_t tgroup;   // rows: not 0: two levels of tickets, groups of RED_TGROUP blocks (0: one counter per output)
     int64_t rstride;  // cols: stride of the reduced axis
     int64_t inner;    // cols: length of the inner (contiguous) iteration dim
     int64_t col_blocks;
     int32_t mark_fill; // NaN-ignoring searches: report "extreme equals the value NaNs count as" as -1 - index
     double param;      // K_NANVAR: delta degrees of freedom
+    // strides of a one-dimensional iteration space (nd_i1 != 0): the rows kernels then never read
+    // RedIndex, whose far part of the kernel-argument segment costs them a dependent fetch at start-up
+    int32_t nd_i1;
+    int64_t istr0, dstr0, astr0;
 };
 
 template <class T> DPX_D T shfl_down_any(T v, int off)
@@ -68,6 +72,36 @@ template <class T> DPX_D T shfl_down_any(T v, int off)
     return u.t;
 }
 
+// v of the lane CTRL selects inside each row of 16 lanes (DPP), word by word; a lane without a
+// source (row_shr by s: the first s lanes of a row) gets its own value back
+template <int CTRL, class T> DPX_D T dpp_any(T v)
+{
+    constexpr int W = (sizeof(T) + 3) / 4;
+    union {
+        T t;
+        int w[W];
+    } u;
+    u.w[W - 1] = 0;
+    u.t = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) u.w[i] = __builtin_amdgcn_update_dpp(u.w[i], u.w[i], CTRL, 0xf, 0xf, false);
+    return u.t;
+}
+// v of lane `lane` (a constant), in every lane
+template <class T> DPX_D T readlane_any(T v, int lane)
+{
+    constexpr int W = (sizeof(T) + 3) / 4;
+    union {
+        T t;
+        int w[W];
+    } u;
+    u.w[W - 1] = 0;
+    u.t = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) u.w[i] = __builtin_amdgcn_readlane(u.w[i], lane);
+    return u.t;
+}
+
 // iteration index -> element offsets of src / dst / aux
 DPX_D void iter_offsets(const RedIndex &ix, int64_t o, int64_t &so, int64_t &dof, int64_t &ao)
 {
@@ -80,6 +114,15 @@ DPX_D void iter_offsets(const RedIndex &ix, int64_t o, int64_t &so, int64_t &dof
         ao += i * ix.aux_str[d];
         o = q;
     }
+}
+DPX_D void iter_offsets(const RedIndex &ix, const RedLaunch &L, int64_t o, int64_t &so, int64_t &dof, int64_t &ao)
+{
+    if (L.nd_i1) {
+        so = o * L.istr0;
+        dof = o * L.dstr0;
+        ao = o * L.astr0;
+    }
+    else iter_offsets(ix, o, so, dof, ao);
 }
 DPX_D int64_t red_offset(const RedIndex &ix, int64_t pos)
 {
@@ -323,8 +366,19 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
 template <class P> DPX_D typename P::Acc group_reduce(typename P::Acc r, bool whole_block, int G)
 {
     using Acc = typename P::Acc;
-    const int wl = whole_block ? 64 : G;
-    for (int off = wl >> 1; off > 0; off >>= 1) r = P::combine(r, shfl_down_any(r, off));
+    if (whole_block) {
+        // a whole wave (all 64 lanes are here): rows of 16 lanes fold through DPP shifts into their
+        // last lane (row_shr:1, 2, 4, 8), the four row results are read from lanes 15, 31, 47, 63 and
+        // combined in that order in every lane.  0.3 us shorter than six lane permutes through LDS.
+        r = P::combine(r, dpp_any<0x111>(r));
+        r = P::combine(r, dpp_any<0x112>(r));
+        r = P::combine(r, dpp_any<0x114>(r));
+        r = P::combine(r, dpp_any<0x118>(r));
+        r = P::combine(P::combine(P::combine(readlane_any(r, 15), readlane_any(r, 31)), readlane_any(r, 47)),
+                       readlane_any(r, 63));
+    }
+    else
+        for (int off = G >> 1; off > 0; off >>= 1) r = P::combine(r, shfl_down_any(r, off));
     if (whole_block) {
         __shared__ Acc sm[16];
         __syncthreads(); // sm may still be read by a previous call
@@ -380,20 +434,19 @@ template <class T> DPX_D T slot_read(const Slot<T> *p)
     return u.t;
 }
 
-// Called by every thread of a block; `zero` is what slot_publish returned in this thread
-// (0 in threads that published nothing).  True, for all threads, in the block that took
-// the last of `splits` tickets for this counter: every partial of the output is then
-// readable.  The counter is left at zero for the next launch.
+// Called by every thread of a block, after the threads that hold a partial have published it with
+// slot_publish; `zero` is what slot_publish returned in thread 0 (0 if it published nothing).  True,
+// for all threads, in the block that took the last of `splits` tickets for this counter: every
+// partial of the output is then readable.  The counter is left at zero for the next launch.
+// Order: a thread leaves slot_publish only when its exchanges have returned (the asm statement there
+// consumes their results), the barrier below is passed when every thread has, and thread 0 draws the
+// ticket after the barrier.
 DPX_D bool last_block_of(unsigned *counter, int splits, uint32_t zero)
 {
-    __shared__ unsigned sh_zero;
     __shared__ int is_last;
-    if (threadIdx.x == 0) sh_zero = 0;
-    __syncthreads();
-    atomicOr(&sh_zero, zero); // consumes `zero`: waits for this thread's exchanges
     __syncthreads();
     if (threadIdx.x == 0) {
-        const unsigned t = __hip_atomic_fetch_add(counter + sh_zero, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = __hip_atomic_fetch_add(counter + zero, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (t == (unsigned)(splits - 1));
         if (is_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -405,24 +458,20 @@ DPX_D bool last_block_of(unsigned *counter, int splits, uint32_t zero)
 
 // The same with two levels of tickets, for outputs that many blocks share: atomics on one
 // address are served one at a time (about 10 ns each on MI355X, 5 us for 512 blocks that
-// finish together), so blocks draw their ticket from a counter per group of `tgroup` blocks
+// finish together), so blocks draw their ticket from a counter per group of RED_TGROUP blocks
 // and only the last block of a group draws from the output's counter.  `group_counters`
 // holds the groups of this output, RED_GROUP_PITCH words apart (separate cache lines).
 constexpr int RED_GROUP_PITCH = 32;
-DPX_D bool last_block_of_grouped(unsigned *counter, unsigned *group_counters, int split, int splits, int tgroup,
-                                 uint32_t zero)
+constexpr int RED_TGROUP_LOG2 = 5, RED_TGROUP = 1 << RED_TGROUP_LOG2;
+DPX_D bool last_block_of_grouped(unsigned *counter, unsigned *group_counters, int split, int splits, uint32_t zero)
 {
-    __shared__ unsigned sh_zero2;
     __shared__ int is_last2;
-    if (threadIdx.x == 0) sh_zero2 = 0;
-    __syncthreads();
-    atomicOr(&sh_zero2, zero);
     __syncthreads();
     if (threadIdx.x == 0) {
-        const int g = split / tgroup, ng = (splits + tgroup - 1) / tgroup;
-        const int in_g = (g == ng - 1) ? splits - g * tgroup : tgroup;
+        const int g = split >> RED_TGROUP_LOG2, ng = (splits + RED_TGROUP - 1) >> RED_TGROUP_LOG2;
+        const int in_g = (g == ng - 1) ? splits - g * RED_TGROUP : RED_TGROUP;
         unsigned *c1 = group_counters + (size_t)g * RED_GROUP_PITCH;
-        const unsigned t = __hip_atomic_fetch_add(c1 + sh_zero2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = __hip_atomic_fetch_add(c1 + zero, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         int last = 0;
         if (t == (unsigned)(in_g - 1)) {
             __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -452,23 +501,25 @@ constexpr size_t RED_COUNTER_BYTES = (RED_MAX_TICKETS + RED_MAX_GROUPS * RED_GRO
 DPX_D bool last_block_of_output(unsigned *counters, const RedLaunch &L, int64_t o, int split, uint32_t zero)
 {
     if (L.tgroup == 0) return last_block_of(counters + o, L.splits, zero);
-    const int ng = (L.splits + L.tgroup - 1) / L.tgroup;
+    const int ng = (L.splits + RED_TGROUP - 1) >> RED_TGROUP_LOG2;
     return last_block_of_grouped(counters + o, counters + RED_MAX_TICKETS + (o * ng) * RED_GROUP_PITCH, split,
-                                 L.splits, L.tgroup, zero);
+                                 L.splits, zero);
 }
 
 template <class P, bool CONTIG>
-__global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L, const typename P::In *src,
-                                                       typename P::Out *dst, Slot<typename P::Acc> *partial,
-                                                       const typename P::Aux *aux, unsigned *counters)
+__global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typename P::In *src, typename P::Out *dst,
+                                                       Slot<typename P::Acc> *partial, const typename P::Aux *aux,
+                                                       unsigned *counters, RedIndex ix)
 {
     using In = typename P::In;
     using Acc = typename P::Acc;
     constexpr int E = 16 / (int)sizeof(In);
     const int G = 1 << L.g_log2;
     const bool whole_block = G == (int)blockDim.x;
-    const int64_t oblock = (int64_t)blockIdx.x / L.splits;
-    const int split = (int)((int64_t)blockIdx.x - oblock * L.splits);
+    // (32-bit: the grid has fewer than 2^32 blocks)
+    const uint32_t ob32 = (L.splits == 1) ? blockIdx.x : blockIdx.x / (uint32_t)L.splits;
+    const int64_t oblock = ob32;
+    const int split = (int)(blockIdx.x - ob32 * (uint32_t)L.splits);
     const int lane = threadIdx.x & (G - 1);
     const int64_t o = whole_block ? oblock : oblock * (blockDim.x >> L.g_log2) + (threadIdx.x >> L.g_log2);
     const bool active = o < L.m;
@@ -479,7 +530,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedIndex ix, RedLaunch L
 
     int64_t so = 0, dof = 0, ao = 0;
     if (active) {
-        iter_offsets(ix, o, so, dof, ao);
+        iter_offsets(ix, L, o, so, dof, ao);
         Acc a = P::identity();
         if constexpr (P::has_aux) a = P::load_aux(aux + ao);
         const int64_t beg = (int64_t)split * L.chunk;
@@ -1045,15 +1096,17 @@ template <class T> DPX_D int64_t arg_result(const RedLaunch &L, int64_t idx, val
 // Position = index along the reduced run.  Linear block id = oblock * splits + split, lanes
 // per output as in red_rows_kernel; partial (value, position) pairs laid out [output][split].
 template <class T, bool IS_MAX, bool CONTIG>
-__global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst,
-                                                       Slot<T> *pval, Slot<int64_t> *pidx, unsigned *counters)
+__global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *src, int64_t *dst, Slot<T> *pval,
+                                                       Slot<int64_t> *pidx, unsigned *counters, RedIndex ix)
 {
     using VT = value_of_t<T>;
     constexpr int E = 16 / (int)sizeof(T);
     const int G = 1 << L.g_log2;
     const bool whole_block = G == (int)blockDim.x;
-    const int64_t oblock = (int64_t)blockIdx.x / L.splits;
-    const int split = (int)((int64_t)blockIdx.x - oblock * L.splits);
+    // (32-bit: the grid has fewer than 2^32 blocks)
+    const uint32_t ob32 = (L.splits == 1) ? blockIdx.x : blockIdx.x / (uint32_t)L.splits;
+    const int64_t oblock = ob32;
+    const int split = (int)(blockIdx.x - ob32 * (uint32_t)L.splits);
     const int lane = threadIdx.x & (G - 1);
     const int64_t o = whole_block ? oblock : oblock * (blockDim.x >> L.g_log2) + (threadIdx.x >> L.g_log2);
     const bool active = o < L.m;
@@ -1062,7 +1115,7 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedIndex ix, RedLaunch L
     int64_t bidx = ARG_NONE;
     int64_t so = 0, dof = 0, ao = 0;
     if (active) {
-        iter_offsets(ix, o, so, dof, ao);
+        iter_offsets(ix, L, o, so, dof, ao);
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         const T *p = src + so;

@@ -107,10 +107,10 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     }
     else if (pl.path == DPX_PATH_RED_GENERIC)
         hipLaunchKernelGGL((red_rows_kernel<P, false>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
-                           pl.ix, pl.L, sp, dp, partial, ap, counters);
+                           pl.L, sp, dp, partial, ap, counters, pl.ix);
     else
-        hipLaunchKernelGGL((red_rows_kernel<P, true>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.ix,
-                           pl.L, sp, dp, partial, ap, counters);
+        hipLaunchKernelGGL((red_rows_kernel<P, true>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.L,
+                           sp, dp, partial, ap, counters, pl.ix);
     return red_launch_status(pl, stream, "reduction launch");
 }
 
@@ -143,10 +143,10 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
                            sp, dp, pval, pidx, counters);
     else if (pl.path == DPX_PATH_RED_GENERIC)
         hipLaunchKernelGGL((arg_rows_kernel<T, IS_MAX, false>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
-                           pl.ix, pl.L, sp, dp, pval, pidx, counters);
+                           pl.L, sp, dp, pval, pidx, counters, pl.ix);
     else
         hipLaunchKernelGGL((arg_rows_kernel<T, IS_MAX, true>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
-                           pl.ix, pl.L, sp, dp, pval, pidx, counters);
+                           pl.L, sp, dp, pval, pidx, counters, pl.ix);
     return red_launch_status(pl, stream, "search launch");
 }
 

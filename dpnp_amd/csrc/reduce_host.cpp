@@ -134,6 +134,10 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         ix.shape_r[d] = d < nd_r ? rshape[d] : 1;
         ix.src_rstr[d] = d < nd_r ? rstr[0][d] : 0;
     }
+    pl.L.nd_i1 = nd_i == 1 ? 1 : 0;
+    pl.L.istr0 = istr[0][0];
+    pl.L.astr0 = istr[1][0];
+    pl.L.dstr0 = istr[2][0];
     pl.src_off = ioff[0] + roff[0];
     pl.aux_off = ioff[1];
     pl.dst_off = ioff[2];
