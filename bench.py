@@ -177,7 +177,9 @@ def build_workload(name, dpnp, torch):
                 8 * h + 4 * (side // 2), h),
                ("where_greater_two_calls", where_unfused, (4 + 1) * h + (1 + 4 + 4) * h + 4 * (side // 2), h),
                ("bitwise_and", lambda: dpnp.bitwise_and(ints[0], ints[1], out=o_i), 12 * 2 * h, 2 * h),
-               ("bitwise_and_V1", lambda: dpnp.bitwise_and(ints[0][:, ::2], ints[1][:, ::2], out=o_ih), 12 * h, h)]
+               ("bitwise_and_V1", lambda: dpnp.bitwise_and(ints[0][:, ::2], ints[1][:, ::2], out=o_ih), 12 * h, h),
+               # plain copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters (--ops ...,copy)
+               ("copy", lambda: dpnp.copyto(o_i, ints[0]), 8 * 2 * h, 2 * h)]
         return ops, "f32/i32/bool", "synthetic (seeded normal(0,1), uniform int32, resident in HBM)"
     if name == "cfg5":
         n = 1 << 26

@@ -50,7 +50,7 @@ REDUCE_ID = {n: i for i, n in enumerate(REDUCE_OPS)}
 SEARCH_ID = {n: i for i, n in enumerate(SEARCH_OPS)}
 
 PATH_NAMES = {
-    0: "noop", 1: "ew_contig", 2: "ew_rows", 4: "ew_tile",
+    0: "noop", 1: "ew_contig", 2: "ew_rows", 3: "ew_rows2", 4: "ew_tile",
     10: "red_rows", 11: "red_rows_split", 12: "red_cols", 13: "red_cols_split",
     14: "red_generic", 15: "red_small", 16: "red_flat", 17: "red_short_rows",
 }

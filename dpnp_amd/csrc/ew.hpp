@@ -172,13 +172,17 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_contig_kernel(Fn fn, int64_t n, u
 // without holes) and the lanes then pull the two packs that hold their elements from their
 // neighbours' registers.  All 64 lanes of the wave must make the call.  Measured on MI355X
 // against two loads at a 32-byte lane pitch: 6.4 vs 5.9 TB/s of physical traffic.
-template <class T, int E> DPX_D pack<T, E> load_stride2_wave(const T *lane_ptr)
+template <class T, int E> DPX_D void stride2_wave_issue(const T *lane_ptr, u32x4 &a, u32x4 &b)
+{
+    const int lane = threadIdx.x & 63;
+    const T *wp = lane_ptr - (int64_t)lane * 2 * E;
+    a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + lane * E));
+    b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + (64 + lane) * E));
+}
+template <class T, int E> DPX_D pack<T, E> stride2_wave_regroup(const u32x4 &a, const u32x4 &b)
 {
     static_assert(E >= 2 && sizeof(T) * E == 16);
     const int lane = threadIdx.x & 63;
-    const T *wp = lane_ptr - (int64_t)lane * 2 * E;
-    const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + lane * E));
-    const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wp + (64 + lane) * E));
     const int s = (2 * lane) & 63;
     const bool first = lane < 32;
     union {
@@ -200,6 +204,14 @@ template <class T, int E> DPX_D pack<T, E> load_stride2_wave(const T *lane_ptr)
 #pragma unroll
     for (int e = 0; e < E; ++e) r.v[e] = (2 * e < E) ? lo.p.v[(2 * e) % E] : hi.p.v[(2 * e) % E];
     return r;
+}
+// issue and regroup are separate so that a thread can have the loads of several rows in flight
+// before the first shuffle waits for data
+template <class T, int E> DPX_D pack<T, E> load_stride2_wave(const T *lane_ptr)
+{
+    u32x4 a, b;
+    stride2_wave_issue<T, E>(lane_ptr, a, b);
+    return stride2_wave_regroup<T, E>(a, b);
 }
 
 // ---- strided, vectorised along the inner dimension -----------------------------
@@ -314,6 +326,140 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_rows_kernel(Fn fn,
 {
     ew_rows_body<Fn, Out, Ins...>(fn, ix, out, in, modes, tx_log2, nrows, col_blocks,
                                   std::index_sequence_for<Ins...>{});
+}
+
+// ---- two rows per thread, the way each input is read fixed at compile time --------------------
+// The kernel for calls with a stride-2 input (x[:, ::2], the real or imaginary parts of a complex
+// array) whose rows are whole waves of packs: A[:, ::2] * row, exp(A[:, ::2]), where(mask, A[:, ::2], row),
+// I[:, ::2] & J[:, ::2].  Such a call moves twice the bytes through the vector memory pipeline that
+// it uses (every 64-byte line of the base array is fetched for half of its elements), and at one
+// row per thread the loads of a row operand cost as much of that pipeline as the output does: on
+// MI355X the pipeline, not HBM, then bounds the kernel (fp32 A[:, ::2] * row, 8192 x 4096 outputs:
+// 73.6 us at one row per thread, 61.3 us at two with the row operand loaded once; HBM time of the
+// 403 MB it moves: 50 us).  The rows kernel above decides how to read each operand at run time,
+// and the branches that takes between its loads keep the compiler from issuing them together, so
+// here the reading is part of the kernel's type:
+//   PAT, 2 bits per input: RC_ROWS  contiguous along the inner dim, moves with the rows: one
+//                                   16-byte (or narrower) pack per row;
+//                          RC_S2    stride 2 along the inner dim: wave-interleaved loads, see
+//                                   stride2_wave_issue;
+//                          RC_ONCE  does not move along dim inner - 1 (a row vector, or a scalar
+//                                   when it does not move along the inner dim either: bit k of
+//                                   `scalar`): loaded once for both rows.
+// A thread owns E consecutive outputs of two neighbouring rows (dim inner - 1, extent even); every
+// wave lies inside one row and has 64 full packs (the host checks ncols % (64 E) == 0); the output
+// is contiguous along the inner dim.  Wave-interleaved loads read one element past the last one a
+// wave uses: the wave that ends the last row of the iteration space reads element by element instead.
+enum : int { RC_ROWS = 0, RC_S2 = 1, RC_ONCE = 2 };
+template <class T> using raw_pair_t = std::pair<u32x4, u32x4>; // the two loads of a stride-2 input
+constexpr int rc_of(int pat, int k) { return (pat >> (2 * k)) & 3; }
+
+template <int PAT, class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_rows2_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out *out,
+                         const InPtrs<sizeof...(Ins)> &in, uint32_t scalar, uint32_t waves_per_row,
+                         int64_t npairs, std::index_sequence<I...>)
+{
+    constexpr int N = sizeof...(Ins);
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * ((int)blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t pair = wave / waves_per_row; // (uniform over the wave)
+    if (pair >= npairs) return;
+    const uint32_t cw = (uint32_t)(wave - pair * waves_per_row);
+    const int inner = ix.nd - 1;
+    const int64_t col0 = ((int64_t)cw * 64 + lane) * E;
+    int64_t off[N + 1];
+#pragma unroll
+    for (int k = 0; k <= N; ++k) off[k] = col0 * ix.strides[k][inner];
+    {
+        int64_t r = pair * 2;
+        for (int d = inner - 1; d >= 0; --d) {
+            const int64_t q = (d == 0) ? 0 : r / ix.shape[d];
+            const int64_t i = r - q * ix.shape[d];
+#pragma unroll
+            for (int k = 0; k <= N; ++k) off[k] += i * ix.strides[k][d];
+            r = q;
+        }
+    }
+    int64_t rstep[N + 1];
+#pragma unroll
+    for (int k = 0; k <= N; ++k) rstep[k] = ix.strides[k][inner - 1];
+
+    if (pair == npairs - 1 && cw == waves_per_row - 1) {
+        // the wave that ends the last row: no read past its last element
+        for (int j = 0; j < 2; ++j)
+            for (int e = 0; e < E; ++e)
+                out[off[N] + j * rstep[N] + e] = to_storage<Out>(fn(to_value(
+                    load_one((const Ins *)in.p[I] + off[I] + j * rstep[I] + e * ix.strides[I][inner]))...));
+        return;
+    }
+    // every load of the thread, then the results
+    std::tuple<pack<Ins, E>...> v0, v1;    // RC_ROWS, and RC_ONCE in v0
+    std::tuple<raw_pair_t<Ins>...> w0, w1; // RC_S2 (the tuple has an entry per input; unused ones vanish)
+    auto issue_rows = [&](auto &v, auto &w, auto *p, int64_t o, int rc) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        if (rc == RC_ROWS) v = load_pack<T, E>(p + o);
+        else if (rc == RC_S2) {
+            if constexpr (E >= 2 && sizeof(T) * E == 16) stride2_wave_issue<T, E>(p + o, w.first, w.second);
+        }
+    };
+    (issue_rows(std::get<I>(v0), std::get<I>(w0), (const Ins *)in.p[I], off[I], rc_of(PAT, (int)I)), ...);
+    (issue_rows(std::get<I>(v1), std::get<I>(w1), (const Ins *)in.p[I], off[I] + rstep[I], rc_of(PAT, (int)I)), ...);
+    auto issue_once = [&](auto &v, auto *p, int64_t o, int rc, bool is_scalar) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        if (rc == RC_ONCE) v = is_scalar ? splat<T, E>(load_one(p + o)) : load_pack<T, E, false>(p + o);
+    };
+    (issue_once(std::get<I>(v0), (const Ins *)in.p[I], off[I], rc_of(PAT, (int)I), (scalar >> I) & 1u), ...);
+    auto value = [&](auto &v_first, auto &v_this, auto &w, auto *p, int rc) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        if constexpr (E >= 2 && sizeof(T) * E == 16) {
+            if (rc == RC_S2) return stride2_wave_regroup<T, E>(w.first, w.second);
+        }
+        return rc == RC_ONCE ? v_first : v_this;
+    };
+    auto produce = [&](std::tuple<pack<Ins, E>...> &v, std::tuple<raw_pair_t<Ins>...> &w, int64_t o) {
+        std::tuple<pack<Ins, E>...> x;
+        ((std::get<I>(x) = value(std::get<I>(v0), std::get<I>(v), std::get<I>(w), (const Ins *)in.p[I],
+                                 rc_of(PAT, (int)I))),
+         ...);
+        (keep_whole(std::get<I>(x)), ...);
+        pack<Out, E> r;
+#pragma unroll
+        for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(x).v[e])...));
+        store_pack<Out, E>(out + o, r);
+    };
+    produce(v0, w0, off[N]);
+    produce(v1, w1, off[N] + rstep[N]);
+}
+
+template <int PAT, class Fn, class Out, class... Ins>
+__global__ __launch_bounds__(EW_BLOCK) void ew_rows2_kernel(Fn fn, NdIndex<sizeof...(Ins) + 1> ix, Out *out,
+                                                           InPtrs<sizeof...(Ins)> in, uint32_t scalar,
+                                                           uint32_t waves_per_row, int64_t npairs)
+{
+    ew_rows2_body<PAT, Fn, Out, Ins...>(fn, ix, out, in, scalar, waves_per_row, npairs,
+                                        std::index_sequence_for<Ins...>{});
+}
+
+// Functors whose calls may take ew_rows2_kernel (each pattern is one more kernel per functor and
+// element type, so the list is short): specialised next to the functors' definitions.
+template <class Fn> struct rows2_enabled : std::false_type {};
+// the patterns instantiated for N inputs
+template <int N> struct rows2_patterns {
+    using seq = std::integer_sequence<int>;
+};
+template <> struct rows2_patterns<1> {
+    using seq = std::integer_sequence<int, RC_S2>;
+};
+template <> struct rows2_patterns<2> {
+    using seq = std::integer_sequence<int, RC_S2 | RC_S2 << 2, RC_S2 | RC_ONCE << 2, RC_ONCE | RC_S2 << 2>;
+};
+template <> struct rows2_patterns<3> { // where(mask, x[:, ::2], row); where(x[:, ::2] > scalar, x[:, ::2], row) fused
+    using seq = std::integer_sequence<int, RC_ROWS | RC_S2 << 2 | RC_ONCE << 4, RC_S2 | RC_ONCE << 2 | RC_ONCE << 4>;
+};
+template <class F, int... P> inline void for_each_pattern(F &&f, std::integer_sequence<int, P...>)
+{
+    (f(std::integral_constant<int, P>{}), ...);
 }
 
 // ---- transposing through an LDS tile ------------------------------------------------------
@@ -506,6 +652,12 @@ struct EwPlan {
     int tx_log2;
     int block; // threads per block
     int64_t nrows, col_blocks, grid;
+    // ew_rows2_kernel (pattern >= 0): the way each input is read, inputs that are scalars along the
+    // inner dim, waves per row, row pairs
+    int rows2_pat;
+    uint32_t rows2_scalar, rows2_waves;
+    int rows2_wpb; // waves per block
+    int64_t rows2_pairs;
     // tile path
     uint32_t tmask; // inputs staged through LDS
     int dT;         // the dim those inputs are contiguous along
@@ -539,6 +691,15 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
         }
     }
     ew_finish_plan(pl, E, ew_packs_per_thread<Fn, Out, Ins...>(), sizes, ptrs);
+    if constexpr (rows2_enabled<Fn>::value && E >= 2 && E <= 4 && N >= 1 && N <= 3) {
+        // a call that fits the two-rows kernel in a pattern this functor is instantiated for
+        if (pl.path == DPX_PATH_EW_ROWS && pl.rows2_pat >= 0)
+            for_each_pattern(
+                [&](auto pat_c) {
+                    if (pl.rows2_pat == decltype(pat_c)::value) pl.path = DPX_PATH_EW_ROWS2;
+                },
+                typename rows2_patterns<N>::seq{});
+    }
     if (pl.path == DPX_PATH_NOOP || dry) return hipSuccess;
     InPtrs<N> in;
     for (int k = 0; k < N; ++k) in.p[k] = ptrs[k];
@@ -563,6 +724,22 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
                                    pl.tiles_i);
             }
             return hipGetLastError();
+        }
+        if constexpr (rows2_enabled<Fn>::value && E >= 2 && E <= 4 && N >= 1 && N <= 3) {
+            if (pl.path == DPX_PATH_EW_ROWS2) {
+                // one wave per block, like the contiguous kernel: waves are independent here
+                const int wpb = pl.rows2_wpb;
+                const unsigned grid = (unsigned)((pl.rows2_pairs * pl.rows2_waves + wpb - 1) / wpb);
+                for_each_pattern(
+                    [&](auto pat_c) {
+                        constexpr int PAT = decltype(pat_c)::value;
+                        if (pl.rows2_pat == PAT)
+                            hipLaunchKernelGGL((ew_rows2_kernel<PAT, Fn, Out, Ins...>), dim3(grid), dim3(64 * wpb), 0,
+                                               stream, fn, ix, out, in, pl.rows2_scalar, pl.rows2_waves, pl.rows2_pairs);
+                    },
+                    typename rows2_patterns<N>::seq{});
+                return hipGetLastError();
+            }
         }
         hipLaunchKernelGGL((ew_rows_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid),
                            dim3(pl.block), 0, stream, fn, ix, out, in, pl.modes, pl.tx_log2,

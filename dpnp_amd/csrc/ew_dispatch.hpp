@@ -38,5 +38,7 @@ template <class Op, class T> struct UnaryFn {
 template <class Op, class T> struct BinaryFn {
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
 };
+template <class Op, class T> struct rows2_enabled<UnaryFn<Op, T>> : std::true_type {};
+template <class Op, class T> struct rows2_enabled<BinaryFn<Op, T>> : std::true_type {};
 
 } // namespace dpx

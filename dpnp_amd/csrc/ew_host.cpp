@@ -51,6 +51,10 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     pl.period = 1;
     pl.bcast = pl.modes = 0;
     pl.tx_log2 = 0;
+    pl.rows2_pat = -1;
+    pl.rows2_scalar = pl.rows2_waves = 0;
+    pl.rows2_pairs = 0;
+    pl.rows2_wpb = 1;
     pl.block = EW_CONTIG_BLOCK;
     pl.nrows = pl.col_blocks = pl.grid = 0;
     for (int k = 0; k < 5; ++k) pl.offsets[k] = 0;
@@ -163,6 +167,27 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
         pl.grid = (pl.n + (int64_t)pl.block * E * U - 1) / ((int64_t)pl.block * E * U);
         return;
     }
+    // A one-dimensional call with a stride-2 input (A[:, ::2] of a contiguous matrix with rows of
+    // even length collapses to one): cut it into rows of one wave of packs, which is what
+    // ew_rows2_kernel works on.
+    if (pl.path == DPX_PATH_EW_ROWS && pl.nd == 1 && E >= 2 && pl.strides[nops - 1][0] == 1) {
+        const int64_t C = 64 * (int64_t)E;
+        bool s2 = false, ok = pl.n % (2 * C) == 0;
+        for (int k = 0; k + 1 < nops && ok; ++k) {
+            const int64_t st = pl.strides[k][0];
+            if (st == 2 && itemsize[k] * E == 16) s2 = true;
+            else ok = st == 0 || st == 1;
+        }
+        if (ok && s2) {
+            pl.nd = 2;
+            pl.shape[0] = pl.n / C;
+            pl.shape[1] = C;
+            for (int k = 0; k < nops; ++k) {
+                pl.strides[k][1] = pl.strides[k][0];
+                pl.strides[k][0] = C * pl.strides[k][1];
+            }
+        }
+    }
     const int inner = pl.nd - 1;
     if (pl.path == DPX_PATH_EW_TILE) {
         // tile = 64 positions along dT x (512 bytes / widest itemsize) positions along the inner dim
@@ -208,6 +233,42 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     const int64_t tx = (int64_t)1 << lg, ty = pl.block / tx;
     pl.col_blocks = (per_row + tx - 1) / tx;
     pl.grid = pl.col_blocks * ((pl.nrows + ty - 1) / ty);
+    // Does the call fit ew_rows2_kernel?  Rows of whole waves of packs, an even number of them along
+    // dim inner - 1, a contiguous output, and every input one of: stride 2 along the inner dim
+    // (elements as wide as a pack allows), contiguous and moving with the rows, or the same for
+    // every row (a row vector or a scalar).
+    pl.rows2_pat = -1;
+    if (E >= 2 && pl.nd >= 2 && pl.strides[nops - 1][inner] == 1 && pl.shape[inner - 1] % 2 == 0 &&
+        ncols % (64 * (int64_t)E) == 0 && nops - 1 <= 3 && tune_int("DPX_EW_ROWS2", 1) != 0) {
+        int pat = 0;
+        uint32_t scalar = 0;
+        bool any_s2 = false;
+        for (int k = 0; k + 1 < nops && pat >= 0; ++k) {
+            const int64_t si = pl.strides[k][inner], sr = pl.strides[k][inner - 1];
+            int rc = -1;
+            if (si == 2 && itemsize[k] * E == 16) {
+                rc = RC_S2;
+                any_s2 = true;
+                // the wave-wide reads go one element past a row's last: only the row at the highest
+                // address may not, and that is the last row when no stride is negative
+                for (int d = 0; d < inner; ++d)
+                    if (pl.strides[k][d] < 0) rc = -1;
+            }
+            else if (si == 1 && sr != 0) rc = RC_ROWS;
+            else if ((si == 1 || si == 0) && sr == 0) {
+                rc = RC_ONCE;
+                if (si == 0) scalar |= 1u << k;
+            }
+            pat = rc < 0 ? -1 : (pat | rc << (2 * k));
+        }
+        if (pat >= 0 && any_s2) {
+            pl.rows2_pat = pat;
+            pl.rows2_scalar = scalar;
+            pl.rows2_waves = (uint32_t)(ncols / (64 * (int64_t)E));
+            pl.rows2_pairs = pl.nrows / 2;
+            pl.rows2_wpb = tune_int("DPX_EW_ROWS2_WAVES", 1) == 4 ? 4 : 1; // sweep override, product build: 1
+        }
+    }
 }
 
 void ew_export_plan(const EwPlan &pl, dpx_plan *out)

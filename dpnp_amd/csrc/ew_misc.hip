@@ -10,6 +10,8 @@ template <class C, class S> struct WhereFn {
     DPX_D S operator()(V<C> c, S a, S b) const { return convert<bool_t, C>(to_storage<C>(c)).v ? a : b; }
 };
 
+template <class S> struct rows2_enabled<WhereFn<bool_t, S>> : std::true_type {};
+
 template <class F> static bool for_size_class(int bytes, F &&f)
 {
     switch (bytes) {
@@ -51,6 +53,8 @@ template <class Cmp, class T, class S> struct WhereCmpFn {
 template <class Cmp, class T> struct WhereCmpSelfFn {
     DPX_D T operator()(T x, T r, T b) const { return Cmp::template apply<T>(x, r) ? x : b; }
 };
+
+template <class Cmp, class T> struct rows2_enabled<WhereCmpSelfFn<Cmp, T>> : std::true_type {};
 
 static int where_compare_call(int cmp_op, const dpx_array_view *lhs, const dpx_array_view *rhs,
                               const dpx_array_view *x1, const dpx_array_view *x2,
