@@ -183,7 +183,17 @@ def test_elementwise_plans():
     # config 4: strided x broadcast row
     p = plan_binary("multiply", view([8192, 4096], [8192, 2]), view([8192, 4096], [0, 1], ptr=P1),
                     view([8192, 4096], ptr=P2))
-    assert L.PATH_NAMES[p.path] == "ew_rows" and p.nd == 2 and list(p.shape[:2]) == [8192, 4096]
+    assert L.PATH_NAMES[p.path] == "ew_rows2" and p.nd == 2 and list(p.shape[:2]) == [8192, 4096]
+    # the same with an odd number of rows, or rows that are no multiple of a wave's 256 floats: the general kernel
+    p = plan_binary("multiply", view([8191, 4096], [8192, 2]), view([8191, 4096], [0, 1], ptr=P1),
+                    view([8191, 4096], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"
+    p = plan_binary("multiply", view([8192, 4000], [8192, 2]), view([8192, 4000], [0, 1], ptr=P1),
+                    view([8192, 4000], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows"
+    # a 1-D stride-2 view is cut into rows for the same kernel
+    p = plan_binary("add", view([1 << 20], [2]), view([1 << 20], [2], ptr=P1), view([1 << 20], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows2" and p.nd == 2
     # a matrix with short rows and a row / a column: the contiguous kernel walks it flat
     p = plan_binary("subtract", view([100000, 17]), view([100000, 17], [0, 1], ptr=P1), view([100000, 17], ptr=P2))
     assert L.PATH_NAMES[p.path] == "ew_contig" and p.nd == 2 and p.grid[0] == -(-100000 * 17 // 256)

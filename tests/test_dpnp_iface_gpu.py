@@ -128,8 +128,38 @@ def test_black_scholes_entry_point():
     d1, d2 = 0.5 + 0.5 * dpnp.erf(w1), 0.5 + 0.5 * dpnp.erf(w2)
     Se = dpnp.exp(b) * S
     r = P * d1 - Se * d2
-    assert_same(call.asnumpy(), r.asnumpy())  # fused == unfused, bit for bit
-    assert_same(put.asnumpy(), (r - P + Se).asnumpy())
+    # fused against unfused: the fused kernel's own elementary functions are each good to an ULP of
+    # their result, which the difference of the two products turns into a few ULP of the larger one
+    scale = np.maximum(p, s)
+    assert np.all(np.abs(call.asnumpy() - r.asnumpy()) <= 8 * np.finfo("f8").eps * scale)
+    assert np.all(np.abs(put.asnumpy() - (r - P + Se).asnumpy()) <= 8 * np.finfo("f8").eps * scale)
+    # inputs the short routines do not take (zero, negative, subnormal, infinite, NaN, huge maturities)
+    # go through the long ones and give what the chain gives, bit for bit
+    bad = np.array([0.0, -1.0, 5e-324, np.inf, np.nan, 30.0, 30.0, 30.0])
+    pb, sb, tb = np.full(8, 30.0), np.full(8, 25.0), np.full(8, 1.5)
+    pb[:5] = bad[:5]
+    sb[5], tb[6], tb[7] = 0.0, np.nan, 1e300
+    for arr in (pb, sb, tb):
+        assert arr.shape == (8,)
+    cb, qb = dpnp.black_scholes(dpnp.array(pb), dpnp.array(sb), dpnp.array(tb), 0.1, 0.2)
+    with np.errstate(all="ignore"):
+        wc, wp = orc.black_scholes(pb, sb, tb, 0.1, 0.2)
+    fin = np.isfinite(wc)
+    assert np.array_equal(np.isnan(cb.asnumpy()), np.isnan(wc)) and np.array_equal(np.isnan(qb.asnumpy()), np.isnan(wp))
+    np.testing.assert_allclose(cb.asnumpy()[fin], wc[fin], rtol=1e-12, atol=1e-12)
+    # the same inputs scattered over full chunks of the long array: their waves take the long routines,
+    # the other waves the short ones
+    where = np.array([3, 1000, 4100, 8191, 8200, 2047, 6000, 10006])
+    p2, s2, t2 = p.copy(), s.copy(), t.copy()
+    p2[where], s2[where], t2[where] = pb, sb, tb
+    c2, q2 = dpnp.black_scholes(dpnp.array(p2), dpnp.array(s2), dpnp.array(t2), 0.1, 0.2)
+    with np.errstate(all="ignore"):
+        wc, wp = orc.black_scholes(p2, s2, t2, 0.1, 0.2)
+    for got, want in ((c2.asnumpy(), wc), (q2.asnumpy(), wp)):
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+        np.testing.assert_allclose(got[fin], want[fin], rtol=1e-12, atol=1e-12)
 
 
 # ---- dpnp-level functions built on the ufunc extension kernels ---------------------------------
