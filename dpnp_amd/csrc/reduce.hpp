@@ -429,8 +429,10 @@ template <class T> DPX_D T slot_read(const Slot<T> *p)
         Slot<T> s;
         T t;
     } u;
+    // atomic loads like the exchanges that wrote the words: served where those were performed
 #pragma unroll
-    for (int i = 0; i < Slot<T>::W; ++i) u.s.w[i] = p->w[i];
+    for (int i = 0; i < Slot<T>::W; ++i)
+        u.s.w[i] = __hip_atomic_load(&p->w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return u.t;
 }
 
