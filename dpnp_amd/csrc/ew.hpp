@@ -18,6 +18,7 @@
 //   * strided kernels keep threads adjacent along the innermost output
 //     dimension and pay one div/mod chain per thread, not per element.
 #pragma once
+#include <atomic>
 #include <tuple>
 #include <utility>
 #include "types.hpp"
@@ -474,8 +475,11 @@ template <class F, int... P> inline void for_each_pattern(F &&f, std::integer_se
 // batch dims decoded from the block index.  Measured on MI355X for exp(A.T) -> C-contiguous,
 // 8192 x 8192 floats: 5.8 TB/s; 64 x 64 tiles with 4-byte accesses 4.2 TB/s.
 // modes: as for the rows kernel; for a flagged input MODE_VEC allows the 16-byte phase-1 reads.
+constexpr int EW_TILE_BLOCK = 512;
+constexpr size_t EW_TILE_LDS_MAX = 160 * 1024;
+constexpr int ew_tile_ti(int widest_itemsize) { return widest_itemsize <= 4 ? 128 : 64; }
 template <class Out, class... Ins> struct tile_traits {
-    static constexpr int TI = 64;
+    static constexpr int TI = ew_tile_ti(max_sizeof<Out, Ins...>());
     static constexpr int TJ = 512 / max_sizeof<Out, Ins...>();
     template <class T> static constexpr int pitch() { return TI + (sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T)); }
     template <class T> static constexpr size_t bytes() { return ((size_t)TJ * pitch<T>() * sizeof(T) + 15) & ~(size_t)15; }
@@ -500,26 +504,31 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     constexpr int E = ew_traits<Out, Ins...>::E;
     constexpr int TI = TT::TI, TJ = TT::TJ;
     const int inner = ix.nd - 1;
-    int64_t b = blockIdx.x;
-    const int64_t ti = b % tiles_i;
-    b /= tiles_i;
+    // the grid has fewer than 2^32 blocks, so every quotient below fits 32 bits (64-bit
+    // division is a long routine on this hardware)
+    uint32_t b = blockIdx.x;
+    const uint32_t nti = (uint32_t)tiles_i, ntt = (uint32_t)tiles_t;
+    const uint32_t ti = b % nti;
+    b /= nti;
     // diagonal order: consecutive blocks step along both tile axes, so neither the reads
     // (strided along `inner`) nor the writes (strided along dT) of the blocks in flight pile
     // up on the memory channels one power-of-two stride selects
-    const int64_t tt = (b % tiles_t + ti) % tiles_t;
-    b /= tiles_t;
+    uint32_t tt = b % ntt + ti % ntt;
+    tt = tt >= ntt ? tt - ntt : tt;
+    b /= ntt;
     int64_t off[N + 1];
 #pragma unroll
     for (int k = 0; k <= N; ++k) off[k] = 0;
-    for (int d = inner - 1; d >= 0; --d) {
+    for (int d = inner - 1; d >= 0 && b != 0; --d) {
         if (d == dT) continue;
-        const int64_t q = b / ix.shape[d];
-        const int64_t i = b - q * ix.shape[d];
+        const uint32_t extent = ix.shape[d] > 0xffffffffll ? 0xffffffffu : (uint32_t)ix.shape[d];
+        const uint32_t q = b / extent;
+        const uint32_t i = b - q * extent;
 #pragma unroll
-        for (int k = 0; k <= N; ++k) off[k] += i * ix.strides[k][d];
+        for (int k = 0; k <= N; ++k) off[k] += (int64_t)i * ix.strides[k][d];
         b = q;
     }
-    const int64_t i0 = tt * TI, j0 = ti * TJ;
+    const int64_t i0 = (int64_t)tt * TI, j0 = (int64_t)ti * TJ;
     const int64_t ni = ix.shape[dT], nj = ix.shape[inner];
     // rows / columns of this tile that exist
     const int ci = (ni - i0 < TI) ? (int)(ni - i0) : TI;
@@ -530,6 +539,7 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         ((lds_off[I] = acc, acc += ((tmask >> I) & 1u) ? TT::template bytes<Ins>() : 0), ...);
         lds_off[N] = acc;
     }
+    const bool full = ci == TI && cj == TJ;
     // phase 1: transposed inputs -> LDS, threads adjacent along dT
     auto stage = [&](auto *p, int k, size_t l_off) {
         using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
@@ -537,7 +547,7 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         constexpr int S = TT::template pitch<T>();
         constexpr int VE = 16 / (int)sizeof(T);      // elements per 16-byte access
         constexpr int VPR = TI / VE;                 // accesses per tile row
-        constexpr int RPP = EW_BLOCK / VPR;          // tile rows per pass
+        constexpr int RPP = EW_TILE_BLOCK / VPR;          // tile rows per pass
         constexpr int PASSES = (TJ + RPP - 1) / RPP;
         T *tile = reinterpret_cast<T *>(smem + l_off);
         const int64_t sj = ix.strides[k][inner];
@@ -547,6 +557,17 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
             const bool col_ok = lv * VE < ci;
             const bool whole = lv * VE + VE <= ci; // else: the pack that holds the end of dim dT
             pack<T, VE> m[PASSES];
+            if (TJ % RPP == 0 && full) {
+                // a whole tile, covered by whole passes: nothing to check, all loads in flight before
+                // the first LDS write
+#pragma unroll
+                for (int q = 0; q < PASSES; ++q) m[q] = load_pack<T, VE>(base + (q * RPP + lr) * sj + lv * VE);
+#pragma unroll
+                for (int q = 0; q < PASSES; ++q)
+#pragma unroll
+                    for (int e = 0; e < VE; ++e) tile[(q * RPP + lr) * S + lv * VE + e] = m[q].v[e];
+                return;
+            }
 #pragma unroll
             for (int q = 0; q < PASSES; ++q) {
                 const int r = q * RPP + lr;
@@ -571,14 +592,14 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         else {
             const int lo = threadIdx.x % TI, hi = threadIdx.x / TI;
             if (lo < ci)
-                for (int r = hi; r < cj; r += EW_BLOCK / TI) tile[r * S + lo] = load_one(base + r * sj + lo);
+                for (int r = hi; r < cj; r += EW_TILE_BLOCK / TI) tile[r * S + lo] = load_one(base + r * sj + lo);
         }
     };
     (stage((const Ins *)in.p[I], (int)I, lds_off[I]), ...);
     __syncthreads();
     // phase 2: compute, threads adjacent along the inner dim
     constexpr int CPR = TJ / E;         // packs per tile row (32)
-    constexpr int RPP2 = EW_BLOCK / CPR; // tile rows per pass (8)
+    constexpr int RPP2 = EW_TILE_BLOCK / CPR; // tile rows per pass (16)
     const int lc = threadIdx.x % CPR, lr = threadIdx.x / CPR;
     const int jj = lc * E;
     if (jj >= cj) return;
@@ -607,6 +628,33 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         return r;
     };
     const bool out_vec = ((modes >> (2 * N)) & 3u) == MODE_VEC && cnt == E;
+    if (full && out_vec && tmask == (1u << N) - 1u) {
+        // a whole tile with every input in LDS (exp(A.T), A.T + B.T): no case to tell apart per
+        // row, so the rows are unrolled and the LDS reads of one row overlap the arithmetic of
+        // the row before
+        static_assert(TI % RPP2 == 0, "passes cover the tile exactly");
+        Out *q = out + col[N] + lr * ix.strides[N][dT];
+        const int64_t qstep = RPP2 * ix.strides[N][dT];
+#pragma unroll
+        for (int it = 0; it < TI / RPP2; ++it) {
+            const int i = it * RPP2 + lr;
+            std::tuple<pack<Ins, E>...> v;
+            auto gather = [&](auto &dstp, size_t l_off) {
+                using T = std::remove_cv_t<std::remove_reference_t<decltype(dstp.v[0])>>;
+                constexpr int S = TT::template pitch<T>();
+                const T *tile = reinterpret_cast<const T *>(smem + l_off);
+#pragma unroll
+                for (int e = 0; e < E; ++e) dstp.v[e] = tile[(jj + e) * S + i];
+            };
+            (gather(std::get<I>(v), lds_off[I]), ...);
+            pack<Out, E> r;
+#pragma unroll
+            for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+            store_pack<Out, E>(q, r);
+            q += qstep;
+        }
+        return;
+    }
 #pragma unroll 2
     for (int i = lr; i < ci; i += RPP2) {
         std::tuple<pack<Ins, E>...> v;
@@ -625,7 +673,7 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
 }
 
 template <class Fn, class Out, class... Ins>
-__global__ __launch_bounds__(EW_BLOCK) void ew_tile_kernel(Fn fn, NdIndex<sizeof...(Ins) + 1> ix, Out *out,
+__global__ __launch_bounds__(EW_TILE_BLOCK) void ew_tile_kernel(Fn fn, NdIndex<sizeof...(Ins) + 1> ix, Out *out,
                                                           InPtrs<sizeof...(Ins)> in, uint32_t tmask, uint32_t modes,
                                                           int dT, int64_t tiles_t, int64_t tiles_i)
 {
@@ -684,8 +732,8 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
         ptrs[k] = (const char *)views[k]->data + pl.offsets[k] * sizes[k];
     if constexpr (N >= 1) {
         if (pl.path == DPX_PATH_EW_TILE) {
-            // a block's tiles must fit 64 KiB of LDS: inputs beyond that are read in place
-            for (int k = N - 1; k >= 0 && tile_traits<Out, Ins...>::lds_bytes(pl.tmask) > 65536; --k)
+            // a block's tiles must fit the CU's LDS: inputs beyond that are read in place
+            for (int k = N - 1; k >= 0 && tile_traits<Out, Ins...>::lds_bytes(pl.tmask) > EW_TILE_LDS_MAX; --k)
                 pl.tmask &= ~(1u << k);
             if (pl.tmask == 0) pl.path = DPX_PATH_EW_ROWS;
         }
@@ -719,9 +767,24 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
         if (pl.path == DPX_PATH_EW_TILE) {
             if constexpr (N >= 1) {
                 using TT = tile_traits<Out, Ins...>;
-                hipLaunchKernelGGL((ew_tile_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(EW_BLOCK),
-                                   TT::lds_bytes(pl.tmask), stream, fn, ix, out, in, pl.tmask, pl.modes, pl.dT, pl.tiles_t,
-                                   pl.tiles_i);
+                const size_t lds = TT::lds_bytes(pl.tmask);
+                if (lds > 65536) {
+                    // more dynamic LDS than a launch may ask for by default: raise the kernel's limit,
+                    // once per device
+                    static std::atomic<uint64_t> raised{0};
+                    int dev = 0;
+                    hipError_t e = hipGetDevice(&dev);
+                    if (e != hipSuccess) return e;
+                    const uint64_t bit = 1ull << (dev & 63);
+                    if (!(raised.load(std::memory_order_acquire) & bit)) {
+                        e = hipFuncSetAttribute((const void *)ew_tile_kernel<Fn, Out, Ins...>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)EW_TILE_LDS_MAX);
+                        if (e != hipSuccess) return e;
+                        raised.fetch_or(bit, std::memory_order_release);
+                    }
+                }
+                hipLaunchKernelGGL((ew_tile_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(EW_TILE_BLOCK), lds,
+                                   stream, fn, ix, out, in, pl.tmask, pl.modes, pl.dT, pl.tiles_t, pl.tiles_i);
             }
             return hipGetLastError();
         }

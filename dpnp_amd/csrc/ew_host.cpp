@@ -190,8 +190,9 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     }
     const int inner = pl.nd - 1;
     if (pl.path == DPX_PATH_EW_TILE) {
-        // tile = 64 positions along dT x (512 bytes / widest itemsize) positions along the inner dim
-        const int64_t TI = 64, TJ = 32 * E;
+        // tile = 128 (64 for 8- and 16-byte elements) positions along dT x (512 bytes / widest itemsize)
+        // positions along the inner dim
+        const int64_t TI = ew_tile_ti(16 / E), TJ = 32 * E;
         pl.modes = 0;
         for (int k = 0; k < nops; ++k) {
             uint32_t mode = MODE_STRIDED;
@@ -203,7 +204,7 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
             pl.modes |= mode << (2 * k);
         }
         pl.modes |= keep_bits(pl);
-        pl.block = EW_BLOCK;
+        pl.block = EW_TILE_BLOCK;
         pl.tiles_t = (pl.shape[pl.dT] + TI - 1) / TI;
         pl.tiles_i = (pl.shape[inner] + TJ - 1) / TJ;
         int64_t batch = 1;

@@ -506,7 +506,7 @@ def _plan_path(fn_name, *arrays):
 
 
 @pytest.mark.parametrize("dt", ["?", "i1", "u2", "f2", "i4", "f4", "i8", "f8", "c8", "c16"])
-@pytest.mark.parametrize("shape", [(64, 128), (200, 333), (17, 1000), (1000, 19), (129, 513)])
+@pytest.mark.parametrize("shape", [(64, 128), (200, 333), (17, 1000), (1000, 19), (129, 513), (256, 1024), (300, 1100)])
 def test_transposed_input_all_widths(dt, shape):
     """out (C-contiguous) = op(A.T): full tiles, ragged edges, lengths that are not a multiple of
     the 16-byte pack (element-wise staging), every item size."""
