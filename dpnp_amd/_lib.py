@@ -6,11 +6,24 @@ module raises; there is no CPU or PyTorch fallback.
 import ctypes
 import os
 
+# Where device memory and the stream come from: DPNP_AMD_MEMORY=torch (PyTorch's caching
+# allocator and current stream), =native (the library's own pool and stream, dpx_mem_* and
+# dpx_stream_*), or unset: torch when it can be imported, else native.
 # PyTorch ships its own HIP runtime (libamdhip64.so.7).  It must be in the process before
 # libdpnp_amd.so is loaded so that both bind to the SAME runtime instance: device memory
 # allocated by torch is then valid in this library's launches, and the stream handles match.
 # Loading in the other order leaves two runtimes in the process and the second one finds no device.
-import torch  # noqa: F401,E402
+MEMORY = os.environ.get("DPNP_AMD_MEMORY", "").lower()
+if MEMORY not in ("", "torch", "native"):
+    raise ImportError("DPNP_AMD_MEMORY must be 'torch' or 'native', not %r" % MEMORY)
+torch = None
+if MEMORY != "native":
+    try:
+        import torch  # noqa: F401,E402
+    except ImportError:
+        if MEMORY == "torch":
+            raise
+    MEMORY = "torch" if torch is not None else "native"
 
 MAX_ND = 12
 NOALLOC_SCRATCH_BYTES = 2 << 20  # DPX_NOALLOC_SCRATCH_BYTES
@@ -119,6 +132,15 @@ SIGNATURES = {
     "dpx_copy_cast": (_i, [_VP, _VP, _vp]),
     "dpx_copy_from_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
     "dpx_copy_to_host": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
+    "dpx_device_count": (_i, [ctypes.POINTER(_i)]),
+    "dpx_device_name": (_i, [_i, ctypes.c_char_p, ctypes.c_size_t]),
+    "dpx_stream_create": (_i, [ctypes.POINTER(_vp)]),
+    "dpx_stream_synchronize": (_i, [_vp]),
+    "dpx_stream_destroy": (_i, [_vp]),
+    "dpx_mem_alloc": (_i, [ctypes.POINTER(_vp), ctypes.c_size_t, _vp]),
+    "dpx_mem_free": (_i, [_vp, _vp]),
+    "dpx_mem_release_cached": (_i, []),
+    "dpx_mem_stats": (_i, [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
     "dpx_fill": (_i, [_VP, _d, _d, _i64, _i, _vp]),
     "dpx_unary_plan": (_i, [_i, _VP, _VP, _PP]),
     "dpx_binary_plan": (_i, [_i, _VP, _VP, _VP, _PP]),

@@ -396,6 +396,30 @@ int dpx_copy_from_host(void *dst_device, const void *src_host, size_t nbytes,
                        void *stream);
 int dpx_copy_to_host(void *dst_host, const void *src_device, size_t nbytes,
                      void *stream);
+/* ---- device, streams and device memory -----------------------------------------------------
+ * For hosts that bring no allocator or stream of their own.  The reference gets both from
+ * dpctl: usm_ndarray allocates a dpctl.memory.MemoryUSMDevice for buffer="device"
+ * (dpnp/tensor/_usmarray.pyx:270-305) and every call runs on a dpctl.SyclQueue
+ * (dpnp/tensor/_device.py:160-175); an array frees its memory when its last reference goes,
+ * also while kernels that use it are still queued.
+ * dpx_mem_alloc hands out device memory of the current device for use on `stream`;
+ * dpx_mem_free takes the stream the block was LAST USED on and makes the block available
+ * again in stream order: at once to later work on that stream, after a device-side wait to
+ * work on another stream.  Neither call waits for the device.  Freed blocks stay cached in the
+ * process until dpx_mem_release_cached() (which waits for the device).  A stream passed to
+ * dpx_mem_free must stay valid while the block is cached: destroy library streams with
+ * dpx_stream_destroy, and call dpx_stream_synchronize(stream) before destroying a foreign
+ * stream that blocks were freed on.  Thread-safe. */
+int dpx_device_count(int *count);                       /* 0 when no device or no driver */
+int dpx_device_name(int device, char *buf, size_t len);
+int dpx_stream_create(void **stream);                   /* default priority, non-blocking */
+int dpx_stream_synchronize(void *stream);
+int dpx_stream_destroy(void *stream);                   /* waits for the stream first */
+int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream);
+int dpx_mem_free(void *ptr, void *stream);
+int dpx_mem_release_cached(void);
+int dpx_mem_stats(size_t *in_use_bytes, size_t *cached_bytes);
+
 /* dst = value (converted to dst's dtype): ti._full_usm_ndarray,
  * libtensor/source/full_ctor.cpp. value_im is used for complex dst only. */
 int dpx_fill(const dpx_array_view *dst, double value_re, double value_im,

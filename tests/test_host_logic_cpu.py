@@ -2,7 +2,6 @@
 of results.  Arrays here sit on a host byte buffer: only descriptors are exercised."""
 import numpy as np
 import pytest
-import torch
 
 import dpnp_amd.tensor as dpt
 from dpnp_amd.tensor import _tensor_elementwise_impl as tei
@@ -14,9 +13,22 @@ from dpnp_amd.tensor._usmarray import usm_ndarray
 ALL = list(dpt._dtypes.ALL_DTYPES)
 
 
+class HostBytes:
+    """Host memory with the two methods this package uses of an allocation."""
+
+    def __init__(self, nbytes):
+        self.a = np.empty(max(int(nbytes), 1), dtype=np.uint8)
+
+    def data_ptr(self):
+        return self.a.ctypes.data
+
+    def numel(self):
+        return self.a.size
+
+
 def host_array(shape, dtype="f4", order="C"):
     n = int(np.prod(shape)) if len(shape) else 1
-    buf = torch.empty(max(n, 1) * np.dtype(dtype).itemsize, dtype=torch.uint8)
+    buf = HostBytes(max(n, 1) * np.dtype(dtype).itemsize)
     return usm_ndarray(shape, dtype=dtype, buffer=buf, order=order)
 
 
@@ -31,7 +43,7 @@ def _host_alloc(monkeypatch):
     # allocations made by the layout helpers go to host bytes in these tests
     from dpnp_amd.tensor import _device
 
-    monkeypatch.setattr(_device, "alloc", lambda nbytes: torch.empty(max(int(nbytes), 1), dtype=torch.uint8))
+    monkeypatch.setattr(_device, "alloc", HostBytes)
 
 
 # ---- promotion ---------------------------------------------------------------------------------------
