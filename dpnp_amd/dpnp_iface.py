@@ -297,6 +297,11 @@ class DPNPUnaryFunc:
         return self._fn.types
 
     def __call__(self, x, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+        if (out is None or type(out) is dpnp_array) and dtype is None and where is True and order == "K" \
+                and subok is True and not kwargs and type(x) is dpnp_array:
+            res = self._fn._fast(x._array_obj, None if out is None else out._array_obj)
+            if res is not None:
+                return _wrap(res) if out is None else out
         _check_ufunc_kwargs(self.name_, where, subok, dtype, out, kwargs)
         if not is_supported_array_type(x):
             raise TypeError(f"Input array must be any of supported type, but got {type(x)}")
@@ -326,6 +331,21 @@ class DPNPBinaryFunc:
         return self._fn.types
 
     def __call__(self, x1, x2, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
+        if (out is None or (type(out) is dpnp_array and out is not x1)) and dtype is None and where is True \
+                and order == "K" and subok is True and not kwargs:
+            # arrays and Python numbers, the keywords at their defaults: the tensor function's own short path
+            t1, t2 = type(x1), type(x2)
+            uo = None if out is None else out._array_obj
+            res = None
+            if t1 is dpnp_array:
+                if t2 is dpnp_array:
+                    res = self._fn._fast(x1._array_obj, x2._array_obj, uo)
+                elif t2 is float or t2 is int:
+                    res = self._fn._fast(x1._array_obj, x2, uo)
+            elif t2 is dpnp_array and (t1 is float or t1 is int):
+                res = self._fn._fast(x1, x2._array_obj, uo)
+            if res is not None:
+                return _wrap(res) if out is None else out
         check_supported_arrays_type(x1, x2, scalar_type=True, all_scalars=False)
         _check_ufunc_kwargs(self.name_, where, subok, dtype, out, kwargs)
         u1, u2 = get_usm_ndarray_or_scalar(x1), get_usm_ndarray_or_scalar(x2)

@@ -29,6 +29,7 @@ from ._type_utils import (
     _find_buf_dtype2,
     _find_buf_dtype_in_place_op,
     _resolve_weak_types,
+    _resolve_weak_types_all_py_ints,
 )
 from ._usmarray import usm_ndarray
 
@@ -137,6 +138,30 @@ def _check_out(out, shape, res_dt):
         raise ValueError(f"Output array of type {res_dt} is needed, got {out.dtype}")
 
 
+def _fast_out_ok(out, shape, dt):
+    """`out` can be written directly by a kernel that produces a C-contiguous `shape` of `dt`."""
+    return type(out) is usm_ndarray and out._dtype == dt and out._shape == shape and out._writable \
+        and out._is_c_contiguous()
+
+
+def _scalar_operand(v, dt, shape):
+    """The cached 0-d device array for Python scalar `v` as dtype `dt`, seen with `shape`
+    (all strides zero).  The last few shapes asked for are kept with the 0-d array."""
+    s = _as_device_array(v, dt)
+    if not shape:
+        return s
+    views = s.__dict__.get("_bviews")
+    if views is None:
+        views = s._bviews = {}
+    r = views.get(shape)
+    if r is None:
+        if len(views) >= 8:
+            views.clear()
+        r = views[shape] = s._view(shape, (0,) * len(shape), s._offset)
+        r._writable = False
+    return r
+
+
 class UnaryElementwiseFunc:
     """Elementwise function of one array.
 
@@ -151,6 +176,7 @@ class UnaryElementwiseFunc:
         self.name_ = name
         self.result_type_resolver_fn_ = result_type_resolver_fn
         self.unary_fn_ = unary_dp_impl_fn
+        self._fast_cache = {}
         self.__doc__ = docs
         self.acceptance_fn_ = acceptance_fn
 
@@ -187,7 +213,32 @@ class UnaryElementwiseFunc:
 
     types_ = types
 
+    def _fast(self, x, out=None):
+        """The result for a C-contiguous array whose dtype the kernel takes as it is, else None:
+        the common call without the general path's checks (nothing to cast, order "K" of a
+        C-contiguous input is C; an `out` must be a writable C-contiguous array of the result's
+        shape and dtype in an allocation of its own)."""
+        if type(x) is not usm_ndarray or not x._is_c_contiguous():
+            return None
+        dt = x._dtype
+        res_dt = self._fast_cache.get(dt)
+        if res_dt is None:
+            buf_dt, r = _find_buf_dtype(dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+            res_dt = self._fast_cache[dt] = r if (r is not None and buf_dt is None) else False
+        if res_dt is False:
+            return None
+        if out is None:
+            out = usm_ndarray._new_contiguous(x._shape, res_dt)
+        elif not _fast_out_ok(out, x._shape, res_dt) or out._buf is x._buf:
+            return None
+        self.unary_fn_(x, out)
+        return out
+
     def __call__(self, x, /, *, out=None, order="K"):
+        if order == "K":
+            r = self._fast(x, out)
+            if r is not None:
+                return r
         if not isinstance(x, usm_ndarray):
             raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")
         order = _norm_order(order)
@@ -238,6 +289,7 @@ class BinaryElementwiseFunc:
         self.acceptance_fn_ = acceptance_fn
         self.weak_type_resolver_ = weak_type_resolver
         self._fused_cache = {}
+        self._fast_cache = {}
 
     def __str__(self):
         return f"<{self.__name__} '{self.name_}'>"
@@ -311,7 +363,56 @@ class BinaryElementwiseFunc:
             hit = self._fused_cache[key] = tei._fused_cast_result_type(self.name_, d1, d2)
         return hit
 
+    def _fast(self, o1, o2, out=None):
+        """The result for two C-contiguous arrays of one shape and one dtype that the kernel
+        takes as it is, or for such an array of a floating or complex dtype and a Python float
+        or int (which then takes the array's dtype whatever its value); else None.  See
+        UnaryElementwiseFunc._fast."""
+        t1, t2 = type(o1), type(o2)
+        scalar = None
+        if t1 is usm_ndarray:
+            arr = o1
+            if t2 is usm_ndarray:
+                if o2._dtype != o1._dtype or o1._shape != o2._shape or not o2._is_c_contiguous():
+                    return None
+            elif (t2 is float or t2 is int) and o1._dtype.kind in "fc":
+                scalar = o2
+            else:
+                return None
+        elif t2 is usm_ndarray and (t1 is float or t1 is int) and o2._dtype.kind in "fc":
+            arr, scalar = o2, o1
+        else:
+            return None
+        if not arr._is_c_contiguous():
+            return None
+        dt = arr._dtype
+        res_dt = self._fast_cache.get(dt)
+        if res_dt is None:
+            b1, b2, r = _find_buf_dtype2(dt, dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+            res_dt = self._fast_cache[dt] = r if (r is not None and b1 is None and b2 is None) else False
+        if res_dt is False:
+            return None
+        if scalar is not None:
+            if self.weak_type_resolver_ is not _resolve_weak_types \
+                    and self.weak_type_resolver_ is not _resolve_weak_types_all_py_ints:
+                return None
+            sv = _scalar_operand(scalar, dt, arr._shape)
+            if arr is o1:
+                o2 = sv
+            else:
+                o1 = sv
+        if out is None:
+            out = usm_ndarray._new_contiguous(arr._shape, res_dt)
+        elif not _fast_out_ok(out, arr._shape, res_dt) or out._buf is o1._buf or out._buf is o2._buf:
+            return None
+        self.binary_fn_(src1=o1, src2=o2, dst=out)
+        return out
+
     def __call__(self, o1, o2, /, *, out=None, order="K"):
+        if order == "K":
+            r = self._fast(o1, o2, out)
+            if r is not None:
+                return r
         order = _norm_order(order)
         res_shape, d1, d2 = self._resolve(o1, o2)
         buf1_dt, buf2_dt, res_dt = _find_buf_dtype2(d1, d2, self.result_type_resolver_fn_, None,

@@ -34,7 +34,7 @@ def _move_reduced_axes_last(x, axis, int_only=False):
 def _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap):
     """Validate a user `out`; returns (array the kernel writes, array the user gets back)."""
     if out is None:
-        r = empty(res_shape, dtype=res_dt)
+        r = usm_ndarray._new_contiguous(tuple(res_shape), res_dt)
         return r, r
     if not isinstance(out, usm_ndarray):
         raise TypeError(f"output array must be of usm_ndarray type, got {type(out)}")

@@ -270,14 +270,27 @@ class usm_ndarray:
         """The C descriptor of this array (borrowed; valid while `self` is alive).  Built once:
         shape, strides, offset and allocation of an array object never change; only the
         writable bit may."""
-        v = self.__dict__.get("_cview")
-        if v is None:
+        try:
+            v = self._cview
+        except AttributeError:
             c, f = _contig_flags(self._shape, self._strides)
             flags = (_lib.C_CONTIGUOUS if c else 0) | (_lib.F_CONTIGUOUS if f else 0)
-            v = _lib.make_view(self._pointer, self._shape, self._strides, dtype_id(self._dtype), flags)
-            self._cview = v
-        v.flags = (v.flags & ~_lib.WRITABLE) | (_lib.WRITABLE if self._writable else 0)
+            v = self._cview = _lib.make_view(self._pointer, self._shape, self._strides, dtype_id(self._dtype), flags)
+            self._cview_c = c
+            self._cview_w = None
+        if self._cview_w is not self._writable:
+            w = self._cview_w = bool(self._writable)
+            self._writable = w
+            v.flags = (v.flags & ~_lib.WRITABLE) | (_lib.WRITABLE if w else 0)
         return v
+
+    def _is_c_contiguous(self):
+        """C-contiguity by NumPy's rules, computed once per array object."""
+        try:
+            return self._cview_c
+        except AttributeError:
+            self._as_view()
+            return self._cview_c
 
     @property
     def T(self):

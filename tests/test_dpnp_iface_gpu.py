@@ -396,3 +396,69 @@ def test_frexp_every_binade_and_special_values(dt):
     assert mi.dtype == np.float64
     assert_same(mi.asnumpy(), np.array([0.5, 0.75]))
     assert_same(ei.asnumpy(), np.array([4, 2], "i4"))
+
+
+# ---- the short call path of the ufunc wrappers against the general one ---------------------------
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "i8", "f2", "f4", "f8", "c8", "c16"])
+def test_short_call_path_gives_what_the_general_path_gives(dt):
+    """Contiguous operands of one dtype (or an array and a Python number) with default keywords
+    skip the general path's promotion search and layout logic; order="C" forces the general
+    path, whose result for these operands must be the same array."""
+    rng = np.random.default_rng(41)
+    shape = (33, 65)
+    if dt == "?":
+        a, b = rng.integers(0, 2, shape).astype(dt), rng.integers(0, 2, shape).astype(dt)
+    elif np.dtype(dt).kind in "iu":
+        a, b = rng.integers(1, 100, shape).astype(dt), rng.integers(1, 100, shape).astype(dt)
+    else:
+        a, b = rng.uniform(1, 9, shape).astype(dt), rng.uniform(1, 9, shape).astype(dt)
+    da, db = dpnp.array(a), dpnp.array(b)
+
+    def same(short, general, c_contiguous=True):
+        assert short.dtype == general.dtype and short.shape == general.shape
+        assert short.flags.c_contiguous == c_contiguous
+        assert_same(short.asnumpy(), general.asnumpy())
+
+    for name in ("add", "multiply", "divide", "greater", "maximum", "logical_and", "bitwise_and", "power"):
+        f = getattr(dpnp, name)
+        try:
+            general = f(da, db, order="C")
+        except (ValueError, TypeError):
+            with pytest.raises((ValueError, TypeError)):
+                f(da, db)
+            continue
+        same(f(da, db), general)
+        out = dpnp.empty(shape, dtype=general.dtype)
+        assert f(da, db, out=out) is out
+        assert_same(out.asnumpy(), general.asnumpy())
+        for s in (2, 2.5):
+            for args in ((da, s), (s, da)):
+                try:
+                    general = f(*args, order="C")
+                except (ValueError, TypeError):
+                    continue
+                same(f(*args), general)
+    for name in ("negative", "exp", "sqrt", "isnan", "abs", "logical_not", "square"):
+        f = getattr(dpnp, name)
+        try:
+            general = f(da, order="C")
+        except (ValueError, TypeError):
+            with pytest.raises((ValueError, TypeError)):
+                f(da)
+            continue
+        same(f(da), general)
+        out = dpnp.empty(shape, dtype=general.dtype)
+        assert f(da, out=out) is out
+        assert_same(out.asnumpy(), general.asnumpy())
+    # operands the short path must leave to the general one
+    same(dpnp.add(da.T, db.T), dpnp.add(dpnp.array(a.T.copy()), dpnp.array(b.T.copy())), False)  # F-contiguous
+    same(dpnp.add(da, db[0]), dpnp.add(da, dpnp.array(np.broadcast_to(b[0], shape).copy())))  # broadcast
+    if dt not in ("?",):
+        x = dpnp.array(a)
+        dpnp.add(x, db, out=x)  # out is an input
+        assert_same(x.asnumpy(), (dpnp.add(da, db, order="C")).asnumpy())
+        y = dpnp.array(b)
+        dpnp.add(da, y, out=y)
+        assert_same(y.asnumpy(), (dpnp.add(da, db, order="C")).asnumpy())
+    with pytest.raises(ValueError):
+        dpnp.add(da, db, out=dpnp.empty((5, 5), dtype=dt))
