@@ -162,6 +162,29 @@ def test_black_scholes_entry_point():
         np.testing.assert_allclose(got[fin], want[fin], rtol=1e-12, atol=1e-12)
 
 
+def test_black_scholes_wide_ranges():
+    """Prices and strikes over five decades, maturities from a thousandth of a year to thirty
+    years: options deep in and out of the money (erf saturates), tiny and large variances."""
+    from oracle import oracle as orc
+
+    rng = np.random.default_rng(8)
+    n = 3 * 4096 + 77
+    p, s = 10.0 ** rng.uniform(-2, 3, n), 10.0 ** rng.uniform(-2, 3, n)
+    t = 10.0 ** rng.uniform(-3, 1.5, n)
+    for rate, vol in ((0.1, 0.2), (0.0, 0.05), (-0.01, 1.5)):
+        call, put = dpnp.black_scholes(dpnp.array(p), dpnp.array(s), dpnp.array(t), rate, vol)
+        wc, wp = orc.black_scholes(p, s, t, rate, vol)
+        scale = np.maximum(p, s * np.exp(-rate * t))
+        # a rounding error of the logarithm (or of rate * t) reaches erf's argument multiplied by
+        # 1 / sqrt(2 vol^2 t), and erf' <= 1.13: the bound any two correct evaluations differ by
+        z = 2 * vol * vol * t
+        cond = (np.abs(np.log(p / s)) + np.abs(rate * t) + 0.25 * z) / np.sqrt(z)
+        tol = np.finfo("f8").eps * scale * (4 + 4 * cond)
+        for got, want in ((call.asnumpy(), wc), (put.asnumpy(), wp)):
+            assert np.all(np.isfinite(got))
+            assert np.all(np.abs(got - want) <= 1e-12 * np.abs(want) + tol)
+
+
 # ---- dpnp-level functions built on the ufunc extension kernels ---------------------------------
 def test_nan_to_num_reference_examples():
     # docstring of dpnp.nan_to_num, dpnp/dpnp_iface_mathematical.py:3640-3670
