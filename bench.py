@@ -48,10 +48,19 @@ def cpu_baseline(n_log2=28, repeats=5):
         oc.argmax(a)
     dt = time.perf_counter() - t0
     nbytes = repeats * n * (12 + 4 + 4 + 4)
+    # second stand-in: NumPy on one thread, one pass of the same calls
+    t0 = time.perf_counter()
+    np.add(a, b, out=out)
+    a.sum()
+    b.sum()
+    a.argmax()
+    dt_np = time.perf_counter() - t0
     return {
         "value": nbytes / dt / 1e9, "unit": "GB/s", "cores": oc.threads, "kind": "port",
         "sample": f"{repeats} passes of add + 2 x sum + argmax over 2^{n_log2} fp32 elements "
                   "(C/OpenMP restatement of the reference's kernels, oracle/oracle_c.c; the metric's own size)",
+        "numpy_one_thread": {"value": n * (12 + 4 + 4 + 4) / dt_np / 1e9, "unit": "GB/s", "cores": 1,
+                             "sample": "one pass of the same calls through NumPy"},
     }
 
 

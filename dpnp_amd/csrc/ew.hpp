@@ -477,7 +477,9 @@ template <class F, int... P> inline void for_each_pattern(F &&f, std::integer_se
 // modes: as for the rows kernel; for a flagged input MODE_VEC allows the 16-byte phase-1 reads.
 constexpr int EW_TILE_BLOCK = 512;
 constexpr size_t EW_TILE_LDS_MAX = 160 * 1024;
-constexpr int ew_tile_ti(int widest_itemsize) { return widest_itemsize <= 4 ? 128 : 64; }
+// positions along dT per tile: 128 (512-byte runs of 4-byte elements; measured best for 2-, 4- and 8-byte
+// elements), 64 for 16-byte elements (1 KiB runs already)
+constexpr int ew_tile_ti(int widest_itemsize) { return widest_itemsize <= 8 ? 128 : 64; }
 template <class Out, class... Ins> struct tile_traits {
     static constexpr int TI = ew_tile_ti(max_sizeof<Out, Ins...>());
     static constexpr int TJ = 512 / max_sizeof<Out, Ins...>();

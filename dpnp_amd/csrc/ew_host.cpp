@@ -190,7 +190,7 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     }
     const int inner = pl.nd - 1;
     if (pl.path == DPX_PATH_EW_TILE) {
-        // tile = 128 (64 for 8- and 16-byte elements) positions along dT x (512 bytes / widest itemsize)
+        // tile = 128 (64 for 16-byte elements) positions along dT x (512 bytes / widest itemsize)
         // positions along the inner dim
         const int64_t TI = ew_tile_ti(16 / E), TJ = 32 * E;
         pl.modes = 0;
