@@ -182,6 +182,44 @@ def test_unary_transcendentals_within_4_ulp(op):
             np.testing.assert_array_equal(np.signbit(got), np.signbit(want(x)))
 
 
+def test_float64_trigonometric_functions_on_hard_arguments():
+    """asin and acos of doubles are the library's own routines, sin, cos and tan the device library's:
+    against an 80-bit evaluation on every binade, next to multiples of pi/2 (where the reduced argument
+    cancels), around 1e6, next to +-1 and +-1/2."""
+    if np.finfo(np.longdouble).nmant < 63:
+        pytest.skip("needs an extended-precision long double")
+    rng = np.random.default_rng(31)
+    tiny = float(np.finfo("f8").tiny)
+    mag = np.exp(rng.uniform(np.log(tiny * 4), np.log(1e15), 60000))
+    k = rng.integers(1, 636000, 40000).astype("f8")
+    near = k * (np.pi / 2) + rng.choice([0.0, 1e-9, -1e-9, 1e-4, -3e-13], k.size)
+    edge = 1e6 + rng.uniform(-50, 50, 2000)
+    a = np.concatenate([mag * rng.choice([-1.0, 1.0], mag.size), near, -near[:5000], edge, -edge,
+                        rng.uniform(-50, 50, 40000)])
+    for op, bound in (("sin", 1.5), ("cos", 1.5), ("tan", 3.0)):
+        got = host(getattr(dpt, op)(dev(a)))
+        assert_ulp(got, orc.hi_precision(op, a), bound)
+    m1 = np.exp(rng.uniform(np.log(tiny * 4), 0.0, 40000))
+    b = np.concatenate([m1, 1.0 - m1[m1 < 0.5], 0.5 + rng.uniform(-1e-3, 1e-3, 5000), rng.uniform(0, 1, 40000),
+                        np.array([0.0, 0.5, 1.0, np.nextafter(1.0, 0), np.nextafter(0.5, 0), np.nextafter(0.5, 1)])])
+    b = np.concatenate([b, -b])
+    for op in ("asin", "acos"):
+        got = host(getattr(dpt, op)(dev(b)))
+        assert_ulp(got, orc.hi_precision(op, b), 1.5)
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0 + 2.0 ** -52, -1.5, 1e300])
+    with np.errstate(all="ignore"):
+        for op, f in (("sin", np.sin), ("cos", np.cos), ("tan", np.tan), ("asin", np.arcsin), ("acos", np.arccos)):
+            got, want = host(getattr(dpt, op)(dev(special))), f(special)
+            np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+            ok = ~np.isnan(want)
+            if op in ("asin", "acos"):
+                np.testing.assert_array_equal(got[ok], want[ok])
+                np.testing.assert_array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+            else:
+                assert_ulp(got[ok], f(special[ok].astype(np.longdouble)), 1.5)
+                np.testing.assert_array_equal(np.signbit(got[:2]), np.signbit(want[:2]))
+
+
 @pytest.mark.parametrize("op", ["log1p", "expm1", "sinh", "tanh", "asinh", "atanh", "acosh", "erf", "cosh", "log2", "log10"])
 def test_own_math_routines_keep_relative_accuracy_at_every_magnitude(op):
     """The library's own fp32 / fp64 routines (log2, log10, log1p, erf, sinh, cosh, tanh, asinh, acosh, atanh) against
