@@ -183,9 +183,9 @@ def test_unary_transcendentals_within_4_ulp(op):
 
 
 def test_float64_trigonometric_functions_on_hard_arguments():
-    """asin and acos of doubles are the library's own routines, sin, cos and tan the device library's:
-    against an 80-bit evaluation on every binade, next to multiples of pi/2 (where the reduced argument
-    cancels), around 1e6, next to +-1 and +-1/2."""
+    """asin, acos and, below 1e6 in magnitude, sin and cos of doubles are the library's own routines, tan
+    and the rest the device library's: against an 80-bit evaluation on every binade, next to multiples of
+    pi/2 (where the reduced argument cancels), across the hand-over at 1e6, next to +-1 and +-1/2."""
     if np.finfo(np.longdouble).nmant < 63:
         pytest.skip("needs an extended-precision long double")
     rng = np.random.default_rng(31)
@@ -196,7 +196,7 @@ def test_float64_trigonometric_functions_on_hard_arguments():
     edge = 1e6 + rng.uniform(-50, 50, 2000)
     a = np.concatenate([mag * rng.choice([-1.0, 1.0], mag.size), near, -near[:5000], edge, -edge,
                         rng.uniform(-50, 50, 40000)])
-    for op, bound in (("sin", 1.5), ("cos", 1.5), ("tan", 3.0)):
+    for op, bound in (("sin", 2.0), ("cos", 2.0), ("tan", 2.0)):
         got = host(getattr(dpt, op)(dev(a)))
         assert_ulp(got, orc.hi_precision(op, a), bound)
     m1 = np.exp(rng.uniform(np.log(tiny * 4), 0.0, 40000))
@@ -216,7 +216,7 @@ def test_float64_trigonometric_functions_on_hard_arguments():
                 np.testing.assert_array_equal(got[ok], want[ok])
                 np.testing.assert_array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
             else:
-                assert_ulp(got[ok], f(special[ok].astype(np.longdouble)), 1.5)
+                assert_ulp(got[ok], f(special[ok].astype(np.longdouble)), 2.0)
                 np.testing.assert_array_equal(np.signbit(got[:2]), np.signbit(want[:2]))
 
 
