@@ -142,6 +142,7 @@ int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream)
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fail_hip(e, "hipGetDevice");
     if (dev < 0 || dev >= MAX_DEVICES) return fail(DPX_ERR_BAD_ARGUMENT, "mem_alloc: device index out of range");
+    if (nbytes > ((size_t)1 << 46)) return fail(DPX_ERR_BAD_ARGUMENT, "mem_alloc: more than 64 TiB asked for");
     const size_t size = round_size(nbytes);
     const hipStream_t s = (hipStream_t)stream;
     Block blk{nullptr, 0, nullptr, true};
