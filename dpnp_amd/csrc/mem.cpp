@@ -146,8 +146,6 @@ int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream)
     const size_t size = round_size(nbytes);
     const hipStream_t s = (hipStream_t)stream;
     Block blk{nullptr, 0, nullptr, true};
-    hipStream_t wait_for = nullptr;
-    bool must_wait = false;
     {
         std::lock_guard<std::mutex> lk(g_mu);
         auto &cache = g_cache[dev];
@@ -162,28 +160,22 @@ int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream)
             if (pick == cache.end()) pick = it;
         }
         if (pick != cache.end()) {
+            if (pick->second.stream != s && !pick->second.idle) {
+                // order this stream after everything queued on the block's old stream so far; under the
+                // lock, so that dpx_stream_destroy of the old stream cannot come in between
+                hipEvent_t ev;
+                e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+                if (e == hipSuccess) {
+                    e = hipEventRecord(ev, pick->second.stream);
+                    if (e == hipSuccess) e = hipStreamWaitEvent(s, ev, 0);
+                    const hipError_t e2 = hipEventDestroy(ev); // deferred until the event has completed
+                    if (e == hipSuccess) e = e2;
+                }
+                if (e != hipSuccess) return fail_hip(e, "mem_alloc: ordering after the block's previous stream");
+            }
             blk = pick->second;
             cache.erase(pick);
             g_cached -= blk.size;
-            if (blk.stream != s && !blk.idle) {
-                must_wait = true;
-                wait_for = blk.stream;
-            }
-        }
-    }
-    if (must_wait) {
-        // order this stream after everything queued on the block's old stream so far
-        hipEvent_t ev;
-        e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
-        if (e == hipSuccess) e = hipEventRecord(ev, wait_for);
-        if (e == hipSuccess) e = hipStreamWaitEvent(s, ev, 0);
-        if (e == hipSuccess) e = hipEventDestroy(ev); // destruction is deferred until the event has completed
-        if (e != hipSuccess) {
-            // keep the block: back to the cache as it was
-            std::lock_guard<std::mutex> lk(g_mu);
-            g_cached += blk.size;
-            g_cache[dev].emplace(blk.size, blk);
-            return fail_hip(e, "mem_alloc: ordering after the block's previous stream");
         }
     }
     if (!blk.ptr) {
