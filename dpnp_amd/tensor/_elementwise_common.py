@@ -144,6 +144,13 @@ def _fast_out_ok(out, shape, dt):
         and out._is_c_contiguous()
 
 
+def _spans_meet(x, y):
+    """Two C-contiguous arrays share at least one byte."""
+    x0, x1 = x._contiguous_span()
+    y0, y1 = y._contiguous_span()
+    return x0 < y1 and y0 < x1
+
+
 def _scalar_operand(v, dt, shape):
     """The cached 0-d device array for Python scalar `v` as dtype `dt`, seen with `shape`
     (all strides zero).  The last few shapes asked for are kept with the 0-d array."""
@@ -229,7 +236,7 @@ class UnaryElementwiseFunc:
             return None
         if out is None:
             out = usm_ndarray._new_contiguous(x._shape, res_dt)
-        elif not _fast_out_ok(out, x._shape, res_dt) or out._buf is x._buf:
+        elif not _fast_out_ok(out, x._shape, res_dt) or _spans_meet(out, x):
             return None
         self.unary_fn_(x, out)
         return out
@@ -403,7 +410,8 @@ class BinaryElementwiseFunc:
                 o1 = sv
         if out is None:
             out = usm_ndarray._new_contiguous(arr._shape, res_dt)
-        elif not _fast_out_ok(out, arr._shape, res_dt) or out._buf is o1._buf or out._buf is o2._buf:
+        elif not _fast_out_ok(out, arr._shape, res_dt) or _spans_meet(out, arr) \
+                or (scalar is None and _spans_meet(out, o2)):
             return None
         self.binary_fn_(src1=o1, src2=o2, dst=out)
         return out

@@ -275,14 +275,27 @@ class usm_ndarray:
         except AttributeError:
             c, f = _contig_flags(self._shape, self._strides)
             flags = (_lib.C_CONTIGUOUS if c else 0) | (_lib.F_CONTIGUOUS if f else 0)
-            v = self._cview = _lib.make_view(self._pointer, self._shape, self._strides, dtype_id(self._dtype), flags)
+            ptr = self._pointer
+            v = self._cview = _lib.make_view(ptr, self._shape, self._strides, dtype_id(self._dtype), flags)
             self._cview_c = c
             self._cview_w = None
+            n = 1
+            for d in self._shape:
+                n *= d
+            self._cview_span = (ptr, ptr + n * self._dtype.itemsize)  # the bytes of a contiguous array
         if self._cview_w is not self._writable:
             w = self._cview_w = bool(self._writable)
             self._writable = w
             v.flags = (v.flags & ~_lib.WRITABLE) | (_lib.WRITABLE if w else 0)
         return v
+
+    def _contiguous_span(self):
+        """(first byte, one past the last byte) of a C- or F-contiguous array."""
+        try:
+            return self._cview_span
+        except AttributeError:
+            self._as_view()
+            return self._cview_span
 
     def _is_c_contiguous(self):
         """C-contiguity by NumPy's rules, computed once per array object."""

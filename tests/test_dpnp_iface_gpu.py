@@ -485,3 +485,16 @@ def test_short_call_path_gives_what_the_general_path_gives(dt):
         assert_same(y.asnumpy(), (dpnp.add(da, db, order="C")).asnumpy())
     with pytest.raises(ValueError):
         dpnp.add(da, db, out=dpnp.empty((5, 5), dtype=dt))
+    if dt != "?":
+        # out overlaps an input without being it: both contiguous, the general path's temporary is needed
+        base = np.arange(1, 201).astype(dt)
+        x = dpnp.array(base)
+        dpnp.add(x[:100], x[:100], out=x[50:150])
+        want = base.copy()
+        want[50:150] = base[:100] + base[:100]
+        assert_same(x.asnumpy(), want)
+        x = dpnp.array(base)
+        dpnp.negative(x[:100], out=x[1:101])
+        want = base.copy()
+        want[1:101] = np.negative(base[:100])
+        assert_same(x.asnumpy(), want)
