@@ -612,13 +612,19 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
 // ecnt columns per thread (ecnt = 16 / sizeof(In) when L.vec, else 1).
 // Linear block id = (outer * splits + split) * col_blocks + col_block.
 // Partials are laid out [split][output] (coalesced to write and to fold).
-constexpr int COLS_MAX_BLOCK = 1024;
+// the planner makes blocks of at most 512 threads; the bound leaves the compiler 256 vector registers per
+// lane, which the kernels of 1-byte inputs (16 columns per pack) need: under a bound of 1024 they spilled
+constexpr int COLS_MAX_BLOCK = 512;
 
-// elements of LDS scratch per thread and loads in flight per thread: wide inputs keep 4
-// packs in flight, 1- and 2-byte inputs (8 or 16 accumulators per pack) keep 2
+// elements of LDS scratch per thread, packs in flight per thread (LOADS) and accumulator sets they are
+// folded into (U): wide inputs keep 4 packs in flight with a set each; 1- and 2-byte inputs, whose packs
+// hold 8 or 16 columns, keep 8 in flight (the rows of a block are only 512 bytes wide, so the loads in
+// flight are what feeds the memory system: bool 16384^2 summed down its columns ran at 29 % of the HBM
+// rate with 2) and fold them into one set, which the registers still hold
 template <class In> struct cols_cfg {
     static constexpr int E = 16 / (int)sizeof(In);
-    static constexpr int U = E >= 8 ? 2 : 4;
+    static constexpr int U = E >= 8 ? 1 : 4;
+    static constexpr int LOADS = E >= 8 ? 8 : 4;
 };
 
 // combines acc over the TY thread rows of the block; result valid for ty == 0
@@ -647,6 +653,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     using Acc = typename P::Acc;
     constexpr int E = cols_cfg<In>::E;
     constexpr int U = cols_cfg<In>::U;
+    constexpr int LOADS = cols_cfg<In>::LOADS;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     Acc *sm = reinterpret_cast<Acc *>(smem_raw);
     const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
@@ -707,14 +714,17 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                         return t;
                     }
                 };
-                for (; r + (U - 1) * TY < end; r += U * TY) {
-                    pack<In, E> v[U];
+                // the element-wise form keeps one pack in flight: its LOADS x E separate loads and their
+                // addresses would set the register count of the whole kernel (and spill for 1-byte inputs)
+                constexpr int NL = WHOLE ? LOADS : 1;
+                for (; r + (NL - 1) * TY < end; r += NL * TY) {
+                    pack<In, E> v[NL];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+                    for (int u = 0; u < NL; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                    for (int u = 0; u < U; ++u)
+                    for (int u = 0; u < NL; ++u)
 #pragma unroll
-                        for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], P::pre(v[u].v[e], a[e]));
+                        for (int e = 0; e < E; ++e) acc[u % U][e] = P::combine(acc[u % U][e], P::pre(v[u].v[e], a[e]));
                 }
                 for (; r < end; r += TY) {
                     pack<In, E> v = load(p + r * L.rstride);
@@ -726,12 +736,12 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             else walk(std::false_type{});
         }
         else {
-            for (; r + (U - 1) * TY < end; r += U * TY) {
-                In v[U];
+            for (; r + (LOADS - 1) * TY < end; r += LOADS * TY) {
+                In v[LOADS];
 #pragma unroll
-                for (int u = 0; u < U; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
+                for (int u = 0; u < LOADS; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                for (int u = 0; u < U; ++u) acc[u][0] = P::combine(acc[u][0], P::pre(v[u], a[0]));
+                for (int u = 0; u < LOADS; ++u) acc[u % U][0] = P::combine(acc[u % U][0], P::pre(v[u], a[0]));
             }
             for (; r < end; r += TY) acc[0][0] = P::combine(acc[0][0], P::pre(load_one(p + r * L.rstride), a[0]));
         }
@@ -1233,7 +1243,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
 {
     using VT = value_of_t<T>;
     constexpr int E = 16 / (int)sizeof(T);
-    constexpr int U = E >= 8 ? 2 : 4; // rows in flight per thread
+    constexpr int U = E >= 8 ? 8 : 4; // rows in flight per thread (see cols_cfg)
     __shared__ VT smv[256 * E];
     __shared__ int64_t smi[256 * E];
     const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
@@ -1301,12 +1311,13 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
                     bl[e] = (uint32_t)(r - beg);
                 }
             }
-            for (; r + (U - 1) * TY < end; r += U * TY) {
-                pack<T, E> v[U];
+            constexpr int NL = WHOLE ? U : 1; // the element-wise form keeps one pack in flight (registers)
+            for (; r + (NL - 1) * TY < end; r += NL * TY) {
+                pack<T, E> v[NL];
 #pragma unroll
-                for (int u = 0; u < U; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+                for (int u = 0; u < NL; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
 #pragma unroll
-                for (int u = 0; u < U; ++u) take(v[u], r + u * TY);
+                for (int u = 0; u < NL; ++u) take(v[u], r + u * TY);
             }
             for (; r < end; r += TY) take(load(p + r * L.rstride), r);
         };

@@ -258,7 +258,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     int block = (int)std::min<int64_t>(arg ? 256 : 512, std::max<int64_t>(64, TX * ty));
     if (!arg) {
         const int fb = tune_int("DPX_COLS_BLOCK", 0); // sweep override, product build: default
-        if (fb == 256 || fb == 512 || fb == 1024) block = fb;
+        if (fb == 256 || fb == 512) block = fb;
     }
     if (block < TX) block = (int)TX;
     const int64_t TY = block / TX;
