@@ -637,7 +637,7 @@ DPX_D void ew_tile_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
         static_assert(TI % RPP2 == 0, "passes cover the tile exactly");
         Out *q = out + col[N] + lr * ix.strides[N][dT];
         const int64_t qstep = RPP2 * ix.strides[N][dT];
-#pragma unroll
+#pragma unroll 2
         for (int it = 0; it < TI / RPP2; ++it) {
             const int i = it * RPP2 + lr;
             std::tuple<pack<Ins, E>...> v;
