@@ -54,7 +54,8 @@ template <class Out, class... Ins> struct ew_traits {
     // input: f8 -> i1 0.224 -> 0.193 ms, isnan(f4) 0.227 -> 0.198 ms; at 24 bytes per pack
     // (f4 -> f8) two packs are slower than one, 0.476 -> 0.521 ms.
     static constexpr int pack_bytes = E * (int)(sizeof(Out) + (size_t(0) + ... + sizeof(Ins)));
-    static constexpr int U = pack_bytes <= 20 ? 2 : 1;
+    // a kernel without inputs (fill) stores one pack per thread, in blocks of four waves
+    static constexpr int U = (sizeof...(Ins) > 0 && pack_bytes <= 20) ? 2 : 1;
 };
 
 // Packs per thread of the contiguous kernel for functor Fn.  A functor may ask for two with a member

@@ -164,6 +164,9 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
         }
         pl.period = pl.flat2d ? (uint32_t)pl.shape[1] : 1u;
         pl.block = env_block("DPX_EW_CONTIG_BLOCK", EW_CONTIG_BLOCK);
+        // a kernel that only stores (fill) is one instruction per wave: one-wave blocks are then bound by the
+        // rate waves are launched at (2^28 floats: 59 % of the HBM rate, with four waves per block 81 %)
+        if (nops == 1) pl.block = 256;
         pl.grid = (pl.n + (int64_t)pl.block * E * U - 1) / ((int64_t)pl.block * E * U);
         return;
     }
