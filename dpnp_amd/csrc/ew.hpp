@@ -65,6 +65,8 @@ template <class Out, class... Ins> struct ew_traits {
 // gain nothing, so it is not the rule).
 template <class Fn, class = void> struct fn_two_packs : std::false_type {};
 template <class Fn> struct fn_two_packs<Fn, std::enable_if_t<Fn::two_packs>> : std::true_type {};
+template <class Fn, class = void> struct fn_two_phase : std::false_type {};
+template <class Fn> struct fn_two_phase<Fn, std::enable_if_t<Fn::two_phase>> : std::true_type {};
 template <class Fn, class Out, class... Ins> constexpr int ew_packs_per_thread()
 {
     return (fn_two_packs<Fn>::value && ew_traits<Out, Ins...>::U == 1) ? 2 : ew_traits<Out, Ins...>::U;
@@ -121,8 +123,21 @@ DPX_D void ew_contig_pack(const Fn &fn, Out *out, int64_t base,
     constexpr int E = ew_traits<Out, Ins...>::E;
     (keep_whole(std::get<I>(v)), ...);
     pack<Out, E> r;
+    if constexpr (fn_two_phase<Fn>::value) {
+        // the straight-line part for every element first, then the rare branches
+        decltype(fn.fast(to_value(std::get<I>(v).v[0])...)) t[E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+        for (int e = 0; e < E; ++e) t[e] = fn.fast(to_value(std::get<I>(v).v[e])...);
+        // the results exist here: without this the compiler moves each element's chain down to its branch
+#pragma unroll
+        for (int e = 0; e < E; ++e) asm volatile("" : "+v"(t[e]));
+#pragma unroll
+        for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn.fixup(t[e], to_value(std::get<I>(v).v[e])...));
+    }
+    else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(v).v[e])...));
+    }
     store_pack<Out, E>(out + base, r);
 }
 

@@ -35,8 +35,17 @@ template <class Op, class T> struct UnaryFn {
     static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
     DPX_D auto operator()(V<T> x) const { return Op::template apply<T>(x); }
 };
+// An op may split its work in two phases for element type T (Op::two_phase<T>): fast(a, b) is
+// straight-line code that gives the result or NaN where it does not apply, fixup(r, a, b) branches to the
+// complete routine for those.  The contiguous kernel runs the first phase for all elements of a pack
+// before the second, so that the chains of the elements interleave (see ew_contig_pack).
+template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
+template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct BinaryFn {
+    static constexpr bool two_phase = op_two_phase<Op, T>::value;
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
+    DPX_D auto fast(V<T> a, V<T> b) const { return Op::template fast<T>(a, b); }
+    DPX_D auto fixup(V<T> r, V<T> a, V<T> b) const { return Op::template fixup<T>(r, a, b); }
 };
 template <class Op, class T> struct rows2_enabled<UnaryFn<Op, T>> : std::true_type {};
 template <class Op, class T> struct rows2_enabled<BinaryFn<Op, T>> : std::true_type {};

@@ -111,6 +111,42 @@ def test_binary_ulp(op):
                 assert_same(host(dpt.pow(dev(a[nonneg]), dev(b[nonneg]))), np.power(a[nonneg], b[nonneg]))
 
 
+def test_float32_pow_over_the_whole_range():
+    """pow of floats takes the library's own routine for a positive normal base with a finite exponent and
+    a normal result, the device library's otherwise: every binade of the base, exponents that overflow,
+    underflow and hit the subnormal range, and the special-value table of C's pow."""
+    rng = np.random.default_rng(23)
+    n = 200000
+    x = np.exp(rng.uniform(np.log(1e-37), np.log(1e37), n)).astype("f4")
+    y = rng.uniform(-40, 40, n).astype("f4")
+    y[: n // 4] = rng.uniform(-2, 2, n // 4).astype("f4")
+    y[n // 4: n // 2] = np.round(y[n // 4: n // 2])          # integer exponents
+    x[n // 2: n // 2 + 5000] = 1.0 + rng.uniform(-1e-3, 1e-3, 5000).astype("f4")   # bases next to 1
+    y[n // 2: n // 2 + 5000] = rng.uniform(-3e4, 3e4, 5000).astype("f4")
+    got = host(dpt.pow(dev(x), dev(y)))
+    with np.errstate(all="ignore"):
+        exact = np.power(x.astype("f8"), y.astype("f8"))
+    own = np.abs(y.astype("f8") * np.log2(x.astype("f8"))) < 125.9   # the library's routine: normal results
+    assert own.sum() > n // 4 and (~own).sum() > n // 10
+    assert_ulp(got[own], exact[own], 0.52)
+    assert_ulp(got[~own], exact[~own], 2.0)                          # the device library's powf
+    for dt in ("f2",):
+        xh, yh = rng.uniform(0.1, 8, 5000).astype(dt), rng.uniform(-4, 4, 5000).astype(dt)
+        with np.errstate(all="ignore"):
+            assert_ulp(host(dpt.pow(dev(xh), dev(yh))), np.power(xh.astype("f8"), yh.astype("f8")), 1.0)
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, 3.0, -3.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45,
+                   3.4e38, 1.1754944e-38], dtype="f4")
+    X, Y = [v.ravel() for v in np.meshgrid(sp, sp)]
+    got = host(dpt.pow(dev(X), dev(Y)))
+    with np.errstate(all="ignore"):
+        want = np.power(X, Y)
+        exact = np.power(X.astype("f8"), Y.astype("f8"))
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    np.testing.assert_array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+    assert_ulp(got[ok], exact[ok], 1.0)
+
+
 @pytest.mark.parametrize("op", EXACT_UNARY)
 def test_unary_exact(op):
     rng = np.random.default_rng(11)
