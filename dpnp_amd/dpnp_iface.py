@@ -596,6 +596,8 @@ def isclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
 
 def where(condition, x=None, y=None, /, *, order="K", out=None):
     """Elements of `x` where `condition` holds, else of `y`."""
+    if out is None and type(condition) is dpnp_array and type(x) is dpnp_array and type(y) is dpnp_array:
+        return _wrap(dpt.where(condition._array_obj, x._array_obj, y._array_obj, order=order))
     missing = (x is None, y is None).count(True)
     if missing == 1:
         raise ValueError("Must provide both 'x' and 'y' or neither.")

@@ -40,6 +40,13 @@ def _resolve_two_weak_types(d1, d2):
 def where(condition, x1, x2, /, *, order="K", out=None):
     """Elements of `x1` where `condition` is true, of `x2` elsewhere; the three operands
     broadcast together and the result has the promoted dtype of `x1` and `x2`."""
+    if out is None and order == "K" and type(condition) is usm_ndarray and type(x1) is usm_ndarray \
+            and type(x2) is usm_ndarray and x1._dtype == x2._dtype and condition._shape == x1._shape == x2._shape \
+            and condition._is_c_contiguous() and x1._is_c_contiguous() and x2._is_c_contiguous() and x1.size:
+        # three C-contiguous arrays of one shape, branches of one dtype: nothing to promote, broadcast or lay out
+        r = usm_ndarray._new_contiguous(x1._shape, x1._dtype)
+        ti._where(condition=condition, x1=x1, x2=x2, dst=r)
+        return r
     if not isinstance(condition, usm_ndarray):
         raise TypeError(f"Expecting dpnp_amd.tensor.usm_ndarray type, got {type(condition)}")
     if order not in ("K", "C", "F", "A"):
