@@ -38,7 +38,9 @@ template <class Op, class T> struct UnaryFn {
 // An op may split its work in two phases for element type T (Op::two_phase<T>): fast(a, b) is
 // straight-line code that gives the result or NaN where it does not apply, fixup(r, a, b) branches to the
 // complete routine for those.  The contiguous kernel runs the first phase for all elements of a pack
-// before the second, so that the chains of the elements interleave (see ew_contig_pack).
+// before the second, so that the chains of the elements interleave (see ew_contig_pack).  Such an op
+// also names arguments with a cheap exact form (cheap_applies / cheap), which a wave takes alone when
+// all its lanes have them.
 template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
 template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct BinaryFn {
@@ -46,6 +48,9 @@ template <class Op, class T> struct BinaryFn {
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
     DPX_D auto fast(V<T> a, V<T> b) const { return Op::template fast<T>(a, b); }
     DPX_D auto fixup(V<T> r, V<T> a, V<T> b) const { return Op::template fixup<T>(r, a, b); }
+    // arguments with a cheap exact form, taken when every lane of the wave has them
+    DPX_D bool cheap_applies(V<T> a, V<T> b) const { return Op::template cheap_applies<T>(a, b); }
+    DPX_D auto cheap(V<T> a, V<T> b) const { return Op::template cheap<T>(a, b); }
 };
 template <class Op, class T> struct rows2_enabled<UnaryFn<Op, T>> : std::true_type {};
 template <class Op, class T> struct rows2_enabled<BinaryFn<Op, T>> : std::true_type {};

@@ -130,6 +130,14 @@ def test_float32_pow_over_the_whole_range():
     assert own.sum() > n // 4 and (~own).sum() > n // 10
     assert_ulp(got[own], exact[own], 0.52)
     assert_ulp(got[~own], exact[~own], 2.0)                          # the device library's powf
+    # x ** 2 is the rounded product, for every float type, array or scalar exponent, special values included
+    for dt in ("f2", "f4", "f8"):
+        b = np.concatenate([random_array(rng, 4000, dt, -300, 300), np.array([0.0, -0.0, np.inf, -np.inf, np.nan], dtype=dt)])
+        with np.errstate(all="ignore"):
+            want = b * b
+        assert_same(host(dpt.pow(dev(b), dev(np.full(b.shape, 2, dtype=dt)))), want)
+        assert_same(host(dpt.pow(dev(b), 2)), want)
+        assert_same(host(dpt.pow(dev(b)[::-1], 2.0)), want[::-1])
     for dt in ("f2",):
         xh, yh = rng.uniform(0.1, 8, 5000).astype(dt), rng.uniform(-4, 4, 5000).astype(dt)
         with np.errstate(all="ignore"):
