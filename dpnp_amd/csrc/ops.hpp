@@ -409,6 +409,24 @@ DPX_D double cos_f64(double x)
     return ((q + 1) & 2) ? -v : v;
 }
 
+// sin and cos of one argument from one reduction (the complex functions need both)
+DPX_D void sincos_both_f64(double x, double &sn, double &cs)
+{
+    const double a = __builtin_fabs(x);
+    if (!(a < TRIG_FAST_LIMIT)) {
+        sn = ::sin(x);
+        cs = ::cos(x);
+        return;
+    }
+    double s, c;
+    const int q = sincos_f64(x, s, c);
+    double vs = (q & 1) ? c : s;
+    vs = (q & 2) ? -vs : vs;
+    sn = a < 0x1p-27 ? x : vs;
+    const double vc = (q & 1) ? s : c;
+    cs = ((q + 1) & 2) ? -vc : vc;
+}
+
 // ---- fp64 asin, acos -----------------------------------------------------------------------------
 // The device library's routines run at 49 % (asin) and 69 % (acos) of the HBM rate on 2^26 doubles:
 // two branches with a full division each and a square root, and a wave whose lanes straddle |x| = 1/2
@@ -611,6 +629,12 @@ template <class T> DPX_D bool m_isinf(T x)
 // reference gets these from the SYCL complex library, results agree to rounding error for
 // finite arguments of moderate size) -----------------------------------------------------------
 template <class R> DPX_D bool m_finite(R v) { return v == v && !m_isinf(v); }
+template <class R> DPX_D void m_sincos(R x, R &s, R &c)
+{
+    if constexpr (std::is_same_v<R, double>) sincos_both_f64(x, s, c);
+    else ::sincosf(x, &s, &c);
+}
+
 // exp with the non-finite cases of libtensor/include/kernels/elementwise_functions/exp.hpp:75-132
 template <class R> DPX_D cplx<R> c_exp(cplx<R> z)
 {
@@ -620,7 +644,9 @@ template <class R> DPX_D cplx<R> c_exp(cplx<R> z)
         if (!m_finite(y)) return {q_nan, q_nan};
         const R e = m_exp(x);
         if (y == R(0)) return {e, y};
-        return {e * m_cos(y), e * m_sin(y)};
+        R sn, cs;
+        m_sincos(y, sn, cs);
+        return {e * cs, e * sn};
     }
     if (x != x) return (y == R(0)) ? z : cplx<R>{x, q_nan};
     if (!m_signbit(x)) { // +inf
@@ -700,7 +726,9 @@ template <class R> DPX_D cplx<R> c_sinh(cplx<R> z)
     const bool xf = m_finite(x), yf = m_finite(y);
     if (xf && yf) {
         if (y == R(0)) return {m_sinh(x), y};
-        return {m_sinh(x) * m_cos(y), m_cosh(x) * m_sin(y)};
+        R sn, cs;
+        m_sincos(y, sn, cs);
+        return {m_sinh(x) * cs, m_cosh(x) * sn};
     }
     if (x == R(0) && !yf) return {m_copysign(R(0), x * (y - y)), y - y};
     if (y == R(0) && !xf) return (x != x) ? cplx<R>{x, y} : cplx<R>{x, m_copysign(R(0), y)};
@@ -718,7 +746,9 @@ template <class R> DPX_D cplx<R> c_cosh(cplx<R> z)
     const bool xf = m_finite(x), yf = m_finite(y);
     if (xf && yf) {
         if (y == R(0)) return {m_cosh(x), x * y};
-        return {m_cosh(x) * m_cos(y), m_sinh(x) * m_sin(y)};
+        R sn, cs;
+        m_sincos(y, sn, cs);
+        return {m_cosh(x) * cs, m_sinh(x) * sn};
     }
     if (x == R(0) && !yf) return {q_nan, m_copysign(R(0), x * q_nan)};
     if (y == R(0) && !xf) return {x * x, m_copysign(R(0), x) * y};
