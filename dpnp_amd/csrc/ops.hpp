@@ -994,12 +994,28 @@ template <int WHICH> struct LogicalOp { // logical_and.hpp / logical_or.hpp / lo
         else return x != y;
     }
 };
+// Truncated quotient of two integers of at most 16 bits, b != 0, through the float reciprocal: the
+// integer division sequence is about 35 instructions and a pack of 1-byte elements holds sixteen.
+// Two such numbers have a quotient that is either an integer or at least 2^-16 away from one in
+// relative terms, the product with the reciprocal is off by 2^-22 at most, and the factor
+// 1 + 2^-20 lifts exact quotients back over the integer without carrying any other across one.
+template <class T> DPX_D int small_int_quotient(T a, T b)
+{
+    static_assert(sizeof(T) <= 2);
+    return (int)(((float)(int)a * __builtin_amdgcn_rcpf((float)(int)b)) * 1.00000095367431640625f);
+}
 struct FloorDivOp { // floor_divide.hpp:63-86: ints (x // 0 == 0) and real fp
     template <class T> static constexpr bool ok = is_int_v<T> || is_fp_v<T>;
     template <class T> using out = T;
     template <class T> DPX_D static T apply(T a, T b)
     {
-        if constexpr (is_int_v<T>) {
+        if constexpr (is_int_v<T> && sizeof(T) <= 2) {
+            // branch-free for the narrow types: 32-bit arithmetic, the quotient of -128 by -1 wraps in the cast
+            const int q = small_int_quotient(a, b), m = (int)a - q * (int)b;
+            const int r = q - ((m != 0) && ((m < 0) != ((int)b < 0)));
+            return b == T(0) ? T(0) : (T)r;
+        }
+        else if constexpr (is_int_v<T>) {
             if (b == T(0)) return T(0);
             if constexpr (std::is_signed_v<T>) {
                 if (b == T(-1)) return (T)(0 - (std::make_unsigned_t<T>)a); // INT_MIN // -1 wraps
@@ -1019,7 +1035,12 @@ struct RemainderOp { // remainder.hpp: Python-style modulo, x % 0 == 0 for ints
     template <class T> using out = T;
     template <class T> DPX_D static T apply(T a, T b)
     {
-        if constexpr (is_int_v<T>) {
+        if constexpr (is_int_v<T> && sizeof(T) <= 2) {
+            const int q = small_int_quotient(a, b), m = (int)a - q * (int)b;
+            const int r = (m != 0 && ((m < 0) != ((int)b < 0))) ? m + (int)b : m;
+            return b == T(0) ? T(0) : (T)r;
+        }
+        else if constexpr (is_int_v<T>) {
             if (b == T(0)) return T(0);
             if constexpr (std::is_signed_v<T>) {
                 if (b == T(-1)) return T(0);

@@ -111,6 +111,33 @@ def test_binary_ulp(op):
                 assert_same(host(dpt.pow(dev(a[nonneg]), dev(b[nonneg]))), np.power(a[nonneg], b[nonneg]))
 
 
+@pytest.mark.parametrize("op", ["floor_divide", "remainder"])
+def test_narrow_integer_division_every_pair(op):
+    """floor_divide and remainder of 1- and 2-byte integers go through the float reciprocal: every
+    (dividend, divisor) pair of int8 and uint8, and 16-bit operands over their whole range with the
+    divisors that sit next to zero and at the ends."""
+    for dt in ("i1", "u1"):
+        info = np.iinfo(dt)
+        v = np.arange(info.min, info.max + 1).astype(dt)
+        a, b = [m.ravel() for m in np.meshgrid(v, v)]
+        assert_same(host(getattr(dpt, op)(dev(a), dev(b))), orc.binary(op, a, b))
+    rng = np.random.default_rng(5)
+    for dt in ("i2", "u2"):
+        info = np.iinfo(dt)
+        n = 400000
+        a = rng.integers(info.min, info.max + 1, n).astype(dt)
+        b = rng.integers(info.min, info.max + 1, n).astype(dt)
+        b[: n // 4] = rng.integers(max(info.min, -40), 41, n // 4).astype(dt)
+        edge = np.array([info.min, info.max, 0, 1, 2, 3, info.max - 1] + ([-1, -2, info.min + 1] if info.min < 0 else []), dtype=dt)
+        ea, eb = [m.ravel() for m in np.meshgrid(edge, edge)]
+        a, b = np.concatenate([a, ea]), np.concatenate([b, eb])
+        # exact multiples, where the reciprocal product must not fall below the integer
+        k = rng.integers(1, 180, 20000)
+        d = rng.integers(1, 180, 20000)
+        a, b = np.concatenate([a, (k * d).astype(dt)]), np.concatenate([b, d.astype(dt)])
+        assert_same(host(getattr(dpt, op)(dev(a), dev(b))), orc.binary(op, a, b))
+
+
 def test_float32_pow_over_the_whole_range():
     """pow of floats takes the library's own routine for a positive normal base with a finite exponent and
     a normal result, the device library's otherwise: every binade of the base, exponents that overflow,
