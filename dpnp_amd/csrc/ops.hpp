@@ -1344,11 +1344,13 @@ struct LogaddexpOp { // logaddexp.hpp with libtensor/include/utils/math_utils.hp
     template <class T> DPX_D static T apply(T x, T y)
     {
         if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x, (float)y);
-        if (x == y) return x + m_log(T(2)); // also handles equal infinities
+        // one evaluation serves both orders of the operands (a wave with lanes of both kinds ran two):
+        // max + log1p(exp(-|d|)); a NaN operand passes
+        // through the arithmetic as NaN and the equal case is picked at the end
         const T d = x - y;
-        if (d > T(0)) return x + m_log1p(m_exp(-d));
-        if (d <= T(0)) return y + m_log1p(m_exp(d));
-        return d; // NaN
+        const T hi = d > T(0) ? x : y;
+        const T r = hi + m_log1p(m_exp(d > T(0) ? -d : d));
+        return (x == y) ? x + T(0.693147180559945309417232121458176568) : r; // equal, also equal infinities
     }
 };
 struct NextafterOp {
@@ -1491,11 +1493,10 @@ struct Logaddexp2Op { // logaddexp2.hpp: log2(2**x + 2**y)
     {
         if constexpr (std::is_same_v<T, half_t>) return (half_t)apply<float>((float)x, (float)y);
         constexpr T log2e = T(1.442695040888963407359924681001892137);
-        if (x == y) return x + T(1); // also equal infinities
-        const T d = x - y;
-        if (d > T(0)) return x + log2e * m_log1p(m_exp2(-d));
-        if (d <= T(0)) return y + log2e * m_log1p(m_exp2(d));
-        return d; // NaN
+        const T d = x - y; // as in LogaddexpOp: one evaluation for both orders
+        const T hi = d > T(0) ? x : y;
+        const T r = hi + log2e * m_log1p(m_exp2(d > T(0) ? -d : d));
+        return (x == y) ? x + T(1) : r; // equal, also equal infinities
     }
 };
 struct HeavisideOp { // heaviside.hpp: NaN -> NaN, 0 -> second argument, else x > 0
