@@ -157,6 +157,10 @@ def test_float32_pow_over_the_whole_range():
     assert own.sum() > n // 4 and (~own).sum() > n // 10
     assert_ulp(got[own], exact[own], 0.52)
     assert_ulp(got[~own], exact[~own], 2.0)                          # the device library's powf
+    # the strided and the transposing kernels evaluate element by element: the same values
+    assert_same(host(dpt.pow(dev(x)[::2], dev(y)[::2])), got[::2])
+    xm, ym = x[:160000].reshape(400, 400), y[:160000].reshape(400, 400)
+    assert_same(host(dpt.pow(dev(xm).T, dev(ym).T, order="C")), got[:160000].reshape(400, 400).T)
     # x ** 2 is the rounded product, for every float type, array or scalar exponent, special values included
     for dt in ("f2", "f4", "f8"):
         b = np.concatenate([random_array(rng, 4000, dt, -300, 300), np.array([0.0, -0.0, np.inf, -np.inf, np.nan], dtype=dt)])
