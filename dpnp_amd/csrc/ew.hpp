@@ -163,6 +163,24 @@ DPX_D void ew_contig_body(const Fn &fn, int64_t n, uint32_t bcast, uint32_t peri
     };
     if (block_base + (int64_t)blockDim.x * E * U <= n) { // the usual case: every load first
         std::tuple<pack<Ins, E>...> v[U];
+        if (bcast == 0) {
+            // every input has an element per output element: a path of its own, because with one element
+            // per pack (16-byte elements) the compiler folds the loads of all modes into one instruction
+            // and the streaming hint of this one is lost (complex128 add: 77 % of the HBM rate)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t base = block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E;
+                ((std::get<I>(v[u]) = load_pack<Ins, E>((const Ins *)in.p[I] + base)), ...);
+            }
+            // nothing to execute; it ends the run of instructions this path has in common with the other one,
+            // which the compiler would otherwise move behind the point where the two meet, the last load included
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                ew_contig_pack<Fn, Out, Ins...>(fn, out, block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E,
+                                                v[u], seq);
+            return; // (a path to the end: loads that met the other modes' loads again would be folded with them)
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u)
             load(block_base + ((int64_t)u * (int)blockDim.x + threadIdx.x) * E, v[u]);
