@@ -56,6 +56,54 @@ struct RedLaunch {
     // RedIndex, whose far part of the kernel-argument segment costs them a dependent fetch at start-up
     int32_t nd_i1;
     int64_t istr0, dstr0, astr0;
+    // reduced dims that do not collapse into one run (walk != 0): the reduced space as three digits
+    // (extents wd, element strides ws; missing leading digits have extent 1), counted in `units` units of the
+    // last digit: 16-byte packs along a unit-stride last dim of `inner` elements (vec != 0: the last extent is
+    // the packs per run, the last one of a run possibly partial), else single elements.  `chunk` is in units.
+    // (The column kernel walks whole rows: its units are the positions of the reduced space.)
+    int32_t walk;
+    int64_t units;
+    int64_t wd[3], ws[3];
+    int64_t istep; // walked column reductions: src stride of the inner iteration dim
+};
+
+// Position in a three-digit reduced space that moves by a fixed number of units per step: the element
+// offset is kept up to date by additions, so that no access needs a division.  Digit 0 never wraps for
+// positions inside the space and is not kept.
+struct RedWalker {
+    int64_t k, i1, off;            // digits 2 and 1, element offset
+    int64_t sk, s1, soff, w2, w1;  // the step's digits and offset; offset corrections of a carry out of digit 2, 1
+    int64_t d2, d1;
+    DPX_D void start(const RedLaunch &L, int64_t q, int64_t step)
+    {
+        d2 = L.wd[2];
+        d1 = L.wd[1];
+        w2 = L.ws[1] - d2 * L.ws[2];
+        w1 = L.ws[0] - d1 * L.ws[1];
+        sk = step % d2;
+        const int64_t t = step / d2;
+        s1 = t % d1;
+        soff = (t / d1) * L.ws[0] + s1 * L.ws[1] + sk * L.ws[2];
+        k = q % d2;
+        const int64_t tq = q / d2;
+        i1 = tq % d1;
+        off = (tq / d1) * L.ws[0] + i1 * L.ws[1] + k * L.ws[2];
+    }
+    DPX_D void advance()
+    {
+        k += sk;
+        i1 += s1;
+        off += soff;
+        if (k >= d2) {
+            k -= d2;
+            i1 += 1;
+            off += w2;
+        }
+        if (i1 >= d1) {
+            i1 -= d1;
+            off += w1;
+        }
+    }
 };
 
 template <class T> DPX_D T shfl_down_any(T v, int off)
@@ -583,6 +631,70 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                 for (; pos < end; pos += G) acc[0] = P::combine(acc[0], P::pre(load_one(p + pos), a));
             }
         }
+        else if (L.walk) {
+            const In *p = src + so;
+            const int64_t uend = (beg + L.chunk < L.units) ? beg + L.chunk : L.units;
+            const int64_t c = L.inner;
+            // MODE 0: units are elements; 1: packs, every run a whole number of them; 2: packs, the last one of
+            // a run partial: it is read as the whole pack that ends with the run's last element (a run holds at
+            // least one pack) and the elements it shares with the pack before are left out, so that every
+            // lane issues the same loads whatever its units are
+            auto walk = [&](auto mode_tag) {
+                constexpr int MODE = decltype(mode_tag)::value;
+                RedWalker w;
+                int64_t q = beg + lane;
+                w.start(L, q, G);
+                auto skipped = [&](int64_t k) {
+                    const int64_t rem = c - k * E;
+                    return rem < E ? E - (int)rem : 0;
+                };
+                for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
+                    if constexpr (MODE == 0) {
+                        In v[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) {
+                            v[u] = load_one(p + w.off);
+                            w.advance();
+                        }
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) acc[u] = P::combine(acc[u], P::pre(v[u], a));
+                    }
+                    else {
+                        pack<In, E> v[RED_U];
+                        int skip[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) {
+                            skip[u] = MODE == 2 ? skipped(w.k) : 0;
+                            v[u] = load_pack<In, E>(p + w.off - skip[u]);
+                            w.advance();
+                        }
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u)
+#pragma unroll
+                            for (int e = 0; e < E; ++e) {
+                                const Acc t = P::combine(acc[u], P::pre(v[u].v[e], a));
+                                acc[u] = (MODE == 2 && e < skip[u]) ? acc[u] : t;
+                            }
+                    }
+                }
+                for (; q < uend; q += G) {
+                    if constexpr (MODE == 0) acc[0] = P::combine(acc[0], P::pre(load_one(p + w.off), a));
+                    else {
+                        const int skip = MODE == 2 ? skipped(w.k) : 0;
+                        const pack<In, E> v = load_pack<In, E>(p + w.off - skip);
+#pragma unroll
+                        for (int e = 0; e < E; ++e) {
+                            const Acc t = P::combine(acc[0], P::pre(v.v[e], a));
+                            acc[0] = (MODE == 2 && e < skip) ? acc[0] : t;
+                        }
+                    }
+                    w.advance();
+                }
+            };
+            if (!L.vec) walk(std::integral_constant<int, 0>{});
+            else if (c % E == 0) walk(std::integral_constant<int, 1>{});
+            else walk(std::integral_constant<int, 2>{});
+        }
         else {
             const In *p = src + so;
             for (int64_t pos = beg + lane; pos < end; pos += G)
@@ -643,7 +755,9 @@ template <class P, int E> DPX_D void cols_block_combine(typename P::Acc (&v)[E],
     }
 }
 
-template <class P>
+// WALK: the rows of the reduced space are found by RedWalker (several reduced dims) and the inner iteration dim
+// may have any src stride (L.istep; not 1: single elements, L.vec == 0)
+template <class P, bool WALK = false>
 __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, RedLaunch L,
                                                                  const typename P::In *src, typename P::Out *dst,
                                                                  Slot<typename P::Acc> *partial,
@@ -696,10 +810,21 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             for (int e = 0; e < E; ++e)
                 if (e < ecnt && col0 + e < L.inner) a[e] = P::load_aux(aux + ao + (col0 + e) * ix.aux_str[last]);
         }
-        const In *p = src + so + col0;
+        const In *p = src + so + col0 * (WALK ? L.istep : 1);
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         int64_t r = beg + ty;
+        RedWalker w;
+        if constexpr (WALK) w.start(L, r, TY);
+        // offset of this thread's next row (each call moves on by TY rows)
+        auto next_row = [&](int64_t row) {
+            if constexpr (WALK) {
+                const int64_t off = w.off;
+                w.advance();
+                return off;
+            }
+            else return row * L.rstride;
+        };
         if (L.vec) {
             // the pack that holds the end of a row is read element by element: its own copy of the
             // loops, so the loads of the usual case stay free of branches
@@ -720,14 +845,14 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                 for (; r + (NL - 1) * TY < end; r += NL * TY) {
                     pack<In, E> v[NL];
 #pragma unroll
-                    for (int u = 0; u < NL; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+                    for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
 #pragma unroll
                     for (int u = 0; u < NL; ++u)
 #pragma unroll
                         for (int e = 0; e < E; ++e) acc[u % U][e] = P::combine(acc[u % U][e], P::pre(v[u].v[e], a[e]));
                 }
                 for (; r < end; r += TY) {
-                    pack<In, E> v = load(p + r * L.rstride);
+                    pack<In, E> v = load(p + next_row(r));
 #pragma unroll
                     for (int e = 0; e < E; ++e) acc[0][e] = P::combine(acc[0][e], P::pre(v.v[e], a[e]));
                 }
@@ -739,11 +864,11 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             for (; r + (LOADS - 1) * TY < end; r += LOADS * TY) {
                 In v[LOADS];
 #pragma unroll
-                for (int u = 0; u < LOADS; ++u) v[u] = load_one(p + (r + u * TY) * L.rstride);
+                for (int u = 0; u < LOADS; ++u) v[u] = load_one(p + next_row(r + u * TY));
 #pragma unroll
                 for (int u = 0; u < LOADS; ++u) acc[u % U][0] = P::combine(acc[u % U][0], P::pre(v[u], a[0]));
             }
-            for (; r < end; r += TY) acc[0][0] = P::combine(acc[0][0], P::pre(load_one(p + r * L.rstride), a[0]));
+            for (; r < end; r += TY) acc[0][0] = P::combine(acc[0][0], P::pre(load_one(p + next_row(r)), a[0]));
         }
     }
     Acc v[E];

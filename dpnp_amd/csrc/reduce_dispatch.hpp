@@ -92,8 +92,12 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         while ((size_t)block * E * sizeof(Acc) > 65536) block /= 2;
         if (block < (1 << pl.L.g_log2)) return fail(DPX_ERR_NOT_IMPLEMENTED, "column reduction: accumulator too wide");
         const size_t smem = (size_t)block * E * sizeof(Acc);
-        hipLaunchKernelGGL((red_cols_kernel<P>), dim3((unsigned)pl.grid), dim3(block), smem, stream, pl.ix, pl.L, sp,
-                           dp, partial, ap, counters);
+        if (pl.L.walk)
+            hipLaunchKernelGGL((red_cols_kernel<P, true>), dim3((unsigned)pl.grid), dim3(block), smem, stream, pl.ix,
+                               pl.L, sp, dp, partial, ap, counters);
+        else
+            hipLaunchKernelGGL((red_cols_kernel<P, false>), dim3((unsigned)pl.grid), dim3(block), smem, stream, pl.ix,
+                               pl.L, sp, dp, partial, ap, counters);
     }
     else if (pl.path == DPX_PATH_RED_SHORT_ROWS) {
         const size_t smem = (size_t)pl.L.chunk * srow_pitch<In>((int)pl.L.n) * sizeof(In); // at most 32 KiB

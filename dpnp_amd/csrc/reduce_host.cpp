@@ -1,4 +1,6 @@
 // Reductions: validation and launch planning (no element types here).
+#include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include "reduce_dispatch.hpp"
 
@@ -153,7 +155,18 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const int last = nd_i - 1;
     const int64_t inner = ishape[last];
     const bool contig_red = nd_r == 1 && (rstr[0][0] == 1 || n == 1);
-    const bool cols_ok = !contig_red && nd_r == 1 && istr[0][last] == 1 && inner > 1;
+    const bool cols_plain = !contig_red && nd_r == 1 && istr[0][last] == 1 && inner > 1;
+    // the same arrangement (threads side by side along the inner iteration dim, rows of the reduced space walked
+    // by offset) when that dim is the one src moves least along, whatever its stride and however many reduced
+    // dims stay apart: axes (0, 2) of a 4-d array, columns of a matrix view that takes every other column
+    bool cols_walk = false;
+    if (!contig_red && !cols_plain && !arg && nd_r <= 3 && inner > 1 && istr[0][last] != 0) {
+        int64_t smin = INT64_MAX;
+        for (int d = 0; d < nd_r; ++d) smin = std::min(smin, rstr[0][d] < 0 ? -rstr[0][d] : rstr[0][d]);
+        const int64_t si = istr[0][last] < 0 ? -istr[0][last] : istr[0][last];
+        cols_walk = si < smin;
+    }
+    const bool cols_ok = cols_plain || cols_walk;
     RedLaunch &L = pl.L;
 
     if (contig_red && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
@@ -173,10 +186,30 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     if (!cols_ok) {
         // ---- rows / generic -------------------------------------------------------
-        const bool vec = contig_red; // packs need no alignment
-        const int e = vec ? E : 1;
+        bool vec = contig_red; // packs need no alignment
+        int e = vec ? E : 1;
+        int64_t work = n; // what lanes and splits share out: elements, or the units of a walked space
+        if (!contig_red && !arg && nd_r <= 3) {
+            // reduced dims that stay apart (a sliced matrix summed whole, axes (0, 2) of a 3-d array, a
+            // strided run): lanes walk the reduced space in units of its last dim, 16-byte packs when that
+            // dim has unit stride and holds at least one
+            const int64_t c = rshape[nd_r - 1], s_in = rstr[0][nd_r - 1];
+            vec = s_in == 1 && c >= E;
+            const int64_t per_run = vec ? cdiv(c, E) : c;
+            for (int j = 0; j < 3; ++j) {
+                const int d = nd_r - 3 + j; // digit j is reduced dim d, or missing
+                L.wd[j] = d < 0 ? 1 : rshape[d];
+                L.ws[j] = d < 0 ? 0 : rstr[0][d];
+            }
+            L.wd[2] = per_run;
+            L.ws[2] = vec ? E : s_in;
+            L.walk = 1;
+            L.inner = c;
+            L.units = work = (n / c) * per_run;
+            e = 1;
+        }
         L.vec = vec ? 1 : 0;
-        rows_geometry(n, e, L.g_log2, pl.block);
+        rows_geometry(work, e, L.g_log2, pl.block);
         const int64_t G = (int64_t)1 << L.g_log2;
         const int64_t opb = (G <= 64) ? 256 / G : 1;
         const int64_t oblocks = cdiv(m, opb);
@@ -185,13 +218,15 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         // splitting needs a whole block per output (G > 64) and one ticket counter per output
         // (the largest split count whose grid stays within the target: a grid a little above it
         // runs a second, nearly empty round of blocks and loses 10-15 points of bandwidth)
-        if (G > 64 && 2 * oblocks <= target && oblocks <= RED_MAX_TICKETS && n >= 2 * per_pass)
-            splits = std::min(target / oblocks, cdiv(n, per_pass));
+        // (single elements in flight instead of packs: more blocks per CU make up for the bytes)
+        const int64_t tgt = (L.walk && !vec) ? target * (in_size >= 16 ? 1 : (in_size == 8 ? 2 : 4)) : target;
+        if (G > 64 && 2 * oblocks <= tgt && oblocks <= RED_MAX_TICKETS && work >= 2 * per_pass)
+            splits = std::min(tgt / oblocks, cdiv(work, per_pass));
         if (arg && G > 64 && oblocks <= RED_MAX_TICKETS)
             splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
-        int64_t chunk = cdiv(n, splits);
+        int64_t chunk = cdiv(work, splits);
         chunk = cdiv(chunk, G * e) * (G * e);
-        splits = cdiv(n, chunk);
+        splits = cdiv(work, chunk);
         L.chunk = chunk;
         L.splits = (int32_t)splits;
         // many blocks per output: two levels of tickets (groups of 32 blocks), while the group
@@ -206,7 +241,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
-    if (!arg && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
+    if (!cols_walk && !arg && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
         tune_int("DPX_RED_FLAT", 1) != 0) { // (sweep override: 0 keeps the column kernel)
         // a row-major matrix with rows shorter than 512 bytes: one flat stream of packs, a block of
         // T threads with T * E a multiple of the row length (see red_flat_kernel)
@@ -240,17 +275,29 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
             }
         }
     }
-    const bool vec = true; // packs need no alignment; the kernels read a row's last pack by element
-    const int e = E;
+    // packs need no alignment; the kernels read a row's last pack by element
+    const bool vec = !cols_walk || istr[0][last] == 1;
+    const int e = vec ? E : 1;
     L.vec = vec ? 1 : 0;
     L.rstride = rstride;
     L.inner = inner;
+    if (cols_walk) {
+        for (int j = 0; j < 3; ++j) {
+            const int d = nd_r - 3 + j; // digit j is reduced dim d, or missing
+            L.wd[j] = d < 0 ? 1 : rshape[d];
+            L.ws[j] = d < 0 ? 0 : rstr[0][d];
+        }
+        L.walk = 1;
+        L.units = n;
+        L.istep = istr[0][last];
+    }
     // TX threads side by side cover 512 contiguous bytes of a row (32 x 16 B); up to 16 thread
     // rows walk down the reduced axis: 512-thread blocks, one per CU when splitting
     // thread rows wanted for n reduced rows (4 or more rows per thread)
     const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
     // with a single thread row a whole wave lies side by side and nothing is combined in LDS
-    int lg = std::min(ty == 1 ? 6 : 5, ceil_log2(cdiv(inner, e)));
+    // (single elements at a stride: a whole wave side by side as well, 64 elements are the least it should span)
+    int lg = std::min((ty == 1 || !vec) ? 6 : 5, ceil_log2(cdiv(inner, e)));
     const int forced = tune_int("DPX_COLS_TX_LOG2", -1); // sweep override, product build: default
     if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(inner, e)), forced);
     L.g_log2 = lg;

@@ -781,3 +781,76 @@ def test_argmax_argmin_along_short_rows(dt):
         out = dpt.zeros(2 * 4001, dtype="i8")
         dpt.argmax(dev(a[:, 1, :]), axis=1, out=out[::2])
         assert_same(host(out)[::2], orc.argreduce("argmax", a[:, 1, :], 1))
+
+
+# Reduced dims that do not collapse into one run: (base shape, view, axes).  The runs of the last reduced dim are
+# whole packs, ragged (a partial pack ends each run), shorter than a pack, strided, reversed; one, few and many
+# outputs; reductions large enough to be split over blocks.
+_WALKED = [
+    ((40, 50), np.s_[:, 1:-1], None),
+    ((40, 50), np.s_[1:-1, 3:], None),
+    ((700, 900), np.s_[:, 1:-1], None),
+    ((700, 900), np.s_[::2, ::2], None),
+    ((700, 900), np.s_[::-1, ::3], None),
+    ((300, 1100), np.s_[:, ::2], 1),
+    ((300, 1100), np.s_[:, ::-2], 1),
+    ((300, 1100), np.s_[:, 5:1001:3], 1),
+    ((9, 1000, 33), np.s_[:], (0, 2)),
+    ((9, 1000, 32), np.s_[:], (0, 2)),
+    ((9, 1000, 3), np.s_[:], (0, 2)),
+    ((9, 1000, 1), np.s_[:, ::2], (0, 2)),
+    ((64, 7, 4096), np.s_[:], (0, 2)),
+    ((33, 5, 4100), np.s_[:, :, 1:-2], (0, 2)),
+    ((5, 3, 70000), np.s_[:, :, 1:], (0, 2)),
+    ((2, 3, 70000), np.s_[:, :, ::2], (0, 2)),
+    ((12, 13, 14, 15), np.s_[:], (0, 2)),
+    ((12, 13, 14, 15), np.s_[:], (1, 3)),
+    ((12, 13, 14, 15), np.s_[:], (0, 3)),
+    ((12, 13, 14, 15), np.s_[:], (0, 1, 3)),
+    ((12, 13, 14, 15), np.s_[:, 1:, :, 2:], (0, 2, 3)),
+    ((12, 13, 14, 15), np.s_[:, 1:, 1:, 2:], (1, 2, 3)),
+    ((12, 13, 14, 16), np.s_[1:, 1:, 1:, ::2], None),
+    ((6, 5, 4, 3, 8), np.s_[:, 1:, 1:, 1:, 1:], None),
+    ((6, 5, 4, 3, 8), np.s_[:, 1:, 1:, 1:, 1:], (0, 2, 4)),
+    ((3, 200000), np.s_[:, 1:], None),
+    ((200000, 3), np.s_[:, 1:], None),
+    ((200000, 3), np.s_[:, :2], 1),
+    # the inner iteration dim is the one src moves least along: columns side by side, rows walked
+    ((300, 1100), np.s_[:, ::2], 0),
+    ((300, 1100), np.s_[:, ::-1], 0),
+    ((300, 1100), np.s_[::2, 7::3], 0),
+    ((12, 13, 14, 16), np.s_[:, :, :, ::2], (0, 2)),
+    ((12, 13, 14, 16), np.s_[:, :, 1:, 1:], (0, 2)),
+    ((64, 5, 64, 130), np.s_[:], (0, 2)),
+    ((3000, 2, 50, 9), np.s_[:], (0, 2)),
+    ((40, 3, 50, 2, 70), np.s_[:], (0, 2)),
+    ((7, 3, 6, 2, 5, 70), np.s_[:], (0, 2, 4)),
+    ((150000, 2, 9), np.s_[:, :, ::2], 0),
+]
+
+
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "i8", "f2", "f4", "f8", "c8", "c16"])
+@pytest.mark.parametrize("case", range(len(_WALKED)))
+def test_reduced_dims_that_stay_apart(case, dt):
+    shape, sl, axis = _WALKED[case]
+    rng = np.random.default_rng(7000 + case)
+    base = random_array(rng, shape, dt, -3, 3)
+    hv = base[sl]
+    v = dev_view_like(hv, base)
+    dt = np.dtype(dt)
+    check_sum(host(dpt.sum(v, axis=axis)), hv, axis)
+    if dt.kind != "c":
+        assert_same(host(dpt.max(v, axis=axis)), np.max(hv, axis=axis))
+        assert_same(host(dpt.min(v, axis=axis)), np.min(hv, axis=axis))
+    assert_same(host(dpt.count_nonzero(v, axis=axis)), np.asarray(np.count_nonzero(hv, axis=axis), dtype="i8"))
+    assert_same(host(dpt.any(v, axis=axis)), np.asarray(np.any(hv, axis=axis)))
+    if dt.kind == "f" and dt.itemsize >= 4:
+        tol = 1e-5 if dt.itemsize == 4 else 1e-12
+        want = np.mean(hv.astype(np.longdouble), axis=axis)
+        np.testing.assert_allclose(host(dpt.mean(v, axis=axis)), want.astype("f8"), rtol=0, atol=4 * tol)
+        want = np.var(hv.astype(np.longdouble), axis=axis)
+        np.testing.assert_allclose(host(dpt.var(v, axis=axis)), want.astype("f8"), rtol=10 * tol, atol=10 * tol)
+    if axis is None or isinstance(axis, int):
+        if dt.kind != "c":
+            assert_same(host(dpt.argmax(v, axis=axis)), np.asarray(np.argmax(hv, axis=axis)))
+            assert_same(host(dpt.argmin(v, axis=axis)), np.asarray(np.argmin(hv, axis=axis)))
