@@ -72,6 +72,7 @@ struct RedLaunch {
 // positions inside the space and is not kept.
 struct RedWalker {
     int64_t k, i1, off;            // digits 2 and 1, element offset
+    int64_t seg, sseg;             // runs of the last digit before this position (digits 0 and 1 as one number); per step
     int64_t sk, s1, soff, w2, w1;  // the step's digits and offset; offset corrections of a carry out of digit 2, 1
     int64_t d2, d1;
     DPX_D void start(const RedLaunch &L, int64_t q, int64_t step)
@@ -83,9 +84,11 @@ struct RedWalker {
         sk = step % d2;
         const int64_t t = step / d2;
         s1 = t % d1;
+        sseg = t;
         soff = (t / d1) * L.ws[0] + s1 * L.ws[1] + sk * L.ws[2];
         k = q % d2;
         const int64_t tq = q / d2;
+        seg = tq;
         i1 = tq % d1;
         off = (tq / d1) * L.ws[0] + i1 * L.ws[1] + k * L.ws[2];
     }
@@ -93,10 +96,12 @@ struct RedWalker {
     {
         k += sk;
         i1 += s1;
+        seg += sseg;
         off += soff;
         if (k >= d2) {
             k -= d2;
             i1 += 1;
+            seg += 1;
             off += w2;
         }
         if (i1 >= d1) {
@@ -1327,6 +1332,88 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
                 }
                 if (have) bidx = beg + bl;
             }
+        }
+        else if (L.walk) {
+            // as in red_rows_kernel; a lane meets its positions in increasing order, so a later value only
+            // replaces the best one when it is better
+            const int64_t uend = (beg + L.chunk < L.units) ? beg + L.chunk : L.units;
+            const int64_t c = L.inner;
+            auto walk = [&](auto mode_tag) {
+                constexpr int MODE = decltype(mode_tag)::value;
+                RedWalker w;
+                int64_t q = beg + lane;
+                w.start(L, q, G);
+                auto skipped = [&](int64_t k) {
+                    const int64_t rem = c - k * E;
+                    return rem < E ? E - (int)rem : 0;
+                };
+                // C-order position of the first element of the unit the walker stands on
+                auto unit_pos = [&]() { return MODE == 0 ? w.seg * c + w.k : w.seg * c + w.k * E; };
+                if (q < uend) {
+                    best = to_value(load_one(p + w.off));
+                    bidx = unit_pos();
+                }
+                auto take_pack = [&](const pack<T, E> &v, int skip, int64_t pos) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        const VT x = to_value(v.v[e]);
+                        if ((MODE != 2 || e >= skip) && arg_better<IS_MAX, VT>(x, best)) {
+                            best = x;
+                            bidx = pos + e;
+                        }
+                    }
+                };
+                for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
+                    int64_t pos[RED_U];
+                    if constexpr (MODE == 0) {
+                        T v[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) {
+                            pos[u] = unit_pos();
+                            v[u] = load_one(p + w.off);
+                            w.advance();
+                        }
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) {
+                            const VT x = to_value(v[u]);
+                            if (arg_better<IS_MAX, VT>(x, best)) {
+                                best = x;
+                                bidx = pos[u];
+                            }
+                        }
+                    }
+                    else {
+                        pack<T, E> v[RED_U];
+                        int skip[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) {
+                            skip[u] = MODE == 2 ? skipped(w.k) : 0;
+                            pos[u] = unit_pos() - skip[u];
+                            v[u] = load_pack<T, E>(p + w.off - skip[u]);
+                            w.advance();
+                        }
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) take_pack(v[u], skip[u], pos[u]);
+                    }
+                }
+                for (; q < uend; q += G) {
+                    if constexpr (MODE == 0) {
+                        const VT x = to_value(load_one(p + w.off));
+                        if (arg_better<IS_MAX, VT>(x, best)) {
+                            best = x;
+                            bidx = unit_pos();
+                        }
+                    }
+                    else {
+                        const int skip = MODE == 2 ? skipped(w.k) : 0;
+                        take_pack(load_pack<T, E>(p + w.off - skip), skip, unit_pos() - skip);
+                    }
+                    w.advance();
+                }
+            };
+            if (!L.vec) walk(std::integral_constant<int, 0>{});
+            else if (c % E == 0) walk(std::integral_constant<int, 1>{});
+            else walk(std::integral_constant<int, 2>{});
         }
         else {
             for (int64_t pos = beg + lane; pos < end; pos += G) {

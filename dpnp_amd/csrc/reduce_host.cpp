@@ -189,7 +189,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         bool vec = contig_red; // packs need no alignment
         int e = vec ? E : 1;
         int64_t work = n; // what lanes and splits share out: elements, or the units of a walked space
-        if (!contig_red && !arg && nd_r <= 3) {
+        if (!contig_red && nd_r <= 3) {
             // reduced dims that stay apart (a sliced matrix summed whole, axes (0, 2) of a 3-d array, a
             // strided run): lanes walk the reduced space in units of its last dim, 16-byte packs when that
             // dim has unit stride and holds at least one

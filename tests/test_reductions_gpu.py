@@ -854,3 +854,11 @@ def test_reduced_dims_that_stay_apart(case, dt):
         if dt.kind != "c":
             assert_same(host(dpt.argmax(v, axis=axis)), np.asarray(np.argmax(hv, axis=axis)))
             assert_same(host(dpt.argmin(v, axis=axis)), np.asarray(np.argmin(hv, axis=axis)))
+        if dt.kind == "f":  # the first NaN wins, as in NumPy
+            base = base.copy()
+            base[rng.random(shape) < 0.001] = np.nan
+            hv = base[sl]
+            v = dev_view_like(hv, base)
+            assert_same(host(dpt.argmax(v, axis=axis)), np.asarray(np.argmax(hv, axis=axis)))
+            assert_same(host(dpt.argmin(v, axis=axis)), np.asarray(np.argmin(hv, axis=axis)))
+            assert_same(host(dpt.max(v, axis=axis)), np.max(hv, axis=axis))
