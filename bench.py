@@ -75,6 +75,8 @@ WORKLOADS = {
             "(fp32 input and fp64 input)",
     "cfg4": "8192x8192 fp32 views A[:, ::2], A.T and a (1,4096) row: multiply, exp, where(A>0, A, B); int32 bitwise_and",
     "cfg5": "Black-Scholes over 2^26 fp64 options, call and put: one fused kernel, and the chain of elementwise calls",
+    "layouts": "fp32 2^28 elements reduced over dims that do not collapse into one run: a sliced matrix summed whole, "
+               "axes (0, 2) of 3-d and 4-d arrays, every other column (sum, max, mean, argmax)",
 }
 
 
@@ -218,6 +220,27 @@ def build_workload(name, dpnp, torch):
         ops = [("black_scholes_fused", lambda: dpnp.black_scholes(price, strike, t, r, vol, call=call, put=put), 40 * n, n),
                ("black_scholes_chain", chain, 40 * n, n)]
         return ops, "f64", "synthetic (seeded uniform price, strike [10,50), T [1,2), resident in HBM)"
+    if name == "layouts":
+        side = 1 << 14
+        n = side * side
+        A = normal((side, side))
+        X3, X3s, X4 = A.reshape(4096, 256, 256), A.reshape(256, 1024, 1024), A.reshape(128, 128, 128, 128)
+        s0, i0 = dpnp.empty((), dtype="f4"), dpnp.empty((), dtype="i8")
+        r256, r1024 = dpnp.empty(256, dtype="f4"), dpnp.empty(1024, dtype="f4")
+        r44 = dpnp.empty((128, 128), dtype="f4")
+        rs, rh, ri = dpnp.empty(side, dtype="f4"), dpnp.empty(side // 2, dtype="f4"), dpnp.empty(side, dtype="i8")
+        inner = (side - 2) * (side - 2)
+        # a [:, ::2] view occupies every line of its base: the bytes moved are the whole matrix
+        ops = [("sum_sliced_matrix", lambda: dpnp.sum(A[1:-1, 1:-1], out=s0), 4 * inner, inner),
+               ("argmax_sliced_matrix", lambda: dpnp.argmax(A[1:-1, 1:-1], out=i0), 4 * inner, inner),
+               ("sum_axes02_4096x256x256", lambda: dpnp.sum(X3, axis=(0, 2), out=r256), 4 * n, n),
+               ("max_axes02_4096x256x256", lambda: dpnp.max(X3, axis=(0, 2), out=r256), 4 * n, n),
+               ("mean_axes02_256x1024x1024", lambda: dpnp.mean(X3s, axis=(0, 2), out=r1024), 4 * n, n),
+               ("sum_axes02_128x128x128x128", lambda: dpnp.sum(X4, axis=(0, 2), out=r44), 4 * n, n),
+               ("sum_every_other_column_axis1", lambda: dpnp.sum(A[:, ::2], axis=1, out=rs), 4 * n, n // 2),
+               ("sum_every_other_column_axis0", lambda: dpnp.sum(A[:, ::2], axis=0, out=rh), 4 * n, n // 2),
+               ("argmax_every_other_column_axis1", lambda: dpnp.argmax(A[:, ::2], axis=1, out=ri), 4 * n, n // 2)]
+        return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
     raise SystemExit(f"--workload: unknown workload {name!r} (one of {', '.join(WORKLOADS)})")
 
 
@@ -229,7 +252,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--dump-steps", action="store_true", help="print every step's per-op times to stderr")
     ap.add_argument("--workload", default="metric",
-                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5, "
+                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5 or layouts, "
                          "measured the same way")
     ap.add_argument("--ops", default=None,
                     help="comma-separated subset of the workload's ops (profiling runs); 'copy' in the metric "

@@ -71,42 +71,48 @@ struct RedLaunch {
 // offset is kept up to date by additions, so that no access needs a division.  Digit 0 never wraps for
 // positions inside the space and is not kept.
 struct RedWalker {
-    int64_t k, i1, off;            // digits 2 and 1, element offset
-    int64_t seg, sseg;             // runs of the last digit before this position (digits 0 and 1 as one number); per step
-    int64_t sk, s1, soff, w2, w1;  // the step's digits and offset; offset corrections of a carry out of digit 2, 1
-    int64_t d2, d1;
-    DPX_D void start(const RedLaunch &L, int64_t q, int64_t step)
+    uint32_t k, i1;                // digits 2 and 1 (the host keeps their extents below 2^31)
+    int64_t off;                   // element offset
+    uint32_t rel;                  // C-order position of the unit's first element minus that of unit `origin`, mod 2^32
+    uint32_t sk, s1, d2, d1;       // the step's digits; extents
+    uint32_t srel, wrel;           // position change of a step; its correction when digit 2 wraps
+    int64_t soff, w2, w1;          // offset change of a step; corrections of a carry out of digit 2, 1
+    // positions: a run of the last digit holds `run` of them, a unit `per_unit` (searches; 0, 0 when not needed)
+    DPX_D void start(const RedLaunch &L, int64_t q, int64_t step, int64_t run = 0, int per_unit = 0, int64_t origin = 0)
     {
-        d2 = L.wd[2];
-        d1 = L.wd[1];
-        w2 = L.ws[1] - d2 * L.ws[2];
-        w1 = L.ws[0] - d1 * L.ws[1];
-        sk = step % d2;
-        const int64_t t = step / d2;
-        s1 = t % d1;
-        sseg = t;
-        soff = (t / d1) * L.ws[0] + s1 * L.ws[1] + sk * L.ws[2];
-        k = q % d2;
-        const int64_t tq = q / d2;
-        seg = tq;
-        i1 = tq % d1;
-        off = (tq / d1) * L.ws[0] + i1 * L.ws[1] + k * L.ws[2];
+        const int64_t D2 = L.wd[2], D1 = L.wd[1];
+        d2 = (uint32_t)D2;
+        d1 = (uint32_t)D1;
+        w2 = L.ws[1] - D2 * L.ws[2];
+        w1 = L.ws[0] - D1 * L.ws[1];
+        const int64_t t = step / D2, tq = q / D2;
+        sk = (uint32_t)(step % D2);
+        s1 = (uint32_t)(t % D1);
+        soff = (t / D1) * L.ws[0] + (int64_t)s1 * L.ws[1] + (int64_t)sk * L.ws[2];
+        k = (uint32_t)(q % D2);
+        i1 = (uint32_t)(tq % D1);
+        off = (tq / D1) * L.ws[0] + (int64_t)i1 * L.ws[1] + (int64_t)k * L.ws[2];
+        srel = (uint32_t)(t * run + (int64_t)sk * per_unit);
+        wrel = (uint32_t)(run - D2 * per_unit);
+        rel = (uint32_t)((tq - origin / D2) * run + ((int64_t)k - origin % D2) * per_unit);
     }
     DPX_D void advance()
     {
         k += sk;
         i1 += s1;
-        seg += sseg;
         off += soff;
-        if (k >= d2) {
-            k -= d2;
-            i1 += 1;
-            seg += 1;
-            off += w2;
-        }
-        if (i1 >= d1) {
-            i1 -= d1;
-            off += w1;
+        rel += srel;
+        // runs much longer than a step: no lane of the wave carries in most steps, and one branch skips the rest
+        // (which is made of selects: as branches per lane they would serialise the loads of a round)
+        if (__builtin_amdgcn_ballot_w64((k >= d2) | (i1 >= d1)) != 0) {
+            const bool c2 = k >= d2;
+            k -= c2 ? d2 : 0;
+            i1 += c2 ? 1 : 0;
+            off += c2 ? w2 : 0;
+            rel += c2 ? wrel : 0;
+            const bool c1 = i1 >= d1;
+            i1 -= c1 ? d1 : 0;
+            off += c1 ? w1 : 0;
         }
     }
 };
@@ -649,9 +655,10 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                 RedWalker w;
                 int64_t q = beg + lane;
                 w.start(L, q, G);
-                auto skipped = [&](int64_t k) {
-                    const int64_t rem = c - k * E;
-                    return rem < E ? E - (int)rem : 0;
+                const uint32_t c32 = (uint32_t)c; // (the host keeps run lengths below 2^31)
+                auto skipped = [&](uint32_t k) {
+                    const uint32_t rem = c32 - k * E;
+                    return rem < (uint32_t)E ? E - (int)rem : 0;
                 };
                 for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
                     if constexpr (MODE == 0) {
@@ -1335,52 +1342,52 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
         }
         else if (L.walk) {
             // as in red_rows_kernel; a lane meets its positions in increasing order, so a later value only
-            // replaces the best one when it is better
+            // replaces the best one when it is better.  Positions are kept relative to the chunk's first one, in
+            // 32 bits (the host keeps a chunk's positions below 2^32), and updated by selects: written as
+            // branches, sixteen dependent ones per round of loads, the kernel ran at 65 % of the HBM rate
             const int64_t uend = (beg + L.chunk < L.units) ? beg + L.chunk : L.units;
             const int64_t c = L.inner;
             auto walk = [&](auto mode_tag) {
                 constexpr int MODE = decltype(mode_tag)::value;
+                constexpr int UE = MODE == 0 ? 1 : E; // positions per unit
                 RedWalker w;
                 int64_t q = beg + lane;
-                w.start(L, q, G);
-                auto skipped = [&](int64_t k) {
-                    const int64_t rem = c - k * E;
-                    return rem < E ? E - (int)rem : 0;
+                w.start(L, q, G, c, UE, beg);
+                const int64_t pbase = (beg / L.wd[2]) * c + (beg % L.wd[2]) * UE;
+                const uint32_t c32 = (uint32_t)c; // (the host keeps run lengths below 2^31)
+                auto skipped = [&](uint32_t k) {
+                    const uint32_t rem = c32 - k * E;
+                    return rem < (uint32_t)E ? E - (int)rem : 0;
                 };
-                // C-order position of the first element of the unit the walker stands on
-                auto unit_pos = [&]() { return MODE == 0 ? w.seg * c + w.k : w.seg * c + w.k * E; };
-                if (q < uend) {
+                // position of the first element of the unit the walker stands on, relative to pbase
+                auto unit_rel = [&]() { return w.rel; };
+                uint32_t bl = 0;
+                const bool have = q < uend;
+                if (have) {
                     best = to_value(load_one(p + w.off));
-                    bidx = unit_pos();
+                    bl = unit_rel();
                 }
-                auto take_pack = [&](const pack<T, E> &v, int skip, int64_t pos) {
+                auto take = [&](VT x, bool counts, uint32_t rel) {
+                    const bool better = counts & arg_better<IS_MAX, VT>(x, best);
+                    best = better ? x : best;
+                    bl = better ? rel : bl;
+                };
+                auto take_pack = [&](const pack<T, E> &v, int skip, uint32_t rel) {
 #pragma unroll
-                    for (int e = 0; e < E; ++e) {
-                        const VT x = to_value(v.v[e]);
-                        if ((MODE != 2 || e >= skip) && arg_better<IS_MAX, VT>(x, best)) {
-                            best = x;
-                            bidx = pos + e;
-                        }
-                    }
+                    for (int e = 0; e < E; ++e) take(to_value(v.v[e]), MODE != 2 || e >= skip, rel + e);
                 };
                 for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
-                    int64_t pos[RED_U];
+                    uint32_t rel[RED_U];
                     if constexpr (MODE == 0) {
                         T v[RED_U];
 #pragma unroll
                         for (int u = 0; u < RED_U; ++u) {
-                            pos[u] = unit_pos();
+                            rel[u] = unit_rel();
                             v[u] = load_one(p + w.off);
                             w.advance();
                         }
 #pragma unroll
-                        for (int u = 0; u < RED_U; ++u) {
-                            const VT x = to_value(v[u]);
-                            if (arg_better<IS_MAX, VT>(x, best)) {
-                                best = x;
-                                bidx = pos[u];
-                            }
-                        }
+                        for (int u = 0; u < RED_U; ++u) take(to_value(v[u]), true, rel[u]);
                     }
                     else {
                         pack<T, E> v[RED_U];
@@ -1388,28 +1395,23 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
 #pragma unroll
                         for (int u = 0; u < RED_U; ++u) {
                             skip[u] = MODE == 2 ? skipped(w.k) : 0;
-                            pos[u] = unit_pos() - skip[u];
+                            rel[u] = unit_rel() - skip[u];
                             v[u] = load_pack<T, E>(p + w.off - skip[u]);
                             w.advance();
                         }
 #pragma unroll
-                        for (int u = 0; u < RED_U; ++u) take_pack(v[u], skip[u], pos[u]);
+                        for (int u = 0; u < RED_U; ++u) take_pack(v[u], skip[u], rel[u]);
                     }
                 }
                 for (; q < uend; q += G) {
-                    if constexpr (MODE == 0) {
-                        const VT x = to_value(load_one(p + w.off));
-                        if (arg_better<IS_MAX, VT>(x, best)) {
-                            best = x;
-                            bidx = unit_pos();
-                        }
-                    }
+                    if constexpr (MODE == 0) take(to_value(load_one(p + w.off)), true, unit_rel());
                     else {
                         const int skip = MODE == 2 ? skipped(w.k) : 0;
-                        take_pack(load_pack<T, E>(p + w.off - skip), skip, unit_pos() - skip);
+                        take_pack(load_pack<T, E>(p + w.off - skip), skip, unit_rel() - skip);
                     }
                     w.advance();
                 }
+                if (have) bidx = pbase + bl;
             };
             if (!L.vec) walk(std::integral_constant<int, 0>{});
             else if (c % E == 0) walk(std::integral_constant<int, 1>{});

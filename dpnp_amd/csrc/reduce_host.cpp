@@ -160,7 +160,8 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     // by offset) when that dim is the one src moves least along, whatever its stride and however many reduced
     // dims stay apart: axes (0, 2) of a 4-d array, columns of a matrix view that takes every other column
     bool cols_walk = false;
-    if (!contig_red && !cols_plain && !arg && nd_r <= 3 && inner > 1 && istr[0][last] != 0) {
+    if (!contig_red && !cols_plain && !arg && nd_r <= 3 && inner > 1 && istr[0][last] != 0 &&
+        rshape[nd_r - 1] < ((int64_t)1 << 31) && (nd_r < 2 || rshape[nd_r - 2] < ((int64_t)1 << 31))) {
         int64_t smin = INT64_MAX;
         for (int d = 0; d < nd_r; ++d) smin = std::min(smin, rstr[0][d] < 0 ? -rstr[0][d] : rstr[0][d]);
         const int64_t si = istr[0][last] < 0 ? -istr[0][last] : istr[0][last];
@@ -189,7 +190,9 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         bool vec = contig_red; // packs need no alignment
         int e = vec ? E : 1;
         int64_t work = n; // what lanes and splits share out: elements, or the units of a walked space
-        if (!contig_red && nd_r <= 3) {
+        // (the kernels keep the two inner digits of a walked space and a run's length in 32 bits)
+        const int64_t lim32 = (int64_t)1 << 31;
+        if (!contig_red && nd_r <= 3 && rshape[nd_r - 1] < lim32 && (nd_r < 2 || rshape[nd_r - 2] < lim32)) {
             // reduced dims that stay apart (a sliced matrix summed whole, axes (0, 2) of a 3-d array, a
             // strided run): lanes walk the reduced space in units of its last dim, 16-byte packs when that
             // dim has unit stride and holds at least one
@@ -222,8 +225,9 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         const int64_t tgt = (L.walk && !vec) ? target * (in_size >= 16 ? 1 : (in_size == 8 ? 2 : 4)) : target;
         if (G > 64 && 2 * oblocks <= tgt && oblocks <= RED_MAX_TICKETS && work >= 2 * per_pass)
             splits = std::min(tgt / oblocks, cdiv(work, per_pass));
+        // 32-bit positions inside a chunk (a walked space counts the whole last pack of every run: below 2 n)
         if (arg && G > 64 && oblocks <= RED_MAX_TICKETS)
-            splits = std::max(splits, cdiv(n, (int64_t)1 << 31)); // 32-bit positions inside a chunk
+            splits = std::max(splits, cdiv(n, (int64_t)1 << (L.walk ? 30 : 31)));
         int64_t chunk = cdiv(work, splits);
         chunk = cdiv(chunk, G * e) * (G * e);
         splits = cdiv(work, chunk);

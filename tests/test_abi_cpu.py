@@ -259,6 +259,24 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] == "red_cols_split"
     p = plan_reduce("sum", view([17, 1 << 20], [1, 18]), 1, view([17], ptr=P1))  # padded rows: column kernel
     assert L.PATH_NAMES[p.path] == "red_cols_split"
+    # reduced dims that do not collapse into one run.  A sliced matrix summed whole, axes (0, 2) of a 3-d array:
+    # lanes along the reduced space, packs along its unit-stride last dim
+    p = plan_reduce("sum", view([16384, 16382], [16384, 1]), 2, view([], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.splits > 1
+    p = plan_reduce("max", view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.grid[0] == 1024
+    # every other column summed along the rows: single elements at a stride
+    p = plan_reduce("sum", view([16384, 8192], [16384, 2]), 1, view([16384], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 1 and p.vec == 0
+    # axes (0, 2) of a 4-d array, every other column summed down the columns: src moves least along the inner
+    # iteration dim, so threads sit side by side along it and walk the rows of the reduced space
+    p = plan_reduce("sum", view([128, 128, 128, 128], [1 << 14, 1, 1 << 21, 128]), 2, view([128, 128], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 2 and p.vec == 1
+    p = plan_reduce("sum", view([8192, 16384], [2, 16384]), 1, view([8192], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 1 and p.vec == 0
+    # searches walk the reduced space too (its dims keep their order)
+    L.check(lib.dpx_argreduce_plan(0, view([16384, 16382], [16384, 1]), 2, view([], dt=L.INT64, ptr=P1), pa))
+    assert L.PATH_NAMES[pa.path] == "red_generic" and pa.red_nd == 2 and pa.vec == 1
 
 
 def test_validation_errors_are_raised_before_any_launch():
