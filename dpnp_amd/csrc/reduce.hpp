@@ -1630,6 +1630,150 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     if (ty == 0 && active) write_out();
 }
 
+// Flat variant (see red_flat_kernel): the row of the extremum of every column of a row-major matrix whose rows
+// are shorter than 512 bytes.  Thread t reads packs t, t + NT, ... of the block's rows, so element e of its packs
+// stays in one column and moves down NT * E / inner rows per pack: a thread keeps, per column, the best value and
+// how many rows below its first pack it stood (32 bits: the host keeps a block's rows below 2^32).  LDS holds
+// NT * E (row, value) pairs, entry k of column k mod inner, folded by a tree; blocks leave (row, value) partials
+// laid out [block][column] for the last one.
+template <bool IS_MAX, class VT> DPX_D void arg_flat_fold(VT *smv, int64_t *smi, int count, int inner)
+{
+    const int J = (count + inner - 1) / inner;
+    int s = 1;
+    while (2 * s < J) s *= 2;
+    if (J < 2) s = 0;
+    for (; s >= 1; s >>= 1) {
+        __syncthreads();
+        const int lim = (count - s * inner < s * inner) ? count - s * inner : s * inner;
+        for (int k = threadIdx.x; k < lim; k += (int)blockDim.x)
+            arg_merge<IS_MAX, VT>(smv[k], smi[k], smv[k + s * inner], smi[k + s * inner]);
+    }
+    __syncthreads();
+}
+
+template <class T, bool IS_MAX>
+__global__ __launch_bounds__(256) void arg_flat_kernel(RedIndex ix, RedLaunch L, const T *src, int64_t *dst,
+                                                      Slot<T> *pval, Slot<int64_t> *pidx, unsigned *counters)
+{
+    using VT = value_of_t<T>;
+    constexpr int E = 16 / (int)sizeof(T);
+    constexpr int U = E >= 8 ? 2 : (E >= 4 ? 4 : 8); // packs in flight per thread
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int NT = (int)blockDim.x, t = (int)threadIdx.x;
+    int64_t *smi = reinterpret_cast<int64_t *>(smem_raw);
+    VT *smv = reinterpret_cast<VT *>(smem_raw + (size_t)NT * E * sizeof(int64_t));
+    const int inner = (int)L.inner;
+    const int split = (int)blockIdx.x;
+    const int64_t row0 = (int64_t)split * L.chunk;
+    const int64_t rows = (row0 + L.chunk < L.n) ? L.chunk : L.n - row0;
+    const int64_t elems = rows * inner;
+    const int64_t packs = elems / E;
+    const T *p = src + row0 * inner;
+    const uint32_t rstep = (uint32_t)(NT * E / inner); // rows between a thread's consecutive packs
+
+    VT best[E];
+    uint32_t bl[E];
+    const bool have = t < packs;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        best[e] = VT{};
+        bl[e] = 0;
+    }
+    if (have) { // the first pack seeds the running extrema (and is then visited once more)
+        const pack<T, E> v = load_pack<T, E>(p + (int64_t)t * E);
+#pragma unroll
+        for (int e = 0; e < E; ++e) best[e] = to_value(v.v[e]);
+    }
+    auto take = [&](const pack<T, E> &v, uint32_t below) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const VT x = to_value(v.v[e]);
+            const bool better = arg_better<IS_MAX, VT>(x, best[e]);
+            best[e] = better ? x : best[e];
+            bl[e] = better ? below : bl[e];
+        }
+    };
+    uint32_t cur = 0; // rows below the thread's first pack
+    int64_t q = t;
+    for (; q + (int64_t)(U - 1) * NT < packs; q += (int64_t)U * NT) {
+        pack<T, E> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = load_pack<T, E>(p + (q + (int64_t)u * NT) * E);
+#pragma unroll
+        for (int u = 0; u < U; ++u) take(v[u], cur + (uint32_t)u * rstep);
+        cur += (uint32_t)U * rstep;
+    }
+    for (; q < packs; q += NT) {
+        take(load_pack<T, E>(p + q * E), cur);
+        cur += rstep;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        smv[t * E + e] = best[e];
+        smi[t * E + e] = have ? row0 + (t * E + e) / inner + bl[e] : ARG_NONE;
+    }
+    __syncthreads();
+    // the elements after the last whole pack of the block (fewer than E), as in red_flat_kernel
+    const int tail = (int)(elems - packs * E);
+    if (t < tail) {
+        const int64_t i = packs * E + t;
+        const int k = (int)(i % ((int64_t)NT * E));
+        arg_merge<IS_MAX, VT>(smv[k], smi[k], to_value(load_one(p + i)), row0 + i / inner);
+    }
+    arg_flat_fold<IS_MAX, VT>(smv, smi, NT * E, inner);
+    if (L.splits == 1) {
+        for (int c = t; c < inner; c += NT) dst[(int64_t)c * ix.dst_str[0]] = arg_result<T>(L, smi[c], smv[c]);
+        return;
+    }
+    uint32_t zero = 0;
+    for (int c = t; c < inner; c += NT) {
+        zero |= slot_publish(pval + (int64_t)split * inner + c, to_storage<T>(smv[c]));
+        zero |= slot_publish(pidx + (int64_t)split * inner + c, smi[c]);
+    }
+    if (!last_block_of(counters, L.splits, zero)) return;
+    if (inner > NT) { // more columns than threads (1-byte elements): a thread folds whole columns
+        for (int c = t; c < inner; c += NT) {
+            VT b{};
+            int64_t bi = ARG_NONE;
+            for (int g = 0; g < L.splits; ++g)
+                arg_merge<IS_MAX, VT>(b, bi, to_value(slot_read(pval + (int64_t)g * inner + c)),
+                                      slot_read(pidx + (int64_t)g * inner + c));
+            dst[(int64_t)c * ix.dst_str[0]] = arg_result<T>(L, bi, b);
+        }
+        return;
+    }
+    // thread t < parts * inner folds blocks part, part + parts, ... of column t mod inner
+    const int parts = NT / inner;
+    VT b{};
+    int64_t bi = ARG_NONE;
+    if (t < parts * inner) {
+        constexpr int FU = 4;
+        const int c = t % inner, part = t / inner;
+        int g = part;
+        for (; g + (FU - 1) * parts < L.splits; g += FU * parts) {
+            T wv[FU];
+            int64_t wi[FU];
+#pragma unroll
+            for (int u = 0; u < FU; ++u) {
+                wv[u] = slot_read(pval + (int64_t)(g + u * parts) * inner + c);
+                wi[u] = slot_read(pidx + (int64_t)(g + u * parts) * inner + c);
+            }
+#pragma unroll
+            for (int u = 0; u < FU; ++u) arg_merge<IS_MAX, VT>(b, bi, to_value(wv[u]), wi[u]);
+        }
+        for (; g < L.splits; g += parts)
+            arg_merge<IS_MAX, VT>(b, bi, to_value(slot_read(pval + (int64_t)g * inner + c)),
+                                  slot_read(pidx + (int64_t)g * inner + c));
+    }
+    __syncthreads(); // every thread has read its column results of the first fold
+    if (t < parts * inner) {
+        smv[t] = b;
+        smi[t] = bi;
+    }
+    arg_flat_fold<IS_MAX, VT>(smv, smi, parts * inner, inner);
+    for (int c = t; c < inner; c += NT) dst[(int64_t)c * ix.dst_str[0]] = arg_result<T>(L, smi[c], smv[c]);
+}
+
 // Short rows variant (see red_short_rows_kernel): position of the extremum of each row of a
 // row-major matrix with rows of at most 256 bytes (the predicted class of each sample).
 template <class T, bool IS_MAX>

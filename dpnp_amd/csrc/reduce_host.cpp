@@ -245,7 +245,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
-    if (!cols_walk && !arg && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
+    if (!cols_walk && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
         tune_int("DPX_RED_FLAT", 1) != 0) { // (sweep override: 0 keeps the column kernel)
         // a row-major matrix with rows shorter than 512 bytes: one flat stream of packs, a block of
         // T threads with T * E a multiple of the row length (see red_flat_kernel)
@@ -260,6 +260,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
             const int64_t T = period * (256 / period);
             const int64_t per_block = T * E * 8; // at least 8 packs per thread
             int64_t blocks = std::max<int64_t>(1, std::min<int64_t>(target, (n * inner) / per_block));
+            if (arg) blocks = std::max(blocks, cdiv(n, (int64_t)1 << 31)); // 32-bit rows inside a block
             {
                 const int64_t chunk = cdiv(n, blocks);
                 blocks = cdiv(n, chunk);

@@ -636,6 +636,42 @@ def test_axis0_of_matrices_with_short_rows(dt):
     assert (host(out)[1::2] == 0).all()
 
 
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "i8", "f2", "f4", "f8", "c8", "c16"])
+def test_argmax_argmin_axis0_of_matrices_with_short_rows(dt):
+    # the flat stream again: the row of each column's extremum; values in -3..3 tie all the time (the first row
+    # wins), NaNs beat every number (the first one wins), enough rows for several blocks
+    rng = np.random.default_rng(43)
+    itemsize = np.dtype(dt).itemsize
+    for cols in FLAT_COLS:
+        if cols * itemsize >= 512:
+            continue
+        # (the oracle compares complex values one by one in Python: fewer rows for them)
+        for rows in ((16, 17, 255, 4099) if np.dtype(dt).kind == "c" else (16, 17, 255, 4099, 60013, 300007)):
+            a = random_array(rng, (rows, cols), dt, lo=-3, hi=3)
+            da = dev(a)
+            assert_same(host(dpt.argmax(da, axis=0)), orc.argreduce("argmax", a.T, 1))
+            assert_same(host(dpt.argmin(da, axis=0)), orc.argreduce("argmin", a.T, 1))
+            if np.dtype(dt).kind in "fc" and rows > 255:
+                a[rng.random(a.shape) < 0.001] = np.nan
+                a[rows // 2:, 0] = 0  # a column whose NaNs, if any, lie in the first half
+                da = dev(a)
+                assert_same(host(dpt.argmax(da, axis=0)), orc.argreduce("argmax", a.T, 1))
+                assert_same(host(dpt.argmin(da, axis=0)), orc.argreduce("argmin", a.T, 1))
+    a = random_array(rng, (3000, 17), dt, lo=-3, hi=3)
+    da = dev(a)
+    assert_same(host(dpt.argmax(da[3:], axis=0)), orc.argreduce("argmax", a[3:].T, 1))
+    out = dpt.zeros(34, dtype="i8")
+    dpt.argmin(da, axis=0, out=out[::2])
+    assert_same(host(out)[::2], orc.argreduce("argmin", a.T, 1))
+    assert (host(out)[1::2] == 0).all()
+    if np.dtype(dt).kind == "f":  # the NaN-ignoring searches take the same kernel
+        a = random_array(rng, (70001, 5), dt, lo=-3, hi=3)
+        a[rng.random(a.shape) < 0.3] = np.nan
+        a[0, :] = 0
+        assert_same(dpnp.asnumpy(dpnp.nanargmax(dpnp.array(a), axis=0)), np.nanargmax(a, axis=0))
+        assert_same(dpnp.asnumpy(dpnp.nanargmin(dpnp.array(a), axis=0)), np.nanargmin(a, axis=0))
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 def test_statistics_over_samples_of_few_features(dt):
     # (samples, features) with few features: mean / var / std / logsumexp / hypot / nan forms over axis 0
