@@ -649,12 +649,20 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
             // MODE 0: units are elements; 1: packs, every run a whole number of them; 2: packs, the last one of
             // a run partial: it is read as the whole pack that ends with the run's last element (a run holds at
             // least one pack) and the elements it shares with the pack before are left out, so that every
-            // lane issues the same loads whatever its units are
+            // lane issues the same loads whatever its units are; 3: a run of every other element (L.walk == 2):
+            // the lines it touches are read as in mode 2 (`inner` is their length, 2 x elements - 1) and the
+            // elements at odd places are left out as well, a quarter of the load instructions of mode 0
             auto walk = [&](auto mode_tag) {
                 constexpr int MODE = decltype(mode_tag)::value;
                 RedWalker w;
                 int64_t q = beg + lane;
                 w.start(L, q, G);
+                // does element e of a pack read `skip` places early count?
+                auto counts = [&](int e, int skip) {
+                    if constexpr (MODE == 2) return e >= skip;
+                    else if constexpr (MODE == 3) return e >= skip && ((e + skip) & 1) == 0;
+                    else return true;
+                };
                 const uint32_t c32 = (uint32_t)c; // (the host keeps run lengths below 2^31)
                 auto skipped = [&](uint32_t k) {
                     const uint32_t rem = c32 - k * E;
@@ -676,7 +684,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                         int skip[RED_U];
 #pragma unroll
                         for (int u = 0; u < RED_U; ++u) {
-                            skip[u] = MODE == 2 ? skipped(w.k) : 0;
+                            skip[u] = MODE >= 2 ? skipped(w.k) : 0;
                             v[u] = load_pack<In, E>(p + w.off - skip[u]);
                             w.advance();
                         }
@@ -685,25 +693,28 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
 #pragma unroll
                             for (int e = 0; e < E; ++e) {
                                 const Acc t = P::combine(acc[u], P::pre(v[u].v[e], a));
-                                acc[u] = (MODE == 2 && e < skip[u]) ? acc[u] : t;
+                                acc[u] = counts(e, skip[u]) ? t : acc[u];
                             }
                     }
                 }
                 for (; q < uend; q += G) {
                     if constexpr (MODE == 0) acc[0] = P::combine(acc[0], P::pre(load_one(p + w.off), a));
                     else {
-                        const int skip = MODE == 2 ? skipped(w.k) : 0;
+                        const int skip = MODE >= 2 ? skipped(w.k) : 0;
                         const pack<In, E> v = load_pack<In, E>(p + w.off - skip);
 #pragma unroll
                         for (int e = 0; e < E; ++e) {
                             const Acc t = P::combine(acc[0], P::pre(v.v[e], a));
-                            acc[0] = (MODE == 2 && e < skip) ? acc[0] : t;
+                            acc[0] = counts(e, skip) ? t : acc[0];
                         }
                     }
                     w.advance();
                 }
             };
             if (!L.vec) walk(std::integral_constant<int, 0>{});
+            else if (L.walk == 2) {
+                if constexpr (E >= 4) walk(std::integral_constant<int, 3>{});
+            }
             else if (c % E == 0) walk(std::integral_constant<int, 1>{});
             else walk(std::integral_constant<int, 2>{});
         }
@@ -790,8 +801,22 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     const int split = (int)(b % L.splits);
     const int64_t outer = b / L.splits;
     const int ecnt = L.vec ? E : 1;
-    const int64_t col0 = (cb * TX + tx) * ecnt;
-    const bool active = col0 < L.inner;
+    const int64_t col_first = (cb * TX + tx) * ecnt;
+    const bool active = col_first < L.inner;
+    // The pack that would cross the end of a row is moved back so that it ends with the row; its first `back`
+    // places belong to the thread before.  (Read element by element instead, one row at a time, that one thread
+    // was a chain of dependent round trips as long as its column: 16384 x 16383 floats summed down the columns took
+    // 369 us, 16384 x 16384 158 us.)  Rows shorter than a pack keep the element-wise form.
+    const int back = (L.vec && active && col_first + E > L.inner && L.inner >= E) ? (int)(col_first + E - L.inner) : 0;
+    const int64_t col0 = col_first - back;
+    // L.walk == 2: every other column of a matrix.  The lines are read whole (L.inner is their length, 2 x
+    // columns - 1; L.istep is not used): place e of a thread's pack is column (col0 + e) / 2 of the view when
+    // col0 + e is even and nothing otherwise
+    const bool half = WALK && L.walk == 2;
+    auto has_out = [&](int e) {
+        return e < ecnt && e >= back && col0 + e < L.inner && !(half && ((col0 + e) & 1));
+    };
+    auto out_col = [&](int e) { return half ? (col0 + e) >> 1 : col0 + e; };
 
     Acc acc[U][E];
 #pragma unroll
@@ -820,9 +845,9 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         if constexpr (P::has_aux) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (e < ecnt && col0 + e < L.inner) a[e] = P::load_aux(aux + ao + (col0 + e) * ix.aux_str[last]);
+                if (has_out(e)) a[e] = P::load_aux(aux + ao + out_col(e) * ix.aux_str[last]);
         }
-        const In *p = src + so + col0 * (WALK ? L.istep : 1);
+        const In *p = src + so + col0 * ((WALK && !half) ? L.istep : 1);
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         int64_t r = beg + ty;
@@ -891,12 +916,14 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         for (int u = 1; u < U; ++u) v[e] = P::combine(v[e], acc[u][e]);
     }
     cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
-    const int64_t out0 = outer * L.inner + col0; // flat output index of this thread's first column
+    // flat output index of this thread's column e
+    const int64_t out_base = half ? outer * ((L.inner + 1) >> 1) : outer * L.inner;
+    auto slot_of = [&](int e) { return out_base + out_col(e); };
     if (L.splits == 1) {
         if (ty == 0 && active) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e], L.param);
+                if (has_out(e)) dst[dof + out_col(e) * ix.dst_str[last]] = P::post(v[e], L.param);
         }
         return;
     }
@@ -904,7 +931,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     if (ty == 0 && active) {
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (e < ecnt && col0 + e < L.inner) zero |= slot_publish(partial + (int64_t)split * L.m + out0 + e, v[e]);
+            if (has_out(e)) zero |= slot_publish(partial + (int64_t)split * L.m + slot_of(e), v[e]);
     }
     if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
     // pass two: thread row ty folds splits ty, ty + TY, ... in increasing order
@@ -921,26 +948,24 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             for (int u = 0; u < FU; ++u)
 #pragma unroll
                 for (int e = 0; e < E; ++e)
-                    if (e < ecnt && col0 + e < L.inner)
-                        t[u][e] = slot_read(partial + (int64_t)(sidx + u * TY) * L.m + out0 + e);
+                    if (has_out(e)) t[u][e] = slot_read(partial + (int64_t)(sidx + u * TY) * L.m + slot_of(e));
 #pragma unroll
             for (int u = 0; u < FU; ++u)
 #pragma unroll
                 for (int e = 0; e < E; ++e)
-                    if (e < ecnt && col0 + e < L.inner) v[e] = P::combine(v[e], t[u][e]);
+                    if (has_out(e)) v[e] = P::combine(v[e], t[u][e]);
         }
         for (; sidx < L.splits; sidx += TY) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (e < ecnt && col0 + e < L.inner)
-                    v[e] = P::combine(v[e], slot_read(partial + (int64_t)sidx * L.m + out0 + e));
+                if (has_out(e)) v[e] = P::combine(v[e], slot_read(partial + (int64_t)sidx * L.m + slot_of(e)));
         }
     }
     cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
     if (ty == 0 && active) {
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (e < ecnt && col0 + e < L.inner) dst[dof + (col0 + e) * ix.dst_str[last]] = P::post(v[e], L.param);
+            if (has_out(e)) dst[dof + out_col(e) * ix.dst_str[last]] = P::post(v[e], L.param);
     }
 }
 
@@ -1348,12 +1373,13 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
             const int64_t uend = (beg + L.chunk < L.units) ? beg + L.chunk : L.units;
             const int64_t c = L.inner;
             auto walk = [&](auto mode_tag) {
-                constexpr int MODE = decltype(mode_tag)::value;
-                constexpr int UE = MODE == 0 ? 1 : E; // positions per unit
+                constexpr int MODE = decltype(mode_tag)::value; // (mode 3: see red_rows_kernel)
+                constexpr int UE = MODE == 0 ? 1 : (MODE == 3 ? E / 2 : E); // positions per unit
+                const int64_t run = MODE == 3 ? (c + 1) / 2 : c;           // positions per run
                 RedWalker w;
                 int64_t q = beg + lane;
-                w.start(L, q, G, c, UE, beg);
-                const int64_t pbase = (beg / L.wd[2]) * c + (beg % L.wd[2]) * UE;
+                w.start(L, q, G, run, UE, beg);
+                const int64_t pbase = (beg / L.wd[2]) * run + (beg % L.wd[2]) * UE;
                 const uint32_t c32 = (uint32_t)c; // (the host keeps run lengths below 2^31)
                 auto skipped = [&](uint32_t k) {
                     const uint32_t rem = c32 - k * E;
@@ -1372,9 +1398,14 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
                     best = better ? x : best;
                     bl = better ? rel : bl;
                 };
+                // `rel`: position of the element at place 0 of the pack as read (`skip` places early)
                 auto take_pack = [&](const pack<T, E> &v, int skip, uint32_t rel) {
 #pragma unroll
-                    for (int e = 0; e < E; ++e) take(to_value(v.v[e]), MODE != 2 || e >= skip, rel + e);
+                    for (int e = 0; e < E; ++e) {
+                        if constexpr (MODE == 3)
+                            take(to_value(v.v[e]), e >= skip && ((e + skip) & 1) == 0, rel + (uint32_t)((e - skip) >> 1));
+                        else take(to_value(v.v[e]), MODE != 2 || e >= skip, rel + e);
+                    }
                 };
                 for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
                     uint32_t rel[RED_U];
@@ -1394,8 +1425,8 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
                         int skip[RED_U];
 #pragma unroll
                         for (int u = 0; u < RED_U; ++u) {
-                            skip[u] = MODE == 2 ? skipped(w.k) : 0;
-                            rel[u] = unit_rel() - skip[u];
+                            skip[u] = MODE >= 2 ? skipped(w.k) : 0;
+                            rel[u] = MODE == 3 ? unit_rel() : unit_rel() - skip[u];
                             v[u] = load_pack<T, E>(p + w.off - skip[u]);
                             w.advance();
                         }
@@ -1406,14 +1437,17 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
                 for (; q < uend; q += G) {
                     if constexpr (MODE == 0) take(to_value(load_one(p + w.off)), true, unit_rel());
                     else {
-                        const int skip = MODE == 2 ? skipped(w.k) : 0;
-                        take_pack(load_pack<T, E>(p + w.off - skip), skip, unit_rel() - skip);
+                        const int skip = MODE >= 2 ? skipped(w.k) : 0;
+                        take_pack(load_pack<T, E>(p + w.off - skip), skip, MODE == 3 ? unit_rel() : unit_rel() - skip);
                     }
                     w.advance();
                 }
                 if (have) bidx = pbase + bl;
             };
             if (!L.vec) walk(std::integral_constant<int, 0>{});
+            else if (L.walk == 2) {
+                if constexpr (E >= 4) walk(std::integral_constant<int, 3>{});
+            }
             else if (c % E == 0) walk(std::integral_constant<int, 1>{});
             else walk(std::integral_constant<int, 2>{});
         }
@@ -1467,9 +1501,14 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     b /= L.col_blocks;
     const int split = (int)(b % L.splits);
     const int64_t outer = b / L.splits;
-    const int64_t col0 = (cb * TX + tx) * E;
-    const bool active = col0 < L.inner;
+    const int64_t col_first = (cb * TX + tx) * E;
+    const bool active = col_first < L.inner;
+    // the pack that would cross the end of a row is moved back to end with it; its first `back` places belong
+    // to the thread before (see red_cols_kernel)
+    const int back = (active && col_first + E > L.inner && L.inner >= E) ? (int)(col_first + E - L.inner) : 0;
+    const int64_t col0 = col_first - back;
     const bool whole = col0 + E <= L.inner;
+    auto mine = [&](int e) { return e >= back && col0 + e < L.inner; };
     int64_t so = 0, dof = 0;
     {
         int64_t o = outer;
@@ -1562,7 +1601,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
         const int last = ix.nd_i - 1;
         int64_t *q = dst + dof + col0 * ix.dst_str[last];
         if constexpr (E >= 2) {
-            if (whole && ix.dst_str[last] == 1) {
+            if (whole && back == 0 && ix.dst_str[last] == 1) {
 #pragma unroll
                 for (int e = 0; e < E; e += 2) {
                     pack<int64_t, 2> t;
@@ -1575,7 +1614,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
         }
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (col0 + e < L.inner) q[e * ix.dst_str[last]] = arg_result<T>(L, bidx[e], best[e]);
+            if (mine(e)) q[e * ix.dst_str[last]] = arg_result<T>(L, bidx[e], best[e]);
     };
     combine_rows();
     const int64_t out0 = outer * L.inner + col0;
@@ -1587,7 +1626,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     if (ty == 0 && active) {
 #pragma unroll
         for (int e = 0; e < E; ++e)
-            if (col0 + e < L.inner) {
+            if (mine(e)) {
                 zero |= slot_publish(pval + (int64_t)split * L.m + out0 + e, to_storage<T>(best[e]));
                 zero |= slot_publish(pidx + (int64_t)split * L.m + out0 + e, bidx[e]);
             }
@@ -1608,7 +1647,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
             for (int u = 0; u < FU; ++u)
 #pragma unroll
                 for (int e = 0; e < E; ++e)
-                    if (col0 + e < L.inner) {
+                    if (mine(e)) {
                         tv[u][e] = slot_read(pval + (int64_t)(sidx + u * TY) * L.m + out0 + e);
                         ti[u][e] = slot_read(pidx + (int64_t)(sidx + u * TY) * L.m + out0 + e);
                     }
@@ -1616,12 +1655,12 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
             for (int u = 0; u < FU; ++u)
 #pragma unroll
                 for (int e = 0; e < E; ++e)
-                    if (col0 + e < L.inner) arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(tv[u][e]), ti[u][e]);
+                    if (mine(e)) arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(tv[u][e]), ti[u][e]);
         }
         for (; sidx < L.splits; sidx += TY) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                if (col0 + e < L.inner)
+                if (mine(e))
                     arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(slot_read(pval + (int64_t)sidx * L.m + out0 + e)),
                                           slot_read(pidx + (int64_t)sidx * L.m + out0 + e));
         }

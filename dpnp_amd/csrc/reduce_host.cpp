@@ -196,8 +196,16 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
             // reduced dims that stay apart (a sliced matrix summed whole, axes (0, 2) of a 3-d array, a
             // strided run): lanes walk the reduced space in units of its last dim, 16-byte packs when that
             // dim has unit stride and holds at least one
-            const int64_t c = rshape[nd_r - 1], s_in = rstr[0][nd_r - 1];
+            int64_t c = rshape[nd_r - 1];
+            const int64_t s_in = rstr[0][nd_r - 1];
             vec = s_in == 1 && c >= E;
+            L.walk = 1;
+            if (s_in == 2 && E >= 4 && c >= E && 2 * c < lim32) {
+                // every other element of a run: the lines it touches are read as packs, half of each is used
+                vec = true;
+                c = 2 * c - 1;
+                L.walk = 2;
+            }
             const int64_t per_run = vec ? cdiv(c, E) : c;
             for (int j = 0; j < 3; ++j) {
                 const int d = nd_r - 3 + j; // digit j is reduced dim d, or missing
@@ -206,9 +214,8 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
             }
             L.wd[2] = per_run;
             L.ws[2] = vec ? E : s_in;
-            L.walk = 1;
             L.inner = c;
-            L.units = work = (n / c) * per_run;
+            L.units = work = (n / rshape[nd_r - 1]) * per_run;
             e = 1;
         }
         L.vec = vec ? 1 : 0;
@@ -281,18 +288,22 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         }
     }
     // packs need no alignment; the kernels read a row's last pack by element
-    const bool vec = !cols_walk || istr[0][last] == 1;
+    // every other column of a matrix (src stride 2 along the inner iteration dim): the lines are read whole, as
+    // packs, and the places in between are dropped: the geometry below is that of the lines (`width` elements)
+    const bool half = cols_walk && istr[0][last] == 2 && E >= 4 && 2 * inner - 1 >= E;
+    const bool vec = !cols_walk || istr[0][last] == 1 || half;
     const int e = vec ? E : 1;
+    const int64_t width = half ? 2 * inner - 1 : inner;
     L.vec = vec ? 1 : 0;
     L.rstride = rstride;
-    L.inner = inner;
+    L.inner = width;
     if (cols_walk) {
         for (int j = 0; j < 3; ++j) {
             const int d = nd_r - 3 + j; // digit j is reduced dim d, or missing
             L.wd[j] = d < 0 ? 1 : rshape[d];
             L.ws[j] = d < 0 ? 0 : rstr[0][d];
         }
-        L.walk = 1;
+        L.walk = half ? 2 : 1;
         L.units = n;
         L.istep = istr[0][last];
     }
@@ -302,9 +313,9 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
     // with a single thread row a whole wave lies side by side and nothing is combined in LDS
     // (single elements at a stride: a whole wave side by side as well, 64 elements are the least it should span)
-    int lg = std::min((ty == 1 || !vec) ? 6 : 5, ceil_log2(cdiv(inner, e)));
+    int lg = std::min((ty == 1 || !vec) ? 6 : 5, ceil_log2(cdiv(width, e)));
     const int forced = tune_int("DPX_COLS_TX_LOG2", -1); // sweep override, product build: default
-    if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(inner, e)), forced);
+    if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(width, e)), forced);
     L.g_log2 = lg;
     const int64_t TX = (int64_t)1 << lg;
     int block = (int)std::min<int64_t>(arg ? 256 : 512, std::max<int64_t>(64, TX * ty));
@@ -314,7 +325,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     if (block < TX) block = (int)TX;
     const int64_t TY = block / TX;
-    L.col_blocks = cdiv(inner, TX * e);
+    L.col_blocks = cdiv(width, TX * e);
     const int64_t outer = m / inner;
     const int64_t base_blocks = L.col_blocks * outer;
     const int64_t want = std::max<int64_t>(target * 256 / block, 1); // same number of threads in flight

@@ -265,14 +265,19 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.splits > 1
     p = plan_reduce("max", view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.grid[0] == 1024
-    # every other column summed along the rows: single elements at a stride
+    # every other column summed along the rows: the lines the run touches are read as packs; every third: single
+    # elements at a stride
     p = plan_reduce("sum", view([16384, 8192], [16384, 2]), 1, view([16384], ptr=P1))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 1 and p.vec == 1
+    p = plan_reduce("sum", view([16384, 5000], [16384, 3]), 1, view([16384], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 1 and p.vec == 0
     # axes (0, 2) of a 4-d array, every other column summed down the columns: src moves least along the inner
     # iteration dim, so threads sit side by side along it and walk the rows of the reduced space
     p = plan_reduce("sum", view([128, 128, 128, 128], [1 << 14, 1, 1 << 21, 128]), 2, view([128, 128], ptr=P1))
     assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 2 and p.vec == 1
     p = plan_reduce("sum", view([8192, 16384], [2, 16384]), 1, view([8192], ptr=P1))
+    assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 1 and p.vec == 1  # whole lines
+    p = plan_reduce("sum", view([5000, 16384], [3, 16384]), 1, view([5000], ptr=P1))
     assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 1 and p.vec == 0
     # searches walk the reduced space too (its dims keep their order)
     L.check(lib.dpx_argreduce_plan(0, view([16384, 16382], [16384, 1]), 2, view([], dt=L.INT64, ptr=P1), pa))
