@@ -1572,7 +1572,15 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
 #pragma unroll
                 for (int u = 0; u < NL; ++u) take(v[u], r + u * TY);
             }
-            for (; r < end; r += TY) take(load(p + r * L.rstride), r);
+            if (r < end) { // fewer than NL rows are left: their loads go out together as well
+                pack<T, E> v[NL];
+#pragma unroll
+                for (int u = 0; u < NL; ++u)
+                    if (r + u * TY < end) v[u] = load(p + (r + u * TY) * L.rstride);
+#pragma unroll
+                for (int u = 0; u < NL; ++u)
+                    if (r + u * TY < end) take(v[u], r + u * TY);
+            }
         };
         if (whole) walk(std::true_type{});
         else walk(std::false_type{});
