@@ -313,7 +313,12 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
     // with a single thread row a whole wave lies side by side and nothing is combined in LDS
     // (single elements at a stride: a whole wave side by side as well, 64 elements are the least it should span)
-    int lg = std::min((ty == 1 || !vec) ? 6 : 5, ceil_log2(cdiv(width, e)));
+    // rows that do not start on 16-byte boundaries (an odd row length): a thread row's run touches one line more
+    // than it fills, which is a quarter more lines for 512 bytes and an eighth for the 1024 bytes of a whole
+    // wave side by side (16385 x 16385 floats summed down the columns: 60 -> 76 % of the HBM rate; 2-byte
+    // elements and searches of 4-byte ones gain nothing or lose)
+    const bool misaligned = !cols_walk && (rstride * in_size) % 16 != 0 && in_size >= (arg ? 8 : 4);
+    int lg = std::min((ty == 1 || !vec || misaligned) ? 6 : 5, ceil_log2(cdiv(width, e)));
     const int forced = tune_int("DPX_COLS_TX_LOG2", -1); // sweep override, product build: default
     if (forced >= 0 && forced <= 8) lg = std::min(ceil_log2(cdiv(width, e)), forced);
     L.g_log2 = lg;
