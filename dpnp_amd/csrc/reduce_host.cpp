@@ -310,7 +310,9 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     // TX threads side by side cover 512 contiguous bytes of a row (32 x 16 B); up to 16 thread
     // rows walk down the reduced axis: 512-thread blocks, one per CU when splitting
     // thread rows wanted for n reduced rows (4 or more rows per thread)
-    const int64_t ty = std::min<int64_t>(16, (int64_t)1 << ceil_log2(cdiv(n, 4)));
+    // (rounded down: with fewer than 4 rows a thread never has its 4 loads in flight together)
+    int64_t ty = 1;
+    while (ty < 16 && 8 * ty <= n) ty *= 2;
     // with a single thread row a whole wave lies side by side and nothing is combined in LDS
     // (single elements at a stride: a whole wave side by side as well, 64 elements are the least it should span)
     // rows that do not start on 16-byte boundaries (an odd row length): a thread row's run touches one line more
