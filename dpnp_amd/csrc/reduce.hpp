@@ -916,15 +916,34 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         for (int u = 1; u < U; ++u) v[e] = P::combine(v[e], acc[u][e]);
     }
     cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
+    // results of v: as 16-byte stores when every place of the pack is a column and they lie side by side (few rows
+    // and many columns write as much as they read: one store per column and lane, 16 bytes apart, was the slower half)
+    auto write_out = [&]() {
+        using Out = typename P::Out;
+        if (ecnt == E && back == 0 && !half && col0 + E <= L.inner && ix.dst_str[last] == 1) {
+            constexpr int PER16 = 16 / (int)sizeof(Out) < 1 ? 1 : 16 / (int)sizeof(Out);
+            constexpr int CE = PER16 < E ? PER16 : E;
+            Out *q = dst + dof + col0;
+#pragma unroll
+            for (int e0 = 0; e0 < E; e0 += CE) {
+                pack<Out, CE> o;
+#pragma unroll
+                for (int j = 0; j < CE; ++j) o.v[j] = P::post(v[e0 + j], L.param);
+                // (results wider than the inputs: a lane's stores are pieces of a line that only meet in the L2, so
+                // they must not bypass it: int8 summed into int64 ran twice as long with streaming stores)
+                store_pack<Out, CE, sizeof(Out) <= sizeof(In)>(q + e0, o);
+            }
+            return;
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (has_out(e)) dst[dof + out_col(e) * ix.dst_str[last]] = P::post(v[e], L.param);
+    };
     // flat output index of this thread's column e
     const int64_t out_base = half ? outer * ((L.inner + 1) >> 1) : outer * L.inner;
     auto slot_of = [&](int e) { return out_base + out_col(e); };
     if (L.splits == 1) {
-        if (ty == 0 && active) {
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                if (has_out(e)) dst[dof + out_col(e) * ix.dst_str[last]] = P::post(v[e], L.param);
-        }
+        if (ty == 0 && active) write_out();
         return;
     }
     uint32_t zero = 0;
@@ -962,11 +981,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
         }
     }
     cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
-    if (ty == 0 && active) {
-#pragma unroll
-        for (int e = 0; e < E; ++e)
-            if (has_out(e)) dst[dof + out_col(e) * ix.dst_str[last]] = P::post(v[e], L.param);
-    }
+    if (ty == 0 && active) write_out();
 }
 
 // ================================ flat columns kernel =========================================
