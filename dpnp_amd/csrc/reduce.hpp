@@ -762,6 +762,14 @@ template <class In> struct cols_cfg {
     static constexpr int LOADS = E >= 8 ? 8 : 4;
 };
 
+// a cast between integer types that also compiles (and is never executed) where one side is not an integer: the
+// narrow accumulation of red_cols_kernel sits in a lambda whose body is checked for every policy
+template <class To, class From> DPX_D To int_cast(From x)
+{
+    if constexpr (std::is_integral_v<To> && std::is_integral_v<From>) return (To)x;
+    else return To{};
+}
+
 // combines acc over the TY thread rows of the block; result valid for ty == 0
 template <class P, int E> DPX_D void cols_block_combine(typename P::Acc (&v)[E], typename P::Acc *sm, int tx, int ty,
                                                         int TX, int TY)
@@ -879,6 +887,35 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                 // the element-wise form keeps one pack in flight: its LOADS x E separate loads and their
                 // addresses would set the register count of the whole kernel (and spill for 1-byte inputs)
                 constexpr int NL = WHOLE ? LOADS : 1;
+                // sums and counts of 1- and 2-byte integers into 64-bit accumulators: 16384 rows of a thread at a
+                // time are added up in 32 bits (a sign extension and an add per element instead of four
+                // instructions, half the registers), then moved on to the wide accumulators
+                constexpr bool NARROW = WHOLE && sizeof(In) <= 2 && sizeof(Acc) == 8 && std::is_integral_v<Acc> &&
+                                        !P::has_aux && (P::kind == K_SUM || P::kind == K_COUNT_NONZERO);
+                if constexpr (NARROW) {
+                    using A32 = std::conditional_t<std::is_signed_v<Acc>, int32_t, uint32_t>;
+                    constexpr int ROUNDS = 16384 / NL;
+                    while (r + (NL - 1) * TY < end) {
+                        A32 n32[U][E];
+#pragma unroll
+                        for (int u = 0; u < U; ++u)
+#pragma unroll
+                            for (int e = 0; e < E; ++e) n32[u][e] = 0;
+                        for (int round = 0; round < ROUNDS && r + (NL - 1) * TY < end; ++round, r += NL * TY) {
+                            pack<In, E> v[NL];
+#pragma unroll
+                            for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
+#pragma unroll
+                            for (int u = 0; u < NL; ++u)
+#pragma unroll
+                                for (int e = 0; e < E; ++e) n32[u % U][e] += int_cast<A32>(P::pre(v[u].v[e], a[e]));
+                        }
+#pragma unroll
+                        for (int u = 0; u < U; ++u)
+#pragma unroll
+                            for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], int_cast<Acc>(n32[u][e]));
+                    }
+                }
                 for (; r + (NL - 1) * TY < end; r += NL * TY) {
                     pack<In, E> v[NL];
 #pragma unroll
