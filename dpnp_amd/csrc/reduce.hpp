@@ -776,13 +776,16 @@ template <class P, int E> DPX_D void cols_block_combine(typename P::Acc (&v)[E],
 {
     if (TY == 1) return;
     __syncthreads(); // sm may still be read by a previous call
+    // place e of all threads side by side: neighbouring lanes then touch neighbouring words (thread by thread, 16
+    // 64-bit sums per thread put the lanes of a wave 128 bytes apart, all on the same banks)
+    const int NT = TX * TY;
 #pragma unroll
-    for (int e = 0; e < E; ++e) sm[threadIdx.x * E + e] = v[e];
+    for (int e = 0; e < E; ++e) sm[e * NT + threadIdx.x] = v[e];
     __syncthreads();
     if (ty == 0) {
         for (int y = 1; y < TY; ++y)
 #pragma unroll
-            for (int e = 0; e < E; ++e) v[e] = P::combine(v[e], sm[(y * TX + tx) * E + e]);
+            for (int e = 0; e < E; ++e) v[e] = P::combine(v[e], sm[e * NT + y * TX + tx]);
     }
 }
 
@@ -990,35 +993,46 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             if (has_out(e)) zero |= slot_publish(partial + (int64_t)split * L.m + slot_of(e), v[e]);
     }
     if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
-    // pass two: thread row ty folds splits ty, ty + TY, ... in increasing order
+    // pass two.  Threads side by side along the block's outputs, so that a wave reads consecutive partials (the
+    // thread that owns a pack would read its E partials 4 or 8 bytes at a time, lanes a pack of partials apart:
+    // 128 blocks of 1001 int8 columns summed into int64 spent 70 of their 104 us here).  With fewer outputs than
+    // threads, `parts` threads share a column: thread (part, c) folds splits part, part + parts, ... in
+    // increasing order, then the parts are folded in order through LDS.
+    const int NT = (int)blockDim.x, t = (int)threadIdx.x;
+    const int64_t pcol0 = cb * TX * ecnt; // first place of the block along the rows, and how many it has
+    const int64_t pcols = (L.inner - pcol0 < (int64_t)TX * ecnt) ? L.inner - pcol0 : (int64_t)TX * ecnt;
+    const int64_t ocol0 = half ? pcol0 >> 1 : pcol0; // the same in columns of the output
+    const int ncol = (int)(half ? (pcols + 1) >> 1 : pcols);
+    const Slot<Acc> *part0 = partial + out_base + ocol0;
+    auto fold_from = [&](int c, int first, int step) {
+        constexpr int FU = 8;
+        Acc r = P::identity();
+        int g = first;
+        for (; g + (FU - 1) * step < L.splits; g += FU * step) {
+            Acc w[FU];
 #pragma unroll
-    for (int e = 0; e < E; ++e) v[e] = P::identity();
-    if (active) {
-        // FU partials per column in flight: with few columns and many splits this loop is the tail
-        // of the kernel (512 splits over 16 thread rows: 32 dependent L2 round trips without it)
-        constexpr int FU = E >= 16 ? 2 : (E >= 8 ? 4 : 8);
-        int sidx = ty;
-        for (; sidx + (FU - 1) * TY < L.splits; sidx += FU * TY) {
-            Acc t[FU][E];
+            for (int u = 0; u < FU; ++u) w[u] = slot_read(part0 + (int64_t)(g + u * step) * L.m + c);
 #pragma unroll
-            for (int u = 0; u < FU; ++u)
-#pragma unroll
-                for (int e = 0; e < E; ++e)
-                    if (has_out(e)) t[u][e] = slot_read(partial + (int64_t)(sidx + u * TY) * L.m + slot_of(e));
-#pragma unroll
-            for (int u = 0; u < FU; ++u)
-#pragma unroll
-                for (int e = 0; e < E; ++e)
-                    if (has_out(e)) v[e] = P::combine(v[e], t[u][e]);
+            for (int u = 0; u < FU; ++u) r = P::combine(r, w[u]);
         }
-        for (; sidx < L.splits; sidx += TY) {
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                if (has_out(e)) v[e] = P::combine(v[e], slot_read(partial + (int64_t)sidx * L.m + slot_of(e)));
-        }
+        for (; g < L.splits; g += step) r = P::combine(r, slot_read(part0 + (int64_t)g * L.m + c));
+        return r;
+    };
+    if (ncol >= NT) { // (a single thread row of wide packs: more outputs than threads)
+        for (int c = t; c < ncol; c += NT)
+            dst[dof + (ocol0 + c) * ix.dst_str[last]] = P::post(fold_from(c, 0, 1), L.param);
+        return;
     }
-    cols_block_combine<P, E>(v, sm, tx, ty, TX, TY);
-    if (ty == 0 && active) write_out();
+    const int parts = NT / ncol;
+    Acc r = P::identity();
+    if (t < parts * ncol) r = fold_from(t % ncol, t / ncol, parts);
+    __syncthreads(); // sm may still be read by the combine above
+    if (t < parts * ncol) sm[t] = r;
+    __syncthreads();
+    if (t < ncol) {
+        for (int q = 1; q < parts; ++q) r = P::combine(r, sm[q * ncol + t]);
+        dst[dof + (ocol0 + t) * ix.dst_str[last]] = P::post(r, L.param);
+    }
 }
 
 // ================================ flat columns kernel =========================================
