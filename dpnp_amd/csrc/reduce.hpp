@@ -1706,41 +1706,55 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
             }
     }
     if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
+    // pass two, as in red_cols_kernel: threads side by side along the block's outputs read consecutive partial
+    // pairs; with fewer outputs than threads, `parts` threads share a column and meet in LDS.  (arg_merge takes the
+    // better value and, of equal ones, the smaller position: the order of the merges does not matter.)
+    const int NT = (int)blockDim.x, t = (int)threadIdx.x;
+    const int last = ix.nd_i - 1;
+    const int64_t ocol0 = cb * TX * E;
+    const int ncol = (int)((L.inner - ocol0 < (int64_t)TX * E) ? L.inner - ocol0 : (int64_t)TX * E);
+    const int64_t slot0 = outer * L.inner + ocol0;
+    auto fold_from = [&](int c, int first, int step, VT &b, int64_t &bi) {
+        constexpr int FU = 4;
+        b = VT{};
+        bi = ARG_NONE;
+        int g = first;
+        for (; g + (FU - 1) * step < L.splits; g += FU * step) {
+            T wv[FU];
+            int64_t wi[FU];
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-        best[e] = VT{};
-        bidx[e] = ARG_NONE;
-    }
-    if (active) {
-        constexpr int FU = E >= 16 ? 1 : (E >= 8 ? 2 : 4); // partial pairs per column in flight
-        int sidx = ty;
-        for (; sidx + (FU - 1) * TY < L.splits; sidx += FU * TY) {
-            T tv[FU][E];
-            int64_t ti[FU][E];
+            for (int u = 0; u < FU; ++u) {
+                wv[u] = slot_read(pval + (int64_t)(g + u * step) * L.m + slot0 + c);
+                wi[u] = slot_read(pidx + (int64_t)(g + u * step) * L.m + slot0 + c);
+            }
 #pragma unroll
-            for (int u = 0; u < FU; ++u)
-#pragma unroll
-                for (int e = 0; e < E; ++e)
-                    if (mine(e)) {
-                        tv[u][e] = slot_read(pval + (int64_t)(sidx + u * TY) * L.m + out0 + e);
-                        ti[u][e] = slot_read(pidx + (int64_t)(sidx + u * TY) * L.m + out0 + e);
-                    }
-#pragma unroll
-            for (int u = 0; u < FU; ++u)
-#pragma unroll
-                for (int e = 0; e < E; ++e)
-                    if (mine(e)) arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(tv[u][e]), ti[u][e]);
+            for (int u = 0; u < FU; ++u) arg_merge<IS_MAX, VT>(b, bi, to_value(wv[u]), wi[u]);
         }
-        for (; sidx < L.splits; sidx += TY) {
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                if (mine(e))
-                    arg_merge<IS_MAX, VT>(best[e], bidx[e], to_value(slot_read(pval + (int64_t)sidx * L.m + out0 + e)),
-                                          slot_read(pidx + (int64_t)sidx * L.m + out0 + e));
+        for (; g < L.splits; g += step)
+            arg_merge<IS_MAX, VT>(b, bi, to_value(slot_read(pval + (int64_t)g * L.m + slot0 + c)),
+                                  slot_read(pidx + (int64_t)g * L.m + slot0 + c));
+    };
+    VT fb{};
+    int64_t fi = ARG_NONE;
+    if (ncol >= NT) {
+        for (int c = t; c < ncol; c += NT) {
+            fold_from(c, 0, 1, fb, fi);
+            dst[dof + (ocol0 + c) * ix.dst_str[last]] = arg_result<T>(L, fi, fb);
         }
+        return;
     }
-    combine_rows();
-    if (ty == 0 && active) write_out();
+    const int parts = NT / ncol;
+    if (t < parts * ncol) fold_from(t % ncol, t / ncol, parts, fb, fi);
+    __syncthreads(); // the LDS may still be read by the combine above
+    if (t < parts * ncol) {
+        smv[t] = fb;
+        smi[t] = fi;
+    }
+    __syncthreads();
+    if (t < ncol) {
+        for (int q = 1; q < parts; ++q) arg_merge<IS_MAX, VT>(fb, fi, smv[q * ncol + t], smi[q * ncol + t]);
+        dst[dof + (ocol0 + t) * ix.dst_str[last]] = arg_result<T>(L, fi, fb);
+    }
 }
 
 // Flat variant (see red_flat_kernel): the row of the extremum of every column of a row-major matrix whose rows
