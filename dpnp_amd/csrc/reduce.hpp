@@ -1005,7 +1005,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     const int ncol = (int)(half ? (pcols + 1) >> 1 : pcols);
     const Slot<Acc> *part0 = partial + out_base + ocol0;
     auto fold_from = [&](int c, int first, int step) {
-        constexpr int FU = 8;
+        constexpr int FU = sizeof(Acc) > 8 ? 8 : 16; // partials in flight: a thread's share is a chain of round trips
         Acc r = P::identity();
         int g = first;
         for (; g + (FU - 1) * step < L.splits; g += FU * step) {
@@ -1715,7 +1715,7 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     const int ncol = (int)((L.inner - ocol0 < (int64_t)TX * E) ? L.inner - ocol0 : (int64_t)TX * E);
     const int64_t slot0 = outer * L.inner + ocol0;
     auto fold_from = [&](int c, int first, int step, VT &b, int64_t &bi) {
-        constexpr int FU = 4;
+        constexpr int FU = sizeof(T) > 8 ? 8 : 16; // pairs in flight: a thread's share is a chain of round trips
         b = VT{};
         bi = ARG_NONE;
         int g = first;
