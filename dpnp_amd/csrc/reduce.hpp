@@ -1558,8 +1558,11 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     using VT = value_of_t<T>;
     constexpr int E = 16 / (int)sizeof(T);
     constexpr int U = E >= 8 ? 8 : 4; // rows in flight per thread (see cols_cfg)
-    __shared__ VT smv[256 * E];
-    __shared__ int64_t smi[256 * E];
+    // (position, value) of every place of every thread: sized by the launch (blockDim.x x E pairs; a block of one
+    // wave that held the LDS of 256 threads left a CU room for 13 waves)
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    int64_t *smi = reinterpret_cast<int64_t *>(smem_raw);
+    VT *smv = reinterpret_cast<VT *>(smem_raw + (size_t)blockDim.x * E * sizeof(int64_t));
     const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
     const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> L.g_log2;
     int64_t b = blockIdx.x;

@@ -148,9 +148,11 @@ inline int arg_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
         hipLaunchKernelGGL((arg_flat_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(pl.block), smem, stream, pl.ix,
                            pl.L, sp, dp, pval, pidx, counters);
     }
-    else if (red_is_cols(pl))
-        hipLaunchKernelGGL((arg_cols_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream, pl.ix, pl.L,
-                           sp, dp, pval, pidx, counters);
+    else if (red_is_cols(pl)) {
+        const size_t smem = (size_t)pl.block * (16 / sizeof(T)) * (sizeof(int64_t) + sizeof(value_of_t<T>));
+        hipLaunchKernelGGL((arg_cols_kernel<T, IS_MAX>), dim3((unsigned)pl.grid), dim3(pl.block), smem, stream, pl.ix,
+                           pl.L, sp, dp, pval, pidx, counters);
+    }
     else if (pl.path == DPX_PATH_RED_GENERIC)
         hipLaunchKernelGGL((arg_rows_kernel<T, IS_MAX, false>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
                            pl.L, sp, dp, pval, pidx, counters, pl.ix);
