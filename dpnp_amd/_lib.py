@@ -55,7 +55,7 @@ BINARY_OPS = [
 ]
 REDUCE_OPS = ["sum", "prod", "max", "min", "sumsqdev", "logsumexp", "hypot",
               "nansum", "nanprod", "nanmax", "nanmin", "nancount", "nansumsqdev",
-              "any", "all", "count_nonzero", "nanmean", "nanvar"]
+              "any", "all", "count_nonzero", "nanmean", "nanvar", "sqdev_onepass"]
 SEARCH_OPS = ["argmax", "argmin", "nanargmax", "nanargmin", "nanargmax_marked", "nanargmin_marked"]
 UNARY_ID = {n: i for i, n in enumerate(UNARY_OPS)}
 BINARY_ID = {n: i for i, n in enumerate(BINARY_OPS)}

@@ -235,9 +235,24 @@ enum {
     K_NANMEAN = 16,
     // variance of the elements that are not NaN around a given mean: squared deviations and count travel
     // together, divided by count - ddof at the end
-    K_NANVAR = 17
+    K_NANVAR = 17,
+    // sum of squared deviations from the mean WITHOUT a given mean, in one pass: (count, mean, sum of squared
+    // deviations) triples merged pairwise (Chan, Golub, LeVeque 1979)
+    K_SQDEV1 = 18
 };
 constexpr bool kind_has_count(int k) { return k == K_NANMEAN || k == K_NANVAR; }
+// accumulator of K_SQDEV1: n elements of mean `mean`, m2 = sum of their squared deviations from it
+template <class A> struct sqdev_acc {
+    A n, mean, m2;
+};
+template <class A> DPX_D sqdev_acc<A> sqdev_merge(sqdev_acc<A> a, sqdev_acc<A> b)
+{
+    const A n = a.n + b.n;
+    if (n == A(0)) return a;
+    const A d = b.mean - a.mean;
+    const A fb = b.n / n;
+    return sqdev_acc<A>{n, a.mean + d * fb, a.m2 + b.m2 + d * d * (a.n * fb)};
+}
 // accumulator of K_NANMEAN
 template <class A> struct mean_acc {
     A s;
@@ -277,14 +292,17 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     using In = In_;
     using Out = Out_;
     using Acc = std::conditional_t<
-        kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
-        std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>;
+        KIND == K_SQDEV1, sqdev_acc<acc_of_t<Out_>>,
+        std::conditional_t<
+            kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
+            std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>;
     using Aux = Out_;
     static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV || KIND == K_NANVAR) && !FINAL;
     static constexpr int kind = KIND;
     DPX_D static Acc identity()
     {
         if constexpr (kind_has_count(KIND)) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
+        else if constexpr (KIND == K_SQDEV1) return Acc{0, 0, 0};
         else if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
         else if constexpr (is_bool_v<Out>) return (KIND == K_PROD || KIND == K_ALL) ? 1 : 0;
         else if constexpr (KIND == K_COUNT_NONZERO) return Acc(0);
@@ -297,6 +315,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc pre(In x, Acc aux)
     {
         if constexpr (FINAL) return x; // In == Acc
+        else if constexpr (KIND == K_SQDEV1) return Acc{1, in_to_acc<In, Out>(x) - aux.mean, 0}; // means are kept relative to aux.mean
         else if constexpr (KIND == K_NANMEAN) {
             const bool skip = isnan_(x);
             return Acc{skip ? red_identity<K_SUM, acc_of_t<Out>>() : in_to_acc<In, Out>(x), skip ? 0 : 1};
@@ -327,6 +346,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc combine(Acc a, Acc b)
     {
         if constexpr (kind_has_count(KIND)) return Acc{a.s + b.s, a.c + b.c};
+        else if constexpr (KIND == K_SQDEV1) return sqdev_merge(a, b);
         else if constexpr (is_bool_v<Out>) {
             if constexpr (KIND == K_PROD || KIND == K_MIN || KIND == K_ALL) return a & b;
             else return a | b;
@@ -386,6 +406,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Out post(Acc a)
     {
         if constexpr (KIND == K_NANVAR) return post(a, 0.0);
+        else if constexpr (KIND == K_SQDEV1) return acc_to_out<acc_of_t<Out>, Out>(a.m2);
         else if constexpr (KIND == K_NANMEAN) {
             // sum / count in the accumulator's type: 0 / 0 = NaN for a run without a number
             using A = acc_of_t<Out>;
@@ -598,6 +619,23 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
         if constexpr (CONTIG) {
             const In *p = src + so;
+            if constexpr (P::kind == K_SQDEV1) {
+                // Means travel relative to a reference k0 that every lane and block of an output computes alike:
+                // merges only use differences of means, and absolute means of data far from zero would round them
+                // away.  k0 is the mean of the run's first 64 elements (a whole block per output: its runs are
+                // longer) or its first element (short runs).  Being the mean of 64 of the run's N elements it lies
+                // within sqrt(N / 64) standard deviations of the run's mean, whatever the data.
+                using A = acc_of_t<typename P::Out>;
+                A k0;
+                if (whole_block) {
+                    k0 = in_to_acc<In, typename P::Out>(load_one(p + (threadIdx.x & 63)));
+#pragma unroll
+                    for (int m = 32; m > 0; m >>= 1) k0 += __shfl_xor(k0, m, 64);
+                    k0 *= A(1.0 / 64);
+                }
+                else k0 = in_to_acc<In, typename P::Out>(load_one(p));
+                a = Acc{0, k0, 0};
+            }
             if (L.vec) {
                 const int64_t vend = beg + ((end - beg) / E) * E;
                 const int64_t step = (int64_t)G * E;
@@ -611,6 +649,49 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                         for (int u = 0; u < RED_U; ++u) acc[u] = P::fold_pack(acc[u], v[u]);
                     }
                     for (; pos < vend; pos += step) acc[0] = P::fold_pack(acc[0], load_words16(p + pos));
+                }
+                else if constexpr (P::kind == K_SQDEV1) {
+                    // A lane's elements as sums of d and d^2, d = x - k, k the lane's first element: two
+                    // operations per element where a merge of triples takes a division.  count, mean and m2
+                    // follow as (n, k + s1 / n, s2 - s1^2 / n).  Because k is one of the elements, s2 is at most
+                    // (n + 1) m2, so the rounding of s2 costs m2 a relative error of at most (n + 1) eps, n being
+                    // the few thousand elements of one lane; the lanes' triples are merged pairwise.
+                    using A = acc_of_t<typename P::Out>;
+                    if (pos < vend) {
+                        const A k = in_to_acc<In, typename P::Out>(load_one(p + pos));
+                        A s1[RED_U], s2[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) s1[u] = s2[u] = A(0);
+                        int64_t cnt = 0;
+                        for (; pos + (RED_U - 1) * step < vend; pos += RED_U * step) {
+                            pack<In, E> v[RED_U];
+#pragma unroll
+                            for (int u = 0; u < RED_U; ++u) v[u] = load_pack<In, E>(p + pos + u * step);
+#pragma unroll
+                            for (int u = 0; u < RED_U; ++u)
+#pragma unroll
+                                for (int e = 0; e < E; ++e) {
+                                    const A d = in_to_acc<In, typename P::Out>(v[u].v[e]) - k;
+                                    s1[u] += d;
+                                    s2[u] += d * d;
+                                }
+                            cnt += RED_U * E;
+                        }
+                        for (; pos < vend; pos += step) {
+                            const pack<In, E> v = load_pack<In, E>(p + pos);
+#pragma unroll
+                            for (int e = 0; e < E; ++e) {
+                                const A d = in_to_acc<In, typename P::Out>(v.v[e]) - k;
+                                s1[0] += d;
+                                s2[0] += d * d;
+                            }
+                            cnt += E;
+                        }
+                        const A t1 = (s1[0] + s1[1]) + (s1[2] + s1[3]), t2 = (s2[0] + s2[1]) + (s2[2] + s2[3]);
+                        const A n = (A)cnt;
+                        const A m2 = t2 - t1 * (t1 / n);
+                        acc[0] = Acc{n, (k - a.mean) + t1 / n, m2 > A(0) ? m2 : A(0)};
+                    }
                 }
                 else {
                     for (; pos + (RED_U - 1) * step < vend; pos += RED_U * step) {

@@ -55,7 +55,9 @@ int truth_run(int, RedPlan &, const dpx_array_view *, const dpx_array_view *, hi
 static bool is_truth_op(int op) { return op == DPX_R_ANY || op == DPX_R_ALL || op == DPX_R_COUNT_NONZERO; }
 static bool is_nan_op(int op)
 {
-    return (op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV) || op == DPX_R_NANMEAN || op == DPX_R_NANVAR;
+    // (the one-pass squared deviations are typed in the same file)
+    return (op >= DPX_R_NANSUM && op <= DPX_R_NANSUMSQDEV) || op == DPX_R_NANMEAN || op == DPX_R_NANVAR ||
+           op == DPX_R_SQDEV_ONEPASS;
 }
 static bool takes_aux(int op) { return op == DPX_R_SUMSQDEV || op == DPX_R_NANSUMSQDEV || op == DPX_R_NANVAR; }
 
@@ -89,7 +91,12 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     const bool empty_ok = op != DPX_R_MAX && op != DPX_R_MIN && op != DPX_R_NANMAX && op != DPX_R_NANMIN;
     if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
     RedPlan pl;
-    red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false);
+    red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false, op == DPX_R_SQDEV_ONEPASS);
+    if (op == DPX_R_SQDEV_ONEPASS && pl.path != DPX_PATH_NOOP && pl.path != DPX_PATH_RED_ROWS &&
+        pl.path != DPX_PATH_RED_ROWS_SPLIT && pl.path != DPX_PATH_RED_SMALL)
+        return fail(DPX_ERR_NOT_IMPLEMENTED,
+                    "one-pass squared deviations are for reduced runs that are contiguous in memory; "
+                    "for this layout reduce with DPX_R_SUM, then DPX_R_SUMSQDEV");
     // bytes of one partial result (the accumulator type of the typed kernel)
     auto acc_bytes = [&]() {
         int acc = itemsize_of(dst->dtype);

@@ -83,7 +83,7 @@ static void rows_geometry(int64_t n, int e, int &g_log2, int &block)
 }
 
 void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
-                   const dpx_array_view *aux, bool keep_order, int in_size, bool arg)
+                   const dpx_array_view *aux, bool keep_order, int in_size, bool arg, bool rows_only)
 {
     pl = RedPlan{};
     const int nd = src->nd, ndi = nd - trailing;
@@ -170,7 +170,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     const bool cols_ok = cols_plain || cols_walk;
     RedLaunch &L = pl.L;
 
-    if (contig_red && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
+    if (!rows_only && contig_red && nd_i == 1 && istr[0][0] == n && n >= 2 && n * in_size <= 256 && m >= 64 &&
         tune_int("DPX_RED_SHORT_ROWS", 1) != 0) { // (sweep override: 0 keeps the rows kernel)
         // ---- short rows: a block stages R whole rows in LDS (see red_short_rows_kernel) ----
         const int64_t pitch_bytes = (int64_t)srow_pitch_for((int)n, in_size) * in_size;

@@ -30,6 +30,9 @@ template <class F> static bool for_nan_pair(int op, int in_dt, int out_dt, F &&f
         DPX_PAIR(half_t, half_t) DPX_PAIR(float, float) DPX_PAIR(double, double) DPX_PAIR(half_t, float)
         DPX_PAIR(float, double)
     }
+    else if (op == DPX_R_SQDEV_ONEPASS) { // (no NaN handling: it shares this file's plumbing)
+        DPX_PAIR(float, double) DPX_PAIR(double, double)
+    }
 #undef DPX_PAIR
     return hit;
 }
@@ -48,7 +51,9 @@ template <int KIND> static int nan_run_kind(int op, RedPlan &pl, const dpx_array
         using O = typename decltype(ot)::type;
         // the pair lists above keep complex inputs away from the ordered and the squared-deviation kinds
         constexpr bool ok = !(is_cplx_v<I> && (kind_is_minmax(KIND) || KIND == K_NANSUMSQDEV || KIND == K_NANVAR)) &&
-                            (KIND == K_NANCOUNT) == std::is_same_v<O, int64_t>;
+                            (KIND == K_NANCOUNT) == std::is_same_v<O, int64_t> &&
+                            (KIND != K_SQDEV1 ||
+                             (std::is_same_v<O, double> && (std::is_same_v<I, float> || std::is_same_v<I, double>)));
         if constexpr (ok) {
             if (acc_size) {
                 *acc_size = (int)sizeof(typename RedPolicy<KIND, I, O>::Acc);
@@ -72,6 +77,7 @@ static int nan_dispatch(int op, RedPlan &pl, const dpx_array_view *src, const dp
     case DPX_R_NANSUMSQDEV: return nan_run_kind<K_NANSUMSQDEV>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANMEAN: return nan_run_kind<K_NANMEAN>(op, pl, src, dst, aux, stream, acc_size);
     case DPX_R_NANVAR: return nan_run_kind<K_NANVAR>(op, pl, src, dst, aux, stream, acc_size);
+    case DPX_R_SQDEV_ONEPASS: return nan_run_kind<K_SQDEV1>(op, pl, src, dst, aux, stream, acc_size);
     default: return DPX_ERR_NOT_IMPLEMENTED;
     }
 }

@@ -73,6 +73,21 @@ def _sumsqdev_over_axis(src, mean, trailing_dims_to_reduce, dst, sycl_queue=None
     return _events(sycl_queue)
 
 
+def _sqdev_onepass_over_axis(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
+    """dst[i] = sum_j (src[i, j] - mean_i)**2 with mean_i the mean of row i, in ONE pass over src (float32 or
+    float64 in, float64 out): count, mean and squared deviations travel together and are merged pairwise.  Fast
+    for a contiguous reduced run only (see DPX_R_SQDEV_ONEPASS)."""
+    vs, vd = src._as_view(), dst._as_view()
+    _lib.check(lib.dpx_reduce(_lib.REDUCE_ID["sqdev_onepass"], vs, int(trailing_dims_to_reduce), vd, None,
+                              _stream(sycl_queue)))
+    return _events(sycl_queue)
+
+
+def _sqdev_onepass_dtype_supported(arg_dtype, out_dtype):
+    return bool(lib.dpx_reduce_dtype_supported(_lib.REDUCE_ID["sqdev_onepass"], dtype_id(arg_dtype),
+                                               dtype_id(out_dtype)))
+
+
 def _sumsqdev_over_axis_dtype_supported(arg_dtype, out_dtype, dst_usm_type=None, sycl_queue=None):
     return bool(lib.dpx_reduce_dtype_supported(_lib.REDUCE_ID["sumsqdev"], dtype_id(arg_dtype),
                                                dtype_id(out_dtype)))

@@ -898,3 +898,54 @@ def test_reduced_dims_that_stay_apart(case, dt):
             assert_same(host(dpt.argmax(v, axis=axis)), np.asarray(np.argmax(hv, axis=axis)))
             assert_same(host(dpt.argmin(v, axis=axis)), np.asarray(np.argmin(hv, axis=axis)))
             assert_same(host(dpt.max(v, axis=axis)), np.max(hv, axis=axis))
+
+
+def _exact_var(a, axis, ddof=0):
+    a = a.astype(np.longdouble)
+    m = a.mean(axis=axis, keepdims=True)
+    n = a.size if axis is None else a.shape[axis]
+    return (((a - m) ** 2).sum(axis=axis) / (n - ddof)).astype("f8")
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+def test_variance_in_one_pass_over_contiguous_runs(dt):
+    # float64 accumulation over the last axes of a C-contiguous array takes the one-pass kernel: data far from
+    # zero, outliers at the places lanes start from, constants, tiny and split runs; 1e-12 of the exact variance
+    rng = np.random.default_rng(97)
+    def check(a, axis, ddof=0):
+        got = host(dpt.var(dev(a), axis=axis, correction=ddof, dtype="f8"))
+        want = _exact_var(a, axis, ddof)
+        np.testing.assert_allclose(got, want, rtol=1e-12, atol=0)
+    for n in (1, 2, 3, 5, 63, 64, 257, 4099, 70001, 2_000_003, 1 << 24):
+        a = rng.standard_normal(n).astype(dt)
+        if n > 1:
+            check(a, None)
+            check(a, None, ddof=1)
+        else:
+            assert host(dpt.var(dev(a), dtype="f8")) == 0.0
+        big = (a.astype("f8") * 3 + 1e6).astype(dt)  # mean / sigma = 3e5
+        if n > 1:
+            check(big, None)
+    a = rng.standard_normal(1 << 22).astype(dt)
+    a[::4096] = 1e6  # outliers where lanes take their shift from
+    check(a, None)
+    a[:] = 7.25
+    assert host(dpt.var(dev(a), dtype="f8")) == 0.0
+    for shape in ((1000, 3), (300, 700), (7, 100003), (64, 65, 66)):
+        a = (rng.standard_normal(shape) * 2 - 50).astype(dt)
+        check(a, -1)
+        check(a, -1, ddof=1)
+        if len(shape) == 3:
+            got = host(dpt.var(dev(a), axis=(1, 2), dtype="f8"))
+            np.testing.assert_allclose(got, _exact_var(a.reshape(shape[0], -1), 1), rtol=1e-12)
+    # non-finite values spread as in the two-pass form
+    a = rng.standard_normal(5000).astype(dt)
+    a[123] = np.nan
+    assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
+    a[123] = np.inf
+    assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
+    # std, and the dpnp layer
+    a = rng.standard_normal((50, 4001)).astype(dt)
+    np.testing.assert_allclose(host(dpt.std(dev(a), axis=1, dtype="f8")), np.sqrt(_exact_var(a, 1)), rtol=1e-12)
+    np.testing.assert_allclose(dpnp.asnumpy(dpnp.var(dpnp.array(a), axis=1, dtype="f8", ddof=1)), _exact_var(a, 1, 1),
+                               rtol=1e-12)
