@@ -971,6 +971,56 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                 // the element-wise form keeps one pack in flight: its LOADS x E separate loads and their
                 // addresses would set the register count of the whole kernel (and spill for 1-byte inputs)
                 constexpr int NL = WHOLE ? LOADS : 1;
+                if constexpr (P::kind == K_SQDEV1 && !WALK) {
+                    // one-pass squared deviations down the columns, as in red_rows_kernel: per column, sums of d
+                    // and d^2 with d = x - k, k the first row this thread meets; means relative to row 0 of the
+                    // reduced axis, which every thread row and block of a column reads alike
+                    using A = acc_of_t<typename P::Out>;
+                    {
+                        const pack<In, E> v0 = load(p);
+#pragma unroll
+                        for (int e = 0; e < E; ++e) a[e] = Acc{0, in_to_acc<In, typename P::Out>(v0.v[e]), 0};
+                    }
+                    if (r < end) {
+                        A k[E], s1[E], s2[E];
+                        {
+                            const pack<In, E> vk = load(p + r * L.rstride);
+#pragma unroll
+                            for (int e = 0; e < E; ++e) {
+                                k[e] = in_to_acc<In, typename P::Out>(vk.v[e]);
+                                s1[e] = s2[e] = A(0);
+                            }
+                        }
+                        int64_t cnt = 0;
+                        auto take = [&](const pack<In, E> &v) {
+#pragma unroll
+                            for (int e = 0; e < E; ++e) {
+                                const A d = in_to_acc<In, typename P::Out>(v.v[e]) - k[e];
+                                s1[e] += d;
+                                s2[e] += d * d;
+                            }
+                        };
+                        for (; r + (NL - 1) * TY < end; r += NL * TY) {
+                            pack<In, E> v[NL];
+#pragma unroll
+                            for (int u = 0; u < NL; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+#pragma unroll
+                            for (int u = 0; u < NL; ++u) take(v[u]);
+                            cnt += NL;
+                        }
+                        for (; r < end; r += TY) {
+                            take(load(p + r * L.rstride));
+                            cnt += 1;
+                        }
+                        const A n = (A)cnt;
+#pragma unroll
+                        for (int e = 0; e < E; ++e) {
+                            const A m2 = s2[e] - s1[e] * (s1[e] / n);
+                            acc[0][e] = Acc{n, (k[e] - a[e].mean) + s1[e] / n, m2 > A(0) ? m2 : A(0)};
+                        }
+                    }
+                    return;
+                }
                 // sums and counts of 1- and 2-byte integers into 64-bit accumulators: 16384 rows of a thread at a
                 // time are added up in 32 bits (a sign extension and an add per element instead of four
                 // instructions, half the registers), then moved on to the wide accumulators

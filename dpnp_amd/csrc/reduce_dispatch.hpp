@@ -52,8 +52,8 @@ inline int red_launch_status(const RedPlan &pl, hipStream_t stream, const char *
 int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *dst,
                  const dpx_array_view *aux, bool empty_ok);
 // keep_order: reduced dims may only be merged, not reordered (searches).
-// rows_only: no kernel but the row kernel of contiguous runs may be chosen for short rows (the caller checks the
-// path for the other layouts)
+// rows_only: the kernels for short rows (staged in LDS, or read as one flat stream) are not to be chosen: such
+// matrices then take the plain row or column kernel (the caller checks the path for the other layouts)
 void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const dpx_array_view *dst,
                    const dpx_array_view *aux, bool keep_order, int in_size, bool arg, bool rows_only = false);
 void red_export_plan(const RedPlan &pl, dpx_plan *out, int acc_size);

@@ -252,7 +252,7 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     }
     // ---- cols -----------------------------------------------------------------------
     const int64_t rstride = rstr[0][0];
-    if (!cols_walk && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
+    if (!rows_only && !cols_walk && nd_i == 1 && rstride == inner && inner * in_size < 512 && n >= 16 &&
         tune_int("DPX_RED_FLAT", 1) != 0) { // (sweep override: 0 keeps the column kernel)
         // a row-major matrix with rows shorter than 512 bytes: one flat stream of packs, a block of
         // T threads with T * E a multiple of the row length (see red_flat_kernel)

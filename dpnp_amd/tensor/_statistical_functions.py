@@ -92,18 +92,19 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
             ti._full_usm_ndarray(0, res)
             tei._divide_by_scalar(src=res, scalar=div, dst=res)
         return res
-    # float64 accumulation over the last axes of a C-contiguous array: one pass over the input instead of the
+    # float64 accumulation over the last axes of a C-contiguous array, or down the columns: one pass over the input instead of the
     # mean's pass plus the deviations' (the reference, dpnp/tensor/_statistical_functions.py:140-230, reads the
     # input twice and a full-size temporary three times)
-    if (nelems > 0 and x.size and tuple(perm) == tuple(range(nd)) and x._is_c_contiguous()
-            and tri._sqdev_onepass_dtype_supported(x.dtype, res_dt)):
-        res_shape = x.shape[: nd - red_nd]
+    if nelems > 0 and x.size and tri._sqdev_onepass_dtype_supported(x.dtype, res_dt):
+        arr = permute_dims(x, perm)
+        res_shape = arr.shape[: nd - red_nd]
         res = empty(res_shape, dtype=res_dt)
-        tri._sqdev_onepass_over_axis(src=x, trailing_dims_to_reduce=red_nd, dst=res)
-        tei._divide_by_scalar(src=res, scalar=div, dst=res)
-        if keepdims:
-            res = _keepdims_view(res, res_shape, red_nd, perm, nd)
-        return res
+        if tri._sqdev_onepass_takes(arr, red_nd, res):
+            tri._sqdev_onepass_over_axis(src=arr, trailing_dims_to_reduce=red_nd, dst=res)
+            tei._divide_by_scalar(src=res, scalar=div, dst=res)
+            if keepdims:
+                res = _keepdims_view(res, res_shape, red_nd, perm, nd)
+            return res
     buf = x
     if not tri._sumsqdev_over_axis_dtype_supported(x.dtype, res_dt):
         buf = empty_like(x, dtype=res_dt)

@@ -279,16 +279,22 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 1 and p.vec == 1  # whole lines
     p = plan_reduce("sum", view([5000, 16384], [3, 16384]), 1, view([5000], ptr=P1))
     assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 1 and p.vec == 0
-    # variance in one pass: contiguous reduced runs only (rows shorter than 256 bytes stay with the row kernel,
-    # whose lanes know the reference the means are kept relative to); other layouts are refused
+    # variance in one pass: contiguous reduced runs and columns (short rows stay with the plain row and column
+    # kernels, whose lanes know the reference the means are kept relative to); other layouts are refused
     op = L.REDUCE_ID["sqdev_onepass"]
     p = L.Plan()
     L.check(lib.dpx_reduce_plan(op, view([1 << 28], dt=L.DOUBLE), 1, view([], dt=L.DOUBLE, ptr=P1), p))
     assert L.PATH_NAMES[p.path] == "red_rows_split" and p.scratch_bytes == 131072 + 24 * p.splits
     L.check(lib.dpx_reduce_plan(op, view([1 << 20, 4]), 1, view([1 << 20], dt=L.DOUBLE, ptr=P1), p))
     assert L.PATH_NAMES[p.path] in ("red_small", "red_rows")
-    assert lib.dpx_reduce_plan(op, view([16384, 16384], [1, 16384]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p) \
+    L.check(lib.dpx_reduce_plan(op, view([16384, 16384], [1, 16384]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] == "red_cols_split"  # down the columns
+    L.check(lib.dpx_reduce_plan(op, view([17, 1 << 20], [1, 17]), 1, view([17], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] == "red_cols_split"  # (not the flat stream of short rows)
+    assert lib.dpx_reduce_plan(op, view([16384, 8192], [16384, 2]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p) \
         == L.ERR_NOT_IMPLEMENTED
+    assert lib.dpx_reduce_plan(op, view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], dt=L.DOUBLE, ptr=P1),
+                               p) == L.ERR_NOT_IMPLEMENTED
     assert [(s, d) for s in range(14) for d in range(14) if lib.dpx_reduce_dtype_supported(op, s, d)] \
         == [(L.FLOAT, L.DOUBLE), (L.DOUBLE, L.DOUBLE)]
     # searches walk the reduced space too (its dims keep their order)

@@ -938,6 +938,17 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
         if len(shape) == 3:
             got = host(dpt.var(dev(a), axis=(1, 2), dtype="f8"))
             np.testing.assert_allclose(got, _exact_var(a.reshape(shape[0], -1), 1), rtol=1e-12)
+    # down the columns (and over the leading axes): the column kernel's one-pass form
+    for shape in ((1000, 3), (300, 700), (100003, 7), (5, 20011), (4099, 1001), (20000, 128)):
+        a = (rng.standard_normal(shape) * 2 + 1e5).astype(dt)
+        a[::97] += 1e4  # outliers
+        check(a, 0)
+        check(a, 0, ddof=1)
+    a = (rng.standard_normal((40, 50, 600)) - 7).astype(dt)
+    got = host(dpt.var(dev(a), axis=(0, 1), dtype="f8"))
+    np.testing.assert_allclose(got, _exact_var(a.reshape(-1, 600), 0), rtol=1e-12)
+    got = host(dpt.var(dev(a), axis=1, dtype="f8"))  # a middle axis: outputs contiguous under it
+    np.testing.assert_allclose(got, _exact_var(a, 1), rtol=1e-12)
     # non-finite values spread as in the two-pass form
     a = rng.standard_normal(5000).astype(dt)
     a[123] = np.nan
