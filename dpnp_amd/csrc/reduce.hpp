@@ -727,6 +727,11 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
             const In *p = src + so;
             const int64_t uend = (beg + L.chunk < L.units) ? beg + L.chunk : L.units;
             const int64_t c = L.inner;
+            // (one-pass squared deviations: as in the contiguous form above, with the first element of the
+            // output's reduced space as the reference of the means)
+            constexpr bool SQ = P::kind == K_SQDEV1;
+            using SA = std::conditional_t<SQ, acc_of_t<typename P::Out>, int>;
+            if constexpr (SQ) a = Acc{0, in_to_acc<In, typename P::Out>(load_one(p)), 0};
             // MODE 0: units are elements; 1: packs, every run a whole number of them; 2: packs, the last one of
             // a run partial: it is read as the whole pack that ends with the run's last element (a run holds at
             // least one pack) and the elements it shares with the pack before are left out, so that every
@@ -749,6 +754,26 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                     const uint32_t rem = c32 - k * E;
                     return rem < (uint32_t)E ? E - (int)rem : 0;
                 };
+                // element x into accumulator set u, if it counts
+                SA sk = 0, s1[RED_U], s2[RED_U];
+                int64_t cnt = 0;
+#pragma unroll
+                for (int u = 0; u < RED_U; ++u) s1[u] = s2[u] = 0;
+                if constexpr (SQ) {
+                    if (q < uend) sk = in_to_acc<In, typename P::Out>(load_one(p + w.off));
+                }
+                auto fold = [&](int u, In x, bool ok) {
+                    if constexpr (SQ) {
+                        const SA d = in_to_acc<In, typename P::Out>(x) - sk;
+                        s1[u] += ok ? d : SA(0);
+                        s2[u] += ok ? d * d : SA(0);
+                        cnt += ok ? 1 : 0;
+                    }
+                    else {
+                        const Acc t = P::combine(acc[u], P::pre(x, a));
+                        acc[u] = ok ? t : acc[u];
+                    }
+                };
                 for (; q + (RED_U - 1) * (int64_t)G < uend; q += RED_U * (int64_t)G) {
                     if constexpr (MODE == 0) {
                         In v[RED_U];
@@ -758,7 +783,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                             w.advance();
                         }
 #pragma unroll
-                        for (int u = 0; u < RED_U; ++u) acc[u] = P::combine(acc[u], P::pre(v[u], a));
+                        for (int u = 0; u < RED_U; ++u) fold(u, v[u], true);
                     }
                     else {
                         pack<In, E> v[RED_U];
@@ -772,24 +797,26 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
 #pragma unroll
                         for (int u = 0; u < RED_U; ++u)
 #pragma unroll
-                            for (int e = 0; e < E; ++e) {
-                                const Acc t = P::combine(acc[u], P::pre(v[u].v[e], a));
-                                acc[u] = counts(e, skip[u]) ? t : acc[u];
-                            }
+                            for (int e = 0; e < E; ++e) fold(u, v[u].v[e], counts(e, skip[u]));
                     }
                 }
                 for (; q < uend; q += G) {
-                    if constexpr (MODE == 0) acc[0] = P::combine(acc[0], P::pre(load_one(p + w.off), a));
+                    if constexpr (MODE == 0) fold(0, load_one(p + w.off), true);
                     else {
                         const int skip = MODE >= 2 ? skipped(w.k) : 0;
                         const pack<In, E> v = load_pack<In, E>(p + w.off - skip);
 #pragma unroll
-                        for (int e = 0; e < E; ++e) {
-                            const Acc t = P::combine(acc[0], P::pre(v.v[e], a));
-                            acc[0] = counts(e, skip) ? t : acc[0];
-                        }
+                        for (int e = 0; e < E; ++e) fold(0, v.v[e], counts(e, skip));
                     }
                     w.advance();
+                }
+                if constexpr (SQ) {
+                    if (cnt > 0) {
+                        const SA t1 = (s1[0] + s1[1]) + (s1[2] + s1[3]), t2 = (s2[0] + s2[1]) + (s2[2] + s2[3]);
+                        const SA n = (SA)cnt;
+                        const SA m2 = t2 - t1 * (t1 / n);
+                        acc[0] = Acc{n, (sk - a.mean) + t1 / n, m2 > SA(0) ? m2 : SA(0)};
+                    }
                 }
             };
             if (!L.vec) walk(std::integral_constant<int, 0>{});

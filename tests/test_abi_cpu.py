@@ -291,10 +291,15 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] == "red_cols_split"  # down the columns
     L.check(lib.dpx_reduce_plan(op, view([17, 1 << 20], [1, 17]), 1, view([17], dt=L.DOUBLE, ptr=P1), p))
     assert L.PATH_NAMES[p.path] == "red_cols_split"  # (not the flat stream of short rows)
-    assert lib.dpx_reduce_plan(op, view([16384, 8192], [16384, 2]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p) \
-        == L.ERR_NOT_IMPLEMENTED
-    assert lib.dpx_reduce_plan(op, view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], dt=L.DOUBLE, ptr=P1),
-                               p) == L.ERR_NOT_IMPLEMENTED
+    L.check(lib.dpx_reduce_plan(op, view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], dt=L.DOUBLE, ptr=P1),
+                                p))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2  # lanes walk the reduced dims
+    L.check(lib.dpx_reduce_plan(op, view([16384, 8192], [16384, 2]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] == "red_generic"
+    assert lib.dpx_reduce_plan(op, view([8192, 16384], [2, 16384]), 1, view([8192], dt=L.DOUBLE, ptr=P1), p) \
+        == L.ERR_NOT_IMPLEMENTED  # columns side by side at a stride: no one-pass form
+    assert lib.dpx_reduce_plan(op, view([128, 128, 128, 128], [1 << 14, 1, 1 << 21, 128]), 2,
+                               view([128, 128], dt=L.DOUBLE, ptr=P1), p) == L.ERR_NOT_IMPLEMENTED
     assert [(s, d) for s in range(14) for d in range(14) if lib.dpx_reduce_dtype_supported(op, s, d)] \
         == [(L.FLOAT, L.DOUBLE), (L.DOUBLE, L.DOUBLE)]
     # searches walk the reduced space too (its dims keep their order)

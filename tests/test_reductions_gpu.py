@@ -949,6 +949,18 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
     np.testing.assert_allclose(got, _exact_var(a.reshape(-1, 600), 0), rtol=1e-12)
     got = host(dpt.var(dev(a), axis=1, dtype="f8"))  # a middle axis: outputs contiguous under it
     np.testing.assert_allclose(got, _exact_var(a, 1), rtol=1e-12)
+    # reduced dims that stay apart (lanes walk them): axes (0, 2), sliced matrices, every other element, ragged runs
+    a = (rng.standard_normal((40, 50, 601)) * 3 + 1e5).astype(dt)
+    np.testing.assert_allclose(host(dpt.var(dev(a), axis=(0, 2), dtype="f8")),
+                               _exact_var(np.moveaxis(a, 1, 0).reshape(50, -1), 1), rtol=1e-12)
+    np.testing.assert_allclose(host(dpt.var(dev(a)[:, :, ::2], axis=(0, 2), dtype="f8")),
+                               _exact_var(np.moveaxis(a[:, :, ::2], 1, 0).reshape(50, -1), 1), rtol=1e-12)
+    m = (rng.standard_normal((700, 900)) - 1e4).astype(dt)
+    m[::31, ::29] = 1e3
+    for sl in (np.s_[1:-1, 1:-1], np.s_[:, ::2], np.s_[::2, 3:], np.s_[:, :5]):
+        np.testing.assert_allclose(host(dpt.var(dev(m)[sl], dtype="f8")), _exact_var(m[sl].reshape(-1), None), rtol=1e-12)
+        np.testing.assert_allclose(host(dpt.var(dev(m)[sl], axis=1, dtype="f8", correction=1)),
+                                   _exact_var(m[sl], 1, 1), rtol=1e-12)
     # non-finite values spread as in the two-pass form
     a = rng.standard_normal(5000).astype(dt)
     a[123] = np.nan
