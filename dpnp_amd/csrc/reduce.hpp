@@ -241,6 +241,25 @@ enum {
     K_SQDEV1 = 18
 };
 constexpr bool kind_has_count(int k) { return k == K_NANMEAN || k == K_NANVAR; }
+// accumulator of K_LOGSUMEXP: log(sum(exp(x))) = m + log(s), m the largest element so far, s = sum(exp(x - m)).
+// Merging costs one exp; the pairwise logaddexp it replaces (logsumexp.cpp with math_utils.hpp:129-150) an exp
+// and a log1p per element.
+template <class A> struct lse_acc {
+    A m, s;
+};
+template <class A> DPX_D A lse_exp(A x) // x <= 0
+{
+    if constexpr (std::is_same_v<A, float>) return __expf(x);
+    else return m_exp(x);
+}
+template <class A> DPX_D lse_acc<A> lse_merge(lse_acc<A> a, lse_acc<A> b)
+{
+    const A d = a.m - b.m;
+    const bool same = a.m == b.m; // also equal infinities, whose difference is NaN
+    const A e = same ? A(1) : lse_exp<A>(d > A(0) ? -d : d);
+    const bool ge = d >= A(0) || same; // a NaN operand: false, and e is NaN, which s keeps
+    return lse_acc<A>{ge ? a.m : b.m, ge ? a.s + b.s * e : a.s * e + b.s};
+}
 // accumulator of K_SQDEV1: n elements of mean `mean`, m2 = sum of their squared deviations from it
 template <class A> struct sqdev_acc {
     A n, mean, m2;
@@ -293,9 +312,10 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     using Out = Out_;
     using Acc = std::conditional_t<
         KIND == K_SQDEV1, sqdev_acc<acc_of_t<Out_>>,
+        std::conditional_t<KIND == K_LOGSUMEXP, lse_acc<acc_of_t<Out_>>,
         std::conditional_t<
             kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
-            std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>;
+            std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>>;
     using Aux = Out_;
     static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV || KIND == K_NANVAR) && !FINAL;
     static constexpr int kind = KIND;
@@ -303,6 +323,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     {
         if constexpr (kind_has_count(KIND)) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
         else if constexpr (KIND == K_SQDEV1) return Acc{0, 0, 0};
+        else if constexpr (KIND == K_LOGSUMEXP) return Acc{-(acc_of_t<Out>)__builtin_inff(), 0};
         else if constexpr (is_bool_v<Out> && (KIND == K_MAX || KIND == K_MIN)) return KIND == K_MAX ? 0 : 1;
         else if constexpr (is_bool_v<Out>) return (KIND == K_PROD || KIND == K_ALL) ? 1 : 0;
         else if constexpr (KIND == K_COUNT_NONZERO) return Acc(0);
@@ -316,6 +337,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     {
         if constexpr (FINAL) return x; // In == Acc
         else if constexpr (KIND == K_SQDEV1) return Acc{1, in_to_acc<In, Out>(x) - aux.mean, 0}; // means are kept relative to aux.mean
+        else if constexpr (KIND == K_LOGSUMEXP) return Acc{in_to_acc<In, Out>(x), 1};
         else if constexpr (KIND == K_NANMEAN) {
             const bool skip = isnan_(x);
             return Acc{skip ? red_identity<K_SUM, acc_of_t<Out>>() : in_to_acc<In, Out>(x), skip ? 0 : 1};
@@ -355,7 +377,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
                            KIND == K_NANSUMSQDEV || KIND == K_COUNT_NONZERO)
             return a + b;
         else if constexpr (KIND == K_PROD || KIND == K_NANPROD) return a * b;
-        else if constexpr (KIND == K_LOGSUMEXP) return LogaddexpOp::apply<Acc>(a, b);
+        else if constexpr (KIND == K_LOGSUMEXP) return lse_merge(a, b);
         else if constexpr (KIND == K_HYPOT) return m_hypot(a, b);
         else if constexpr (KIND == K_MAX) return max_nan(a, b);
         else if constexpr (KIND == K_NANMAX) return isnan_(a) ? b : (isnan_(b) ? a : (a > b ? a : b));
@@ -407,6 +429,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     {
         if constexpr (KIND == K_NANVAR) return post(a, 0.0);
         else if constexpr (KIND == K_SQDEV1) return acc_to_out<acc_of_t<Out>, Out>(a.m2);
+        else if constexpr (KIND == K_LOGSUMEXP) return acc_to_out<acc_of_t<Out>, Out>(a.m + m_log(a.s));
         else if constexpr (KIND == K_NANMEAN) {
             // sum / count in the accumulator's type: 0 / 0 = NaN for a run without a number
             using A = acc_of_t<Out>;
@@ -649,6 +672,40 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                         for (int u = 0; u < RED_U; ++u) acc[u] = P::fold_pack(acc[u], v[u]);
                     }
                     for (; pos < vend; pos += step) acc[0] = P::fold_pack(acc[0], load_words16(p + pos));
+                }
+                else if constexpr (P::kind == K_LOGSUMEXP) {
+                    // a round of loads at a time: its largest element first, then one exp per element (and one to
+                    // rescale the running sum) instead of a merge, with its compare and select, per element
+                    using A = acc_of_t<typename P::Out>;
+                    auto take = [&](const A (&x)[RED_U * E], int cnt) {
+                        A bm = acc[0].m;
+#pragma unroll
+                        for (int i = 0; i < RED_U * E; ++i)
+                            if (i < cnt) bm = x[i] > bm ? x[i] : bm;
+                        A sum = acc[0].m == bm ? acc[0].s : acc[0].s * lse_exp<A>(acc[0].m - bm);
+#pragma unroll
+                        for (int i = 0; i < RED_U * E; ++i)
+                            if (i < cnt) sum += x[i] == bm ? A(1) : lse_exp<A>(x[i] - bm); // (a NaN element: NaN)
+                        acc[0] = Acc{bm, sum};
+                    };
+                    for (; pos + (RED_U - 1) * step < vend; pos += RED_U * step) {
+                        pack<In, E> v[RED_U];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u) v[u] = load_pack<In, E>(p + pos + u * step);
+                        A x[RED_U * E];
+#pragma unroll
+                        for (int u = 0; u < RED_U; ++u)
+#pragma unroll
+                            for (int e = 0; e < E; ++e) x[u * E + e] = in_to_acc<In, typename P::Out>(v[u].v[e]);
+                        take(x, RED_U * E);
+                    }
+                    for (; pos < vend; pos += step) {
+                        const pack<In, E> v = load_pack<In, E>(p + pos);
+                        A x[RED_U * E];
+#pragma unroll
+                        for (int e = 0; e < E; ++e) x[e] = in_to_acc<In, typename P::Out>(v.v[e]);
+                        take(x, E);
+                    }
                 }
                 else if constexpr (P::kind == K_SQDEV1) {
                     // A lane's elements as sums of d and d^2, d = x - k, k the lane's first element: two

@@ -106,6 +106,7 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
         if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
+        if (op == DPX_R_LOGSUMEXP) acc *= 2; // (largest element, sum of exponentials relative to it)
         if (is_nan_op(op)) acc = nan_acc_size(op, src, dst);
         if (is_truth_op(op)) acc = op == DPX_R_COUNT_NONZERO ? 8 : 4;
         return acc;

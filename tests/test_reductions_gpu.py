@@ -972,3 +972,43 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
     np.testing.assert_allclose(host(dpt.std(dev(a), axis=1, dtype="f8")), np.sqrt(_exact_var(a, 1)), rtol=1e-12)
     np.testing.assert_allclose(dpnp.asnumpy(dpnp.var(dpnp.array(a), axis=1, dtype="f8", ddof=1)), _exact_var(a, 1, 1),
                                rtol=1e-12)
+
+
+@pytest.mark.parametrize("dt", ["f2", "f4", "f8"])
+def test_logsumexp_every_kernel_family_and_special_values(dt):
+    # (largest element, sum of exponentials relative to it) pairs: rows, columns, flat and walked kernels, split
+    # runs, infinities and NaN
+    rng = np.random.default_rng(211)
+    rtol = {"f2": 2e-3, "f4": 1e-5, "f8": 1e-12}[dt]
+    def want(a, axis):
+        a = a.astype(np.longdouble)
+        m = np.max(a, axis=axis, keepdims=True)
+        m = np.where(np.isfinite(m), m, 0)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            r = np.log(np.sum(np.exp(a - m), axis=axis)) + np.squeeze(m, axis=axis) if axis is not None \
+                else np.log(np.sum(np.exp(a - m))) + m.reshape(())
+        return np.asarray(r)
+    for shape, axis in (((2_000_003,), None), ((4099,), None), ((300, 700), 1), ((300, 700), 0), ((100003, 7), 0),
+                        ((1000, 3), 1), ((40, 50, 60), (0, 2)), ((5, 20011), 0), ((700, 900), None)):
+        a = (rng.standard_normal(shape) * (3 if dt == "f2" else 30)).astype(dt)
+        got = host(dpt.logsumexp(dev(a), axis=axis)).astype(np.longdouble)
+        np.testing.assert_allclose(got, want(a, axis), rtol=rtol, atol=rtol)
+    a = (rng.standard_normal((700, 900)) * 5).astype(dt)
+    got = host(dpt.logsumexp(dev(a)[1:-1, 1:-1])).astype(np.longdouble)  # a sliced matrix: the walked kernel
+    np.testing.assert_allclose(got, want(a[1:-1, 1:-1], None), rtol=rtol)
+    # special values, alone and among numbers, in runs long enough for the batched path
+    base = (rng.standard_normal(5000) * 3).astype(dt)
+    for v, res in ((-np.inf, None), (np.inf, np.inf), (np.nan, np.nan)):
+        a = base.copy()
+        a[[0, 17, 4999]] = v
+        got = float(dpt.logsumexp(dev(a)))
+        if res is None:
+            np.testing.assert_allclose(got, float(want(a, None)), rtol=rtol)
+        elif np.isnan(res):
+            assert np.isnan(got)
+        else:
+            assert got == res
+    assert float(dpt.logsumexp(dev(np.full(3000, -np.inf, dtype=dt)))) == -np.inf
+    assert float(dpt.logsumexp(dev(np.full(3000, np.inf, dtype=dt)))) == np.inf
+    assert np.isnan(float(dpt.logsumexp(dev(np.array([np.inf, -np.inf, np.nan], dtype=dt)))))
+    assert float(dpt.logsumexp(dev(np.array([np.inf, -np.inf], dtype=dt)))) == np.inf
