@@ -95,13 +95,18 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
     # float64 accumulation over the last axes of a C-contiguous array, or down the columns: one pass over the input instead of the
     # mean's pass plus the deviations' (the reference, dpnp/tensor/_statistical_functions.py:140-230, reads the
     # input twice and a full-size temporary three times)
-    if nelems > 0 and x.size and tri._sqdev_onepass_dtype_supported(x.dtype, res_dt):
+    # A float32 result of float32 input goes the same way: accumulated in float64 (never less accurate than the
+    # float32 accumulation of the reference), then rounded; the result arrays are small.
+    acc_dt = float64 if (x.dtype == _as_dtype("f4") and res_dt == _as_dtype("f4")) else res_dt
+    if nelems > 0 and x.size and tri._sqdev_onepass_dtype_supported(x.dtype, acc_dt):
         arr = permute_dims(x, perm)
         res_shape = arr.shape[: nd - red_nd]
-        res = empty(res_shape, dtype=res_dt)
+        res = empty(res_shape, dtype=acc_dt)
         if tri._sqdev_onepass_takes(arr, red_nd, res):
             tri._sqdev_onepass_over_axis(src=arr, trailing_dims_to_reduce=red_nd, dst=res)
             tei._divide_by_scalar(src=res, scalar=div, dst=res)
+            if acc_dt != res_dt:
+                res = astype(res, res_dt, copy=False)
             if keepdims:
                 res = _keepdims_view(res, res_shape, red_nd, perm, nd)
             return res
