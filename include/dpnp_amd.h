@@ -230,8 +230,8 @@ typedef enum dpx_reduce_op {
      * dpnp/dpnp_iface_nanfunctions.py:1188-1391).  ddof is 0 through dpx_reduce; dpx_nan_variance
      * takes it as an argument. */
     DPX_R_NANVAR,
-    /* sum((x - mean(x))^2) in ONE pass over the input, without a given mean: float32 or float64 in, float64
-     * out.  The reference's var reads the input for the mean, then again for the deviations
+    /* sum((x - mean(x))^2) in ONE pass over the input, without a given mean: float32, float64 or an integer
+     * type in, float64 out.  The reference's var reads the input for the mean, then again for the deviations
      * (dpnp/tensor/_statistical_functions.py:140-230: sum, divide, subtract, multiply, sum); this op carries
      * (count, mean, sum of squared deviations) triples and merges them pairwise.  For reduced runs that are
      * contiguous in memory (last axes of a C-contiguous array), for one strided reduced axis whose outputs

@@ -967,6 +967,11 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
     assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
     a[123] = np.inf
     assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
+    # integer input: float64 result straight from the integers
+    for idt in ("i1", "u2", "i4", "u8"):
+        a = rng.integers(0, 100, (300, 700)).astype(idt)
+        for ax in (None, 0, 1):
+            np.testing.assert_allclose(host(dpt.var(dev(a), axis=ax)), _exact_var(a, ax), rtol=1e-12)
     # std, and the dpnp layer
     a = rng.standard_normal((50, 4001)).astype(dt)
     np.testing.assert_allclose(host(dpt.std(dev(a), axis=1, dtype="f8")), np.sqrt(_exact_var(a, 1)), rtol=1e-12)
