@@ -1015,6 +1015,20 @@ struct FloorDivOp { // floor_divide.hpp:63-86: ints (x // 0 == 0) and real fp
             const int r = q - ((m != 0) && ((m < 0) != ((int)b < 0)));
             return b == T(0) ? T(0) : (T)r;
         }
+        else if constexpr (is_int_v<T> && sizeof(T) == 4) {
+            // 32-bit operands through the double quotient, branch-free: both are exact as doubles, and a
+            // quotient that is not an integer lies at least 1 / |b| from the next one, 2^-31 of its size and
+            // more, so the correctly rounded double quotient never lands on an integer it does not equal and
+            // its floor is the floored quotient (a third of the instructions of the integer division with its
+            // sign cases; int32 // scalar: 67 % of the HBM rate before)
+            const double q = __builtin_floor((double)a / (double)b);
+            T r;
+            if constexpr (std::is_signed_v<T>) {
+                r = (T)(int64_t)q; // (-2^31 // -1 = 2^31 wraps to -2^31 in the cast)
+            }
+            else r = (T)q;
+            return b == T(0) ? T(0) : r;
+        }
         else if constexpr (is_int_v<T>) {
             if (b == T(0)) return T(0);
             if constexpr (std::is_signed_v<T>) {

@@ -841,3 +841,29 @@ def test_mixed_dtype_arithmetic_equals_cast_then_compute(op, pair):
     if op == "add":
         d2 += dev(b)
         assert_same(host(d2), a + b.astype(wide))
+
+
+@pytest.mark.parametrize("dt", ["i4", "u4"])
+def test_floor_divide_of_32_bit_integers_on_hard_quotients(dt):
+    """32-bit floor_divide goes through the double quotient: extremes, divisors of every size and sign, quotients
+    that miss an integer by 1 / b, zero divisors (result 0, floor_divide.hpp:63-86), -2^31 // -1 (wraps)."""
+    rng = np.random.default_rng(4242)
+    info = np.iinfo(dt)
+    edge = np.array([info.min, info.min + 1, -2, -1, 0, 1, 2, 3, 7, 46341, 65535, 65536, info.max - 1, info.max],
+                    dtype=np.int64)
+    edge = edge[(edge >= info.min) & (edge <= info.max)]
+    a = np.concatenate([np.repeat(edge, len(edge)), rng.integers(info.min, info.max, 200000, endpoint=True)])
+    b = np.concatenate([np.tile(edge, len(edge)), rng.integers(info.min, info.max, 200000, endpoint=True)])
+    # k * b - 1, k * b, k * b + 1: quotients next to an integer
+    bb = rng.integers(1, 1 << 16, 100000)
+    kk = rng.integers(0, (info.max // (1 << 16)), 100000)
+    for off in (-1, 0, 1):
+        a = np.concatenate([a, np.clip(kk * bb + off, info.min, info.max)])
+        b = np.concatenate([b, bb if dt == "u4" else bb * rng.choice([-1, 1], bb.size)])
+    a, b = a.astype(dt), b.astype(dt)
+    want = orc.binary("floor_divide", a, b)
+    assert_same(host(dpt.floor_divide(dev(a), dev(b))), want)
+    # against a scalar divisor and in place
+    for d in ((7, 1, 3) if dt == "u4" else (7, -7, -1, 1)):
+        x = dev(a)
+        assert_same(host(dpt.floor_divide(x, d)), orc.binary("floor_divide", a, np.full_like(a, d)))
