@@ -1054,6 +1054,16 @@ struct RemainderOp { // remainder.hpp: Python-style modulo, x % 0 == 0 for ints
             const int r = (m != 0 && ((m < 0) != ((int)b < 0))) ? m + (int)b : m;
             return b == T(0) ? T(0) : (T)r;
         }
+        else if constexpr (is_int_v<T> && sizeof(T) == 4) {
+            // a - floor(a / b) * b with the floored quotient of FloorDivOp (exact for 32-bit operands), in
+            // wrapping 32-bit arithmetic: the sign follows the divisor, -2^31 % -1 comes out as 0
+            using U = std::make_unsigned_t<T>;
+            const double q = __builtin_floor((double)a / (double)b);
+            U qi;
+            if constexpr (std::is_signed_v<T>) qi = (U)(int64_t)q;
+            else qi = (U)q;
+            return b == T(0) ? T(0) : (T)((U)a - qi * (U)b);
+        }
         else if constexpr (is_int_v<T>) {
             if (b == T(0)) return T(0);
             if constexpr (std::is_signed_v<T>) {

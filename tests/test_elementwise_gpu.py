@@ -863,7 +863,9 @@ def test_floor_divide_of_32_bit_integers_on_hard_quotients(dt):
     a, b = a.astype(dt), b.astype(dt)
     want = orc.binary("floor_divide", a, b)
     assert_same(host(dpt.floor_divide(dev(a), dev(b))), want)
-    # against a scalar divisor and in place
+    assert_same(host(dpt.remainder(dev(a), dev(b))), orc.binary("remainder", a, b))  # the same quotient
+    # against a scalar divisor
     for d in ((7, 1, 3) if dt == "u4" else (7, -7, -1, 1)):
         x = dev(a)
         assert_same(host(dpt.floor_divide(x, d)), orc.binary("floor_divide", a, np.full_like(a, d)))
+        assert_same(host(dpt.remainder(x, d)), orc.binary("remainder", a, np.full_like(a, d)))
