@@ -28,7 +28,18 @@ def _move_reduced_axes_last(x, axis, int_only=False):
         axis = (axis,)
     axis = normalize_axis_tuple(axis, nd, "axis")
     perm = [i for i in range(nd) if i not in axis] + list(axis)
-    return permute_dims(x, perm), axis, perm
+    if perm == list(range(nd)):
+        return x, axis, perm  # the reduced axes are the last ones already: x and its cached descriptor serve
+    # the permuted view of an array is kept with it: the next call with the same axes finds the view and the
+    # descriptor it has built
+    cache = x.__dict__.get("_perm_views")
+    if cache is None:
+        cache = x.__dict__["_perm_views"] = {}
+    key = tuple(perm)
+    arr = cache.get(key)
+    if arr is None:
+        arr = cache[key] = x._view([x._shape[a] for a in perm], [x._strides[a] for a in perm], x._offset)
+    return arr, axis, perm
 
 
 def _prepare_out(x, out, axis, keepdims, res_shape, res_dt, guard_overlap):

@@ -201,6 +201,7 @@ class usm_ndarray:
         r = reshape(self, new_shape, copy=False)
         self._shape, self._strides = r._shape, r._strides
         self.__dict__.pop("_cview", None)
+        self.__dict__.pop("_perm_views", None)
 
     @property
     def strides(self):
