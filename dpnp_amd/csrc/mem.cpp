@@ -30,6 +30,7 @@ struct Block {
     size_t size;
     hipStream_t stream; // the stream of its last use; meaningful while cached
     bool idle;          // its last use is known to have completed (the stream was synchronized or destroyed)
+    uint64_t stamp;     // value of the free counter when it was cached: orders frees against stream waits
 };
 
 constexpr int MAX_DEVICES = 64;
@@ -39,6 +40,7 @@ std::multimap<size_t, Block> g_cache[MAX_DEVICES];       // free, by size
 std::unordered_map<void *, int> g_device_of;             // every block the pool owns -> device
 std::unordered_set<hipStream_t> g_streams;               // streams made by dpx_stream_create
 size_t g_in_use = 0, g_cached = 0;
+uint64_t g_free_seq = 0;                                 // counts dpx_mem_free calls
 
 size_t round_size(size_t n)
 {
@@ -107,13 +109,20 @@ int dpx_stream_create(void **stream)
 
 int dpx_stream_synchronize(void *stream)
 {
+    // Blocks freed on this stream BEFORE the wait starts have completed when it returns.  Another thread may
+    // free a block on the stream while this one waits or before it takes the lock again: that block's work
+    // may still be queued, so it must not be marked.
+    uint64_t seen;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        seen = g_free_seq;
+    }
     hipError_t e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return fail_hip(e, "hipStreamSynchronize");
-    // everything freed on this stream so far has completed
     std::lock_guard<std::mutex> lk(g_mu);
     for (auto &cache : g_cache)
         for (auto &kv : cache)
-            if (kv.second.stream == (hipStream_t)stream) kv.second.idle = true;
+            if (kv.second.stream == (hipStream_t)stream && kv.second.stamp <= seen) kv.second.idle = true;
     return DPX_OK;
 }
 
@@ -145,7 +154,7 @@ int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream)
     if (nbytes > ((size_t)1 << 46)) return fail(DPX_ERR_BAD_ARGUMENT, "mem_alloc: more than 64 TiB asked for");
     const size_t size = round_size(nbytes);
     const hipStream_t s = (hipStream_t)stream;
-    Block blk{nullptr, 0, nullptr, true};
+    Block blk{nullptr, 0, nullptr, true, 0};
     {
         std::lock_guard<std::mutex> lk(g_mu);
         auto &cache = g_cache[dev];
@@ -196,7 +205,7 @@ int dpx_mem_alloc(void **ptr, size_t nbytes, void *stream)
                 return fail(DPX_ERR_HIP, "mem_alloc: hipMalloc of " + std::to_string(size) + " bytes: " + hipGetErrorString(e));
             }
         }
-        blk = Block{p, size, s, false};
+        blk = Block{p, size, s, false, 0};
     }
     blk.stream = s;
     blk.idle = false;
@@ -220,6 +229,7 @@ int dpx_mem_free(void *ptr, void *stream)
     g_live.erase(it);
     blk.stream = (hipStream_t)stream;
     blk.idle = false;
+    blk.stamp = ++g_free_seq;
     g_in_use -= blk.size;
     g_cached += blk.size;
     g_cache[g_device_of[ptr]].emplace(blk.size, blk);

@@ -316,9 +316,20 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         std::conditional_t<
             kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
             std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>>;
-    using Aux = Out_;
+    // sum(|z - mean|^2) of complex input into a real result (variance of complex data,
+    // dpnp/dpnp_iface_statistics.py:1849-1851: x * conj(x), real part): the mean is a complex number of the
+    // result's precision, the deviation's two parts are squared and added in the real accumulator
+    static constexpr bool cplx_dev = KIND == K_SUMSQDEV && is_cplx_v<In_> && !is_cplx_v<Out_> && !FINAL;
+    using Aux = std::conditional_t<cplx_dev, cplx<Out_>, Out_>;
+    // what a kernel keeps of an output's side input while it reads that output's elements
+    using AuxAcc = std::conditional_t<cplx_dev, cplx<acc_of_t<Out_>>, Acc>;
     static constexpr bool has_aux = (KIND == K_SUMSQDEV || KIND == K_NANSUMSQDEV || KIND == K_NANVAR) && !FINAL;
     static constexpr int kind = KIND;
+    DPX_D static AuxAcc aux_identity()
+    {
+        if constexpr (cplx_dev) return AuxAcc{0, 0};
+        else return identity();
+    }
     DPX_D static Acc identity()
     {
         if constexpr (kind_has_count(KIND)) return Acc{red_identity<K_SUM, acc_of_t<Out>>(), 0};
@@ -333,9 +344,13 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         else if constexpr (KIND == K_NANPROD) return red_identity<K_PROD, Acc>();
         else return red_identity<KIND, Acc>();
     }
-    DPX_D static Acc pre(In x, Acc aux)
+    DPX_D static Acc pre(In x, AuxAcc aux)
     {
         if constexpr (FINAL) return x; // In == Acc
+        else if constexpr (cplx_dev) {
+            const Acc dr = (Acc)x.re - aux.re, di = (Acc)x.im - aux.im;
+            return dr * dr + di * di;
+        }
         else if constexpr (KIND == K_SQDEV1) return Acc{1, in_to_acc<In, Out>(x) - aux.mean, 0}; // means are kept relative to aux.mean
         else if constexpr (KIND == K_LOGSUMEXP) return Acc{in_to_acc<In, Out>(x), 1};
         else if constexpr (KIND == K_NANMEAN) {
@@ -451,9 +466,10 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         }
         else return post(a);
     }
-    DPX_D static Acc load_aux(const Aux *p)
+    DPX_D static AuxAcc load_aux(const Aux *p)
     {
-        if constexpr (KIND == K_NANVAR) return Acc{(acc_of_t<Out>)*p, 0};
+        if constexpr (cplx_dev) return AuxAcc{(Acc)p->re, (Acc)p->im};
+        else if constexpr (KIND == K_NANVAR) return Acc{(acc_of_t<Out>)*p, 0};
         else if constexpr (std::is_same_v<Aux, half_t>) return (float)*p;
         else if constexpr (is_bool_v<Aux>) return (int32_t)p->v;
         else return (Acc)*p;
@@ -636,7 +652,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
     int64_t so = 0, dof = 0, ao = 0;
     if (active) {
         iter_offsets(ix, L, o, so, dof, ao);
-        Acc a = P::identity();
+        typename P::AuxAcc a = P::aux_identity();
         if constexpr (P::has_aux) a = P::load_aux(aux + ao);
         const int64_t beg = (int64_t)split * L.chunk;
         const int64_t end = (beg + L.chunk < L.n) ? beg + L.chunk : L.n;
@@ -747,7 +763,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                         const A t1 = (s1[0] + s1[1]) + (s1[2] + s1[3]), t2 = (s2[0] + s2[1]) + (s2[2] + s2[3]);
                         const A n = (A)cnt;
                         const A m2 = t2 - t1 * (t1 / n);
-                        acc[0] = Acc{n, (k - a.mean) + t1 / n, m2 > A(0) ? m2 : A(0)};
+                        acc[0] = Acc{n, (k - a.mean) + t1 / n, m2 < A(0) ? A(0) : m2};
                     }
                 }
                 else {
@@ -872,7 +888,7 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
                         const SA t1 = (s1[0] + s1[1]) + (s1[2] + s1[3]), t2 = (s2[0] + s2[1]) + (s2[2] + s2[3]);
                         const SA n = (SA)cnt;
                         const SA m2 = t2 - t1 * (t1 / n);
-                        acc[0] = Acc{n, (sk - a.mean) + t1 / n, m2 > SA(0) ? m2 : SA(0)};
+                        acc[0] = Acc{n, (sk - a.mean) + t1 / n, m2 < SA(0) ? SA(0) : m2};
                     }
                 }
             };
@@ -1015,9 +1031,9 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
     }
     const int last = ix.nd_i - 1;
     if (active) {
-        Acc a[E];
+        typename P::AuxAcc a[E];
 #pragma unroll
-        for (int e = 0; e < E; ++e) a[e] = P::identity();
+        for (int e = 0; e < E; ++e) a[e] = P::aux_identity();
         if constexpr (P::has_aux) {
 #pragma unroll
             for (int e = 0; e < E; ++e)
@@ -1100,7 +1116,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
 #pragma unroll
                         for (int e = 0; e < E; ++e) {
                             const A m2 = s2[e] - s1[e] * (s1[e] / n);
-                            acc[0][e] = Acc{n, (k[e] - a[e].mean) + s1[e] / n, m2 > A(0) ? m2 : A(0)};
+                            acc[0][e] = Acc{n, (k[e] - a[e].mean) + s1[e] / n, m2 < A(0) ? A(0) : m2};
                         }
                     }
                     return;
@@ -1293,9 +1309,9 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     const int64_t packs = elems / E;
     const In *p = src + row0 * inner;
 
-    Acc a[E];
+    typename P::AuxAcc a[E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) a[e] = P::identity();
+    for (int e = 0; e < E; ++e) a[e] = P::aux_identity();
     if constexpr (P::has_aux) {
         int c = (int)(((int64_t)t * E) % inner);
 #pragma unroll
@@ -1338,7 +1354,7 @@ __global__ __launch_bounds__(256) void red_flat_kernel(RedIndex ix, RedLaunch L,
     if (t < tail) {
         const int64_t i = packs * E + t;
         const int k = (int)(i % ((int64_t)T * E));
-        Acc ax = P::identity();
+        typename P::AuxAcc ax = P::aux_identity();
         if constexpr (P::has_aux) ax = P::load_aux(aux + (int64_t)(k % inner) * ix.aux_str[0]);
         sm[k] = P::combine(sm[k], P::pre(load_one(p + i), ax));
     }
@@ -1451,7 +1467,7 @@ __global__ __launch_bounds__(256) void red_short_rows_kernel(RedIndex ix, RedLau
     __syncthreads();
     for (int r = t; r < R; r += 256) { // very short rows: several rows per thread
         const int64_t o = row0 + r;
-        Acc a = P::identity();
+        typename P::AuxAcc a = P::aux_identity();
         if constexpr (P::has_aux) a = P::load_aux(aux + o * ix.aux_str[0]);
         const In *row = sm + r * pitch;
         Acc acc = P::identity();

@@ -40,6 +40,7 @@ int sum_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream
 int prod_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 int sqdev_run(RedPlan &, const dpx_array_view *, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 int sum_acc_size(int, int);
+int sqdev_acc_size(int, int);
 int prod_acc_size(int, int);
 int minmax_run(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
 int arg_run_any(bool, RedPlan &, const dpx_array_view *, const dpx_array_view *, hipStream_t);
@@ -84,12 +85,16 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
 {
     if (op < 0 || op >= DPX_R_NUM_OPS) return fail(DPX_ERR_BAD_ARGUMENT, "unknown reduction op id");
     if (!view_ok(src) || !view_ok(dst)) return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
-    if (takes_aux(op) != (aux != nullptr))
+    if (!plan_out && takes_aux(op) != (aux != nullptr))
         return fail(DPX_ERR_BAD_ARGUMENT, "aux must be given for the squared-deviation ops and only for them");
     if (!reduce_supported(op, src->dtype, dst->dtype))
         return fail(DPX_ERR_NOT_IMPLEMENTED, "Datatypes are not supported");
     const bool empty_ok = op != DPX_R_MAX && op != DPX_R_MIN && op != DPX_R_NANMAX && op != DPX_R_NANMIN;
-    if (int rc = red_validate(src, trailing, dst, aux, empty_ok)) return rc;
+    // deviations of complex input from a complex mean, squared magnitudes summed into a real result
+    const int aux_dt = (op == DPX_R_SUMSQDEV && (src->dtype == DPX_CFLOAT || src->dtype == DPX_CDOUBLE))
+                           ? (dst->dtype == DPX_FLOAT ? DPX_CFLOAT : DPX_CDOUBLE)
+                           : -1;
+    if (int rc = red_validate(src, trailing, dst, aux, empty_ok, aux_dt)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false, op == DPX_R_SQDEV_ONEPASS);
     if (op == DPX_R_SQDEV_ONEPASS && pl.path != DPX_PATH_NOOP && pl.path != DPX_PATH_RED_ROWS &&
@@ -102,10 +107,11 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     // bytes of one partial result (the accumulator type of the typed kernel)
     auto acc_bytes = [&]() {
         int acc = itemsize_of(dst->dtype);
-        if (op == DPX_R_SUM || op == DPX_R_SUMSQDEV) acc = sum_acc_size(src->dtype, dst->dtype) ? sum_acc_size(src->dtype, dst->dtype) : acc;
+        if (op == DPX_R_SUM) acc = sum_acc_size(src->dtype, dst->dtype);
+        if (op == DPX_R_SUMSQDEV) acc = sqdev_acc_size(src->dtype, dst->dtype);
         if (op == DPX_R_PROD) acc = prod_acc_size(src->dtype, dst->dtype);
         if ((op == DPX_R_MAX || op == DPX_R_MIN) && dst->dtype == DPX_BOOL) acc = 4;
-        if ((op == DPX_R_SUMSQDEV || op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
+        if ((op == DPX_R_LOGSUMEXP || op == DPX_R_HYPOT) && dst->dtype == DPX_HALF) acc = 4;
         if (op == DPX_R_LOGSUMEXP) acc *= 2; // (largest element, sum of exponentials relative to it)
         if (is_nan_op(op)) acc = nan_acc_size(op, src, dst);
         if (is_truth_op(op)) acc = op == DPX_R_COUNT_NONZERO ? 8 : 4;
@@ -124,12 +130,10 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
                         "dpx_reduce_noalloc: the partial results of this reduction need " + std::to_string(need) +
                             " bytes of scratch, the static scratch holds " +
                             std::to_string((size_t)DPX_NOALLOC_SCRATCH_BYTES) + "; use dpx_reduce");
-        // the static block instead of the pool's; its ticket counters must be zero when the kernel
-        // starts, whatever an earlier call left (a fill kernel: legal under stream capture)
+        // the static block instead of the pool's (red_scratch checks the typed kernel's own slot size against it
+        // once more and clears the ticket counters, in that order)
         if (int rc = noalloc_scratch(&pl.ext_scratch)) return rc;
         pl.ext_scratch_bytes = DPX_NOALLOC_SCRATCH_BYTES;
-        const hipError_t e = zero_fill_async(pl.ext_scratch, RED_COUNTER_BYTES / 16, s);
-        if (e != hipSuccess) return fail_hip(e, "clearing the static scratch counters");
     }
     if (is_nan_op(op)) return nan_run(op, pl, src, dst, aux, s);
     if (is_truth_op(op)) return truth_run(op, pl, src, dst, s);
@@ -192,10 +196,7 @@ int dpx_reduce_plan(int op, const dpx_array_view *src, int trailing_dims_to_redu
                     dpx_plan *plan)
 {
     if (!plan) return fail(DPX_ERR_BAD_ARGUMENT, "plan is null");
-    // a plan for a squared-deviation op is that of the matching sum with the same dtypes
-    if (op == DPX_R_SUMSQDEV) op = DPX_R_SUM;
-    if (op == DPX_R_NANSUMSQDEV) op = DPX_R_NANSUM;
-    if (op == DPX_R_NANVAR) op = DPX_R_NANMEAN;
+    // (the ops with a side input are planned without it: its layout follows the destination's)
     return reduce_call(op, src, trailing_dims_to_reduce, dst, nullptr, nullptr, plan);
 }
 int dpx_nan_variance(const dpx_array_view *src, int trailing_dims_to_reduce, const dpx_array_view *mean, double ddof,

@@ -32,6 +32,11 @@ inline int red_scratch(const RedPlan &pl, hipStream_t stream, size_t need, char 
                         "this reduction needs " + std::to_string(need) + " bytes of scratch for its partial results; "
                         "the static scratch of the entry point that allocates nothing holds " +
                         std::to_string(pl.ext_scratch_bytes) + ": use dpx_reduce");
+        // the size is known to fit (from the typed kernel's own slot size): only now is anything launched.
+        // The ticket counters must be zero when the kernel starts, whatever an earlier call left
+        // (a fill kernel: legal under stream capture)
+        const hipError_t e = zero_fill_async(pl.ext_scratch, RED_COUNTER_BYTES / 16, stream);
+        if (e != hipSuccess) return fail_hip(e, "clearing the static scratch counters");
         *out = pl.ext_scratch;
         return DPX_OK;
     }
@@ -49,8 +54,9 @@ inline int red_launch_status(const RedPlan &pl, hipStream_t stream, const char *
 
 // Validation shared by reductions and searches, in the order of py_reduction_over_axis
 // (libtensor/source/reductions/reduction_over_axis.hpp:188-238).
+// aux_dt: the dtype aux must have (-1: the destination's)
 int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *dst,
-                 const dpx_array_view *aux, bool empty_ok);
+                 const dpx_array_view *aux, bool empty_ok, int aux_dt = -1);
 // keep_order: reduced dims may only be merged, not reordered (searches).
 // rows_only: the kernels for short rows (staged in LDS, or read as one flat stream) are not to be chosen: such
 // matrices then take the plain row or column kernel (the caller checks the path for the other layouts)
@@ -71,7 +77,7 @@ inline int red_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view 
     using Acc = typename P::Acc;
     const In *sp = (const In *)src->data + pl.src_off;
     Out *dp = (Out *)dst->data + pl.dst_off;
-    const Out *ap = aux ? (const Out *)aux->data + pl.aux_off : nullptr;
+    const typename P::Aux *ap = aux ? (const typename P::Aux *)aux->data + pl.aux_off : nullptr;
     if (pl.path == DPX_PATH_NOOP) return DPX_OK;
     if (pl.L.n == 0) {
         hipLaunchKernelGGL((red_fill_kernel<P>), dim3((unsigned)((pl.L.m + 255) / 256)), dim3(256), 0, stream,

@@ -7,7 +7,7 @@
 namespace dpx {
 
 int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *dst,
-                 const dpx_array_view *aux, bool empty_ok)
+                 const dpx_array_view *aux, bool empty_ok, int aux_dt)
 {
     if (!view_ok(src) || !view_ok(dst) || (aux && !view_ok(aux)))
         return fail(DPX_ERR_BAD_ARGUMENT, "malformed array descriptor");
@@ -24,7 +24,10 @@ int red_validate(const dpx_array_view *src, int trailing, const dpx_array_view *
     if (!(dst->flags & DPX_WRITABLE)) return fail(DPX_ERR_NOT_WRITABLE, "output array is read-only.");
     if (aux) {
         if (!same_shape(aux, dst)) return fail(DPX_ERR_SHAPE_MISMATCH, "aux shape does not match destination shape");
-        if (aux->dtype != dst->dtype) return fail(DPX_ERR_BAD_DTYPE, "aux dtype does not match destination dtype");
+        if (aux_dt < 0 && aux->dtype != dst->dtype)
+            return fail(DPX_ERR_BAD_DTYPE, "aux dtype does not match destination dtype");
+        if (aux_dt >= 0 && aux->dtype != aux_dt)
+            return fail(DPX_ERR_BAD_DTYPE, "aux of complex input must be complex, of the destination's precision");
     }
     const int64_t m = view_size(dst);
     int64_t n = 1;

@@ -112,12 +112,22 @@ template <class F> static bool for_sqdev_pair(int in_dt, int out_dt, F &&f)
     DPX_PAIR(double, double) DPX_PAIR(bool_t, double) DPX_PAIR(int8_t, double) DPX_PAIR(uint8_t, double)
     DPX_PAIR(int16_t, double) DPX_PAIR(uint16_t, double) DPX_PAIR(int32_t, double) DPX_PAIR(uint32_t, double)
     DPX_PAIR(int64_t, double) DPX_PAIR(uint64_t, double)
+    // complex input, complex aux: sum(|z - aux|^2), a real result
+    DPX_PAIR(c64, float) DPX_PAIR(c64, double) DPX_PAIR(c128, double)
 #undef DPX_PAIR
     return hit;
 }
 bool sqdev_pair_supported(int in_dt, int out_dt)
 {
     return for_sqdev_pair(in_dt, out_dt, [](auto, auto) {});
+}
+int sqdev_acc_size(int in_dt, int out_dt)
+{
+    int sz = 0;
+    for_sqdev_pair(in_dt, out_dt, [&](auto it, auto ot) {
+        sz = (int)sizeof(typename RedPolicy<K_SUMSQDEV, typename decltype(it)::type, typename decltype(ot)::type>::Acc);
+    });
+    return sz;
 }
 int sqdev_run(RedPlan &pl, const dpx_array_view *src, const dpx_array_view *dst, const dpx_array_view *aux,
               hipStream_t stream)

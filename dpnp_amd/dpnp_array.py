@@ -159,15 +159,19 @@ class dpnp_array:
 
         return dpnp.mean(self, axis=axis, dtype=dtype, out=out, keepdims=keepdims, where=where)
 
-    def var(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True):
+    def var(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
+            correction=None):
         from . import dpnp_iface as dpnp
 
-        return dpnp.var(self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims, where=where)
+        return dpnp.var(self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims, where=where,
+                        mean=mean, correction=correction)
 
-    def std(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True):
+    def std(self, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
+            correction=None):
         from . import dpnp_iface as dpnp
 
-        return dpnp.std(self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims, where=where)
+        return dpnp.std(self, axis=axis, dtype=dtype, out=out, ddof=ddof, keepdims=keepdims, where=where,
+                        mean=mean, correction=correction)
 
     def all(self, axis=None, out=None, keepdims=False, *, where=True):
         from . import dpnp_iface as dpnp

@@ -725,20 +725,73 @@ def mean(a, /, axis=None, dtype=None, out=None, keepdims=False, *, where=True):
     return get_result_array(res, out, casting="unsafe")
 
 
-def var(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
-        correction=None):
-    check_limitations(where=where)
-    if mean is not None:
-        raise NotImplementedError("var(..., mean=) is outside this library's scope")
+_mean = mean  # (var and std have a parameter of that name)
+
+
+def _check_ddof(ddof, correction):
     if correction is not None:
         if ddof != 0:
             raise ValueError("ddof and correction can't be provided simultaneously.")
         ddof = correction
     if not isinstance(ddof, (int, float)):
         raise TypeError(f"An integer or float is required, but got {type(ddof)}")
+    return ddof
+
+
+def _var_around_mean(a, u, axis, dtype, out, ddof, keepdims, mean):
+    """Variance of complex data, or around a mean the caller brings: dpnp/dpnp_iface_statistics.py:1832-1869.
+
+    sum(|a - mean|**2) / (N - ddof), with the reference's dtype rules (integer and bool input computes in
+    the default floating type; the deviations live in the type `a - mean` promotes to; the sum is taken
+    in `dtype` when given) and its divisor (N - ddof as it comes, NaN when that is zero).  The common
+    shapes run as one kernel (tensor._sum_abs_sqdev); anything else as the reference's own sequence of calls.
+    """
+    if dtype is None and u.dtype.kind not in "fc":
+        dtype = dpt.float64
+    um = None if mean is None else get_usm_ndarray(mean)
+    fused = None
+    if u.dtype.kind == "c":
+        if dtype is None:
+            m = um if um is not None else dpt.mean(u, axis=axis, keepdims=True)
+            fused = dpt._statistical_functions._sum_abs_sqdev(u, m, axis, keepdims)
+    elif um is not None and um.dtype.kind != "c":
+        # the type the reference's deviations and their sum would have
+        res_dt = dpt.dtype(dtype) if dtype is not None else np.result_type(u.dtype, um.dtype)
+        if res_dt.kind == "f":
+            fused = dpt._statistical_functions._sum_abs_sqdev(u, um, axis, keepdims, dtype=res_dt)
+    if fused is not None:
+        result = get_result_array(fused, out, casting="unsafe")
+    else:
+        arrmean = mean if mean is not None else _mean(a, axis=axis, dtype=dtype, keepdims=True)
+        x = subtract(a, arrmean)
+        if x.dtype.kind == "c":
+            x = multiply(x, x.conj(), out=x).real
+        else:
+            x = square(x, out=x)
+        result = sum(x, axis=axis, dtype=dtype, out=out, keepdims=keepdims)
+    axes = range(u.ndim) if axis is None else (axis if isinstance(axis, (tuple, list)) else (axis,))
+    items = 1
+    for ax in axes:
+        items *= u.shape[ax]
+    # (the reference writes numpy.max(items - ddof, 0): the 0 is an axis, nothing is clamped)
+    cnt = np.asarray(np.intp(items) - ddof).astype(result.dtype, casting="same_kind").item()
+    ur = get_usm_ndarray(result)
+    if ur.size:
+        tei._divide_by_scalar(src=ur, scalar=cnt if cnt else np.nan, dst=ur)
+    return result
+
+
+def var(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
+        correction=None):
+    check_supported_arrays_type(a)
+    check_limitations(where=where)
+    ddof = _check_ddof(ddof, correction)
     u = get_usm_ndarray(a)
-    res = dpt.var(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
-    result = get_result_array(res, out)
+    if u.dtype.kind == "c" or mean is not None:
+        result = _var_around_mean(a, u, axis, dtype, out, ddof, keepdims, mean)
+    else:
+        res = dpt.var(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
+        result = get_result_array(res, out)
     if out is None and dtype is not None:
         result = result.astype(dtype, casting="same_kind")
     return result
@@ -746,18 +799,17 @@ def var(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=
 
 def std(a, /, axis=None, dtype=None, out=None, ddof=0, keepdims=False, *, where=True, mean=None,
         correction=None):
+    check_supported_arrays_type(a)
     check_limitations(where=where)
-    if mean is not None:
-        raise NotImplementedError("std(..., mean=) is outside this library's scope")
-    if correction is not None:
-        if ddof != 0:
-            raise ValueError("ddof and correction can't be provided simultaneously.")
-        ddof = correction
-    if not isinstance(ddof, (int, float)):
-        raise TypeError(f"An integer or float is required, but got {type(ddof)}")
+    ddof = _check_ddof(ddof, correction)
     u = get_usm_ndarray(a)
-    res = dpt.std(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
-    result = get_result_array(res, out)
+    if u.dtype.kind == "c" or mean is not None:
+        # dpnp/dpnp_iface_statistics.py:1644-1656: the variance in its own type, then the root in place
+        result = var(a, axis=axis, dtype=None, out=out, ddof=ddof, keepdims=keepdims, where=where, mean=mean)
+        sqrt(result, out=result)
+    else:
+        res = dpt.std(u, axis=axis, correction=ddof, keepdims=keepdims, dtype=_wider_float(u, dtype))
+        result = get_result_array(res, out)
     if out is None and dtype is not None:
         result = result.astype(dtype, casting="same_kind")
     return result

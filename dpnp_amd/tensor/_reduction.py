@@ -38,7 +38,13 @@ def _move_reduced_axes_last(x, axis, int_only=False):
     key = tuple(perm)
     arr = cache.get(key)
     if arr is None:
-        arr = cache[key] = x._view([x._shape[a] for a in perm], [x._strides[a] for a in perm], x._offset)
+        arr = x._view([x._shape[a] for a in perm], [x._strides[a] for a in perm], x._offset)
+        if arr._base is x:
+            # an internal view, never handed out: it holds the allocation itself, not the array that keeps it
+            # (x -> cache -> view -> x would be a cycle, and the memory of a dropped array would wait for the
+            # cycle collector instead of being freed with the last reference)
+            arr._base = None
+        cache[key] = arr
     return arr, axis, perm
 
 

@@ -127,6 +127,50 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
     return res
 
 
+def _sum_abs_sqdev(x, mean, axis=None, keepdims=False, *, dtype=None):
+    """sum(|x - mean|**2) over `axis` in ONE kernel, or None when this call has no fused form.
+
+    The tail of dpnp.var when the caller brings the mean or the data is complex
+    (dpnp/dpnp_iface_statistics.py:1843-1860: subtract, square or multiply by the conjugate, real part,
+    sum: three or four kernels over full-size temporaries there).  Fused when `mean` broadcasts against
+    `x` with extent 1 along every reduced axis (the keepdims=True shape the reference documents, or fewer
+    dims), the result type is a real floating one with a kernel for this input type, and a complex mean
+    meets complex data; the mean is cast to the result's precision (a small array).
+    """
+    nd = x.ndim
+    axis, perm, nelems = _split_axes(x, axis)
+    red_nd = len(axis)
+    if red_nd == 0 or nelems == 0 or x.size == 0 or mean.ndim > nd:
+        return None
+    if x.dtype.kind == "c":
+        res_dt = _as_dtype("f4" if x.dtype == _as_dtype("c8") else "f8") if dtype is None else _as_dtype(dtype)
+    else:
+        if mean.dtype.kind == "c":
+            return None
+        res_dt = _as_dtype(dtype) if dtype is not None else None
+        if res_dt is None:
+            return None
+    if res_dt.kind != "f" or not tri._sumsqdev_over_axis_dtype_supported(x.dtype, res_dt):
+        return None
+    mshape = (1,) * (nd - mean.ndim) + tuple(mean.shape)
+    for d in range(nd):
+        if mshape[d] != 1 and (d in axis or mshape[d] != x.shape[d]):
+            return None
+    aux_dt = res_dt if x.dtype.kind != "c" else _as_dtype("c8" if res_dt == _as_dtype("f4") else "c16")
+    if mean.dtype != aux_dt:
+        mean = astype(mean, aux_dt)
+    mstrides = (0,) * (nd - mean.ndim) + tuple(mean.strides)
+    arr = permute_dims(x, perm)
+    res_shape = arr.shape[: nd - red_nd]
+    keep = [d for d in range(nd) if d not in axis]
+    aux = mean._view(list(res_shape), [0 if mshape[d] == 1 else mstrides[d] for d in keep], mean._offset)
+    res = empty(res_shape, dtype=res_dt)
+    tri._sumsqdev_over_axis(src=arr, mean=aux, trailing_dims_to_reduce=red_nd, dst=res)
+    if keepdims:
+        res = _keepdims_view(res, res_shape, red_nd, perm, nd)
+    return res
+
+
 def _check_var_args(x, correction, name):
     if not isinstance(x, usm_ndarray):
         raise TypeError(f"Expected dpnp_amd.tensor.usm_ndarray, got {type(x)}")

@@ -202,7 +202,8 @@ typedef enum dpx_reduce_op {
     DPX_R_PROD,
     DPX_R_MAX,
     DPX_R_MIN,
-    DPX_R_SUMSQDEV, /* sum((x - aux)^2): second pass of var, see dpx_reduce */
+    DPX_R_SUMSQDEV, /* sum(|x - aux|^2): second pass of var (also with a caller's mean, also of complex
+                     * input: dpnp/dpnp_iface_statistics.py:1832-1869), see dpx_reduce */
     DPX_R_LOGSUMEXP, /* log(sum(exp(x))), libtensor/source/reductions/logsumexp.cpp */
     DPX_R_HYPOT,     /* sqrt(sum(x^2)) by pairwise hypot, libtensor/source/reductions/reduce_hypot.cpp */
     /* NaN-ignoring forms, floating inputs only.  The reference composes them from a masked copy
@@ -415,7 +416,9 @@ int dpx_copy_to_host(void *dst_host, const void *src_device, size_t nbytes,
  * dpx_mem_alloc hands out device memory of the current device for use on `stream`;
  * dpx_mem_free takes the stream the block was LAST USED on and makes the block available
  * again in stream order: at once to later work on that stream, after a device-side wait to
- * work on another stream.  Neither call waits for the device.  Freed blocks stay cached in the
+ * work on another stream.  Neither call waits for the device, with one exception: when the driver is
+ * out of memory dpx_mem_alloc waits for the device (hipDeviceSynchronize), returns every cached block to
+ * the driver and tries once more.  Freed blocks stay cached in the
  * process until dpx_mem_release_cached() (which waits for the device).  A stream passed to
  * dpx_mem_free must stay valid while the block is cached: destroy library streams with
  * dpx_stream_destroy, and call dpx_stream_synchronize(stream) before destroying a foreign
@@ -468,7 +471,9 @@ int dpx_black_scholes(const void *price, const void *strike, const void *t,
  * _max_over_axis, _min_over_axis).  The last `trailing_dims_to_reduce` axes of
  * src are reduced; dst has the leading src.nd - trailing axes.
  * op == DPX_R_SUMSQDEV (and DPX_R_NANSUMSQDEV) additionally takes `aux` (same shape and dtype as dst,
- * any strides): dst[i] = sum_j (src[i,j] - aux[i])^2; aux is NULL otherwise. */
+ * any strides): dst[i] = sum_j (src[i,j] - aux[i])^2; aux is NULL otherwise.  DPX_R_SUMSQDEV of complex
+ * src gives the real dst[i] = sum_j |src[i,j] - aux[i]|^2 (float32 or float64 from complex64, float64 from
+ * complex128), with aux complex of dst's precision (complex64 for a float32 dst, else complex128). */
 int dpx_reduce(int op, const dpx_array_view *src, int trailing_dims_to_reduce,
                const dpx_array_view *dst, const dpx_array_view *aux,
                void *stream);

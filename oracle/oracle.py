@@ -604,6 +604,40 @@ def var(a, trailing, correction=0.0, out_dtype=None):
         return (((x - mu) ** 2).sum(axis=-1) / div).astype(dt)
 
 
+def var_around_mean(a, trailing, mean=None, ddof=0, out_dtype=None):
+    """dpnp/dpnp_iface_statistics.py:1832-1869, the branch dpnp.var takes for complex input or a
+    caller's `mean`: x = a - mean (mean of the run when none is given), |x|^2 (x * conj(x), real part,
+    for complex x; x^2 otherwise), summed over the last `trailing` axes, divided by N - ddof.
+    `mean` has the leading shape of `a` (one value per run), or broadcasts to it.
+    The divisor is N - ddof as it comes (line 1864 writes numpy.max(cnt - ddof, 0): the 0 is an axis
+    argument, not a lower bound) and NaN when it is zero.  Result dtype: `out_dtype`, else the real type
+    of what `a - mean` promotes to (float64 for integer and bool input).  Evaluated in long double, rounded once."""
+    a = np.asarray(a)
+    a2, lead, n = _split(a, trailing)
+    wide = np.clongdouble if (a2.dtype.kind == "c" or (mean is not None and np.asarray(mean).dtype.kind == "c")) \
+        else np.longdouble
+    x = a2.astype(wide)
+    if mean is None:
+        mdt = a2.dtype
+        with np.errstate(all="ignore"):
+            mu = x.mean(axis=-1, keepdims=True) if n else np.full(lead + (1,), np.nan, dtype=wide)
+    else:
+        m = np.asarray(mean)
+        mdt = m.dtype
+        mu = np.broadcast_to(m, lead).astype(wide)[..., None]
+    if out_dtype is not None:
+        dt = np.dtype(out_dtype)
+    else:
+        base = a2.dtype if a2.dtype.kind in "fc" else np.dtype("f8")
+        dt = np.result_type(base, mdt)
+        dt = np.dtype({"c8": "f4", "c16": "f8"}.get(dt.str[1:], dt.str[1:]))
+    div = n - ddof
+    with np.errstate(all="ignore"):
+        d = x - mu
+        sq = (d.real * d.real + d.imag * d.imag) if wide is np.clongdouble else d * d
+        return (sq.sum(axis=-1) / (np.longdouble(div) if div else np.nan)).astype(dt)
+
+
 # ---------------------------------------------------------------------------------------------
 # NaN-ignoring reductions: dpnp/dpnp_iface_nanfunctions.py
 # ---------------------------------------------------------------------------------------------

@@ -227,3 +227,30 @@ def test_errors_raised_by_the_python_layer_before_any_kernel():
         dpt.var(host_array((3,), "c8"))
     with pytest.raises(IndexError):
         dpt.sum(x, axis=2)
+
+
+def test_reduction_over_leading_axis_leaves_no_reference_cycle():
+    # the permuted view a reduction keeps with its input must not keep the input alive: dropping the last
+    # reference frees the allocation at once, with the cycle collector switched off
+    import gc
+    import weakref
+
+    from dpnp_amd.tensor._reduction import _move_reduced_axes_last
+
+    was = gc.isenabled()
+    gc.disable()
+    try:
+        for axis in (0, 1, (0, 2), None):
+            x = host_array((4, 5, 6))
+            alive = weakref.ref(x._buf.a.base if x._buf.a.base is not None else x._buf)
+            buf_alive = weakref.ref(x._buf)
+            arr, _, _ = _move_reduced_axes_last(x, axis)
+            again, _, _ = _move_reduced_axes_last(x, axis)
+            assert again is arr  # kept with the array
+            v = x[1:]  # a view of x: its own permuted view refers to x, not to v
+            _move_reduced_axes_last(v, 0)
+            del arr, again, v, x
+            assert buf_alive() is None and alive() is None, axis
+    finally:
+        if was:
+            gc.enable()

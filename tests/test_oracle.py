@@ -17,6 +17,9 @@ Oracle function -> what pins it here (none of the pins calls NumPy for the rule 
   maximum / minimum                       test_maximum_minimum_nan_rule
   promote_binary                          test_promotion_matches_numpy_result_type,
                                           test_promotion_with_acceptance_hooks
+  var_around_mean                         test_var_around_mean_identities_and_docstring_values (exact
+                                          rational arithmetic, var(z) = var(Re z) + var(Im z), the shift
+                                          identity, dpnp_iface_statistics.py:1815-1826,1625-1634)
   cast, where, reductions, collapse       the tests of those names below
 """
 from fractions import Fraction
@@ -623,3 +626,45 @@ def test_clip_matches_numpy_and_the_reference_special_cases():
     z = np.array([1 + 1j, 1 + 5j, 3 + 0j, 0 + 9j], "c8")
     got = orc.clip(z, np.complex64(1 + 2j), np.complex64(2 + 0j))
     np.testing.assert_array_equal(got, np.array([1 + 2j, 1 + 5j, 2 + 0j, 1 + 2j], "c8"))
+
+
+def test_var_around_mean_identities_and_docstring_values():
+    # the reference's documented values (dpnp_iface_statistics.py:1821-1826 and 1629-1634)
+    a = np.array([[14, 8, 11, 10], [7, 9, 10, 11], [10, 15, 5, 10]])
+    m = a.mean(axis=1)
+    v = orc.var_around_mean(a, 1, mean=m)
+    assert v.dtype == np.dtype("f8")
+    assert np.array_equal(v, [4.6875, 2.1875, 12.5])
+    np.testing.assert_allclose(np.sqrt(v), [2.16506351, 1.47901995, 3.53553391], rtol=1e-8)
+    # exact rational arithmetic on small integer data, real and complex, with and without a given mean
+    rng = np.random.default_rng(5)
+    re, im = rng.integers(-9, 10, (4, 7)), rng.integers(-9, 10, (4, 7))
+    z = (re + 1j * im).astype("c16")
+    for ddof in (0, 1, 2.5, 7, 9):
+        for r in range(4):
+            mr, mi = Fraction(int(re[r].sum()), 7), Fraction(int(im[r].sum()), 7)
+            tot = sum((Fraction(int(p)) - mr) ** 2 + (Fraction(int(q)) - mi) ** 2 for p, q in zip(re[r], im[r]))
+            got = orc.var_around_mean(z, 1, ddof=ddof)[r]
+            div = Fraction(7) - Fraction(ddof)
+            if div == 0:
+                assert np.isnan(got)
+            else:  # (a negative divisor is kept: the reference does not clamp it)
+                assert got == pytest.approx(float(tot / div), rel=1e-14)
+    given = np.array([1.5 - 2j, 0, 3j, -1])
+    for r in range(4):
+        tot = sum((Fraction(int(p)) - Fraction(given[r].real)) ** 2 + (Fraction(int(q)) - Fraction(given[r].imag)) ** 2
+                  for p, q in zip(re[r], im[r]))
+        assert orc.var_around_mean(z, 1, mean=given, ddof=1)[r] == pytest.approx(float(tot / 6), rel=1e-14)
+    # var(z) = var(Re z) + var(Im z); var(x, mean=m) = var(x) + (mean(x) - m)^2
+    x = rng.normal(3, 2, (5, 64))
+    w = (x + 1j * rng.normal(-1, 0.5, (5, 64))).astype("c16")
+    np.testing.assert_allclose(orc.var_around_mean(w, 1), orc.var(w.real.copy(), 1) + orc.var(w.imag.copy(), 1),
+                               rtol=1e-13)
+    shift = rng.normal(0, 1, 5)
+    np.testing.assert_allclose(orc.var_around_mean(x, 1, mean=x.mean(axis=1) + shift),
+                               orc.var(x, 1) + shift ** 2, rtol=1e-13)
+    # dtypes: complex64 -> float32, integers -> float64, float32 data with a float32 mean stays float32
+    assert orc.var_around_mean(w.astype("c8"), 1).dtype == np.dtype("f4")
+    assert orc.var_around_mean(re.astype("i2"), 1, mean=np.zeros(4, "f4")).dtype == np.dtype("f8")
+    assert orc.var_around_mean(x.astype("f4"), 1, mean=np.zeros(5, "f4")).dtype == np.dtype("f4")
+    assert np.isnan(orc.var_around_mean(np.zeros((2, 0)), 1)).all()

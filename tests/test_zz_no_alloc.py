@@ -50,6 +50,12 @@ CASES = [
     ("full sum int8 -> int64", "sum", "i1", "i8", (1 << 24,), (1 << 21,), 1, False),
     ("full count_nonzero u8", "count_nonzero", "u1", "i8", (1 << 24,), (1 << 19,), 1, False),
     ("full nanmean f32", "nanmean", "f4", "f4", (1 << 23,), (1 << 19,), 1, False),
+    # partials wider than the result: (largest element, sum of exponentials) pairs, (count, mean, M2) triples
+    ("full logsumexp f32", "logsumexp", "f4", "f4", (1 << 23,), (1 << 19,), 1, False),
+    ("rows logsumexp f64", "logsumexp", "f8", "f8", (3, 1 << 21), (2, 1 << 18), 1, False),
+    ("cols logsumexp f32", "logsumexp", "f4", "f4", (1 << 14, 1 << 10), (1 << 12, 200), 1, True),
+    ("full one-pass squared deviations f32 -> f64", "sqdev_onepass", "f4", "f8", (1 << 24,), (1 << 20,), 1, False),
+    ("cols one-pass squared deviations f64", "sqdev_onepass", "f8", "f8", (1 << 14, 1 << 10), (1 << 12, 200), 1, True),
 ]
 
 
@@ -83,6 +89,12 @@ def test_noalloc_matches_dpx_reduce_twice_in_a_row(case):
             assert np.array_equal(got, ah.max(axis=-1))
         elif op == "count_nonzero":
             assert np.array_equal(got, np.count_nonzero(ah, axis=-1))
+        elif op == "logsumexp":
+            h = ah.astype("f8")
+            ref = np.log(np.exp(h - h.max(axis=-1, keepdims=True)).sum(axis=-1)) + h.max(axis=-1)
+            np.testing.assert_allclose(got, ref, rtol=1e-5)
+        elif op == "sqdev_onepass":
+            np.testing.assert_allclose(got, ah.astype("f8").var(axis=-1) * ah.shape[-1], rtol=1e-10)
     assert split_seen, "no case exercised the scratch buffer"
 
 
@@ -95,6 +107,23 @@ def test_noalloc_with_aux_and_one_block_plans():
     got = host(_reduce(L.lib.dpx_reduce_noalloc, "sumsqdev", x, 1, "f4", aux=mean))
     assert np.array_equal(_bits(got), _bits(want))
     np.testing.assert_allclose(got, ((a.astype("f8") - a.mean(axis=1, dtype="f8")[:, None]) ** 2).sum(axis=1), rtol=1e-5)
+    # the NaN-ignoring variance around a given mean: (sum, count) pairs in scratch
+    a[rng.random(a.shape) < 0.01] = np.nan
+    x = dev(a)
+    mean = dev(np.nanmean(a.astype("f8"), axis=1).astype("f4"))
+    assert _plan("nanvar", x, 1, "f4").splits > 1
+    want = host(_reduce(L.lib.dpx_reduce, "nanvar", x, 1, "f4", aux=mean))
+    got = host(_reduce(L.lib.dpx_reduce_noalloc, "nanvar", x, 1, "f4", aux=mean))
+    assert np.array_equal(_bits(got), _bits(want))
+    np.testing.assert_allclose(got, np.nanvar(a.astype("f8"), axis=1), rtol=1e-5)
+    # complex input around a complex mean, a real result
+    z = (rng.standard_normal((3, 1 << 20)) + 1j * rng.standard_normal((3, 1 << 20))).astype("c8")
+    x, mean = dev(z), dev(z.mean(axis=1, dtype="c16").astype("c8"))
+    assert _plan("sumsqdev", x, 1, "f4").splits > 1
+    want = host(_reduce(L.lib.dpx_reduce, "sumsqdev", x, 1, "f4", aux=mean))
+    got = host(_reduce(L.lib.dpx_reduce_noalloc, "sumsqdev", x, 1, "f4", aux=mean))
+    assert np.array_equal(_bits(got), _bits(want))
+    np.testing.assert_allclose(got, z.astype("c16").var(axis=1) * z.shape[1], rtol=1e-5)
     # plans without scratch (one block per output) go the same way through both entry points
     b = dev(rng.standard_normal((4096, 512)).astype("f4"))
     assert _plan("sum", b, 1, "f4").splits == 1
