@@ -65,6 +65,7 @@ def cpu_baseline(n_log2=28, repeats=5):
 
 
 PRIME_STEPS = 24
+CONFIG_STEPS = 12  # timed steps of each of cfg1..cfg5 inside the default run
 MALL_BYTES = 256 << 20  # last-level (memory-side) cache of the MI355X
 
 WORKLOADS = {
@@ -81,16 +82,24 @@ WORKLOADS = {
 
 
 def _device_array(dpnp, torch, t):
-    """A dpnp array holding the bytes of torch tensor t (handed over by a byte copy, before timing)."""
+    """A dpnp array (memory of the library's own pool) holding the values of torch tensor t.  torch only
+    generates the synthetic data: its tensor is viewed as an array of this package without a copy (any
+    object with data_ptr() and numel() serves as a buffer) and copied by the library's copy kernel on the
+    library's stream, before anything is timed."""
+    from dpnp_amd.tensor._usmarray import usm_ndarray
+
     names = {torch.float32: "f4", torch.float64: "f8", torch.int32: "i4", torch.bool: "?"}
+    t = t.contiguous()
     arr = dpnp.empty(tuple(t.shape), dtype=names[t.dtype])
-    nbytes = t.numel() * t.element_size()
-    arr.get_array()._buf[:nbytes].copy_(t.contiguous().view(-1).view(torch.uint8))
+    torch.cuda.synchronize()  # t is complete (torch's stream) before the library's stream reads it
+    src = usm_ndarray(tuple(t.shape), dtype=names[t.dtype], buffer=t.view(-1).view(torch.uint8))
+    dpnp.copyto(arr, dpnp.ndarray._create_from_usm_ndarray(src))
+    dpnp.synchronize()  # ... and the copy is complete before torch frees or reuses t
     return arr
 
 
 def build_workload(name, dpnp, torch):
-    """-> (ops, dtype, data): ops = [(label, callable, algorithmic bytes, elements)].
+    """-> (ops, dtype, data): ops = [(label, callable, algorithmic bytes, elements[, physical bytes])].
     Algorithmic bytes = every input element read once + every output element written once."""
     g = torch.Generator(device="cuda").manual_seed(0)
 
@@ -138,13 +147,14 @@ def build_workload(name, dpnp, torch):
     if name == "cfg3":
         n = 1 << 28
         t = torch.randn(n, device="cuda", generator=g)
-        pick = torch.randint(0, n, (n // 100,), device="cuda", generator=g)
-        t[pick] = t.max()
-        pick = torch.randint(0, n, (n // 100,), device="cuda", generator=g)
-        t[pick] = t.min()
+        # distinct places (a choice without replacement): 1 % maxima, 1 % minima, then 0.1 % NaN
+        perm = torch.randperm(n, device="cuda", generator=g)
+        t[perm[: n // 100]] = t.max()
+        t[perm[n // 100: 2 * (n // 100)]] = t.min()
         clean = _device_array(dpnp, torch, t)
         clean64 = _device_array(dpnp, torch, t.double())
-        pick = torch.randint(0, n, (n // 1000,), device="cuda", generator=g)
+        pick = perm[2 * (n // 100): 2 * (n // 100) + n // 1000]
+        del perm
         t[pick] = float("nan")
         x = _device_array(dpnp, torch, t)
         del t, pick
@@ -181,15 +191,19 @@ def build_workload(name, dpnp, torch):
             dpnp.greater(V1, 0, out=o_b)
             dpnp.where(o_b, V1, B, out=o_half)
 
-        ops = [("multiply_V1_B", lambda: dpnp.multiply(V1, B, out=o_half), 8 * h + 4 * (side // 2), h),
-               ("exp_V1", lambda: dpnp.exp(V1, out=o_half), 8 * h, h),
+        # fifth field: the bytes moved physically.  A [:, ::2] view occupies every 128-byte line of its base
+        # matrix, so reading it reads the whole matrix (8 bytes per element of the view instead of 4)
+        row = 4 * (side // 2)
+        ops = [("multiply_V1_B", lambda: dpnp.multiply(V1, B, out=o_half), 8 * h + row, h, 12 * h + row),
+               ("exp_V1", lambda: dpnp.exp(V1, out=o_half), 8 * h, h, 12 * h),
                ("exp_AT_keep_layout", lambda: dpnp.exp(V2, out=o_f), 8 * 2 * h, 2 * h),
                ("exp_AT_to_C", lambda: dpnp.exp(V2, out=o_c), 8 * 2 * h, 2 * h),
                ("where_greater_fused", lambda: dpnp.where_compare("greater", V1, 0, V1, B, out=o_half),
-                8 * h + 4 * (side // 2), h),
-               ("where_greater_two_calls", where_unfused, (4 + 1) * h + (1 + 4 + 4) * h + 4 * (side // 2), h),
+                8 * h + row, h, 12 * h + row),
+               ("where_greater_two_calls", where_unfused, (4 + 1) * h + (1 + 4 + 4) * h + row, h,
+                (8 + 1) * h + (1 + 8 + 4) * h + row),
                ("bitwise_and", lambda: dpnp.bitwise_and(ints[0], ints[1], out=o_i), 12 * 2 * h, 2 * h),
-               ("bitwise_and_V1", lambda: dpnp.bitwise_and(ints[0][:, ::2], ints[1][:, ::2], out=o_ih), 12 * h, h),
+               ("bitwise_and_V1", lambda: dpnp.bitwise_and(ints[0][:, ::2], ints[1][:, ::2], out=o_ih), 12 * h, h, 20 * h),
                # plain copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters (--ops ...,copy)
                ("copy", lambda: dpnp.copyto(o_i, ints[0]), 8 * 2 * h, 2 * h)]
         return ops, "f32/i32/bool", "synthetic (seeded normal(0,1), uniform int32, resident in HBM)"
@@ -245,49 +259,79 @@ def build_workload(name, dpnp, torch):
     raise SystemExit(f"--workload: unknown workload {name!r} (one of {', '.join(WORKLOADS)})")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--dump-steps", action="store_true", help="print every step's per-op times to stderr")
-    ap.add_argument("--workload", default="metric",
-                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5 or layouts, "
-                         "measured the same way")
-    ap.add_argument("--ops", default=None,
-                    help="comma-separated subset of the workload's ops (profiling runs); 'copy' in the metric "
-                         "workload is a plain copy of known size")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
-        sys.exit(2)
+def dpnp_cpu_probe():
+    """Looks for an installed dpnp (the reference itself, with its SYCL CPU device) on this box, in a child
+    process; when there is one, times the metric's calls on its CPU device there.  The expected answer is
+    "unavailable on this box": the record then says that the reference path was looked for."""
+    import subprocess
 
-    import torch
+    code = r"""
+import importlib.util, json, sys, time
+if importlib.util.find_spec("dpnp") is None or importlib.util.find_spec("dpctl") is None:
+    print(json.dumps("unavailable on this box")); sys.exit(0)
+try:
+    import dpctl, dpnp
+    dev = dpctl.SyclDevice("cpu")
+    n = 1 << 24
+    a = dpnp.random.uniform(-1, 1, n, device=dev).astype(dpnp.float32)
+    b = dpnp.random.uniform(-1, 1, n, device=dev).astype(dpnp.float32)
+    q = a.sycl_queue
+    def timed(f):
+        for _ in range(5): f(); q.wait()
+        ts = []
+        for _ in range(20):
+            t0 = time.perf_counter(); f(); q.wait(); ts.append(time.perf_counter() - t0)
+        return sorted(ts)[10]
+    out = {"cores": dev.max_compute_units, "elements": n,
+           "add_GB/s": 12 * n / timed(lambda: dpnp.add(a, b)) / 1e9,
+           "sum_GB/s": 4 * n / timed(lambda: dpnp.sum(a)) / 1e9,
+           "argmax_GB/s": 4 * n / timed(lambda: dpnp.argmax(a)) / 1e9}
+    print(json.dumps(out))
+except Exception as e:
+    print(json.dumps("present but not usable: %s: %s" % (type(e).__name__, e)))
+"""
+    try:
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+        return json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:  # the probe must never take the bench down
+        return f"probe failed: {type(e).__name__}: {e}"
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(1)
-    import dpnp_amd as dpnp
+
+def _pool_bytes_in_use():
+    import ctypes
+
+    from dpnp_amd import _lib
+
+    used, cached = ctypes.c_size_t(), ctypes.c_size_t()
+    _lib.check(_lib.lib.dpx_mem_stats(ctypes.byref(used), ctypes.byref(cached)))
+    return used.value
+
+
+def measure(name, dpnp, torch, steps, warmup, prime, ops_filter=None, dump=False):
+    """Runs workload `name`: `prime` + `warmup` untimed steps, then exactly `steps` timed ones.  Every op is
+    bracketed by HIP events recorded on the library's own stream (the one its kernels are launched on)."""
+    from dpnp_amd.tensor import _device
+
+    stream = torch.cuda.ExternalStream(_device.current_stream_ptr())
 
     def select(all_ops):
-        if args.ops is None:
+        if ops_filter is None:
             return [o for o in all_ops if o[0] != "copy"]
-        wanted = [w for w in args.ops.split(",") if w]
+        wanted = [w for w in ops_filter.split(",") if w]
         sel = [o for o in all_ops if o[0] in wanted]
         if not sel or len(sel) != len(wanted):
-            print(f"--ops: unknown op in {wanted}; {args.workload} has {[o[0] for o in all_ops]}", file=sys.stderr)
+            print(f"--ops: unknown op in {wanted}; {name} has {[o[0] for o in all_ops]}", file=sys.stderr)
             sys.exit(2)
         return sel
 
-    mem0 = torch.cuda.memory_allocated()
-    all_ops, dtype, data = build_workload(args.workload, dpnp, torch)
-    working_set = torch.cuda.memory_allocated() - mem0
+    mem0 = _pool_bytes_in_use()
+    all_ops, dtype, data = build_workload(name, dpnp, torch)
+    working_set = _pool_bytes_in_use() - mem0
     # A workload whose arrays fit the 256 MiB memory-side cache would be served from it when every
     # step reuses the same buffers: such a workload gets several buffer sets, enough that a set has
     # left the cache (3 x its size has streamed through) when its turn comes again.
     nsets = 1 if working_set >= MALL_BYTES else min(8, -(-3 * MALL_BYTES // max(working_set, 1)) + 1)
-    op_sets = [select(all_ops)] + [select(build_workload(args.workload, dpnp, torch)[0]) for _ in range(nsets - 1)]
+    op_sets = [select(all_ops)] + [select(build_workload(name, dpnp, torch)[0]) for _ in range(nsets - 1)]
     ops = op_sets[0]
     step_bytes = sum(o[2] for o in ops)
 
@@ -297,60 +341,113 @@ def main():
     def step(events=None):
         cur = op_sets[step_no[0] % nsets]
         step_no[0] += 1
-        for k, (_, fn, _, _) in enumerate(cur):
+        for k, o in enumerate(cur):
             if events is not None:
-                events[k][0].record()
+                events[k][0].record(stream)
             h0 = time.perf_counter()
-            fn()
+            o[1]()
             host_us.append((time.perf_counter() - h0) * 1e6)
             if events is not None:
-                events[k][1].record()
+                events[k][1].record(stream)
+
+    def sync():
+        dpnp.synchronize()
+        torch.cuda.synchronize()
 
     # Process start-up, not steady state: the first launch of each kernel loads its code object,
     # and the HIP runtime stalls the submitting thread once, for 30-40 ms, a few dozen launches
     # into a process (seen on the host clock around a launch, with the GPU idle).  Both are kept
     # out of the W + K steps whatever W is.
-    for _ in range(PRIME_STEPS):
+    for _ in range(prime):
         step()
-    torch.cuda.synchronize()
-    for _ in range(args.warmup):
+    sync()
+    for _ in range(warmup):
         step()
-    torch.cuda.synchronize()
+    sync()
     ev = [[[torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)] for _ in ops]
-          for _ in range(args.steps)]
+          for _ in range(steps)]
     t_begin, t_end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
+    sync()
     del host_us[:]
     wall0 = time.perf_counter()
-    t_begin.record()
-    for s in range(args.steps):
+    t_begin.record(stream)
+    for s in range(steps):
         step(ev[s])
-    t_end.record()
-    torch.cuda.synchronize()
+    t_end.record(stream)
+    sync()
     wall = time.perf_counter() - wall0
     gpu_ms = t_begin.elapsed_time(t_end)
-    ms_per_step = max(gpu_ms, wall * 1e3) / args.steps
+    ms_per_step = max(gpu_ms, wall * 1e3) / steps
     per_op = {}
-    for k, (name, _, nb, nel) in enumerate(ops):
-        times = sorted(ev[s][k][0].elapsed_time(ev[s][k][1]) for s in range(args.steps))
-        ms = sum(times) / args.steps
-        med = times[args.steps // 2] if args.steps % 2 else 0.5 * (times[args.steps // 2 - 1] + times[args.steps // 2])
-        host = sorted(host_us[s * len(ops) + k] for s in range(args.steps))
+    for k, o in enumerate(ops):
+        label, nb, nel = o[0], o[2], o[3]
+        times = sorted(ev[s][k][0].elapsed_time(ev[s][k][1]) for s in range(steps))
+        ms = sum(times) / steps
+        med = times[steps // 2] if steps % 2 else 0.5 * (times[steps // 2 - 1] + times[steps // 2])
+        host = sorted(host_us[s * len(ops) + k] for s in range(steps))
         # host_us_median: time the submitting thread spends inside the call (Python layer, C ABI,
         # launch), which bounds the rate of calls whose kernels are shorter than that
-        per_op[name] = {"ms": round(ms, 5), "ms_median": round(med, 5), "host_us_median": round(host[args.steps // 2], 1),
-                        "GB/s": round(nb / ms / 1e6, 1),
-                        "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4),
-                        "frac_of_peak_median": round(nb / med / 1e6 / HBM_PEAK_GBS, 4),
-                        "elements/s": round(nel / ms * 1e3)}
-    if args.dump_steps:
-        for s in range(args.steps):
+        per_op[label] = {"ms": round(ms, 5), "ms_median": round(med, 5), "host_us_median": round(host[steps // 2], 1),
+                         "GB/s": round(nb / ms / 1e6, 1),
+                         "frac_of_peak": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4),
+                         "frac_of_peak_median": round(nb / med / 1e6 / HBM_PEAK_GBS, 4),
+                         "elements/s": round(nel / ms * 1e3)}
+        if len(o) > 4:  # bytes the call moves physically (whole lines of a strided view)
+            per_op[label]["frac_physical"] = round(o[4] / ms / 1e6 / HBM_PEAK_GBS, 4)
+    if dump:
+        for s in range(steps):
             print(s, " ".join("%s=%.4f(host %.0fus)" % (ops[k][0], ev[s][k][0].elapsed_time(ev[s][k][1]),
                                                          host_us[s * len(ops) + k]) for k in range(len(ops))),
                   file=sys.stderr)
+    del op_sets, all_ops
+    return {"ops": [(o[0], o[2]) for o in ops], "dtype": dtype, "data": data, "nsets": nsets,
+            "step_bytes": step_bytes, "ms_per_step": ms_per_step, "per_op": per_op}
+
+
+def release_memory(torch):
+    import gc
+
+    from dpnp_amd import _lib
+
+    gc.collect()
+    _lib.check(_lib.lib.dpx_mem_release_cached())
+    torch.cuda.empty_cache()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="metric workload only: leave out the short runs of cfg1..cfg5 that fill `configs`")
+    ap.add_argument("--dump-steps", action="store_true", help="print every step's per-op times to stderr")
+    ap.add_argument("--workload", default="metric",
+                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5, layouts "
+                         "or floors, measured the same way")
+    ap.add_argument("--ops", default=None,
+                    help="comma-separated subset of the workload's ops (profiling runs); 'copy' in the metric "
+                         "workload is a plain copy of known size")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    # torch generates the synthetic data and provides the timing events; it is imported before the package so
+    # that both use one HIP runtime.  The package itself runs on its own memory pool and stream.
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    import dpnp_amd as dpnp
+    from dpnp_amd import _lib
+
+    m = measure(args.workload, dpnp, torch, args.steps, args.warmup, PRIME_STEPS, args.ops, args.dump_steps)
+    per_op, ms_per_step, step_bytes = m["per_op"], m["ms_per_step"], m["step_bytes"]
     # the roofline object describes the op with the largest share of the step
-    dom = max(range(len(ops)), key=lambda k: per_op[ops[k][0]]["ms"])
-    dom_name, _, dom_bytes, _ = ops[dom]
+    dom_name, dom_bytes = max(m["ops"], key=lambda o: per_op[o[0]]["ms"])
     dom_ms = per_op[dom_name]["ms"]
     kernel = ("ew_contig_kernel<add,f32> (c = a + b, 2^28 elements)" if (args.workload, dom_name) == ("metric", "add")
               else f"{args.workload}:{dom_name}")
@@ -363,14 +460,15 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "primed": PRIME_STEPS,  # untimed steps before the warm-up (process start-up, see below)
-        "buffer_sets": nsets,   # distinct sets of arrays the steps cycle through
+        "primed": PRIME_STEPS,  # untimed steps before the warm-up (process start-up, see above)
+        "buffer_sets": m["nsets"],   # distinct sets of arrays the steps cycle through
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": dtype,
-        "data": data,
+        "dtype": m["dtype"],
+        "data": m["data"],
+        "memory_and_stream": _lib.MEMORY,  # "native": dpx_mem_alloc / dpx_stream_create
         "config": {"workload": workload, "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(step_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4)},
         "per_op": per_op,
@@ -383,8 +481,25 @@ def main():
         # HBM bytes per launch from the committed rocprofv3 --pmc summary
         out["roofline"]["traffic"] = json.load(open(traffic_file)).get("bytes_per_launch")
         out["roofline"]["traffic_source"] = "profiles/add_f32_2p28_traffic.json (rocprofv3 --pmc, not measured in this run)"
+    if args.workload == "metric" and args.ops is None and not args.no_configs:
+        # the other configurations, a few steps each (parity cases, not the headline: their own lines come
+        # from --workload cfgN): per op, time and share of the HBM peak on algorithmic bytes, and on the
+        # bytes physically moved where a strided view makes the two differ
+        configs = {}
+        for cfg in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+            release_memory(torch)
+            c = measure(cfg, dpnp, torch, CONFIG_STEPS, 3, 4)
+            configs[cfg] = {
+                "workload": WORKLOADS[cfg], "steps": CONFIG_STEPS, "buffer_sets": c["nsets"],
+                "ms_per_step": round(c["ms_per_step"], 5),
+                "sum_of_op_ms": round(sum(v["ms"] for v in c["per_op"].values()), 5),  # event times of the ops, launch gaps excluded
+                "per_op": {k: {f: v[f] for f in ("ms", "host_us_median", "frac_of_peak", "frac_physical") if f in v}
+                           for k, v in c["per_op"].items()}}
+        out["configs"] = configs
+        release_memory(torch)
     if not args.no_cpu_baseline and args.workload == "metric":
         out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"]["dpnp_cpu"] = dpnp_cpu_probe()
     print(json.dumps(out))
 
 

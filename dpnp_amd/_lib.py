@@ -6,24 +6,21 @@ module raises; there is no CPU or PyTorch fallback.
 import ctypes
 import os
 
-# Where device memory and the stream come from: DPNP_AMD_MEMORY=torch (PyTorch's caching
-# allocator and current stream), =native (the library's own pool and stream, dpx_mem_* and
-# dpx_stream_*), or unset: torch when it can be imported, else native.
+# Where device memory and the stream come from: the library's own pool and stream (dpx_mem_* and
+# dpx_stream_*, "native") unless DPNP_AMD_MEMORY=torch asks for PyTorch's caching allocator and current
+# stream (for processes that mix this package's calls with torch work on the same data).
 # PyTorch ships its own HIP runtime (libamdhip64.so.7).  It must be in the process before
 # libdpnp_amd.so is loaded so that both bind to the SAME runtime instance: device memory
 # allocated by torch is then valid in this library's launches, and the stream handles match.
 # Loading in the other order leaves two runtimes in the process and the second one finds no device.
-MEMORY = os.environ.get("DPNP_AMD_MEMORY", "").lower()
-if MEMORY not in ("", "torch", "native"):
+# A process that uses torch for something else beside this package (on the native provider) imports
+# torch first for the same reason.
+MEMORY = os.environ.get("DPNP_AMD_MEMORY", "").lower() or "native"
+if MEMORY not in ("torch", "native"):
     raise ImportError("DPNP_AMD_MEMORY must be 'torch' or 'native', not %r" % MEMORY)
 torch = None
-if MEMORY != "native":
-    try:
-        import torch  # noqa: F401,E402
-    except ImportError:
-        if MEMORY == "torch":
-            raise
-    MEMORY = "torch" if torch is not None else "native"
+if MEMORY == "torch":
+    import torch  # noqa: F401,E402
 
 MAX_ND = 12
 NOALLOC_SCRATCH_BYTES = 2 << 20  # DPX_NOALLOC_SCRATCH_BYTES

@@ -2,12 +2,12 @@
 
 Two providers, chosen once per process (``dpnp_amd._lib.MEMORY``):
 
-* ``torch``: PyTorch as plumbing.  Its caching allocator hands out device memory (a uint8
-  CUDA tensor per allocation) and its current stream is the hipStream_t every kernel of
-  the library is enqueued on, so this library's work interleaves correctly with torch work
-  of the same process.
-* ``native``: the library's own pool and stream (``dpx_mem_alloc`` / ``dpx_mem_free`` /
-  ``dpx_stream_create``), used when torch cannot be imported or DPNP_AMD_MEMORY=native.
+* ``native`` (the default): the library's own pool and stream (``dpx_mem_alloc`` /
+  ``dpx_mem_free`` / ``dpx_stream_create``).
+* ``torch`` (DPNP_AMD_MEMORY=torch): PyTorch as plumbing.  Its caching allocator hands out
+  device memory (a uint8 CUDA tensor per allocation) and its current stream is the hipStream_t
+  every kernel of the library is enqueued on, so this library's work interleaves correctly
+  with torch work of the same process.
 
 Both allocators are stream-ordered: a temporary released right after a launch is not
 reused before that launch has run.

@@ -134,3 +134,41 @@ def test_mean_var_of_integer_arrays_in_one_pass(dt):
     assert L.lib.dpx_reduce_dtype_supported(L.REDUCE_ID["sum"], dtype_id(np.dtype(dt)), dtype_id(np.dtype("f8"))) == 1
     s = dpt.sum(d, dtype="f4")
     np.testing.assert_allclose(float(s), float(np.sum(a.astype("f8"))), rtol=1e-5, atol=1e-2)
+
+
+@pytest.mark.parametrize("dt", ["f4", "f8"])
+def test_one_pass_variance_propagates_inf_and_nan_in_every_kernel_form(dt):
+    """inf or NaN anywhere in a run gives NaN (inf - mean is inf, inf * 0 in the merge is NaN), a run without
+    them its variance: short rows (one lane per row), long rows, columns, reduced dims that stay apart, a
+    sliced matrix.  The one-pass kernels keep (count, mean, M2) triples; a clamp of a NaN M2 to zero, or a merge
+    with an untouched accumulator skipped, would give a finite result here."""
+    rng = np.random.default_rng(83)
+    cases = [((600, 5), 1), ((600, 8), 1), ((40, 3000), 1), ((3, 200000), 1), ((3000, 70), 0), ((40000, 6), 0),
+             ((6, 300, 40), (0, 2)), ((50, 40, 30), (0, 2))]
+    for shape, axis in cases:
+        a = rng.standard_normal(shape).astype(dt) + 5
+        out_shape = np.var(a, axis=axis).shape
+        for bad in (np.inf, -np.inf, np.nan):
+            h = a.copy()
+            hit = np.zeros(out_shape, bool)
+            for o in rng.choice(hit.size, size=min(3, hit.size), replace=False):
+                oi = np.unravel_index(o, out_shape)
+                hit[oi] = True
+                # one element of that output's run, first, last or inside
+                full = [slice(None)] * len(shape)
+                keep = [d for d in range(len(shape)) if d not in (axis if isinstance(axis, tuple) else (axis,))]
+                for d, i in zip(keep, oi):
+                    full[d] = i
+                run = np.ascontiguousarray(h[tuple(full)])
+                run.reshape(-1)[rng.choice([0, run.size - 1, run.size // 2])] = bad
+                h[tuple(full)] = run
+            got = host(dpt.var(dev(h), axis=axis, dtype="f8"))
+            assert np.isnan(got[hit]).all(), (shape, axis, bad)
+            np.testing.assert_allclose(got[~hit], np.var(a.astype("f8"), axis=axis)[~hit], rtol=1e-10)
+    # a sliced matrix reduced whole, the bad element at a corner of the slice and just outside it
+    h = rng.standard_normal((300, 400)).astype(dt)
+    h[0, 0] = np.nan  # outside the slice
+    d = dev(h)
+    assert np.isfinite(float(dpt.var(d[1:-1, 1:-1], dtype="f8")))
+    h[1, 1] = np.inf
+    assert np.isnan(float(dpt.var(dev(h)[1:-1, 1:-1], dtype="f8")))
