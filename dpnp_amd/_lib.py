@@ -174,6 +174,14 @@ def _load():
 lib = _load()
 
 
+try:
+    from . import _dpx_ext as ext  # noqa: E402  (the pybind11 binding; links the library loaded above)
+except ImportError as e:  # pragma: no cover
+    raise ImportError(
+        "dpnp_amd/_dpx_ext extension module is not built (or was built for another Python): run "
+        "`make -C dpnp_amd/csrc`; there is no fallback path.  " + str(e)) from e
+
+
 class DpxError(Exception):
     """Base for errors reported by the library."""
 

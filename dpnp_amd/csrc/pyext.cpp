@@ -30,8 +30,9 @@ namespace {
 
 PyObject *s_cview, *s_as_view, *s_writable, *s_array_obj; // interned attribute names
 PyTypeObject *g_usm_type = nullptr, *g_dpnp_type = nullptr;
-PyObject *g_stream_fn = nullptr; // callable(device_index) -> hipStream_t as int (torch's current stream), or null
-void *g_stream = nullptr;        // the library's own stream otherwise
+PyObject *g_stream_fn = nullptr; // callable(device_index) -> hipStream_t as int
+bool g_stream_fixed = false;     // the callable always gives the same stream (the library's own): asked once
+void *g_stream = nullptr;        // that stream, once known
 PyObject *g_events = nullptr;    // the (event, event) pair of the default queue
 PyObject *g_events_fn = nullptr; // callable(queue) -> (event, event)
 PyObject *g_alloc = nullptr;     // callable(shape tuple, dtype id) -> freshly allocated C-contiguous usm_ndarray
@@ -105,7 +106,7 @@ dpx_array_view *view_arg(py::handle h, const char *what)
 void *stream_of(py::handle queue)
 {
     if (!queue.is_none()) return (void *)py::cast<uintptr_t>(queue.attr("stream_ptr"));
-    if (!g_stream_fn) return g_stream;
+    if (g_stream) return g_stream;
     PyObject *zero = PyLong_FromLong(0);
     PyObject *r = PyObject_CallOneArg(g_stream_fn, zero);
     Py_DECREF(zero);
@@ -113,6 +114,7 @@ void *stream_of(py::handle queue)
     void *s = PyLong_AsVoidPtr(r);
     Py_DECREF(r);
     if (!s && PyErr_Occurred()) throw py::error_already_set();
+    if (g_stream_fixed) g_stream = s; // the library's own stream: one per process, created at first use
     return s;
 }
 
@@ -169,51 +171,114 @@ py::object fresh_result(PyObject *like, const int64_t *shape, int nd, int dt, dp
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// f(x, out=out) for a C-contiguous x whose dtype the kernel takes as it is
+// Broadcast descriptors of `n` operands against each other: extent 1 -> stride 0.  False when the shapes do
+// not broadcast (the general path words the error) or the result is empty.
+bool broadcast_views(const dpx_array_view *const *in, int n, dpx_array_view *b, int64_t *shape, int *nd_out, bool *plain)
+{
+    int nd = 0;
+    for (int i = 0; i < n; ++i) nd = in[i]->nd > nd ? in[i]->nd : nd;
+    for (int d = 0; d < nd; ++d) shape[d] = 1;
+    for (int i = 0; i < n; ++i)
+        for (int d = 0; d < in[i]->nd; ++d) {
+            const int k = nd - in[i]->nd + d;
+            if (in[i]->shape[d] == 1) continue;
+            if (shape[k] == 1) shape[k] = in[i]->shape[d];
+            else if (shape[k] != in[i]->shape[d]) return false;
+        }
+    int64_t total = 1;
+    for (int d = 0; d < nd; ++d) total *= shape[d];
+    if (total == 0) return false;
+    *plain = true; // nothing broadcast, all C-contiguous
+    for (int i = 0; i < n; ++i) {
+        b[i] = *in[i];
+        b[i].nd = nd;
+        bool same = in[i]->nd == nd;
+        for (int d = 0; d < nd; ++d) {
+            const int k = d - (nd - in[i]->nd);
+            const int64_t ext = k >= 0 ? in[i]->shape[k] : 1;
+            b[i].shape[d] = shape[d];
+            b[i].strides[d] = (k >= 0 && ext == shape[d]) ? in[i]->strides[k] : 0;
+            same = same && ext == shape[d];
+        }
+        if (!same) b[i].flags &= ~(DPX_C_CONTIGUOUS | DPX_F_CONTIGUOUS);
+        b[i].flags &= ~DPX_WRITABLE;
+        *plain = *plain && same && (in[i]->flags & DPX_C_CONTIGUOUS);
+    }
+    *nd_out = nd;
+    return true;
+}
+
+// `out` as the destination of a kernel that produces `shape` of dtype `dt`: right type and shape, writable, and
+// sharing no memory with an input (the in-place and temporary cases belong to the general path)
+dpx_array_view *checked_out(py::handle out, PyObject *like, const int64_t *shape, int nd, int dt,
+                            const dpx_array_view *const *in, int n)
+{
+    PyObject *uo = usm_of(out.ptr());
+    if (!uo || Py_TYPE(out.ptr()) != Py_TYPE(like)) return nullptr;
+    dpx_array_view *vo = view_of(uo);
+    if (vo->dtype != dt || !(vo->flags & DPX_WRITABLE) || vo->nd != nd) return nullptr;
+    for (int d = 0; d < nd; ++d)
+        if (vo->shape[d] != shape[d]) return nullptr;
+    for (int i = 0; i < n; ++i)
+        if (dpx_array_overlap(in[i], vo)) return nullptr;
+    return vo;
+}
+
+// f(x, out=out) for an array whose dtype the kernel takes as it is.  A fresh result is made here only for a
+// C-contiguous x (its layout is then C); with `out` any layout of x goes.
 py::object unary_call(int op, py::handle x, py::handle out)
 {
     PyObject *ux = usm_of(x.ptr());
     if (!ux || op < 0 || op >= 128) return not_implemented();
     dpx_array_view *vx = view_of(ux);
-    if (!(vx->flags & DPX_C_CONTIGUOUS)) return not_implemented();
     const int rdt = g_unary_res[op][vx->dtype];
     if (rdt < 0) return not_implemented();
     dpx_array_view *vo;
     py::object res;
-    if (out.is_none()) res = fresh_result(x.ptr(), vx->shape, vx->nd, rdt, &vo);
+    if (out.is_none()) {
+        if (!(vx->flags & DPX_C_CONTIGUOUS)) return not_implemented();
+        res = fresh_result(x.ptr(), vx->shape, vx->nd, rdt, &vo);
+    }
     else {
-        PyObject *uo = usm_of(out.ptr());
-        if (!uo || Py_TYPE(out.ptr()) != Py_TYPE(x.ptr())) return not_implemented();
-        vo = view_of(uo);
-        if (!plain_out(vo, vx, rdt) || spans_meet(vo, vx)) return not_implemented();
+        if (view_elems(vx) == 0) return not_implemented();
+        const dpx_array_view *in[1] = {vx};
+        vo = checked_out(out, x.ptr(), vx->shape, vx->nd, rdt, in, 1);
+        if (!vo) return not_implemented();
         res = py::reinterpret_borrow<py::object>(out);
     }
     if (int rc = dpx_unary(op, vx, vo, stream_of(py::none()))) raise_status(rc);
     return res;
 }
 
-// f(x1, x2, out=out) for two C-contiguous arrays of one shape and one dtype the kernel takes as it is
+// f(x1, x2, out=out) for two arrays of one dtype that the kernel takes as it is.  A fresh result is made here
+// only for two C-contiguous arrays of one shape; with `out` the operands may have any layout and broadcast.
 py::object binary_call(int op, py::handle x1, py::handle x2, py::handle out)
 {
     PyObject *u1 = usm_of(x1.ptr()), *u2 = usm_of(x2.ptr());
     if (!u1 || !u2 || Py_TYPE(x1.ptr()) != Py_TYPE(x2.ptr()) || op < 0 || op >= 128) return not_implemented();
     dpx_array_view *v1 = view_of(u1), *v2 = view_of(u2);
-    if (v1->dtype != v2->dtype || !(v1->flags & v2->flags & DPX_C_CONTIGUOUS) || !same_shape(v1, v2))
-        return not_implemented();
+    if (v1->dtype != v2->dtype) return not_implemented();
     const int rdt = g_binary_res[op][v1->dtype];
     if (rdt < 0) return not_implemented();
     dpx_array_view *vo;
     py::object res;
-    if (out.is_none()) res = fresh_result(x1.ptr(), v1->shape, v1->nd, rdt, &vo);
-    else {
-        PyObject *uo = usm_of(out.ptr());
-        if (!uo || Py_TYPE(out.ptr()) != Py_TYPE(x1.ptr()) || out.ptr() == x1.ptr()) return not_implemented();
-        vo = view_of(uo);
-        if (!plain_out(vo, v1, rdt) || spans_meet(vo, v1) || spans_meet(vo, v2)) return not_implemented();
-        res = py::reinterpret_borrow<py::object>(out);
+    if (out.is_none()) {
+        if (!(v1->flags & v2->flags & DPX_C_CONTIGUOUS) || !same_shape(v1, v2)) return not_implemented();
+        res = fresh_result(x1.ptr(), v1->shape, v1->nd, rdt, &vo);
+        if (int rc = dpx_binary(op, v1, v2, vo, stream_of(py::none()))) raise_status(rc);
+        return res;
     }
-    if (int rc = dpx_binary(op, v1, v2, vo, stream_of(py::none()))) raise_status(rc);
-    return res;
+    if (out.ptr() == x1.ptr()) return not_implemented(); // x1 op= x2: the in-place kernels, general path
+    const dpx_array_view *in[2] = {v1, v2};
+    dpx_array_view b[2];
+    int64_t shape[DPX_MAX_ND];
+    int nd;
+    bool plain;
+    if (!broadcast_views(in, 2, b, shape, &nd, &plain)) return not_implemented();
+    vo = checked_out(out, x1.ptr(), shape, nd, rdt, in, 2);
+    if (!vo) return not_implemented();
+    if (int rc = dpx_binary(op, plain ? v1 : &b[0], plain ? v2 : &b[1], vo, stream_of(py::none()))) raise_status(rc);
+    return py::reinterpret_borrow<py::object>(out);
 }
 
 // sum(x, axis=axis, out=out) and its siblings with dtype=None, keepdims=False: `axis` None, an int or a
@@ -300,6 +365,36 @@ py::object reduce_call(int op, bool search, py::handle x, py::handle axis, py::h
     return res;
 }
 
+// where(condition, x1, x2, out=out) for arrays whose branches share a dtype: the three operands are broadcast
+// on their descriptors (extent 1 -> stride 0).  A fresh result is only made here when nothing is broadcast and
+// all three are C-contiguous (its layout is then C whatever the order rule); other layouts are the general path's.
+py::object where_call(py::handle cond, py::handle x1, py::handle x2, py::handle out)
+{
+    PyObject *uc = usm_of(cond.ptr()), *u1 = usm_of(x1.ptr()), *u2 = usm_of(x2.ptr());
+    if (!uc || !u1 || !u2 || Py_TYPE(x1.ptr()) != Py_TYPE(cond.ptr()) || Py_TYPE(x2.ptr()) != Py_TYPE(cond.ptr()))
+        return not_implemented();
+    const dpx_array_view *in[3] = {view_of(uc), view_of(u1), view_of(u2)};
+    if (in[1]->dtype != in[2]->dtype) return not_implemented();
+    dpx_array_view b[3];
+    int64_t shape[DPX_MAX_ND];
+    int nd;
+    bool plain;
+    if (!broadcast_views(in, 3, b, shape, &nd, &plain)) return not_implemented();
+    dpx_array_view *vo;
+    py::object res;
+    if (out.is_none()) {
+        if (!plain) return not_implemented();
+        res = fresh_result(cond.ptr(), shape, nd, in[1]->dtype, &vo);
+    }
+    else {
+        vo = checked_out(out, cond.ptr(), shape, nd, in[1]->dtype, in, 3);
+        if (!vo) return not_implemented();
+        res = py::reinterpret_borrow<py::object>(out);
+    }
+    if (int rc = dpx_where(&b[0], &b[1], &b[2], vo, stream_of(py::none()))) raise_status(rc);
+    return res;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 py::cpp_function make_unary(int op, const std::string &name)
 {
@@ -379,23 +474,17 @@ PYBIND11_MODULE(_dpx_ext, m)
     std::memset(g_search_res, -2, sizeof g_search_res);
 
     m.def("init",
-          [](py::object usm_type, py::object dpnp_type, py::object stream, py::object events_fn, py::object alloc,
-             py::object wrap) {
+          [](py::object usm_type, py::object stream_fn, bool stream_fixed, py::object events_fn, py::object alloc) {
               g_usm_type = (PyTypeObject *)usm_type.release().ptr();
-              g_dpnp_type = dpnp_type.is_none() ? nullptr : (PyTypeObject *)dpnp_type.release().ptr();
-              if (PyLong_Check(stream.ptr())) {
-                  g_stream = PyLong_AsVoidPtr(stream.ptr());
-                  g_stream_fn = nullptr;
-              }
-              else g_stream_fn = stream.release().ptr();
+              g_stream_fn = stream_fn.release().ptr();
+              g_stream_fixed = stream_fixed;
+              g_stream = nullptr;
               g_events = events_fn(py::none()).release().ptr();
               g_events_fn = events_fn.release().ptr();
               g_alloc = alloc.release().ptr();
-              if (!wrap.is_none()) g_wrap = wrap.release().ptr();
           },
-          "init(usm_ndarray type, dpnp_array type or None, stream (int: the library's stream; callable(device) -> "
-          "int: the current stream), events(queue) -> (event, event), alloc(shape, dtype id) -> usm_ndarray, "
-          "wrap(usm_ndarray) -> dpnp_array or None)");
+          "init(usm_ndarray type, stream(device index) -> hipStream_t as int, whether that is always the same "
+          "stream, events(queue) -> (event, event), alloc(shape, dtype id) -> usm_ndarray)");
     m.def("set_array_class", [](py::object dpnp_type, py::object wrap) {
         g_dpnp_type = (PyTypeObject *)dpnp_type.release().ptr();
         g_wrap = wrap.release().ptr();
@@ -417,6 +506,7 @@ PYBIND11_MODULE(_dpx_ext, m)
           py::arg("op"), py::arg("x"), py::arg("axis") = py::none(), py::arg("out") = py::none());
     m.def("search_call", [](int op, py::handle x, py::handle axis, py::handle out) { return reduce_call(op, true, x, axis, out); },
           py::arg("op"), py::arg("x"), py::arg("axis") = py::none(), py::arg("out") = py::none());
+    m.def("where_call", &where_call, py::arg("condition"), py::arg("x1"), py::arg("x2"), py::arg("out") = py::none());
     m.def(
         "_where",
         [](py::handle condition, py::handle x1, py::handle x2, py::handle dst, py::handle sycl_queue, py::handle) {

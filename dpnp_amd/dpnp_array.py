@@ -297,5 +297,14 @@ class dpnp_array:
         return dpnp.invert(self)
 
 
+def _register_with_ext():
+    from . import _lib
+
+    _lib.ext.set_array_class(dpnp_array, dpnp_array._create_from_usm_ndarray)
+
+
+_register_with_ext()
+
+
 def _np_scalar_or(x):
     return x.item() if isinstance(x, np.generic) else x

@@ -19,6 +19,9 @@ from .tensor import _tensor_elementwise_impl as tei
 from .tensor import _tensor_impl as ti
 from .tensor._type_utils import _default_accumulation_dtype
 from .tensor._usmarray import usm_ndarray
+from . import _lib
+
+_ext = _lib.ext
 
 # dtypes and constants under their NumPy names
 bool = bool_ = dpt.bool  # noqa: A001
@@ -299,6 +302,12 @@ class DPNPUnaryFunc:
     def __call__(self, x, /, out=None, *, where=True, order="K", dtype=None, subok=True, **kwargs):
         if (out is None or type(out) is dpnp_array) and dtype is None and where is True and order == "K" \
                 and subok is True and not kwargs and type(x) is dpnp_array:
+            fn = self._fn
+            if not fn._ext_types_known:
+                fn._tell_ext_types()
+            res = _ext.unary_call(fn._op_id, x, out)  # the plain case, checked on the descriptors
+            if res is not NotImplemented:
+                return res
             res = self._fn._fast(x._array_obj, None if out is None else out._array_obj)
             if res is not None:
                 return _wrap(res) if out is None else out
@@ -335,6 +344,13 @@ class DPNPBinaryFunc:
                 and order == "K" and subok is True and not kwargs:
             # arrays and Python numbers, the keywords at their defaults: the tensor function's own short path
             t1, t2 = type(x1), type(x2)
+            if t1 is dpnp_array and t2 is dpnp_array:
+                fn = self._fn
+                if not fn._ext_types_known:
+                    fn._tell_ext_types()
+                res = _ext.binary_call(fn._op_id, x1, x2, out)  # the plain case, checked on the descriptors
+                if res is not NotImplemented:
+                    return res
             uo = None if out is None else out._array_obj
             res = None
             if t1 is dpnp_array:
@@ -596,6 +612,10 @@ def isclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
 
 def where(condition, x=None, y=None, /, *, order="K", out=None):
     """Elements of `x` where `condition` holds, else of `y`."""
+    if order == "K" and x is not None and y is not None:
+        r = _ext.where_call(condition, x, y, out)  # arrays with branches of one dtype, on the descriptors
+        if r is not NotImplemented:
+            return r
     if out is None and type(condition) is dpnp_array and type(x) is dpnp_array and type(y) is dpnp_array:
         return _wrap(dpt.where(condition._array_obj, x._array_obj, y._array_obj, order=order))
     missing = (x is None, y is None).count(True)
@@ -612,6 +632,8 @@ def where(condition, x=None, y=None, /, *, order="K", out=None):
 
 
 # -- reductions ---------------------------------------------------------------------------------------------
+_R_SUM, _R_PROD, _R_MAX, _R_MIN = (_lib.REDUCE_ID[n] for n in ("sum", "prod", "max", "min"))
+_S_ARGMAX, _S_ARGMIN = _lib.SEARCH_ID["argmax"], _lib.SEARCH_ID["argmin"]
 def _wrap_reduction_call(usm_a, out, fn, res_dt, **kwargs):
     """Run a tensor-level reduction; an `out` of another dtype gets an unsafe cast of the result."""
     usm_out = None
@@ -629,6 +651,10 @@ def _reduction_res_dt(a, dtype):
 
 
 def sum(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    if dtype is None and keepdims is False and initial is None and where is True:
+        r = _ext.reduce_call(_R_SUM, a, axis, out)  # the plain call, on the descriptors; else the general path
+        if r is not NotImplemented:
+            return r
     check_limitations(initial=initial, where=where)
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.sum, _reduction_res_dt(u, dtype), axis=axis, dtype=dtype,
@@ -636,6 +662,10 @@ def sum(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where=
 
 
 def prod(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where=True):
+    if dtype is None and keepdims is False and initial is None and where is True:
+        r = _ext.reduce_call(_R_PROD, a, axis, out)
+        if r is not NotImplemented:
+            return r
     check_limitations(initial=initial, where=where)
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.prod, _reduction_res_dt(u, dtype), axis=axis, dtype=dtype,
@@ -643,12 +673,20 @@ def prod(a, axis=None, dtype=None, out=None, keepdims=False, initial=None, where
 
 
 def max(a, axis=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    if keepdims is False and initial is None and where is True:
+        r = _ext.reduce_call(_R_MAX, a, axis, out)
+        if r is not NotImplemented:
+            return r
     check_limitations(initial=initial, where=where)
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.max, u.dtype, axis=axis, keepdims=keepdims)
 
 
 def min(a, axis=None, out=None, keepdims=False, initial=None, where=True):  # noqa: A001
+    if keepdims is False and initial is None and where is True:
+        r = _ext.reduce_call(_R_MIN, a, axis, out)
+        if r is not NotImplemented:
+            return r
     check_limitations(initial=initial, where=where)
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.min, u.dtype, axis=axis, keepdims=keepdims)
@@ -694,11 +732,19 @@ def _search_res_dt(out):
 
 
 def argmax(a, axis=None, out=None, *, keepdims=False):
+    if keepdims is False:
+        r = _ext.search_call(_S_ARGMAX, a, axis, out)
+        if r is not NotImplemented:
+            return r
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.argmax, _search_res_dt(out), axis=axis, keepdims=keepdims)
 
 
 def argmin(a, axis=None, out=None, *, keepdims=False):
+    if keepdims is False:
+        r = _ext.search_call(_S_ARGMIN, a, axis, out)
+        if r is not NotImplemented:
+            return r
     u = get_usm_ndarray(a)
     return _wrap_reduction_call(u, out, dpt.argmin, _search_res_dt(out), axis=axis, keepdims=keepdims)
 
@@ -820,29 +866,32 @@ def where_compare(cmp_name, lhs, rhs, x, y, out=None):
     """`where(lhs CMP rhs, x, y)` in one pass; cmp_name in equal/not_equal/less/less_equal/
     greater/greater_equal.  All four operands must share a shape after broadcasting; lhs/rhs
     share a dtype and x/y share a dtype (scalars adopt the array operand's dtype)."""
-    arrs = [o for o in (lhs, rhs, x, y) if is_supported_array_type(o)]
-    if not arrs:
-        raise TypeError("at least one operand must be an array")
-    from .tensor._manipulation_functions import _broadcast_shape_impl
+    from .tensor._elementwise_common import _scalar_operand
 
-    shape = _broadcast_shape_impl([get_usm_ndarray(o).shape if is_supported_array_type(o) else ()
-                                   for o in (lhs, rhs, x, y)])
+    us = [o._array_obj if type(o) is dpnp_array else (o if type(o) is usm_ndarray else None) for o in (lhs, rhs, x, y)]
+    if us[0] is None and us[1] is None or us[2] is None and us[3] is None:
+        if not _builtins.any(u is not None for u in us):
+            raise TypeError("at least one operand must be an array")
+        raise TypeError("each of (lhs, rhs) and (x, y) needs an array operand")
+    shapes = [u._shape for u in us if u is not None]
+    shape = shapes[0]
+    if _builtins.any(sh != shape for sh in shapes[1:]):
+        from .tensor._manipulation_functions import _broadcast_shape_impl
 
-    def pair(a, b):
-        ua = get_usm_ndarray(a) if is_supported_array_type(a) else None
-        ub = get_usm_ndarray(b) if is_supported_array_type(b) else None
-        if ua is None and ub is None:
-            raise TypeError("each of (lhs, rhs) and (x, y) needs an array operand")
-        dt = (ua if ua is not None else ub).dtype
-        ua = dpt.full((), a, dtype=dt) if ua is None else ua
-        ub = dpt.full((), b, dtype=dt) if ub is None else ub
-        if ua.dtype != ub.dtype:
+        shape = _broadcast_shape_impl(shapes)
+
+    def pair(a, b, ua, ub):
+        dt = (ua if ua is not None else ub)._dtype
+        # a Python number becomes the kept 0-d device array of that value, seen with the result's shape
+        ua = _scalar_operand(a, dt, shape) if ua is None else (ua if ua._shape == shape else dpt.broadcast_to(ua, shape))
+        ub = _scalar_operand(b, dt, shape) if ub is None else (ub if ub._shape == shape else dpt.broadcast_to(ub, shape))
+        if ua._dtype != ub._dtype:
             raise ValueError("operands of a pair must have one dtype")
-        return dpt.broadcast_to(ua, shape), dpt.broadcast_to(ub, shape)
+        return ua, ub
 
-    ul, ur = pair(lhs, rhs)
-    ux, uy = pair(x, y)
-    res = dpt.empty(shape, dtype=ux.dtype) if out is None else get_usm_ndarray(out)
+    ul, ur = pair(lhs, rhs, us[0], us[1])
+    ux, uy = pair(x, y, us[2], us[3])
+    res = usm_ndarray._new_contiguous(tuple(shape), ux._dtype) if out is None else get_usm_ndarray(out)
     ti._where_compare(cmp_name, ul, ur, ux, uy, res)
     return out if out is not None else _wrap(res)
 

@@ -11,12 +11,14 @@ from collections import OrderedDict
 
 import numpy as np
 
+from .. import _lib
 from . import _tensor_impl as ti
 from ._copy_utils import _empty_like_orderK, _empty_like_pair_orderK
 from ._ctors import empty, empty_like, full
 from ._device import ExecutionPlacementError  # noqa: F401  (re-exported)
 from ._device import current_stream_ptr
 from ._dtypes import dtype as _as_dtype
+from ._dtypes import ALL_DTYPES, dtype_id
 from ._manipulation_functions import _broadcast_shape_impl, broadcast_to
 from ._type_utils import (
     WeakBooleanType,
@@ -32,6 +34,10 @@ from ._type_utils import (
     _resolve_weak_types_all_py_ints,
 )
 from ._usmarray import usm_ndarray
+
+
+_ext_unary_call = _lib.ext.unary_call
+_ext_binary_call = _lib.ext.binary_call
 
 
 def _operand_dtype(o):
@@ -183,6 +189,8 @@ class UnaryElementwiseFunc:
         self.name_ = name
         self.result_type_resolver_fn_ = result_type_resolver_fn
         self.unary_fn_ = unary_dp_impl_fn
+        self._op_id = _lib.UNARY_ID.get(name, -1)  # the extension module's plain-call path is keyed by it
+        self._ext_types_known = False
         self._fast_cache = {}
         self.__doc__ = docs
         self.acceptance_fn_ = acceptance_fn
@@ -220,11 +228,27 @@ class UnaryElementwiseFunc:
 
     types_ = types
 
+    def _tell_ext_types(self):
+        """Enter this function's result dtype for every input dtype it takes without a cast into the extension
+        module's table (the type search stays here; the module's plain-call path only looks the answer up)."""
+        self._ext_types_known = True
+        if self._op_id < 0:
+            return
+        for dt in ALL_DTYPES:
+            buf_dt, r = _find_buf_dtype(dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+            ok = r is not None and buf_dt is None
+            _lib.ext.set_unary_type(self._op_id, dtype_id(dt), dtype_id(r) if ok else -1)
+
     def _fast(self, x, out=None):
         """The result for a C-contiguous array whose dtype the kernel takes as it is, else None:
         the common call without the general path's checks (nothing to cast, order "K" of a
         C-contiguous input is C; an `out` must be a writable C-contiguous array of the result's
         shape and dtype in an allocation of its own)."""
+        if not self._ext_types_known:
+            self._tell_ext_types()
+        r = _ext_unary_call(self._op_id, x, out)  # the same checks, on the descriptors
+        if r is not NotImplemented:
+            return r
         if type(x) is not usm_ndarray or not x._is_c_contiguous():
             return None
         dt = x._dtype
@@ -295,6 +319,8 @@ class BinaryElementwiseFunc:
         self.__doc__ = docs
         self.acceptance_fn_ = acceptance_fn
         self.weak_type_resolver_ = weak_type_resolver
+        self._op_id = _lib.BINARY_ID.get(name, -1)
+        self._ext_types_known = False
         self._fused_cache = {}
         self._fast_cache = {}
 
@@ -370,11 +396,26 @@ class BinaryElementwiseFunc:
             hit = self._fused_cache[key] = tei._fused_cast_result_type(self.name_, d1, d2)
         return hit
 
+    def _tell_ext_types(self):
+        """See UnaryElementwiseFunc._tell_ext_types."""
+        self._ext_types_known = True
+        if self._op_id < 0:
+            return
+        for dt in ALL_DTYPES:
+            b1, b2, r = _find_buf_dtype2(dt, dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+            ok = r is not None and b1 is None and b2 is None
+            _lib.ext.set_binary_type(self._op_id, dtype_id(dt), dtype_id(r) if ok else -1)
+
     def _fast(self, o1, o2, out=None):
         """The result for two C-contiguous arrays of one shape and one dtype that the kernel
         takes as it is, or for such an array of a floating or complex dtype and a Python float
         or int (which then takes the array's dtype whatever its value); else None.  See
         UnaryElementwiseFunc._fast."""
+        if not self._ext_types_known:
+            self._tell_ext_types()
+        r = _ext_binary_call(self._op_id, o1, o2, out)  # two arrays: the same checks, on the descriptors
+        if r is not NotImplemented:
+            return r
         t1, t2 = type(o1), type(o2)
         scalar = None
         if t1 is usm_ndarray:

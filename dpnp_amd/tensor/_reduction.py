@@ -152,36 +152,92 @@ def _search_over_axis(x, axis, keepdims, out, _reduction_fn):
     return _finish(out, user, keepdims, res_shape, red_nd, perm, nd)
 
 
+def _fill_ext_type_tables():
+    """Default result dtype of each reduction per input dtype, for the extension module's plain-call path
+    (reduce_call / search_call): only pairs with a direct kernel are entered."""
+    from .. import _lib
+    from ._dtypes import ALL_DTYPES, bool as _bool, dtype_id, int64
+
+    ext, lib = _lib.ext, _lib.lib
+    rules = {"sum": _default_accumulation_dtype, "prod": _default_accumulation_dtype,
+             "max": lambda dt, q: dt, "min": lambda dt, q: dt,
+             "logsumexp": _default_accumulation_dtype_fp_types, "hypot": _default_accumulation_dtype_fp_types,
+             "any": lambda dt, q: _bool, "all": lambda dt, q: _bool, "count_nonzero": lambda dt, q: int64}
+    for name, rule in rules.items():
+        op = _lib.REDUCE_ID[name]
+        for dt in ALL_DTYPES:
+            if name in ("logsumexp", "hypot") and dt.kind == "c":
+                continue
+            res = rule(dt, None)
+            ok = res is not None and lib.dpx_reduce_dtype_supported(op, dtype_id(dt), dtype_id(res))
+            ext.set_reduce_type(op, dtype_id(dt), dtype_id(res) if ok else -1)
+    for name in ("argmax", "argmin"):
+        op = _lib.SEARCH_ID[name]
+        for dt in ALL_DTYPES:
+            ok = lib.dpx_search_dtype_supported(op, dtype_id(dt), dtype_id(int64))
+            ext.set_search_type(op, dtype_id(dt), dtype_id(int64) if ok else -1)
+    return ext.reduce_call, ext.search_call, _lib.REDUCE_ID, _lib.SEARCH_ID
+
+
+_ext_reduce, _ext_search, _RID, _SID = _fill_ext_type_tables()
+
+
+def _plain(op, x, axis, dtype, keepdims, out, search=False):
+    """The call for the plain case (default result dtype, no keepdims), done on the descriptors by the extension
+    module; NotImplemented for anything else."""
+    if dtype is not None or keepdims is not False:
+        return NotImplemented
+    return _ext_search(op, x, axis, out) if search else _ext_reduce(op, x, axis, out)
+
+
 def sum(x, /, *, axis=None, dtype=None, keepdims=False, out=None):  # noqa: A001
     """Sum of the elements of `x` over `axis` (all axes when None)."""
+    r = _plain(_RID["sum"], x, axis, dtype, keepdims, out)
+    if r is not NotImplemented:
+        return r
     return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._sum_over_axis,
                                 tri._sum_over_axis_dtype_supported, _default_accumulation_dtype)
 
 
 def prod(x, /, *, axis=None, dtype=None, keepdims=False, out=None):
     """Product of the elements of `x` over `axis`."""
+    r = _plain(_RID["prod"], x, axis, dtype, keepdims, out)
+    if r is not NotImplemented:
+        return r
     return _reduction_over_axis(x, axis, dtype, keepdims, out, tri._prod_over_axis,
                                 tri._prod_over_axis_dtype_supported, _default_accumulation_dtype)
 
 
 def max(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
     """Maximum over `axis`; NaN propagates."""
+    r = _plain(_RID["max"], x, axis, None, keepdims, out)
+    if r is not NotImplemented:
+        return r
     return _comparison_over_axis(x, axis, keepdims, out, tri._max_over_axis)
 
 
 def min(x, /, *, axis=None, keepdims=False, out=None):  # noqa: A001
     """Minimum over `axis`; NaN propagates."""
+    r = _plain(_RID["min"], x, axis, None, keepdims, out)
+    if r is not NotImplemented:
+        return r
     return _comparison_over_axis(x, axis, keepdims, out, tri._min_over_axis)
 
 
 def argmax(x, /, *, axis=None, keepdims=False, out=None):
     """Index of the maximum along `axis` (flat C-order index when None); first occurrence,
     NaN counts as the maximum."""
+    r = _plain(_SID["argmax"], x, axis, None, keepdims, out, search=True)
+    if r is not NotImplemented:
+        return r
     return _search_over_axis(x, axis, keepdims, out, tri._argmax_over_axis)
 
 
 def argmin(x, /, *, axis=None, keepdims=False, out=None):
     """Index of the minimum along `axis`; first occurrence, NaN counts as the minimum."""
+    r = _plain(_SID["argmin"], x, axis, None, keepdims, out, search=True)
+    if r is not NotImplemented:
+        return r
     return _search_over_axis(x, axis, keepdims, out, tri._argmin_over_axis)
 
 

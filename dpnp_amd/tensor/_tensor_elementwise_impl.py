@@ -8,39 +8,27 @@ from ._dtypes import dtype_from_id, dtype_id
 from ._tensor_impl import _events, _stream
 
 lib = _lib.lib
+ext = _lib.ext
 
 
 def _make_unary(name, op_id):
-    def fn(src, dst, sycl_queue=None, depends=()):
-        vs, vd = src._as_view(), dst._as_view()
-        _lib.check(lib.dpx_unary(op_id, vs, vd, _stream(sycl_queue)))
-        return _events(sycl_queue)
+    fn = ext.make_unary(op_id, "_" + name)  # _X(src, dst, sycl_queue=None, depends=()) -> (event, event)
 
     def result_type(dt):
         return dtype_from_id(lib.dpx_unary_result_type(op_id, dtype_id(dt)))
 
-    fn.__name__ = "_" + name
     result_type.__name__ = f"_{name}_result_type"
     return fn, result_type
 
 
 def _make_binary(name, op_id):
-    def fn(src1, src2, dst, sycl_queue=None, depends=()):
-        v1, v2, vd = src1._as_view(), src2._as_view(), dst._as_view()
-        _lib.check(lib.dpx_binary(op_id, v1, v2, vd, _stream(sycl_queue)))
-        return _events(sycl_queue)
+    fn = ext.make_binary(op_id, "_" + name)  # _X(src1, src2, dst, sycl_queue=None, depends=())
+    inplace = ext.make_binary_inplace(op_id, f"_{name}_inplace")  # _X_inplace(lhs, rhs, sycl_queue=None, depends=())
 
     def result_type(dt1, dt2):
         return dtype_from_id(lib.dpx_binary_result_type(op_id, dtype_id(dt1), dtype_id(dt2)))
 
-    def inplace(lhs, rhs, sycl_queue=None, depends=()):
-        vl, vr = lhs._as_view(), rhs._as_view()
-        _lib.check(lib.dpx_binary_inplace(op_id, vl, vr, _stream(sycl_queue)))
-        return _events(sycl_queue)
-
-    fn.__name__ = "_" + name
     result_type.__name__ = f"_{name}_result_type"
-    inplace.__name__ = f"_{name}_inplace"
     return fn, result_type, inplace
 
 
@@ -55,10 +43,7 @@ for _n, _i in _lib.BINARY_ID.items():
     globals()[f"_{_n}_inplace"] = _ip
 
 
-def _divide_by_scalar(src, scalar, dst, sycl_queue=None, depends=()):
-    vs, vd = src._as_view(), dst._as_view()
-    _lib.check(lib.dpx_divide_by_scalar(vs, float(scalar), vd, _stream(sycl_queue)))
-    return _events(sycl_queue)
+_divide_by_scalar = ext._divide_by_scalar  # (src, scalar, dst, sycl_queue=None, depends=())
 
 
 def _fused_cast_result_type(name, dt1, dt2):

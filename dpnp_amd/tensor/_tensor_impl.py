@@ -23,10 +23,7 @@ def _stream(q):
     return _current_stream_ptr(0) if q is None else q.stream_ptr
 
 
-def _where(condition, x1, x2, dst, sycl_queue=None, depends=()):
-    vc, v1, v2, vd = condition._as_view(), x1._as_view(), x2._as_view(), dst._as_view()
-    _lib.check(lib.dpx_where(vc, v1, v2, vd, _stream(sycl_queue)))
-    return _events(sycl_queue)
+_where = _lib.ext._where  # (condition, x1, x2, dst, sycl_queue=None, depends=()) -> (event, event)
 
 
 def _clip(src, min, max, dst, sycl_queue=None, depends=()):  # noqa: A002
@@ -39,15 +36,10 @@ def _clip(src, min, max, dst, sycl_queue=None, depends=()):  # noqa: A002
 
 def _where_compare(cmp_name, lhs, rhs, x1, x2, dst, sycl_queue=None, depends=()):
     """dst = (lhs CMP rhs) ? x1 : x2 in one pass (no counterpart in the reference)."""
-    views = [a._as_view() for a in (lhs, rhs, x1, x2, dst)]
-    _lib.check(lib.dpx_where_compare(_lib.BINARY_ID[cmp_name], *views, _stream(sycl_queue)))
-    return _events(sycl_queue)
+    return _lib.ext._where_compare(_lib.BINARY_ID[cmp_name], lhs, rhs, x1, x2, dst, sycl_queue, depends)
 
 
-def _copy_usm_ndarray_into_usm_ndarray(src, dst, sycl_queue=None, depends=()):
-    vs, vd = src._as_view(), dst._as_view()
-    _lib.check(lib.dpx_copy_cast(vs, vd, _stream(sycl_queue)))
-    return _events(sycl_queue)
+_copy_usm_ndarray_into_usm_ndarray = _lib.ext._copy_usm_ndarray_into_usm_ndarray  # (src, dst, sycl_queue=None, depends=())
 
 
 def _full_usm_ndarray(fill_value, dst, sycl_queue=None, depends=()):
@@ -64,14 +56,8 @@ def _full_usm_ndarray(fill_value, dst, sycl_queue=None, depends=()):
     return _events(sycl_queue)
 
 
-def _array_overlap(a, b):
-    va, vb = a._as_view(), b._as_view()
-    return bool(lib.dpx_array_overlap(va, vb))
-
-
-def _same_logical_tensors(a, b):
-    va, vb = a._as_view(), b._as_view()
-    return bool(lib.dpx_same_logical(va, vb))
+_array_overlap = _lib.ext._array_overlap
+_same_logical_tensors = _lib.ext._same_logical_tensors
 
 
 # device_support_queries.cpp: MI355X has fp16 and fp64, so the defaults are NumPy's

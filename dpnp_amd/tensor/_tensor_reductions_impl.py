@@ -10,26 +10,17 @@ lib = _lib.lib
 
 
 def _make_reduction(name, op_id):
-    def fn(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
-        vs, vd = src._as_view(), dst._as_view()
-        _lib.check(lib.dpx_reduce(op_id, vs, int(trailing_dims_to_reduce), vd, None, _stream(sycl_queue)))
-        return _events(sycl_queue)
+    # _X_over_axis(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()) -> (event, event)
+    fn = _lib.ext.make_reduction(op_id, f"_{name}_over_axis")
 
     def supported(arg_dtype, out_dtype, dst_usm_type=None, sycl_queue=None):
         return bool(lib.dpx_reduce_dtype_supported(op_id, dtype_id(arg_dtype), dtype_id(out_dtype)))
 
-    fn.__name__ = f"_{name}_over_axis"
     return fn, supported
 
 
 def _make_search(name, op_id):
-    def fn(src, trailing_dims_to_reduce, dst, sycl_queue=None, depends=()):
-        vs, vd = src._as_view(), dst._as_view()
-        _lib.check(lib.dpx_argreduce(op_id, vs, int(trailing_dims_to_reduce), vd, _stream(sycl_queue)))
-        return _events(sycl_queue)
-
-    fn.__name__ = f"_{name}_over_axis"
-    return fn
+    return _lib.ext.make_search(op_id, f"_{name}_over_axis")
 
 
 _sum_over_axis, _sum_over_axis_dtype_supported = _make_reduction("sum", _lib.REDUCE_ID["sum"])

@@ -514,3 +514,21 @@ class usm_ndarray:
     def __ixor__(self, o): return self._fn("bitwise_xor")._inplace_op(self, o)
     def __ilshift__(self, o): return self._fn("bitwise_left_shift")._inplace_op(self, o)
     def __irshift__(self, o): return self._fn("bitwise_right_shift")._inplace_op(self, o)
+
+
+def _ext_alloc(shape, dt_id):
+    """Fresh C-contiguous array for the extension module's calls that make their own result."""
+    from ._dtypes import ALL_DTYPES
+
+    return usm_ndarray._new_contiguous(shape, ALL_DTYPES[dt_id])
+
+
+def _init_ext():
+    from ._tensor_impl import _events
+
+    # the stream: the library's own is one per process (asked for once, at the first call that needs it);
+    # PyTorch's current stream is asked for at every call
+    _lib.ext.init(usm_ndarray, _device.current_stream_ptr, _lib.MEMORY == "native", _events, _ext_alloc)
+
+
+_init_ext()

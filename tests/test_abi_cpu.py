@@ -351,3 +351,34 @@ def test_overlap_predicates():
     assert lib.dpx_same_logical(a, view([10], ptr=FAKE)) == 1
     assert lib.dpx_same_logical(a, view([10], [2], ptr=FAKE)) == 0
     assert lib.dpx_same_logical(a, view([10], ptr=FAKE, dt=L.INT32)) == 0
+
+
+def test_extension_module_binds_the_same_library_and_names_its_functions_like_the_reference():
+    """dpnp_amd._dpx_ext (pybind11) links libdpnp_amd.so and makes the boundary functions under the
+    reference's names and keyword arguments (tensor_elementwise.cpp:42, elementwise_common.cpp:118-188,
+    reductions/sum.cpp: `_sum_over_axis(src, trailing_dims_to_reduce, dst, sycl_queue, depends)`)."""
+    import dpnp_amd._lib as L
+    from dpnp_amd.tensor import _tensor_elementwise_impl as tei
+    from dpnp_amd.tensor import _tensor_impl as ti
+    from dpnp_amd.tensor import _tensor_reductions_impl as tri
+
+    ext = L.ext
+    for fn, name, args in ((tei._add, "_add", ("src1", "src2", "dst", "sycl_queue", "depends")),
+                           (tei._exp, "_exp", ("src", "dst", "sycl_queue", "depends")),
+                           (tei._add_inplace, "_add_inplace", ("lhs", "rhs", "sycl_queue", "depends")),
+                           (tri._sum_over_axis, "_sum_over_axis", ("src", "trailing_dims_to_reduce", "dst", "sycl_queue", "depends")),
+                           (tri._argmax_over_axis, "_argmax_over_axis", ("src", "trailing_dims_to_reduce", "dst", "sycl_queue", "depends")),
+                           (ti._where, "_where", ("condition", "x1", "x2", "dst", "sycl_queue", "depends")),
+                           (ti._copy_usm_ndarray_into_usm_ndarray, "_copy_usm_ndarray_into_usm_ndarray", ("src", "dst", "sycl_queue", "depends"))):
+        assert type(fn).__name__ == "builtin_function_or_method" and fn.__name__ == name
+        sig = fn.__doc__.splitlines()[0]
+        assert all(f"{a}:" in sig for a in args), sig
+    # a wrong argument is a TypeError before anything reaches the library, as with the reference's bindings
+    with pytest.raises(TypeError):
+        tei._add(1, 2, 3)
+    # the plain-call functions decline what they do not handle instead of guessing
+    assert ext.binary_call(L.BINARY_ID["add"], 1.0, 2.0, None) is NotImplemented
+    assert ext.reduce_call(L.REDUCE_ID["sum"], object(), None, None) is NotImplemented
+    assert ext.where_call(None, None, None, None) is NotImplemented
+    with pytest.raises(ValueError):
+        ext.set_binary_type(10 ** 6, 0, 0)

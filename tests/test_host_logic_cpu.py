@@ -254,3 +254,73 @@ def test_reduction_over_leading_axis_leaves_no_reference_cycle():
     finally:
         if was:
             gc.enable()
+
+
+# ---- the extension module's plain-call path: what it takes and what it leaves to the general path ---------
+def test_plain_call_path_declines_everything_but_the_plain_case():
+    """binary_call / unary_call / reduce_call / where_call decide on the array descriptors alone.  Every case
+    here is one they must hand back (NotImplemented) BEFORE anything is launched: no GPU is present, and a
+    launch would raise."""
+    import dpnp_amd._lib as L
+
+    ext = L.ext
+    add, exp, rsum, amax = L.BINARY_ID["add"], L.UNARY_ID["exp"], L.REDUCE_ID["sum"], L.SEARCH_ID["argmax"]
+    f4, i4 = 10, 5
+    ext.set_binary_type(add, f4, f4)
+    ext.set_unary_type(exp, f4, f4)
+    a, b, c = host_array((4, 6)), host_array((4, 6)), host_array((4, 6))
+    assert ext.binary_call(add, a, host_array((4, 6), "f8"), c) is NotImplemented  # mixed dtypes: promotion
+    assert ext.binary_call(add, a, host_array((6,)), None) is NotImplemented  # broadcasting without out: layout rules
+    assert ext.binary_call(add, a.T, b.T, None) is NotImplemented  # not C-contiguous without out: order "K"
+    assert ext.binary_call(add, a, host_array((5,)), c) is NotImplemented  # shapes that do not broadcast
+    assert ext.binary_call(add, a, b, host_array((4, 6), "f8")) is NotImplemented  # out of another dtype
+    assert ext.binary_call(add, a, b, host_array((6, 4))) is NotImplemented  # out of another shape
+    assert ext.binary_call(add, a, b, a) is NotImplemented  # in place
+    assert ext.binary_call(add, a, b, a[1:]) is NotImplemented  # out overlaps an input
+    ro = host_array((4, 6))
+    ro.flags.writable = False
+    assert ext.binary_call(add, a, b, ro) is NotImplemented  # read-only out: the general path raises
+    assert ext.binary_call(add, a, 2.0, c) is NotImplemented  # scalars stay with the Python layer
+    assert ext.binary_call(L.BINARY_ID["hypot"], a, b, c) is NotImplemented  # type not looked up yet
+    ia = host_array((4, 6), "i4")
+    assert ext.unary_call(exp, ia, None) is NotImplemented  # needs a cast
+    assert ext.unary_call(exp, a.T, None) is NotImplemented
+    assert ext.unary_call(exp, a, a) is NotImplemented
+    assert ext.unary_call(exp, a.T, c) is NotImplemented  # out of another shape
+    # reductions: axis forms, out checks, empty extents
+    r = host_array((4,))
+    assert ext.reduce_call(rsum, a, [1], r) is NotImplemented  # a list: normalised by the general path
+    assert ext.reduce_call(rsum, a, 2, r) is NotImplemented  # out of range: the general path raises
+    assert ext.reduce_call(rsum, a, (1, 1), r) is NotImplemented  # repeated axis
+    assert ext.reduce_call(rsum, a, (), None) is NotImplemented  # nothing reduced: a copy
+    assert ext.reduce_call(rsum, a, 1, host_array((6,))) is NotImplemented  # out of another shape
+    assert ext.reduce_call(rsum, a, 1, host_array((4,), "f8")) is NotImplemented  # out of another dtype
+    assert ext.reduce_call(rsum, a, 1, a[:, 0]) is NotImplemented  # out inside the input
+    assert ext.reduce_call(rsum, host_array((0, 6)), 0, None) is NotImplemented  # empty reduced axis
+    assert ext.reduce_call(rsum, host_array((4, 0)), 0, None) is NotImplemented  # empty result
+    assert ext.reduce_call(rsum, host_array(()), None, None) is NotImplemented  # 0-d
+    assert ext.search_call(amax, a, (0, 1), None) is NotImplemented  # a search takes one axis
+    assert ext.search_call(amax, a, 1, host_array((4,), "i4")) is NotImplemented  # the index type is int64
+    # where: branches of different dtypes, shapes that do not broadcast, out mismatches, overlap
+    m = host_array((4, 6), "?")
+    assert ext.where_call(m, a, host_array((4, 6), "f8"), None) is NotImplemented
+    assert ext.where_call(m, a, host_array((5,)), None) is NotImplemented
+    assert ext.where_call(m, a, host_array((6,)), None) is NotImplemented  # broadcast without out: layout rules
+    assert ext.where_call(m, a, b, host_array((4, 6), "f8")) is NotImplemented
+    assert ext.where_call(m, a, b, a) is NotImplemented
+    assert ext.where_call(m, a, 1.0, c) is NotImplemented
+    assert ext.where_call(host_array((0,), "?"), host_array((0,)), host_array((0,)), None) is NotImplemented
+    # the plain cases reach the library; where no device is present the launch error comes back as RuntimeError
+    # (with a device these arrays of host memory must not be launched on at all)
+    import ctypes
+
+    n = ctypes.c_int(0)
+    L.check(L.lib.dpx_device_count(ctypes.byref(n)))
+    if n.value:
+        return
+    for call in (lambda: ext.binary_call(add, a, b, c), lambda: ext.unary_call(exp, a, c),
+                 lambda: ext.binary_call(add, a[:, ::2], host_array((1, 3)), host_array((4, 3))),
+                 lambda: ext.unary_call(exp, a.T, host_array((6, 4))),
+                 lambda: ext.where_call(m, a, host_array((6,)), c)):
+        with pytest.raises(RuntimeError):
+            call()
