@@ -76,6 +76,9 @@ WORKLOADS = {
             "(fp32 input and fp64 input)",
     "cfg4": "8192x8192 fp32 views A[:, ::2], A.T and a (1,4096) row: multiply, exp, where(A>0, A, B); int32 bitwise_and",
     "cfg5": "Black-Scholes over 2^26 fp64 options, call and put: one fused kernel, and the chain of elementwise calls",
+    "floors": "access patterns and instruction streams on their own (dpnp_amd/csrc/floors.hip), each beside the product "
+              "call it bounds: Black-Scholes split into its memory streams and its arithmetic, the 2^24 read with and "
+              "without a cross-block step, every-other-column reads, 512-byte runs on both sides of a transposition",
     "layouts": "fp32 2^28 elements reduced over dims that do not collapse into one run: a sliced matrix summed whole, "
                "axes (0, 2) of 3-d and 4-d arrays, every other column (sum, max, mean, argmax)",
 }
@@ -256,7 +259,72 @@ def build_workload(name, dpnp, torch):
                ("sum_every_other_column_axis0", lambda: dpnp.sum(A[:, ::2], axis=0, out=rh), 4 * n, n // 2),
                ("argmax_every_other_column_axis1", lambda: dpnp.argmax(A[:, ::2], axis=1, out=ri), 4 * n, n // 2)]
         return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
+    if name == "floors":
+        return build_floors(dpnp, torch, uniform, normal)
     raise SystemExit(f"--workload: unknown workload {name!r} (one of {', '.join(WORKLOADS)})")
+
+
+def build_floors(dpnp, torch, uniform, normal):
+    """Each measurement kernel of libdpx_floors.so (label "floor:<name>") next to the product call whose time it
+    bounds (label "product:<call>").  The kernels run on the library's stream, on workspaces of the package's pool."""
+    import ctypes
+
+    from dpnp_amd.tensor import _device
+
+    path = os.path.join(ROOT, "dpnp_amd", "libdpx_floors.so")
+    if not os.path.exists(path):
+        raise SystemExit("dpnp_amd/libdpx_floors.so is not built: make -C dpnp_amd/csrc")
+    fl = ctypes.CDLL(path)
+    fl.dpx_floors_name.restype = fl.dpx_floors_about.restype = ctypes.c_char_p
+    fl.dpx_floors_bytes.restype = ctypes.c_double
+    fl.dpx_floors_workspace.restype = ctypes.c_size_t
+    fl.dpx_floors_prepare.argtypes = fl.dpx_floors_launch.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    stream = _device.current_stream_ptr()
+    index = {fl.dpx_floors_name(i).decode(): i for i in range(fl.dpx_floors_count())}
+
+    def floor(name):
+        i = index[name]
+        ws = dpnp.empty(fl.dpx_floors_workspace(i), dtype="u1")
+        ptr = ws.get_array()._buf.data_ptr()
+        if fl.dpx_floors_prepare(i, ptr, stream):
+            raise SystemExit(f"floors: preparing {name} failed")
+
+        def run(ws=ws):  # (the closure keeps the workspace alive)
+            if fl.dpx_floors_launch(i, ptr, stream):
+                raise RuntimeError(f"floors: launch of {name} failed")
+        nb = fl.dpx_floors_bytes(i)
+        return (f"floor:{name}", run, nb, 0)
+
+    n26, n24, side = 1 << 26, 1 << 24, 8192
+    # the product calls the floors stand beside
+    price, strike = uniform(n26, 10.0, 50.0, torch.float64), uniform(n26, 10.0, 50.0, torch.float64)
+    t = uniform(n26, 1.0, 2.0, torch.float64)
+    call, put = dpnp.empty(n26, dtype="f8"), dpnp.empty(n26, dtype="f8")
+    c24, s24 = uniform(n24), dpnp.empty((), dtype="f4")
+    A, A2, B = normal((side, side)), normal((side, side)), normal((1, side // 2))
+    o_half, o_b = dpnp.empty((side, side // 2), dtype="f4"), dpnp.empty((side, side // 2), dtype="?")
+    o_c = dpnp.empty((side, side), dtype="f4")
+    V1, V1b = A[:, ::2], A2[:, ::2]
+    h = side * side // 2
+    ops = [
+        floor("launch"),
+        floor("bs_streams"), floor("stream5_f64"), floor("bs_arithmetic"),
+        ("product:black_scholes_fused", lambda: dpnp.black_scholes(price, strike, t, 0.1, 0.2, call=call, put=put), 40 * n26, n26),
+        floor("read_f32_2p24"), floor("read_f32_2p24_tickets"),
+        ("product:sum_f32_2p24", lambda: dpnp.sum(c24, out=s24), 4 * n24, n24),
+        floor("stride2_one_input"),
+        ("product:multiply_V1_row", lambda: dpnp.multiply(V1, B, out=o_half), 12 * h, h),
+        floor("stride2_predicate"),
+        ("product:greater_V1_0", lambda: dpnp.greater(V1, 0, out=o_b), 9 * h, h),
+        floor("stride2_two_inputs"),
+        ("product:multiply_V1_V1b", lambda: dpnp.multiply(V1, V1b, out=o_half), 20 * h, h),
+        floor("tile_runs_8192"),
+        ("product:exp_AT_to_C", lambda: dpnp.exp(A.T, out=o_c), 16 * h, 2 * h),
+    ]
+    ops[0] = (ops[0][0], ops[0][1], 1, 0)  # (no bytes: keep the ratio defined)
+    ops[3] = (ops[3][0], ops[3][1], 1, 0)
+    return ops, "f64/f32", "synthetic; bytes of the strided calls are the whole lines they touch (physical bytes)"
+
 
 
 def dpnp_cpu_probe():

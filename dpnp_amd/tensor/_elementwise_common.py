@@ -235,8 +235,11 @@ class UnaryElementwiseFunc:
         if self._op_id < 0:
             return
         for dt in ALL_DTYPES:
-            buf_dt, r = _find_buf_dtype(dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
-            ok = r is not None and buf_dt is None
+            try:
+                buf_dt, r = _find_buf_dtype(dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+                ok = r is not None and buf_dt is None
+            except Exception:  # a type the function refuses with an error of its own: the general path raises it
+                ok = False
             _lib.ext.set_unary_type(self._op_id, dtype_id(dt), dtype_id(r) if ok else -1)
 
     def _fast(self, x, out=None):
@@ -402,8 +405,11 @@ class BinaryElementwiseFunc:
         if self._op_id < 0:
             return
         for dt in ALL_DTYPES:
-            b1, b2, r = _find_buf_dtype2(dt, dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
-            ok = r is not None and b1 is None and b2 is None
+            try:
+                b1, b2, r = _find_buf_dtype2(dt, dt, self.result_type_resolver_fn_, None, acceptance_fn=self.acceptance_fn_)
+                ok = r is not None and b1 is None and b2 is None
+            except Exception:  # e.g. subtract of bool: the general path raises the function's own error
+                ok = False
             _lib.ext.set_binary_type(self._op_id, dtype_id(dt), dtype_id(r) if ok else -1)
 
     def _fast(self, o1, o2, out=None):

@@ -324,3 +324,23 @@ def test_plain_call_path_declines_everything_but_the_plain_case():
                  lambda: ext.where_call(m, a, host_array((6,)), c)):
         with pytest.raises(RuntimeError):
             call()
+
+
+def test_every_function_can_tell_the_extension_module_its_types():
+    """The per-function type tables of the plain-call path are filled from the Python layer's own type search,
+    for every dtype, also those a function refuses with an error of its own (subtract and negative of bool)."""
+    import dpnp_amd._lib as L
+    from dpnp_amd.tensor import _elementwise_funcs as ef
+    from dpnp_amd.tensor._elementwise_common import BinaryElementwiseFunc, UnaryElementwiseFunc
+
+    seen = 0
+    for f in vars(ef).values():
+        if isinstance(f, (BinaryElementwiseFunc, UnaryElementwiseFunc)):
+            f._tell_ext_types()
+            assert f._ext_types_known and f._op_id >= 0
+            seen += 1
+    assert seen >= 70
+    assert L.ext.binary_type(L.BINARY_ID["subtract"], 0) == -1 and L.ext.binary_type(L.BINARY_ID["subtract"], 10) == 10
+    assert L.ext.binary_type(L.BINARY_ID["less"], 11) == 0  # comparisons give bool
+    assert L.ext.unary_type(L.UNARY_ID["negative"], 0) == -1 and L.ext.unary_type(L.UNARY_ID["exp"], 5) == -1
+    assert L.ext.unary_type(L.UNARY_ID["abs"], 13) == 11  # |complex128| is float64
