@@ -254,9 +254,11 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
                 rc = RC_S2;
                 any_s2 = true;
                 // the wave-wide reads go one element past a row's last: only the row at the highest
-                // address may not, and that is the last row when no stride is negative
+                // address may not, and that is the last row when no stride is negative and rows do not
+                // interleave (every other row then begins at or beyond the element after its predecessor's
+                // last; views with explicit strides smaller than a row's extent take the general kernel)
                 for (int d = 0; d < inner; ++d)
-                    if (pl.strides[k][d] < 0) rc = -1;
+                    if (pl.strides[k][d] < 0 || (pl.shape[d] > 1 && pl.strides[k][d] < 2 * ncols - 1)) rc = -1;
             }
             else if (si == 1 && sr != 0) rc = RC_ROWS;
             else if ((si == 1 || si == 0) && sr == 0) {

@@ -104,6 +104,23 @@ def test_shapes_next_to_the_conditions_stay_generic():
     out = dpt.empty((16, 256), dtype="f4")
     assert _path("negative", da[::-1, ::2], out) == "ew_rows"
     assert_same(host(dpt.negative(da[::-1, ::2])), -a[::-1, ::2])
+    # overlapping windows (row stride smaller than a row's extent, explicit strides): rows interleave, so a
+    # row's wave-wide read could end past the last element the view addresses; generic kernel
+    from dpnp_amd.tensor._usmarray import usm_ndarray
+
+    flat = random_array(rng, (4 * 100 + 2 * 256 - 1,), "f4")
+    dflat = dev(flat)
+    win = usm_ndarray((4, 256), dtype="f4", buffer=dflat, strides=(100, 2))
+    out = dpt.empty((4, 256), dtype="f4")
+    assert _path("negative", win, out) == "ew_rows"
+    want = np.lib.stride_tricks.as_strided(flat, (4, 256), (400, 8))
+    assert_same(host(dpt.negative(win)), -want)
+    # rows exactly one extent apart (the closest that do not interleave) keep the two-rows kernel
+    flat = random_array(rng, (4 * 511,), "f4")
+    dflat = dev(flat)
+    win = usm_ndarray((4, 256), dtype="f4", buffer=dflat, strides=(511, 2))
+    assert _path("negative", win, out) == "ew_rows2"
+    assert_same(host(dpt.negative(win)), -np.lib.stride_tricks.as_strided(flat, (4, 256), (2044, 8)))
     # narrow element types keep the generic kernel (two-byte packs of eight)
     h = random_array(rng, (8, 2048), "f2")
     assert_same(host(dpt.negative(dev(h)[:, ::2])), -h[:, ::2])
