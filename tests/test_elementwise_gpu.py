@@ -772,6 +772,19 @@ def test_extension_fmax_fmin_all_types(dt):
             a[1::13] = complex(1, np.nan)
     for name in ("fmax", "fmin"):
         assert_same(host(getattr(dpt, name)(dev(a), dev(b))), orc.binary(name, a, b))
+    if np.dtype(dt).kind == "c":
+        # every pair of a grid with signed zeros, infinities and NaN parts (the oracle's rule is pinned on the same
+        # grid against a scalar transcription of math_utils.hpp:73-95)
+        vals = [0.0, -0.0, 1.0, -1.0, 2.5, np.inf, -np.inf, np.nan]
+        grid = np.array([complex(re, im) for re in vals for im in vals], dtype=dt)
+        ga, gb = (g.ravel() for g in np.meshgrid(grid, grid, indexing="ij"))
+        for name in ("fmax", "fmin", "less_equal", "greater_equal", "less", "greater", "maximum", "minimum"):
+            got, want = host(getattr(dpt, name)(dev(ga), dev(gb))), orc.binary(name, ga, gb)
+            if want.dtype.kind == "c":
+                assert_same(got.real, want.real)
+                assert_same(got.imag, want.imag)
+            else:
+                assert_same(got, want)
 
 
 def test_extension_binary_misc():

@@ -17,6 +17,11 @@ Oracle function -> what pins it here (none of the pins calls NumPy for the rule 
   maximum / minimum                       test_maximum_minimum_nan_rule
   promote_binary                          test_promotion_matches_numpy_result_type,
                                           test_promotion_with_acceptance_hooks
+  black_scholes                           test_black_scholes_against_the_textbook_formula_in_40_digits (mpmath ncdf)
+  fmax / fmin / <= / >= of complex        test_complex_fmax_fmin_ordering_brute_force (scalar transcription of
+                                          math_utils.hpp:73-95 and fmax.hpp:57-70 on a grid with NaN parts)
+  binary pow (floats)                     test_float_pow_special_values (C99 F.10.4.4 written out; the reference's
+                                          list, test_binary_ufuncs.py:972-994)
   var_around_mean                         test_var_around_mean_identities_and_docstring_values (exact
                                           rational arithmetic, var(z) = var(Re z) + var(Im z), the shift
                                           identity, dpnp_iface_statistics.py:1815-1826,1625-1634)
@@ -324,19 +329,97 @@ def test_where_known_answer():
     assert (orc.where(np.array([0.0, -0.0, np.nan, 2.0]), np.ones(4), np.zeros(4)) == [0, 0, 1, 1]).all()
 
 
-def test_black_scholes_put_call_parity():
+def test_black_scholes_against_the_textbook_formula_in_40_digits():
+    """The oracle restates the reference example's expression tree (erf of w1, w2).  Pinned against the textbook
+    form written independently of it: call = S0 Phi(d1) - K exp(-rT) Phi(d2), put = K exp(-rT) Phi(-d2) -
+    S0 Phi(-d1), d1 = (ln(S0/K) + (r + sigma^2/2) T) / (sigma sqrt(T)), d2 = d1 - sigma sqrt(T), with Phi the
+    normal distribution function of mpmath (ncdf) at 40 digits.  A dropped term, a wrong sign of r or a swapped
+    price and strike changes the prices by far more than the bound."""
+    import mpmath
+
     rng = np.random.default_rng(4)
-    p, s, t = rng.uniform(10, 50, 1000), rng.uniform(10, 50, 1000), rng.uniform(1, 2, 1000)
-    call, put = orc.black_scholes(p, s, t, 0.1, 0.2)
-    np.testing.assert_allclose(call - put, p - s * np.exp(-0.1 * t), rtol=1e-12, atol=1e-12)
-    # closed form of the same expression tree with the normal CDF written through erf:
-    # call = P*N(d1') - S*exp(-rT)*N(d2') with N(x) = (1 + erf(x)) / 2 applied to w1, w2
-    z = t * (0.2 * 0.2 * 2)
-    w1 = (np.log(p / s) + 0.1 * t + 0.25 * z) / np.sqrt(z)
-    w2 = (np.log(p / s) + 0.1 * t - 0.25 * z) / np.sqrt(z)
-    erf = np.vectorize(math.erf)
-    want = p * (0.5 + 0.5 * erf(w1)) - s * np.exp(-0.1 * t) * (0.5 + 0.5 * erf(w2))
-    np.testing.assert_allclose(call, want, rtol=1e-11, atol=1e-11)
+    n = 200
+    p, s, t = rng.uniform(10, 50, n), rng.uniform(10, 50, n), rng.uniform(1, 2, n)
+    r, sigma = 0.1, 0.2
+    call, put = orc.black_scholes(p, s, t, r, sigma)
+    with mpmath.workdps(40):
+        rr, sg = mpmath.mpf(r), mpmath.mpf(sigma)
+        for i in range(n):
+            s0, k, tt = mpmath.mpf(float(p[i])), mpmath.mpf(float(s[i])), mpmath.mpf(float(t[i]))
+            d1 = (mpmath.log(s0 / k) + (rr + sg * sg / 2) * tt) / (sg * mpmath.sqrt(tt))
+            d2 = d1 - sg * mpmath.sqrt(tt)
+            disc = k * mpmath.exp(-rr * tt)
+            c = s0 * mpmath.ncdf(d1) - disc * mpmath.ncdf(d2)
+            q = disc * mpmath.ncdf(-d2) - s0 * mpmath.ncdf(-d1)
+            scale = max(float(s0), float(k))
+            assert abs(float(call[i]) - float(c)) <= 1e-13 * scale, (i, float(call[i]), float(c))
+            assert abs(float(put[i]) - float(q)) <= 1e-13 * scale, (i, float(put[i]), float(q))
+    # deep in and out of the money, where one of the two products dominates
+    p2, s2, t2 = np.array([1.0, 1000.0, 50.0]), np.array([1000.0, 1.0, 50.0]), np.array([0.25, 0.25, 30.0])
+    c2, q2 = orc.black_scholes(p2, s2, t2, r, sigma)
+    assert c2[0] < 1e-100 and abs(q2[0] - (1000 * math.exp(-0.025) - 1)) < 1e-9
+    assert q2[1] < 1e-100 and abs(c2[1] - (1000 - math.exp(-0.025))) < 1e-9
+
+
+def test_complex_fmax_fmin_ordering_brute_force():
+    """fmax / fmin of complex operands (dpnp/backend/kernels/elementwise_functions/fmax.hpp:57-70, fmin.hpp): the
+    first operand is kept when the second holds a NaN or when first >= second (<=) in the order of
+    math_utils.hpp:73-95.  Checked against a scalar transcription written with Python floats, on every pair of
+    a grid with signed zeros, infinities and NaN parts."""
+    vals = [0.0, -0.0, 1.0, -1.0, 2.5, np.inf, -np.inf, np.nan]
+    grid = np.array([complex(re, im) for re in vals for im in vals], dtype="c16")
+
+    def ge(x, y):  # greater_equal_complex
+        return (x.imag >= y.imag) if x.real == y.real else (x.real > y.real and not math.isnan(x.imag) and not math.isnan(y.imag))
+
+    def le(x, y):  # less_equal_complex
+        return (x.imag <= y.imag) if x.real == y.real else (x.real < y.real and not math.isnan(x.imag) and not math.isnan(y.imag))
+
+    a, b = np.meshgrid(grid, grid, indexing="ij")
+    a, b = a.ravel(), b.ravel()
+    for name, cmp in (("fmax", ge), ("fmin", le)):
+        got = orc.binary(name, a, b)
+        for x, y, g in zip(a, b, got):
+            x, y = complex(x), complex(y)
+            want = x if (math.isnan(y.real) or math.isnan(y.imag) or cmp(x, y)) else y
+            same = (g.real == want.real or (math.isnan(g.real) and math.isnan(want.real))) and \
+                   (g.imag == want.imag or (math.isnan(g.imag) and math.isnan(want.imag)))
+            assert same and math.copysign(1, g.real) == math.copysign(1, want.real) \
+                and math.copysign(1, g.imag) == math.copysign(1, want.imag), (name, x, y, g, want)
+    # the ordering functions themselves, on the same grid (less_equal / greater_equal of complex arrays)
+    for name, cmp in (("greater_equal", ge), ("less_equal", le)):
+        got = orc.binary(name, a, b)
+        assert [bool(g) for g in got] == [cmp(complex(x), complex(y)) for x, y in zip(a, b)], name
+
+
+def test_float_pow_special_values():
+    """Real pow is the C library's (pow.hpp:93-95: sycl::pow): the special values of C99 F.10.4.4, written out here,
+    and the reference's own list (dpnp/tests/test_binary_ufuncs.py:972-994: finite and infinite bases to
+    infinite exponents)."""
+    inf, nan = np.inf, np.nan
+    cases = [  # (x, y, pow(x, y))
+        (1.0, inf, 1.0), (1.0, -inf, 1.0), (2.0, inf, inf), (2.0, -inf, 0.0), (-2.0, inf, inf), (-2.0, -inf, 0.0),
+        (inf, inf, inf), (-inf, -inf, 0.0),  # the reference's list
+        (0.5, inf, 0.0), (0.5, -inf, inf), (-0.5, inf, 0.0), (-1.0, inf, 1.0), (-1.0, -inf, 1.0),
+        (nan, 0.0, 1.0), (nan, -0.0, 1.0), (1.0, nan, 1.0), (inf, 0.0, 1.0), (0.0, 0.0, 1.0),
+        (0.0, 3.0, 0.0), (-0.0, 3.0, -0.0), (-0.0, 2.0, 0.0), (0.0, -3.0, inf), (-0.0, -3.0, -inf), (-0.0, -2.0, inf),
+        (0.0, -inf, inf), (0.0, inf, 0.0),
+        (-inf, 3.0, -inf), (-inf, 2.0, inf), (-inf, -3.0, -0.0), (-inf, -2.0, 0.0), (inf, -1.0, 0.0), (inf, 0.5, inf),
+        (-8.0, 1.0 / 3, nan), (-2.0, 0.5, nan), (nan, 2.0, nan), (2.0, nan, nan),
+        (-2.0, 3.0, -8.0), (-2.0, -2.0, 0.25), (4.0, 0.5, 2.0), (10.0, -2.0, 0.01),
+    ]
+    for dt in ("f4", "f8"):
+        x = np.array([c[0] for c in cases], dtype=dt)
+        y = np.array([c[1] for c in cases], dtype=dt)
+        want = np.array([c[2] for c in cases], dtype=dt)
+        with np.errstate(all="ignore"):
+            got = orc.binary("pow", x, y)
+        assert got.dtype == np.dtype(dt)
+        for c, g, w in zip(cases, got, want):
+            if math.isnan(w):
+                assert math.isnan(g), c
+            else:
+                assert g == w and math.copysign(1, g) == math.copysign(1, w), (c, g)
 
 
 # ---- reductions ----------------------------------------------------------------------------------
