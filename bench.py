@@ -79,6 +79,11 @@ WORKLOADS = {
     "floors": "access patterns and instruction streams on their own (dpnp_amd/csrc/floors.hip), each beside the product "
               "call it bounds: Black-Scholes split into its memory streams and its arithmetic, the 2^24 read with and "
               "without a cross-block step, every-other-column reads, 512-byte runs on both sides of a transposition",
+    "survey": "functions outside the named configurations that run furthest below the HBM rate: fp64 pow / asinh / atanh / "
+              "log1p / tan over 2^26 elements, complex128 exp / sin / cos / sinh / tanh / expm1 over 2^25, float16 sin / sinh "
+              "over 2^27, column sums of a 16384x16384 int8 matrix",
+    "colsearch": "argmax and max down the columns of fp32 matrices of 2^28 elements with 128 to 4096 columns, and argmax "
+                 "along the middle axis of 65536x32x128",
     "layouts": "fp32 2^28 elements reduced over dims that do not collapse into one run: a sliced matrix summed whole, "
                "axes (0, 2) of 3-d and 4-d arrays, every other column (sum, max, mean, argmax)",
 }
@@ -261,6 +266,41 @@ def build_workload(name, dpnp, torch):
         return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
     if name == "floors":
         return build_floors(dpnp, torch, uniform, normal)
+    if name == "survey":
+        n, n2, n3 = 1 << 26, 1 << 25, 1 << 27
+        x, y, xs = uniform(n, 0.1, 10.0, torch.float64), uniform(n, -3.0, 3.0, torch.float64), uniform(n, -1.0, 1.0, torch.float64)
+        o = dpnp.empty(n, dtype="f8")
+        z = dpnp.empty(n2, dtype="c16")
+        z.real[...] = uniform(n2, -2.0, 2.0, torch.float64)
+        z.imag[...] = uniform(n2, -2.0, 2.0, torch.float64)
+        oz = dpnp.empty(n2, dtype="c16")
+        xh = dpnp.astype(uniform(n3), "f2")
+        oh = dpnp.empty(n3, dtype="f2")
+        B8 = _device_array(dpnp, torch, torch.randint(0, 100, (1 << 14, 1 << 14), device="cuda", generator=g,
+                                                      dtype=torch.int32)).astype("i1")
+        o8 = dpnp.empty(1 << 14, dtype="i8")
+        ops = [("pow_f64", lambda: dpnp.power(x, y, out=o), 24 * n, n)]
+        for fn in ("arcsinh", "arctanh", "log1p", "tan"):
+            ops.append((f"{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))
+        for fn in ("exp", "sin", "cos", "sinh", "tanh", "expm1"):
+            ops.append((f"{fn}_c128", lambda f=getattr(dpnp, fn): f(z, out=oz), 32 * n2, n2))
+        for fn in ("sin", "sinh"):
+            ops.append((f"{fn}_f16", lambda f=getattr(dpnp, fn): f(xh, out=oh), 4 * n3, n3))
+        ops.append(("sum_axis0_int8_16384sq", lambda: dpnp.sum(B8, axis=0, out=o8), 1 << 28, 1 << 28))
+        return ops, "f64/c128/f16/i8", "synthetic (seeded uniform, resident in HBM)"
+    if name == "colsearch":
+        n = 1 << 28
+        ops, keep = [], []
+        A = normal((1 << 14, 1 << 14))
+        for cols in (128, 256, 512, 1024, 4096):
+            M = A.reshape(n // cols, cols)
+            oi, of = dpnp.empty(cols, dtype="i8"), dpnp.empty(cols, dtype="f4")
+            ops.append((f"argmax_axis0_{n // cols}x{cols}", lambda M=M, oi=oi: dpnp.argmax(M, axis=0, out=oi), 4 * n, n))
+            ops.append((f"max_axis0_{n // cols}x{cols}", lambda M=M, of=of: dpnp.max(M, axis=0, out=of), 4 * n, n))
+        X = A.reshape(65536, 32, 128)
+        om = dpnp.empty((65536, 128), dtype="i8")
+        ops.append(("argmax_axis1_65536x32x128", lambda: dpnp.argmax(X, axis=1, out=om), 4 * n + 8 * 65536 * 128, n))
+        return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
     raise SystemExit(f"--workload: unknown workload {name!r} (one of {', '.join(WORKLOADS)})")
 
 

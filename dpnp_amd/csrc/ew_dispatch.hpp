@@ -30,6 +30,9 @@ template <class Op> struct op_two_packs : std::false_type {};
 #define DPX_TWO_PACKS(OP) \
     template <> struct op_two_packs<OP> : std::true_type {};
 DPX_TWO_PACKS(Expm1Op) DPX_TWO_PACKS(Log2Op) DPX_TWO_PACKS(SinhOp) DPX_TWO_PACKS(TanhOp)
+// (pow of doubles: a table look-up that waits for the base sits in every element's chain; a second pack per
+// thread keeps the memory system busy meanwhile)
+DPX_TWO_PACKS(PowOp)
 #undef DPX_TWO_PACKS
 template <class Op, class T> struct UnaryFn {
     static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
@@ -44,6 +47,7 @@ template <class Op, class T> struct UnaryFn {
 template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
 template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct BinaryFn {
+    static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
     static constexpr bool two_phase = op_two_phase<Op, T>::value;
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
     DPX_D auto fast(V<T> a, V<T> b) const { return Op::template fast<T>(a, b); }

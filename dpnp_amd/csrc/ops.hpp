@@ -8,6 +8,7 @@
 #pragma once
 #include "types.hpp"
 #include "erf_table.hpp"
+#include "pow_log_table.hpp"
 
 namespace dpx {
 
@@ -596,6 +597,83 @@ DPX_D float pow_f32(float x, float y)
     return (r != r) ? ::powf(x, y) : r;
 }
 
+// ---- fp64 pow ------------------------------------------------------------------------------------
+// pow of the device library runs at 37 % of the HBM rate (2^26 doubles, 24 bytes per element).  For a
+// positive normal base and a finite exponent whose result is far from the ends of the normal range,
+// x^y = exp(y log x) is evaluated here with the logarithm carried as a sum of two doubles:
+//  * log x = k ln 2 + log c + log1p(r): the mantissa z of x (scaled into [0.705, 1.41), so that k = 0 around 1)
+//    falls into one of 128 intervals (pow_log_table.hpp, 16 bytes per interval: 1/c as a float, log c as a
+//    double that is a multiple of 2^-42 and a float for the rest, 1/c chosen so that this rest is below 2^-54);
+//    r = z / c - 1 is formed without error as (z * invc - 1) + the product's rounding error (|r| <= 2^-8);
+//    k LN2_HI + log c is exact (both multiples of 2^-42), the sums with r and with -r^2/2 keep their
+//    rounding errors (the larger term first), and r^3/3 - ... - r^8/8 follows in plain arithmetic.
+//    Relative error of the logarithm about 2^-66, also next to x = 1, where the interval around 1 has
+//    c = 1 and log c = 0;
+//  * t = y log x as a product of the two-term logarithm with y, again in two terms;
+//  * exp t = 2^n exp(f), n = rint(t / ln 2), f = t - n ln 2 in two steps plus the low term of t, |f| <= 0.35,
+//    Taylor polynomial of degree 13.
+// Measured on the host against long double powl over 2.8e7 arguments (ordinary ranges, |t| up to 690, bases
+// within 0.03 and within a few thousand ULP of 1 with huge exponents, every binade, interval edges, integer
+// exponents): mean 0.26, worst 1.71 ULP.  About 85 vector instructions and one 16-byte table look-up per element.
+// Straight-line code: NaN where it does not apply (pow_f64 then asks the device library).
+DPX_D double pow_f64_fast(double x, double y)
+{
+    auto K = [](double v) { return scalar_const(v); };
+    constexpr double LN2_HI = 0x1.62e42fefa3800p-1, LN2_LO = 0x1.ef35793c76730p-45, LOG2E = 0x1.71547652b82fep+0;
+    const uint64_t ix = (uint64_t)__double_as_longlong(x), tmp = ix - POW_LOG_OFF;
+    const int i = (int)((tmp >> 45) & 127);
+    const double kd = (double)(int)((int64_t)tmp >> 52);
+    const double z = __longlong_as_double((long long)(ix - (tmp & (0xfffull << 52))));
+    const pow_log_entry ent = pow_log_table[i]; // one 16-byte look-up
+    const double invc = (double)ent.invc, logc = ent.logc, logctail = (double)ent.logctail;
+    const double ph = z * invc, r_lo = __builtin_fma(z, invc, -ph); // z * invc = ph + r_lo exactly
+    const double r = ph - 1.0;                                       // exact: ph lies within 2^-8 of 1
+    const double t1 = __builtin_fma(kd, K(LN2_HI), logc);            // exact
+    const double t2 = t1 + r;
+    const double lo1 = __builtin_fma(kd, K(LN2_LO), logctail);
+    const double lo2 = t1 - t2 + r; // |t1| >= |r| or t1 == 0: the sum's rounding error
+    const double ar = -0.5 * r, ar2 = r * ar, ar3 = r * ar2;
+    const double hi = t2 + ar2;
+    const double lo3 = __builtin_fma(ar, r, -ar2);
+    const double lo4 = t2 - hi + ar2;
+    double q = __builtin_fma(r, K(1.0 / 4), K(-2.0 / 7));
+    q = __builtin_fma(r, q, K(1.0 / 3));
+    q = __builtin_fma(r, q, K(-2.0 / 5));
+    q = __builtin_fma(r, q, K(1.0 / 2));
+    q = __builtin_fma(r, q, K(-2.0 / 3));
+    const double lo = lo1 + lo2 + lo3 + lo4 + __builtin_fma(-r, r_lo, r_lo) + ar3 * q;
+    const double lhi = hi + lo, llo = hi - lhi + lo;
+    const double ehi = y * lhi, elo = __builtin_fma(y, llo, __builtin_fma(y, lhi, -ehi));
+    const double ec = __builtin_fmin(__builtin_fmax(ehi, -745.0), 745.0); // keeps the conversion of n in range
+    const double n = __builtin_rint(ec * K(LOG2E));
+    double f = __builtin_fma(-n, K(LN2_HI), ec);
+    f = __builtin_fma(-n, K(LN2_LO), f);
+    f += elo;
+    double p = K(1.0 / 6227020800.0);
+    p = __builtin_fma(p, f, K(1.0 / 479001600.0));
+    p = __builtin_fma(p, f, K(1.0 / 39916800.0));
+    p = __builtin_fma(p, f, K(1.0 / 3628800.0));
+    p = __builtin_fma(p, f, K(1.0 / 362880.0));
+    p = __builtin_fma(p, f, K(1.0 / 40320.0));
+    p = __builtin_fma(p, f, K(1.0 / 5040.0));
+    p = __builtin_fma(p, f, K(1.0 / 720.0));
+    p = __builtin_fma(p, f, K(1.0 / 120.0));
+    p = __builtin_fma(p, f, K(1.0 / 24.0));
+    p = __builtin_fma(p, f, K(1.0 / 6.0));
+    p = __builtin_fma(p, f, 0.5);
+    p = __builtin_fma(p, f, 1.0);
+    p = __builtin_fma(p, f, 1.0);
+    const double res = __builtin_amdgcn_ldexp(p, (int)n);
+    // +normal base, finite exponent, result well inside the normal range; NaN in ehi fails the comparison
+    const bool own = __builtin_amdgcn_class(x, 0x100) && __builtin_amdgcn_class(y, 0x1f8) && __builtin_fabs(ehi) < 700.0;
+    return own ? res : (double)__builtin_nanf("");
+}
+DPX_D double pow_f64(double x, double y)
+{
+    const double r = pow_f64_fast(x, y);
+    return (r != r) ? ::pow(x, y) : r;
+}
+
 #define DPX_FP_FN2(NAME, F32, F64)                                          \
     template <class T> DPX_D T NAME(T x, T y)                               \
     {                                                                       \
@@ -603,7 +681,7 @@ DPX_D float pow_f32(float x, float y)
         else if constexpr (std::is_same_v<T, float>) return F32(x, y);      \
         else return (T)F32((float)x, (float)y);                             \
     }
-DPX_FP_FN2(m_pow, pow_f32, ::pow)
+DPX_FP_FN2(m_pow, pow_f32, pow_f64)
 DPX_FP_FN2(m_atan2, ::atan2f, ::atan2)
 DPX_FP_FN2(m_hypot, ::hypotf, ::hypot)
 DPX_FP_FN2(m_copysign, ::copysignf, ::copysign)
@@ -1118,16 +1196,22 @@ struct PowOp { // pow.hpp: ints by repeated squaring (negative exponent -> 0), f
             return m_pow(a, b);
         }
     }
-    // float and half: pow_f32_fast for the whole pack first, powf for what it leaves
-    template <class T> static constexpr bool two_phase = is_fp_v<T> && sizeof(T) <= 4;
+    // the short routine (pow_f32_fast, pow_f64_fast) for the whole pack first, the device library for what it leaves
+    template <class T> static constexpr bool two_phase = is_fp_v<T>;
     template <class T, class R> DPX_D static R fast(R a, R b)
     {
-        const R r = (R)pow_f32_fast((float)a, (float)b);
+        R r;
+        if constexpr (std::is_same_v<R, double>) r = pow_f64_fast(a, b);
+        else r = (R)pow_f32_fast((float)a, (float)b);
         return b == R(2) ? a * a : r; // squares as in apply()
     }
     template <class T, class R> DPX_D static bool cheap_applies(R, R b) { return b == R(2); }
     template <class T, class R> DPX_D static R cheap(R a, R) { return a * a; }
-    template <class T, class R> DPX_D static R fixup(R r, R a, R b) { return (r != r) ? (R)::powf((float)a, (float)b) : r; }
+    template <class T, class R> DPX_D static R fixup(R r, R a, R b)
+    {
+        if constexpr (std::is_same_v<R, double>) return (r != r) ? ::pow(a, b) : r;
+        else return (r != r) ? (R)::powf((float)a, (float)b) : r;
+    }
 };
 struct Atan2Op {
     template <class T> static constexpr bool ok = is_fp_v<T>;

@@ -138,6 +138,60 @@ def test_narrow_integer_division_every_pair(op):
         assert_same(host(getattr(dpt, op)(dev(a), dev(b))), orc.binary(op, a, b))
 
 
+def test_float64_pow_over_the_whole_range():
+    """pow of doubles takes the library's own routine (two-term logarithm from a 128-interval table, pow_f64_fast)
+    for a positive normal base with a finite exponent and |y log x| < 700, the device library's otherwise.  Against
+    an 80-bit evaluation: ordinary arguments, results up to the ends of that range, bases next to 1 with huge
+    exponents (where the logarithm's relative error is multiplied by up to 2^10), every binade of the base, the
+    edges of the table's intervals, integer exponents; then what the routine leaves to the device library."""
+    rng = np.random.default_rng(29)
+    n = 120000
+    parts = []
+    parts.append((rng.uniform(0.1, 10, n), rng.uniform(-3, 3, n)))
+    x = np.exp(rng.uniform(-700, 700, n))
+    parts.append((x, rng.uniform(-1, 1, n) * 690 / np.maximum(np.abs(np.log(x)), 1e-3)))
+    x = 1 + rng.uniform(-0.015, 0.015, n)
+    parts.append((x, rng.uniform(-1, 1, n) * 600 / np.maximum(np.abs(np.log(x)), 1e-300)))
+    x = (np.float64(1).view("i8") + rng.integers(-2000, 2000, n)).view("f8")  # a few thousand ULP around 1
+    lg = np.log1p(x - 1)
+    y = np.where(lg != 0, rng.uniform(-1, 1, n) * 690 / np.where(lg != 0, lg, 1), rng.uniform(-1e18, 1e18, n))
+    parts.append((x, y))
+    parts.append((np.ldexp(rng.uniform(0.5, 1.5, n), rng.integers(-1020, 1020, n)), rng.uniform(-0.65, 0.65, n)))
+    edge = 0.705078125 * (1 + rng.uniform(-5e-7, 5e-7, n)) * rng.choice([1.0, 2.0], n)
+    parts.append((edge, rng.uniform(-50, 50, n)))
+    parts.append((rng.uniform(1, 2, n), rng.integers(-100, 100, n).astype("f8")))
+    x = np.concatenate([p[0] for p in parts])
+    y = np.concatenate([p[1] for p in parts])
+    got = host(dpt.pow(dev(x), dev(y)))
+    with np.errstate(all="ignore"):
+        exact = np.power(x.astype(np.longdouble), y.astype(np.longdouble))
+        t = y * np.log(x)
+    own = np.abs(t) < 699
+    assert own.sum() > 0.95 * x.size
+    assert_ulp(got[own], exact[own], 2.0)   # measured on the host: mean 0.26, worst 1.71 ULP
+    rest = ~own & np.isfinite(exact.astype("f8")) & (np.abs(exact) > 1e-300)
+    assert_ulp(got[rest], exact[rest], 2.0)  # the device library's pow
+    assert float(dpt.pow(dev(np.array([1.0])), dev(np.array([5.0])))[0]) == 1.0
+    assert_same(host(dpt.pow(dev(np.array([2.0, 4.0, 10.0, 7.0])), dev(np.array([3.0, 0.5, -2.0, 0.0])))),
+                np.array([8.0, 2.0, 0.01, 1.0]))
+    # the special values of C's pow, negative bases, subnormals, overflow and underflow: what the routine declines
+    sp = [0.0, -0.0, 1.0, -1.0, 2.0, -2.0, 0.5, -0.5, np.inf, -np.inf, np.nan, 5e-324, -5e-324, 1e-310, 1e308, -8.0, 3.0]
+    sx, sy = (g.ravel() for g in np.meshgrid(np.array(sp), np.array(sp + [1 / 3, 1e3, -1e3, 2.0 ** 60]), indexing="ij"))
+    with np.errstate(all="ignore"):
+        want = np.power(sx, sy)
+    g = host(dpt.pow(dev(sx), dev(sy)))
+    fin = np.isfinite(want) & (want != 0)
+    assert np.array_equal(np.isnan(g), np.isnan(want)) and np.array_equal(g[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+    assert np.array_equal(np.signbit(g[~np.isnan(want)]), np.signbit(want[~np.isnan(want)]))
+    assert_ulp(g[fin], np.power(sx[fin].astype(np.longdouble), sy[fin].astype(np.longdouble)), 2.0)
+    # the strided and the transposing kernels evaluate element by element: the same values
+    assert_same(host(dpt.pow(dev(x)[::2], dev(y)[::2])), got[::2])
+    xm, ym = x[:160000].reshape(400, 400), y[:160000].reshape(400, 400)
+    assert_same(host(dpt.pow(dev(xm).T, dev(ym).T, order="C")), got[:160000].reshape(400, 400).T)
+    # a scalar exponent (broadcast operand)
+    assert_same(host(dpt.pow(dev(x[:5000]), 1.75)), host(dpt.pow(dev(x[:5000]), dev(np.full(5000, 1.75)))))
+
+
 def test_float32_pow_over_the_whole_range():
     """pow of floats takes the library's own routine for a positive normal base with a finite exponent and
     a normal result, the device library's otherwise: every binade of the base, exponents that overflow,
