@@ -287,6 +287,9 @@ def build_workload(name, dpnp, torch):
         for fn in ("sin", "sinh"):
             ops.append((f"{fn}_f16", lambda f=getattr(dpnp, fn): f(xh, out=oh), 4 * n3, n3))
         ops.append(("sum_axis0_int8_16384sq", lambda: dpnp.sum(B8, axis=0, out=o8), 1 << 28, 1 << 28))
+        # the real functions the complex ones are built from (only with --ops: for instruction counts)
+        for fn in ("exp", "sin", "cos", "sinh", "cosh", "expm1", "log"):
+            ops.append((f"ref:{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))
         return ops, "f64/c128/f16/i8", "synthetic (seeded uniform, resident in HBM)"
     if name == "colsearch":
         n = 1 << 28
@@ -424,7 +427,7 @@ def measure(name, dpnp, torch, steps, warmup, prime, ops_filter=None, dump=False
 
     def select(all_ops):
         if ops_filter is None:
-            return [o for o in all_ops if o[0] != "copy"]
+            return [o for o in all_ops if o[0] != "copy" and not o[0].startswith("ref:")]
         wanted = [w for w in ops_filter.split(",") if w]
         sel = [o for o in all_ops if o[0] in wanted]
         if not sel or len(sel) != len(wanted):

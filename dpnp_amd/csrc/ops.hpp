@@ -415,6 +415,9 @@ DPX_D void sincos_both_f64(double x, double &sn, double &cs)
 {
     const double a = __builtin_fabs(x);
     if (!(a < TRIG_FAST_LIMIT)) {
+        // (a statement the compiler may not execute speculatively: without it both device-library routines, about
+        // 160 vector instructions, were evaluated for every element ahead of this test and their results selected)
+        asm volatile("" ::: "memory");
         sn = ::sin(x);
         cs = ::cos(x);
         return;
@@ -713,26 +716,56 @@ template <class R> DPX_D void m_sincos(R x, R &s, R &c)
     else ::sincosf(x, &s, &c);
 }
 
+// In the complex functions below every real function is evaluated ONCE, ahead of the case analysis, and the
+// cases only choose among products of the values: written with the calls inside the branches (sin y and cos y of
+// the finite case, again in the cases of an infinite real part), the compiler moved the branches' calls in front
+// of the case analysis and kept the finite case's own copy, so that every element paid for sin and cos twice
+// (complex128 exp: 257 vector instructions per element, 108 for the function on its own).
+
+// sinh and cosh of one argument from one expm1 (the forms of sinh_via and cosh_via above): t = expm1(|x|),
+// w = t + 1 = exp(|x|), sinh = (t + t/w)/2, cosh = (w + 1/w)/2.  Host check against long double over 2e7
+// arguments: sinh 1.9, cosh 1.3 ULP.
+template <class R> DPX_D void m_sinhcosh(R x, R &sh, R &ch)
+{
+    if constexpr (std::is_same_v<R, double>) {
+        const R a = __builtin_fabs(x);
+        if (!(a <= R(709))) { // rare: where exp overflows and the functions do not yet, infinities, NaN
+            asm volatile("" ::: "memory"); // (not to be executed speculatively, see sincos_both_f64)
+            sh = sinh_f64(x);
+            ch = cosh_f64(x);
+            return;
+        }
+        const R t = ::expm1(a), w = t + R(1);
+        const R rc = div_moderate<R>(R(1), w), q = t * rc;
+        R s = R(0.5) * ((a < R(1)) ? R(2) * t - t * q : t + q);
+        s = (a == R(0)) ? a : s;
+        sh = __builtin_copysign(s, x);
+        ch = R(0.5) * w + R(0.5) * rc;
+    }
+    else {
+        sh = m_sinh(x);
+        ch = m_cosh(x);
+    }
+}
+
 // exp with the non-finite cases of libtensor/include/kernels/elementwise_functions/exp.hpp:75-132
 template <class R> DPX_D cplx<R> c_exp(cplx<R> z)
 {
     const R x = z.re, y = z.im;
+    R sn, cs;
+    m_sincos(y, sn, cs);
+    const R e = m_exp(x);
+    const bool xf = m_finite(x), yf = m_finite(y);
+    if (xf && yf) return (y == R(0)) ? cplx<R>{e, y} : cplx<R>{e * cs, e * sn};
     const R q_nan = (R)__builtin_nanf("");
-    if (m_finite(x)) {
-        if (!m_finite(y)) return {q_nan, q_nan};
-        const R e = m_exp(x);
-        if (y == R(0)) return {e, y};
-        R sn, cs;
-        m_sincos(y, sn, cs);
-        return {e * cs, e * sn};
-    }
+    if (xf) return {q_nan, q_nan};
     if (x != x) return (y == R(0)) ? z : cplx<R>{x, q_nan};
     if (!m_signbit(x)) { // +inf
         if (y == R(0)) return {x, y};
-        if (m_finite(y)) return {x * m_cos(y), x * m_sin(y)};
+        if (yf) return {x * cs, x * sn};
         return {x, q_nan};
     }
-    if (m_finite(y)) return {R(0) * m_cos(y), R(0) * m_sin(y)}; // exp(-inf) = 0
+    if (yf) return {R(0) * cs, R(0) * sn}; // exp(-inf) = 0
     return {R(0), R(0)};
 }
 // 2^z = exp(z ln 2) (exp2.hpp:75-133)
@@ -743,26 +776,31 @@ template <class R> DPX_D cplx<R> c_exp2(cplx<R> z)
     if (t.re != t.re && t.im == R(0)) return z; // the reference hands back its argument here
     return c_exp(t);
 }
-// expm1(x + iy) = expm1(x) cos y - 2 sin^2(y/2) + i exp(x) sin y (expm1.hpp:75-138)
+// expm1(x + iy) = expm1(x) cos y - 2 sin^2(y/2) + i exp(x) sin y (expm1.hpp:75-138), with
+// 2 sin^2(y/2) = 1 - cos y = sin^2 y / (1 + cos y): the quotient where cos y >= 0 (no cancellation), the
+// difference elsewhere
 template <class R> DPX_D cplx<R> c_expm1(cplx<R> z)
 {
     const R x = z.re, y = z.im;
+    R sn, cs;
+    m_sincos(y, sn, cs);
+    const R t = m_expm1(x), e = m_exp(x);
     const R q_nan = (R)__builtin_nanf("");
+    const bool yf = m_finite(y);
     if (m_isinf(x)) {
         if (x > R(0)) {
-            if (!m_finite(y)) return {x, q_nan};
+            if (!yf) return {x, q_nan};
             if (y == R(0)) return z;
-            return {m_copysign(x, m_cos(y)), m_copysign(x, m_sin(y))};
+            return {m_copysign(x, cs), m_copysign(x, sn)};
         }
-        if (!m_finite(y)) return {R(-1), m_copysign(R(0), y)};
-        return {R(-1), m_copysign(R(0), m_sin(y))};
+        if (!yf) return {R(-1), m_copysign(R(0), y)};
+        return {R(-1), m_copysign(R(0), sn)};
     }
     if (x != x) return (y == R(0)) ? z : cplx<R>{q_nan, q_nan};
     if (x == R(0) && y == R(0)) return {R(0), y};
-    const R cy = m_cos(y);
-    const R sy = (y == R(0)) ? y : m_sin(y);
-    const R sh = (y == R(0)) ? y : m_sin(y / R(2));
-    return {m_expm1(x) * cy - R(2) * sh * sh, m_exp(x) * sy};
+    const R h = (cs >= R(0)) ? div_moderate<R>(sn * sn, R(1) + cs) : R(1) - cs; // NaN y: NaN either way
+    const R sy = (y == R(0)) ? y : sn;
+    return {t * cs - h, e * sy};
 }
 template <class R> DPX_D cplx<R> c_log(cplx<R> z) { return {m_log(m_hypot(z.re, z.im)), m_atan2(z.im, z.re)}; }
 // log1p.hpp:75-100, log2.hpp:75-83, log10.hpp:75-84
@@ -801,61 +839,66 @@ template <class R> DPX_D cplx<R> c_sqrt(cplx<R> z)
 template <class R> DPX_D cplx<R> c_sinh(cplx<R> z)
 {
     const R x = z.re, y = z.im;
+    R sn, cs, sh, ch;
+    m_sincos(y, sn, cs);
+    m_sinhcosh(x, sh, ch);
     const bool xf = m_finite(x), yf = m_finite(y);
-    if (xf && yf) {
-        if (y == R(0)) return {m_sinh(x), y};
-        R sn, cs;
-        m_sincos(y, sn, cs);
-        return {m_sinh(x) * cs, m_cosh(x) * sn};
-    }
+    if (xf && yf) return (y == R(0)) ? cplx<R>{sh, y} : cplx<R>{sh * cs, ch * sn};
     if (x == R(0) && !yf) return {m_copysign(R(0), x * (y - y)), y - y};
     if (y == R(0) && !xf) return (x != x) ? cplx<R>{x, y} : cplx<R>{x, m_copysign(R(0), y)};
     if (xf && !yf) return {y - y, x * (y - y)};
     if (x == x) { // +-inf
         if (!yf) return {x * x, x * (y - y)};
-        return {x * m_cos(y), (R)__builtin_inff() * m_sin(y)};
+        return {x * cs, (R)__builtin_inff() * sn};
     }
     return {(x * x) * (y - y), (x + x) * (y - y)};
 }
 template <class R> DPX_D cplx<R> c_cosh(cplx<R> z)
 {
     const R x = z.re, y = z.im;
+    R sn, cs, sh, ch;
+    m_sincos(y, sn, cs);
+    m_sinhcosh(x, sh, ch);
     const R q_nan = (R)__builtin_nanf("");
     const bool xf = m_finite(x), yf = m_finite(y);
-    if (xf && yf) {
-        if (y == R(0)) return {m_cosh(x), x * y};
-        R sn, cs;
-        m_sincos(y, sn, cs);
-        return {m_cosh(x) * cs, m_sinh(x) * sn};
-    }
+    if (xf && yf) return (y == R(0)) ? cplx<R>{ch, x * y} : cplx<R>{ch * cs, sh * sn};
     if (x == R(0) && !yf) return {q_nan, m_copysign(R(0), x * q_nan)};
     if (y == R(0) && !xf) return {x * x, m_copysign(R(0), x) * y};
     if (xf && !yf) return {q_nan, x * q_nan};
     if (m_isinf(x)) {
         if (!yf) return {x * x, x * q_nan};
-        return {(x * x) * m_cos(y), x * m_sin(y)};
+        return {(x * x) * cs, x * sn};
     }
     return {(x * x) * (y - y), (x + x) * (y - y)};
 }
 template <class R> DPX_D cplx<R> c_tanh(cplx<R> z)
 {
     const R x = z.re, y = z.im;
+    // Kahan's formulation: no cancellation near the poles at x = 0, y = pi/2 + k pi.  rho = sqrt(1 + sinh^2 x) is
+    // cosh x; the sign of sin y cos y and of sin 2y, which the large and infinite cases ask for, is that of tan y
+    R t;
+    if constexpr (std::is_same_v<R, double>) {
+        // the quotient of this library's sin and cos (about 65 vector instructions; the device library's tan takes 185
+        // inside this kernel); cos y is accurate to 1.5 ULP also next to its zeros, where tan y has its poles
+        R sn, cs;
+        sincos_both_f64(y, sn, cs);
+        t = (sn == R(0)) ? sn * cs : div_moderate<R>(sn, cs); // (the short division would turn -0 into +0)
+    }
+    else t = m_tan(y);
+    R sh, rho;
+    m_sinhcosh(x, sh, rho);
     const R q_nan = (R)__builtin_nanf("");
     if (!m_finite(x)) {
         if (x != x) return {q_nan, (y == R(0)) ? y : q_nan};
-        return {m_copysign(R(1), x), m_copysign(R(0), m_isinf(y) ? y : m_sin(y) * m_cos(y))};
+        return {m_copysign(R(1), x), m_copysign(R(0), m_isinf(y) ? y : t)};
     }
     if (!m_finite(y)) return (x == R(0)) ? cplx<R>{x, q_nan} : cplx<R>{q_nan, q_nan};
-    // Kahan's formulation: no cancellation near the poles at x = 0, y = pi/2 + k pi
     const R ax = x < R(0) ? -x : x;
-    if (ax > R(20)) return {m_copysign(R(1), x), m_copysign(R(0), m_sin(y + y))};
-    const R t = m_tan(y);
+    if (ax > R(20)) return {m_copysign(R(1), x), m_copysign(R(0), t)};
     const R beta = R(1) + t * t;
-    const R sh = m_sinh(x);
-    const R rho = m_sqrt(R(1) + sh * sh);
     if (m_isinf(t)) return {rho / sh, R(1) / t};
-    const R d = R(1) + beta * sh * sh;
-    return {beta * rho * sh / d, t / d};
+    const R rd = div_moderate<R>(R(1), R(1) + beta * sh * sh);
+    return {(beta * rho * sh) * rd, t * rd};
 }
 // sin z = -i sinh(iz), cos z = cosh(iz), tan z = -i tanh(iz)
 template <class R> DPX_D cplx<R> c_sin(cplx<R> z)
