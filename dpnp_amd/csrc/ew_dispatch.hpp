@@ -30,6 +30,9 @@ template <class Op> struct op_two_packs : std::false_type {};
 #define DPX_TWO_PACKS(OP) \
     template <> struct op_two_packs<OP> : std::true_type {};
 DPX_TWO_PACKS(Expm1Op) DPX_TWO_PACKS(Log2Op) DPX_TWO_PACKS(SinhOp) DPX_TWO_PACKS(TanhOp)
+// (log1p and the inverse hyperbolic functions through it: a table look-up that waits for the argument sits in
+// the element's chain, a wave with one pack spends most of its life waiting)
+DPX_TWO_PACKS(Log1pOp) DPX_TWO_PACKS(AsinhOp) DPX_TWO_PACKS(AcoshOp) DPX_TWO_PACKS(AtanhOp)
 // (pow of doubles: a table look-up that waits for the base sits in every element's chain; a second pack per
 // thread keeps the memory system busy meanwhile)
 DPX_TWO_PACKS(PowOp)
