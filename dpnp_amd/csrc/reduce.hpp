@@ -1939,56 +1939,85 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
                 zero |= slot_publish(pidx + (int64_t)split * L.m + out0 + e, bidx[e]);
             }
     }
-    if (!last_block_of(counters + (outer * L.col_blocks + cb), L.splits, zero)) return;
     // pass two, as in red_cols_kernel: threads side by side along the block's outputs read consecutive partial
     // pairs; with fewer outputs than threads, `parts` threads share a column and meet in LDS.  (arg_merge takes the
     // better value and, of equal ones, the smaller position: the order of the merges does not matter.)
+    // With many blocks per output (tgroup != 0) the pass has two levels: the last block of every group of
+    // RED_TGROUP splits folds the group's pairs and leaves the result in the place of the group's first split,
+    // and the last of those blocks folds the groups' results.  One block folding 512 pairs per column took
+    // 35 us of a 200 us launch (2^21 x 128 floats), a chain of 16 round trips to memory per thread.
     const int NT = (int)blockDim.x, t = (int)threadIdx.x;
     const int last = ix.nd_i - 1;
     const int64_t ocol0 = cb * TX * E;
     const int ncol = (int)((L.inner - ocol0 < (int64_t)TX * E) ? L.inner - ocol0 : (int64_t)TX * E);
     const int64_t slot0 = outer * L.inner + ocol0;
-    auto fold_from = [&](int c, int first, int step, VT &b, int64_t &bi) {
+    // pairs first, first + step, ... of the `count` pairs of column c that stand `scale` splits apart from `base`
+    auto fold_from = [&](int c, int base, int count, int scale, int first, int step, VT &b, int64_t &bi) {
         constexpr int FU = sizeof(T) > 8 ? 8 : 16; // pairs in flight: a thread's share is a chain of round trips
         b = VT{};
         bi = ARG_NONE;
+        auto at = [&](int g) { return (int64_t)(base + g * scale) * L.m + slot0 + c; };
         int g = first;
-        for (; g + (FU - 1) * step < L.splits; g += FU * step) {
+        for (; g + (FU - 1) * step < count; g += FU * step) {
             T wv[FU];
             int64_t wi[FU];
 #pragma unroll
             for (int u = 0; u < FU; ++u) {
-                wv[u] = slot_read(pval + (int64_t)(g + u * step) * L.m + slot0 + c);
-                wi[u] = slot_read(pidx + (int64_t)(g + u * step) * L.m + slot0 + c);
+                wv[u] = slot_read(pval + at(g + u * step));
+                wi[u] = slot_read(pidx + at(g + u * step));
             }
 #pragma unroll
             for (int u = 0; u < FU; ++u) arg_merge<IS_MAX, VT>(b, bi, to_value(wv[u]), wi[u]);
         }
-        for (; g < L.splits; g += step)
-            arg_merge<IS_MAX, VT>(b, bi, to_value(slot_read(pval + (int64_t)g * L.m + slot0 + c)),
-                                  slot_read(pidx + (int64_t)g * L.m + slot0 + c));
+        for (; g < count; g += step)
+            arg_merge<IS_MAX, VT>(b, bi, to_value(slot_read(pval + at(g))), slot_read(pidx + at(g)));
     };
-    VT fb{};
-    int64_t fi = ARG_NONE;
-    if (ncol >= NT) {
-        for (int c = t; c < ncol; c += NT) {
-            fold_from(c, 0, 1, fb, fi);
-            dst[dof + (ocol0 + c) * ix.dst_str[last]] = arg_result<T>(L, fi, fb);
+    // every column of the block folded over those pairs; emit(c, value, position) in one thread per column
+    auto fold_block = [&](int base, int count, int scale, auto &&emit) {
+        VT fb{};
+        int64_t fi = ARG_NONE;
+        if (ncol >= NT) {
+            for (int c = t; c < ncol; c += NT) {
+                fold_from(c, base, count, scale, 0, 1, fb, fi);
+                emit(c, fb, fi);
+            }
+            return;
         }
+        const int parts = NT / ncol;
+        if (t < parts * ncol) fold_from(t % ncol, base, count, scale, t / ncol, parts, fb, fi);
+        __syncthreads(); // the LDS may still be read by an earlier combine
+        if (t < parts * ncol) {
+            smv[t] = fb;
+            smi[t] = fi;
+        }
+        __syncthreads();
+        if (t < ncol) {
+            for (int q = 1; q < parts; ++q) arg_merge<IS_MAX, VT>(fb, fi, smv[q * ncol + t], smi[q * ncol + t]);
+            emit(t, fb, fi);
+        }
+    };
+    auto to_dst = [&](int c, VT fb, int64_t fi) {
+        dst[dof + (ocol0 + c) * ix.dst_str[last]] = arg_result<T>(L, fi, fb);
+    };
+    unsigned *ticket = counters + (outer * L.col_blocks + cb);
+    if (L.tgroup == 0) {
+        if (!last_block_of(ticket, L.splits, zero)) return;
+        fold_block(0, L.splits, 1, to_dst);
         return;
     }
-    const int parts = NT / ncol;
-    if (t < parts * ncol) fold_from(t % ncol, t / ncol, parts, fb, fi);
-    __syncthreads(); // the LDS may still be read by the combine above
-    if (t < parts * ncol) {
-        smv[t] = fb;
-        smi[t] = fi;
-    }
-    __syncthreads();
-    if (t < ncol) {
-        for (int q = 1; q < parts; ++q) arg_merge<IS_MAX, VT>(fb, fi, smv[q * ncol + t], smi[q * ncol + t]);
-        dst[dof + (ocol0 + t) * ix.dst_str[last]] = arg_result<T>(L, fi, fb);
-    }
+    const int grp = split >> RED_TGROUP_LOG2, ngrp = (L.splits + RED_TGROUP - 1) >> RED_TGROUP_LOG2;
+    const int g_first = grp << RED_TGROUP_LOG2;
+    const int g_count = (L.splits - g_first < RED_TGROUP) ? L.splits - g_first : RED_TGROUP;
+    unsigned *gticket = counters + RED_MAX_TICKETS + ((outer * L.col_blocks + cb) * ngrp + grp) * RED_GROUP_PITCH;
+    if (!last_block_of(gticket, g_count, zero)) return;
+    zero = 0;
+    // (a thread overwrites the pair of the group's first split only after reading it: it is among those it folds)
+    fold_block(g_first, g_count, 1, [&](int c, VT fb, int64_t fi) {
+        zero |= slot_publish(pval + (int64_t)g_first * L.m + slot0 + c, to_storage<T>(fb));
+        zero |= slot_publish(pidx + (int64_t)g_first * L.m + slot0 + c, fi);
+    });
+    if (!last_block_of(ticket, ngrp, zero)) return;
+    fold_block(0, ngrp, RED_TGROUP, to_dst);
 }
 
 // Flat variant (see red_flat_kernel): the row of the extremum of every column of a row-major matrix whose rows

@@ -223,6 +223,17 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
         }
         L.vec = vec ? 1 : 0;
         rows_geometry(work, e, L.g_log2, pl.block);
+        if (L.walk && vec && pl.block == 256 && L.g_log2 == 8 && m > target && m <= 8 * target &&
+            tune_int("DPX_ROWS_G_LOG2", -1) < 0) {
+            // A walked space with more outputs than split plans have blocks: a wave's loads of one round go to
+            // runs that lie far apart, and with every output on a whole 256-thread block four times as many waves
+            // as a split plan runs stream from that many places at once (256 x 1024 x 1024 floats summed over
+            // axes 0 and 2: 74 % of the HBM rate; 128 x 2048 x 1024: 71 %).  Fewer lanes per output, for as many
+            // waves as a split plan has (4 per block, `target` blocks): 86 % and 90 %; half as many waves again
+            // lose 20 points.
+            L.g_log2 = ceil_log2(cdiv(64 * 4 * target, m));
+            pl.block = L.g_log2 >= 7 ? 1 << L.g_log2 : 256;
+        }
         const int64_t G = (int64_t)1 << L.g_log2;
         const int64_t opb = (G <= 64) ? 256 / G : 1;
         const int64_t oblocks = cdiv(m, opb);
@@ -349,6 +360,8 @@ void red_make_plan(RedPlan &pl, const dpx_array_view *src, int trailing, const d
     splits = cdiv(n, chunk);
     L.chunk = chunk;
     L.splits = (int32_t)splits;
+    // searches over few columns (many blocks per column block): the partial pairs are folded in two levels
+    L.tgroup = (arg && splits >= 64 && base_blocks * cdiv(splits, 32) <= RED_MAX_GROUPS) ? 32 : 0;
     pl.block = block;
     pl.grid = base_blocks * splits;
     pl.path = splits > 1 ? DPX_PATH_RED_COLS_SPLIT : DPX_PATH_RED_COLS;

@@ -265,6 +265,12 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.splits > 1
     p = plan_reduce("max", view([1024, 256, 1024], [1024, 1 << 20, 1]), 2, view([1024], ptr=P1))
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2 and p.vec == 1 and p.grid[0] == 1024
+    # (512 to 4096 outputs: lanes per output for as many waves as a split plan runs, not a whole 256-thread block)
+    assert p.block == 128
+    p = plan_reduce("sum", view([2048, 128, 1024], [1024, 1 << 21, 1]), 2, view([2048], ptr=P1))
+    assert p.grid[0] == 512 and p.block == 256  # a wave per output
+    p = plan_reduce("sum", view([512, 512, 1024], [1024, 1 << 19, 1]), 2, view([512], ptr=P1))
+    assert p.grid[0] == 512 and p.block == 256 and p.splits == 1  # a block per output
     # every other column summed along the rows: the lines the run touches are read as packs; every third: single
     # elements at a stride
     p = plan_reduce("sum", view([16384, 8192], [16384, 2]), 1, view([16384], ptr=P1))

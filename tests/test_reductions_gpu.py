@@ -672,6 +672,45 @@ def test_argmax_argmin_axis0_of_matrices_with_short_rows(dt):
         assert_same(dpnp.asnumpy(dpnp.nanargmin(dpnp.array(a), axis=0)), np.nanargmin(a, axis=0))
 
 
+@pytest.mark.parametrize("dt", ["i1", "i4", "f2", "f4", "f8", "c16"])
+def test_argmax_argmin_down_few_long_columns(dt):
+    # rows of 512 bytes and more, few column blocks, so many blocks per column: their (value, row) pairs are
+    # folded group by group and then across the groups.  Ties all over (the first row wins, in whichever block
+    # it lies), the extremum planted in the first and in the last block, NaNs that beat every number
+    import dpnp_amd._lib as L
+    rng = np.random.default_rng(44)
+    itemsize = np.dtype(dt).itemsize
+    for cols, rows in ((512 // itemsize, 150_000), (512 // itemsize + 3, 70_001), (1024 // itemsize, 40_000)):
+        if np.dtype(dt).kind == "c":  # (the oracle compares complex values one by one in Python)
+            rows = 4200 + rows // 100
+        a = random_array(rng, (rows, cols), dt, lo=-3, hi=3)
+        da = dev(a)
+        p = L.Plan()
+        res = dpt.empty(cols, dtype="i8")
+        L.check(L.lib.dpx_argreduce_plan(L.SEARCH_ID["argmax"], da.T._as_view(), 1, res._as_view(), p))
+        assert L.PATH_NAMES[p.path] == "red_cols_split" and p.splits >= 64, (cols, p.splits)
+        assert_same(host(dpt.argmax(da, axis=0)), orc.argreduce("argmax", a.T, 1))
+        assert_same(host(dpt.argmin(da, axis=0)), orc.argreduce("argmin", a.T, 1))
+        if np.dtype(dt).kind != "c":
+            b = a.copy()
+            b[5, 0], b[rows - 2, 1], b[rows // 2, 2] = 100, 100, 100
+            b[7, 3], b[rows - 1, 4] = -100, -100
+            db = dev(b)
+            got = host(dpt.argmax(db, axis=0))
+            assert_same(got, np.argmax(b, axis=0))
+            assert (got[0], got[1], got[2]) == (5, rows - 2, rows // 2)
+            assert_same(host(dpt.argmin(db, axis=0)), np.argmin(b, axis=0))
+        if np.dtype(dt).kind in "fc":
+            a[rng.random(a.shape) < 0.0005] = np.nan
+            a[rows // 2:, 0] = 0
+            da = dev(a)
+            assert_same(host(dpt.argmax(da, axis=0)), orc.argreduce("argmax", a.T, 1))
+            assert_same(host(dpt.argmin(da, axis=0)), orc.argreduce("argmin", a.T, 1))
+        if np.dtype(dt).kind == "f":
+            a[0, :] = 0
+            assert_same(dpnp.asnumpy(dpnp.nanargmax(dpnp.array(a), axis=0)), np.nanargmax(a, axis=0))
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 def test_statistics_over_samples_of_few_features(dt):
     # (samples, features) with few features: mean / var / std / logsumexp / hypot / nan forms over axis 0
@@ -862,6 +901,11 @@ _WALKED = [
     ((40, 3, 50, 2, 70), np.s_[:], (0, 2)),
     ((7, 3, 6, 2, 5, 70), np.s_[:], (0, 2, 4)),
     ((150000, 2, 9), np.s_[:, :, ::2], 0),
+    # more outputs than a split plan has blocks, long walked spaces: fewer lanes per output than a whole block
+    ((8, 1024, 1024), np.s_[:], (0, 2)),
+    ((8, 2048, 512), np.s_[:], (0, 2)),
+    ((8, 4096, 512), np.s_[:, :, 1:], (0, 2)),
+    ((1024, 4100), np.s_[:, ::2], 1),
 ]
 
 
