@@ -262,7 +262,11 @@ def build_workload(name, dpnp, torch):
                ("sum_axes02_128x128x128x128", lambda: dpnp.sum(X4, axis=(0, 2), out=r44), 4 * n, n),
                ("sum_every_other_column_axis1", lambda: dpnp.sum(A[:, ::2], axis=1, out=rs), 4 * n, n // 2),
                ("sum_every_other_column_axis0", lambda: dpnp.sum(A[:, ::2], axis=0, out=rh), 4 * n, n // 2),
-               ("argmax_every_other_column_axis1", lambda: dpnp.argmax(A[:, ::2], axis=1, out=ri), 4 * n, n // 2)]
+               ("argmax_every_other_column_axis1", lambda: dpnp.argmax(A[:, ::2], axis=1, out=ri), 4 * n, n // 2),
+               # (variance in one pass, float64 accumulation; the time includes the division and the rounding of
+               # the 8192 results to float32, two small launches)
+               ("var_every_other_column_axis0", lambda: dpnp.var(A[:, ::2], axis=0, out=rh), 4 * n, n // 2),
+               ("var_axes02_256x1024x1024", lambda: dpnp.var(X3s, axis=(0, 2), out=r1024), 4 * n, n)]
         return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
     if name == "floors":
         return build_floors(dpnp, torch, uniform, normal)

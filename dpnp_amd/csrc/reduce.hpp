@@ -901,8 +901,30 @@ __global__ __launch_bounds__(1024) void red_rows_kernel(RedLaunch L, const typen
         }
         else {
             const In *p = src + so;
-            for (int64_t pos = beg + lane; pos < end; pos += G)
-                acc[0] = P::combine(acc[0], P::pre(load_one(p + red_offset(ix, pos)), a));
+            if constexpr (P::kind == K_SQDEV1) {
+                // (as above: the first element of the output's reduced space is the reference of the means)
+                using A = acc_of_t<typename P::Out>;
+                a = Acc{0, in_to_acc<In, typename P::Out>(load_one(p + red_offset(ix, 0))), 0};
+                int64_t pos = beg + lane;
+                if (pos < end) {
+                    const A k = in_to_acc<In, typename P::Out>(load_one(p + red_offset(ix, pos)));
+                    A s1 = 0, s2 = 0;
+                    int64_t cnt = 0;
+                    for (; pos < end; pos += G) {
+                        const A d = in_to_acc<In, typename P::Out>(load_one(p + red_offset(ix, pos))) - k;
+                        s1 += d;
+                        s2 += d * d;
+                        cnt += 1;
+                    }
+                    const A n = (A)cnt;
+                    const A m2 = s2 - s1 * (s1 / n);
+                    acc[0] = Acc{n, (k - a.mean) + s1 / n, m2 < A(0) ? A(0) : m2};
+                }
+            }
+            else {
+                for (int64_t pos = beg + lane; pos < end; pos += G)
+                    acc[0] = P::combine(acc[0], P::pre(load_one(p + red_offset(ix, pos)), a));
+            }
         }
     }
     Acc r = P::combine(P::combine(acc[0], acc[1]), P::combine(acc[2], acc[3]));
@@ -1071,10 +1093,11 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                 // the element-wise form keeps one pack in flight: its LOADS x E separate loads and their
                 // addresses would set the register count of the whole kernel (and spill for 1-byte inputs)
                 constexpr int NL = WHOLE ? LOADS : 1;
-                if constexpr (P::kind == K_SQDEV1 && !WALK) {
+                if constexpr (P::kind == K_SQDEV1) {
                     // one-pass squared deviations down the columns, as in red_rows_kernel: per column, sums of d
                     // and d^2 with d = x - k, k the first row this thread meets; means relative to row 0 of the
-                    // reduced axis, which every thread row and block of a column reads alike
+                    // reduced space (offset 0), which every thread row and block of a column reads alike.  (Places
+                    // of a pack that are no column of the view carry numbers nobody reads.)
                     using A = acc_of_t<typename P::Out>;
                     {
                         const pack<In, E> v0 = load(p);
@@ -1084,7 +1107,9 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                     if (r < end) {
                         A k[E], s1[E], s2[E];
                         {
-                            const pack<In, E> vk = load(p + r * L.rstride);
+                            int64_t off_k = r * L.rstride;
+                            if constexpr (WALK) off_k = w.off; // (the row is met again below: d = 0)
+                            const pack<In, E> vk = load(p + off_k);
 #pragma unroll
                             for (int e = 0; e < E; ++e) {
                                 k[e] = in_to_acc<In, typename P::Out>(vk.v[e]);
@@ -1103,13 +1128,13 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                         for (; r + (NL - 1) * TY < end; r += NL * TY) {
                             pack<In, E> v[NL];
 #pragma unroll
-                            for (int u = 0; u < NL; ++u) v[u] = load(p + (r + u * TY) * L.rstride);
+                            for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
 #pragma unroll
                             for (int u = 0; u < NL; ++u) take(v[u]);
                             cnt += NL;
                         }
                         for (; r < end; r += TY) {
-                            take(load(p + r * L.rstride));
+                            take(load(p + next_row(r)));
                             cnt += 1;
                         }
                         const A n = (A)cnt;
@@ -1167,6 +1192,39 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
             };
             if (col0 + E <= L.inner) walk(std::true_type{});
             else walk(std::false_type{});
+        }
+        else if constexpr (P::kind == K_SQDEV1) {
+            // the same with one column per thread (columns at a stride, rows shorter than a pack)
+            using A = acc_of_t<typename P::Out>;
+            a[0] = Acc{0, in_to_acc<In, typename P::Out>(load_one(p)), 0};
+            if (r < end) {
+                int64_t off_k = r * L.rstride;
+                if constexpr (WALK) off_k = w.off;
+                const A k = in_to_acc<In, typename P::Out>(load_one(p + off_k));
+                A s1[2] = {A(0), A(0)}, s2[2] = {A(0), A(0)};
+                int64_t cnt = 0;
+                for (; r + (LOADS - 1) * TY < end; r += LOADS * TY) {
+                    In v[LOADS];
+#pragma unroll
+                    for (int u = 0; u < LOADS; ++u) v[u] = load_one(p + next_row(r + u * TY));
+#pragma unroll
+                    for (int u = 0; u < LOADS; ++u) {
+                        const A d = in_to_acc<In, typename P::Out>(v[u]) - k;
+                        s1[u & 1] += d;
+                        s2[u & 1] += d * d;
+                    }
+                    cnt += LOADS;
+                }
+                for (; r < end; r += TY) {
+                    const A d = in_to_acc<In, typename P::Out>(load_one(p + next_row(r))) - k;
+                    s1[0] += d;
+                    s2[0] += d * d;
+                    cnt += 1;
+                }
+                const A t1 = s1[0] + s1[1], t2 = s2[0] + s2[1], n = (A)cnt;
+                const A m2 = t2 - t1 * (t1 / n);
+                acc[0][0] = Acc{n, (k - a[0].mean) + t1 / n, m2 < A(0) ? A(0) : m2};
+            }
         }
         else {
             for (; r + (LOADS - 1) * TY < end; r += LOADS * TY) {

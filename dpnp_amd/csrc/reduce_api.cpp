@@ -97,13 +97,8 @@ static int reduce_call(int op, const dpx_array_view *src, int trailing, const dp
     if (int rc = red_validate(src, trailing, dst, aux, empty_ok, aux_dt)) return rc;
     RedPlan pl;
     red_make_plan(pl, src, trailing, dst, aux, false, itemsize_of(src->dtype), false, op == DPX_R_SQDEV_ONEPASS);
-    if (op == DPX_R_SQDEV_ONEPASS && pl.path != DPX_PATH_NOOP && pl.path != DPX_PATH_RED_ROWS &&
-        pl.path != DPX_PATH_RED_ROWS_SPLIT && pl.path != DPX_PATH_RED_SMALL &&
-        !((pl.path == DPX_PATH_RED_COLS || pl.path == DPX_PATH_RED_COLS_SPLIT) && !pl.L.walk) &&
-        !(pl.path == DPX_PATH_RED_GENERIC && pl.L.walk))
-        return fail(DPX_ERR_NOT_IMPLEMENTED,
-                    "one-pass squared deviations have no kernel for this layout (more than three reduced dims that "
-                    "stay apart, or a strided inner iteration dim): reduce with DPX_R_SUM, then DPX_R_SUMSQDEV");
+    // (one-pass squared deviations: every layout has a kernel; the plan above keeps away from the flat stream and
+    // the staged short rows, whose lanes do not know the reference the means are kept relative to)
     // bytes of one partial result (the accumulator type of the typed kernel)
     auto acc_bytes = [&]() {
         int acc = itemsize_of(dst->dtype);

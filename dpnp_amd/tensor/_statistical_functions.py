@@ -92,8 +92,8 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
             ti._full_usm_ndarray(0, res)
             tei._divide_by_scalar(src=res, scalar=div, dst=res)
         return res
-    # float64 accumulation over the last axes of a C-contiguous array, or down the columns: one pass over the input instead of the
-    # mean's pass plus the deviations' (the reference, dpnp/tensor/_statistical_functions.py:140-230, reads the
+    # float64 accumulation: one pass over the input, whatever its layout, instead of the mean's pass plus the
+    # deviations' (the reference, dpnp/tensor/_statistical_functions.py:140-230, reads the
     # input twice and a full-size temporary three times)
     # A float32 result of float32 input goes the same way: accumulated in float64 (never less accurate than the
     # float32 accumulation of the reference), then rounded; the result arrays are small.
@@ -102,14 +102,13 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
         arr = permute_dims(x, perm)
         res_shape = arr.shape[: nd - red_nd]
         res = empty(res_shape, dtype=acc_dt)
-        if tri._sqdev_onepass_takes(arr, red_nd, res):
-            tri._sqdev_onepass_over_axis(src=arr, trailing_dims_to_reduce=red_nd, dst=res)
-            tei._divide_by_scalar(src=res, scalar=div, dst=res)
-            if acc_dt != res_dt:
-                res = astype(res, res_dt, copy=False)
-            if keepdims:
-                res = _keepdims_view(res, res_shape, red_nd, perm, nd)
-            return res
+        tri._sqdev_onepass_over_axis(src=arr, trailing_dims_to_reduce=red_nd, dst=res)
+        tei._divide_by_scalar(src=res, scalar=div, dst=res)
+        if acc_dt != res_dt:
+            res = astype(res, res_dt, copy=False)
+        if keepdims:
+            res = _keepdims_view(res, res_shape, red_nd, perm, nd)
+        return res
     buf = x
     if not tri._sumsqdev_over_axis_dtype_supported(x.dtype, res_dt):
         buf = empty_like(x, dtype=res_dt)

@@ -74,13 +74,6 @@ def _sqdev_onepass_over_axis(src, trailing_dims_to_reduce, dst, sycl_queue=None,
     return _events(sycl_queue)
 
 
-def _sqdev_onepass_takes(src, trailing_dims_to_reduce, dst):
-    """Whether the one-pass kernel takes this layout (it refuses those it has no fast form for)."""
-    plan = _lib.Plan()
-    return lib.dpx_reduce_plan(_lib.REDUCE_ID["sqdev_onepass"], src._as_view(), int(trailing_dims_to_reduce),
-                               dst._as_view(), plan) == _lib.OK
-
-
 def _sqdev_onepass_dtype_supported(arg_dtype, out_dtype):
     return bool(lib.dpx_reduce_dtype_supported(_lib.REDUCE_ID["sqdev_onepass"], dtype_id(arg_dtype),
                                                dtype_id(out_dtype)))

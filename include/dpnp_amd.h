@@ -234,12 +234,11 @@ typedef enum dpx_reduce_op {
     /* sum((x - mean(x))^2) in ONE pass over the input, without a given mean: float32, float64 or an integer
      * type in, float64 out.  The reference's var reads the input for the mean, then again for the deviations
      * (dpnp/tensor/_statistical_functions.py:140-230: sum, divide, subtract, multiply, sum); this op carries
-     * (count, mean, sum of squared deviations) triples and merges them pairwise.  For reduced runs that are
-     * contiguous in memory (last axes of a C-contiguous array), for one strided reduced axis whose outputs
-     * are contiguous (axis 0 of a C-contiguous matrix) and for up to three reduced dims that stay apart
-     * with lanes along them (axes (0, 2) of a 3-d array, a sliced matrix), where it runs at the rate of
-     * sum; the remaining layouts are refused (DPX_ERR_NOT_IMPLEMENTED): reduce them with SUM, then
-     * SUMSQDEV.  dpx_reduce_plan tells which it is without launching anything. */
+     * (count, mean, sum of squared deviations) triples and merges them pairwise.  Every layout dpx_reduce
+     * takes for DPX_R_SUM is taken, at the rate of that sum: reduced runs that are contiguous in memory,
+     * columns (outputs side by side, plain or at a stride), reduced dims that stay apart.  A thread sums
+     * d and d^2 with d = x - k, k being the first element it meets; means travel relative to the first
+     * element of the output's reduced space. */
     DPX_R_SQDEV_ONEPASS,
     DPX_R_NUM_OPS
 } dpx_reduce_op;

@@ -302,10 +302,14 @@ def test_reduction_plans():
     assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 2  # lanes walk the reduced dims
     L.check(lib.dpx_reduce_plan(op, view([16384, 8192], [16384, 2]), 1, view([16384], dt=L.DOUBLE, ptr=P1), p))
     assert L.PATH_NAMES[p.path] == "red_generic"
-    assert lib.dpx_reduce_plan(op, view([8192, 16384], [2, 16384]), 1, view([8192], dt=L.DOUBLE, ptr=P1), p) \
-        == L.ERR_NOT_IMPLEMENTED  # columns side by side at a stride: no one-pass form
-    assert lib.dpx_reduce_plan(op, view([128, 128, 128, 128], [1 << 14, 1, 1 << 21, 128]), 2,
-                               view([128, 128], dt=L.DOUBLE, ptr=P1), p) == L.ERR_NOT_IMPLEMENTED
+    L.check(lib.dpx_reduce_plan(op, view([8192, 16384], [2, 16384]), 1, view([8192], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] == "red_cols_split"  # columns side by side at a stride, rows walked
+    L.check(lib.dpx_reduce_plan(op, view([3, 4, 5, 6, 7, 8], [40320, 6720, 1008, 144, 16, 1]), 5,
+                                view([3], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] == "red_generic" and p.red_nd == 5  # five reduced dims that stay apart
+    L.check(lib.dpx_reduce_plan(op, view([128, 128, 128, 128], [1 << 14, 1, 1 << 21, 128]), 2,
+                                view([128, 128], dt=L.DOUBLE, ptr=P1), p))
+    assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 2
     assert [(s, d) for s in range(14) for d in range(14) if lib.dpx_reduce_dtype_supported(op, s, d)] \
         == [(s, L.DOUBLE) for s in (L.INT8, L.UINT8, L.INT16, L.UINT16, L.INT32, L.UINT32, L.INT64, L.UINT64, L.FLOAT,
                                     L.DOUBLE)]

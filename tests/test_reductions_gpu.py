@@ -1005,6 +1005,30 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
         np.testing.assert_allclose(host(dpt.var(dev(m)[sl], dtype="f8")), _exact_var(m[sl].reshape(-1), None), rtol=1e-12)
         np.testing.assert_allclose(host(dpt.var(dev(m)[sl], axis=1, dtype="f8", correction=1)),
                                    _exact_var(m[sl], 1, 1), rtol=1e-12)
+    # columns side by side with the rows of the reduced space walked (every other column, every third, a 4-d
+    # array over axes (0, 2)), and reduced dims the kernels index one element at a time (more than three apart)
+    import dpnp_amd._lib as L
+    for sl in (np.s_[:, ::2], np.s_[:, 7::3], np.s_[::2, ::-1], np.s_[:, :3:2]):
+        v = dev(m)[sl]
+        p = L.Plan()
+        res = dpt.empty(v.shape[1], dtype="f8")
+        L.check(L.lib.dpx_reduce_plan(L.REDUCE_ID["sqdev_onepass"], v.T._as_view(), 1, res._as_view(), p))
+        assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split", "red_generic"), L.PATH_NAMES[p.path]
+        np.testing.assert_allclose(host(dpt.var(v, axis=0, dtype="f8")), _exact_var(m[sl], 0), rtol=1e-12)
+        np.testing.assert_allclose(host(dpt.var(v, axis=0, dtype="f8", correction=1)), _exact_var(m[sl], 0, 1), rtol=1e-12)
+    big = (rng.standard_normal((60013, 40)) * 2 + 1e5).astype(dt)  # columns split over blocks
+    np.testing.assert_allclose(host(dpt.var(dev(big)[:, ::2], axis=0, dtype="f8")), _exact_var(big[:, ::2], 0), rtol=1e-12)
+    np.testing.assert_allclose(host(dpt.var(dev(big)[:, ::3], axis=0, dtype="f8")), _exact_var(big[:, ::3], 0), rtol=1e-12)
+    a4 = (rng.standard_normal((12, 13, 14, 16)) * 3 - 1e4).astype(dt)
+    np.testing.assert_allclose(host(dpt.var(dev(a4), axis=(0, 2), dtype="f8")),
+                               _exact_var(a4.transpose(1, 3, 0, 2).reshape(13, 16, -1), 2), rtol=1e-12)
+    a6 = (rng.standard_normal((5, 4, 6, 3, 7, 9)) * 3 + 1e4).astype(dt)
+    for sl6, axes in ((np.s_[:, 1:, 1:, 1:, 1:, 1:], None), (np.s_[:, 1:, 1:, 1:, 1:, 1:], (1, 2, 3, 4, 5)),
+                      (np.s_[1:, :, 1:, :, 1:, :], (0, 2, 4))):
+        h6 = a6[sl6]
+        keep = [d for d in range(6) if axes is not None and d not in axes]
+        flat = h6.transpose(keep + [d for d in range(6) if d not in keep]).reshape([h6.shape[d] for d in keep] + [-1])
+        np.testing.assert_allclose(host(dpt.var(dev(a6)[sl6], axis=axes, dtype="f8")), _exact_var(flat, -1), rtol=1e-12)
     # non-finite values spread as in the two-pass form
     a = rng.standard_normal(5000).astype(dt)
     a[123] = np.nan
