@@ -381,6 +381,17 @@ class DPNPBinaryFunc:
             return out
         return _wrap(res)
 
+    def outer(self, x1, x2, out=None, where=True, order="K", dtype=None, subok=True, **kwargs):
+        """The op over all pairs (a, b), a in x1 and b in x2: result shape x1.shape + x2.shape (a broadcast call on
+        x1[..., None * x2.ndim] and x2[None * x1.ndim, ...]; DPNPBinaryFunc.outer,
+        dpnp/dpnp_algo/dpnp_elementwise_common.py:741-847)."""
+        check_supported_arrays_type(x1, x2, scalar_type=True, all_scalars=False)
+        if not (np.isscalar(x1) or np.isscalar(x2)):
+            n1, n2 = x1.ndim, x2.ndim
+            x1 = x1[(Ellipsis,) + (None,) * n2]
+            x2 = x2[(None,) * n1 + (Ellipsis,)]
+        return self.__call__(x1, x2, out=out, where=where, order=order, dtype=dtype, subok=subok, **kwargs)
+
 
 _UNARY = {
     "abs": ef.abs, "absolute": ef.abs, "negative": ef.negative, "positive": ef.positive,

@@ -61,6 +61,30 @@ def test_ufunc_keywords():
     assert_same((i ** 2).asnumpy(), np.arange(10, dtype="i4") ** 2)
 
 
+@pytest.mark.parametrize("x_shape", [(), (2,), (3, 4), (3, 4, 5)])
+@pytest.mark.parametrize("y_shape", [(), (2,), (3, 4), (3, 4, 5)])
+def test_elementwise_outer(x_shape, y_shape):
+    # (the cases of test_elemenwise_outer and test_elemenwise_outer_scalar, dpnp/tests/test_mathematical.py:2833-2862;
+    # the products and sums of two float64 numbers are exact or rounded once, alike on both sides)
+    rng = np.random.default_rng(len(x_shape) * 4 + len(y_shape))
+    a, b = rng.random(x_shape), rng.random(y_shape)
+    x, y = dpnp.asarray(a), dpnp.asarray(b)
+    for name in ("multiply", "add", "greater", "maximum"):
+        got = getattr(dpnp, name).outer(x, y)
+        want = getattr(np, name).outer(a, b)
+        assert got.shape == want.shape == tuple(x_shape) + tuple(y_shape)
+        assert_same(got.asnumpy(), want)
+    out = dpnp.empty(tuple(x_shape) + tuple(y_shape), dtype="f8")
+    assert dpnp.subtract.outer(x, y, out=out) is out
+    assert_same(out.asnumpy(), np.subtract.outer(a, b))
+    assert_same(dpnp.add.outer(x, 5).asnumpy(), a + 5)
+    assert_same(dpnp.add.outer(5, y).asnumpy(), 5 + b)
+    with pytest.raises(TypeError):
+        dpnp.add.outer(2, 3)
+    with pytest.raises(NotImplementedError):
+        dpnp.add.outer(x, y, where=False)
+
+
 def test_where():
     a = np.array([[0, 1, 2], [0, 2, 4], [0, 3, 6]])
     x = dpnp.array(a)
