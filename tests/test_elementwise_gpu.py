@@ -138,6 +138,103 @@ def test_narrow_integer_division_every_pair(op):
         assert_same(host(getattr(dpt, op)(dev(a), dev(b))), orc.binary(op, a, b))
 
 
+def test_float32_hyperbolic_functions_over_the_whole_range():
+    """float32 sinh / cosh, asinh / acosh / atanh and log1p are the library's own routines (the argument of the
+    logarithm formed in double, hardware log2 / reciprocal / rsqrt seeds).  Against a float64 evaluation: magnitudes
+    spread over every binade the function is finite on, both signs, the places where the routines change form
+    (2^-12, 1, 88, 2^30), arguments next to the ends of the domain, and the special values."""
+    rng = np.random.default_rng(31)
+    n = 400000
+    def spread(lo, hi):  # log-uniform magnitudes
+        return np.exp(rng.uniform(np.log(lo), np.log(hi), n)).astype("f4")
+    def around(c, rel=1e-3):
+        return (c * (1 + rng.uniform(-rel, rel, n // 10))).astype("f4")
+    sign = rng.choice(np.array([-1, 1], dtype="f4"), n)
+    cases = {
+        "sinh": np.concatenate([spread(1e-30, 89.4) * sign, around(1.0), around(88.0), around(2.0 ** -12)]),
+        "cosh": np.concatenate([spread(1e-30, 89.4) * sign, around(88.0), rng.uniform(-2, 2, n).astype("f4")]),
+        "asinh": np.concatenate([spread(1e-30, 3e38) * sign, spread(1e-5, 100) * sign, around(2.0 ** -12), around(2.0 ** 30)]),
+        "acosh": np.concatenate([spread(1.0, 3e38), 1 + spread(1e-7, 1.0), around(2.0 ** 30),
+                                 np.nextafter(np.float32(1), np.float32(2)) * np.ones(1, "f4")]),
+        "atanh": np.concatenate([spread(1e-30, 1.0) * sign, 1 - spread(6e-8, 0.1), around(2.0 ** -12), around(0.5)]),
+        "log1p": np.concatenate([spread(1e-30, 3e38), -spread(1e-30, 1.0), -1 + spread(6e-8, 0.1), around(2.0 ** -12),
+                                 -around(2.0 ** -12)]),
+    }
+    ref = {"sinh": np.sinh, "cosh": np.cosh, "asinh": np.arcsinh, "acosh": np.arccosh, "atanh": np.arctanh,
+           "log1p": np.log1p}
+    worst = {}
+    for name, x in cases.items():
+        x = x[np.isfinite(x)]
+        if name == "atanh":
+            x = x[np.abs(x) < 1]
+        if name == "acosh":
+            x = x[x >= 1]
+        if name == "log1p":
+            x = x[x > -1]
+        got = host(getattr(dpt, name)(dev(x)))
+        assert got.dtype == np.float32
+        with np.errstate(all="ignore"):
+            exact = ref[name](x.astype("f8"))
+        fin = np.isfinite(exact.astype("f4"))
+        assert fin.sum() > 0.99 * x.size
+        worst[name] = float(np.max(orc.ulp_error(got[fin], exact[fin])))
+        assert_same(got[~fin], exact[~fin].astype("f4"))  # overflow to infinity at the same arguments
+    assert max(worst.values()) <= 3.0, worst
+    # special values and signed zeros
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e-45, -1e-45, 1.2e-38, 3.4028235e38, -3.4028235e38,
+                   2.0, -2.0, 0.5, -0.5, 89.0, -89.0, 90.0, -90.0, 1e10, -1e10], dtype="f4")
+    for name in cases:
+        got = host(getattr(dpt, name)(dev(sp)))
+        with np.errstate(all="ignore"):
+            want = ref[name](sp.astype("f8")).astype("f4")
+        assert (np.isnan(got) == np.isnan(want)).all(), name
+        ok = ~np.isnan(want)
+        assert (np.signbit(got[ok]) == np.signbit(want[ok])).all(), name
+        inf = np.isinf(want) | (want == 0)
+        assert_same(got[inf], want[inf])
+        fin = ok & ~inf
+        assert_ulp(got[fin], ref[name](sp.astype("f8"))[fin], 3.0)
+    # float16 goes through the same routines
+    xh = rng.uniform(-8, 8, 50000).astype("f2")
+    for name in ("sinh", "cosh", "asinh"):
+        assert_ulp(host(getattr(dpt, name)(dev(xh))), ref[name](xh.astype("f8")), 1.0)
+
+
+_HALF_TABLE_OPS = ["sin", "cos", "tan", "tanh", "expm1", "log1p", "sinh", "asinh", "acosh", "atanh", "sinc", "exp"]
+
+
+@pytest.mark.parametrize("name", _HALF_TABLE_OPS)
+def test_float16_functions_through_their_table(name):
+    """Large contiguous float16 arrays go through a table of the function's 65536 results, staged in LDS; smaller
+    and strided ones, and those of cheap functions (exp here), through the plain kernel.  Every bit pattern (NaNs with their payloads, subnormals, both
+    zeros, infinities) must give the same bits both ways, whatever the alignment and the tail."""
+    fn = getattr(dpt, name)
+    every = np.arange(65536, dtype="u2")
+    small = host(fn(dev(every.view("f2")))).view("u2")   # the plain kernel: 65536 elements
+    # against the host for the numbers (the plain kernel's own accuracy tests are elsewhere: a loose bound here)
+    x = every.view("f2")
+    with np.errstate(all="ignore"):
+        ref = {"rsqrt": lambda v: 1 / np.sqrt(v), "asin": np.arcsin, "acos": np.arccos, "asinh": np.arcsinh,
+               "acosh": np.arccosh, "atanh": np.arctanh}.get(name, getattr(np, name, None))(x.astype("f8"))
+    got = small.view("f2")
+    fin = np.isfinite(ref) & np.isfinite(ref.astype("f2")) & (np.abs(ref) > 6.2e-5)
+    assert_ulp(got[fin], ref[fin], 2.0)
+    rng = np.random.default_rng(5)
+    n = (1 << 23) + 13
+    bits = np.concatenate([np.tile(every, 8), rng.integers(0, 65536, n - 8 * 65536).astype("u2")])
+    rng.shuffle(bits)
+    d = dev(bits.view("f2"))
+    for view, hv in ((d, bits), (d[1:], bits[1:]), (d[3:-2], bits[3:-2])):
+        assert view.size >= 1 << 23
+        got = host(fn(view)).view("u2")
+        assert np.array_equal(got, small[hv]), name
+    out = dpt.empty(n - 1, dtype="f2")
+    fn(d[:-1], out=out)  # into a given array
+    assert np.array_equal(host(out).view("u2"), small[bits[:-1]])
+    got = host(fn(d[::2])).view("u2")  # strided: the plain kernel
+    assert np.array_equal(got, small[bits[::2]])
+
+
 def test_float64_pow_over_the_whole_range():
     """pow of doubles takes the library's own routine (two-term logarithm from a 128-interval table, pow_f64_fast)
     for a positive normal base with a finite exponent and |y log x| < 700, the device library's otherwise.  Against
