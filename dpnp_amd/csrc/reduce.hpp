@@ -65,6 +65,7 @@ struct RedLaunch {
     int64_t units;
     int64_t wd[3], ws[3];
     int64_t istep; // walked column reductions: src stride of the inner iteration dim
+    int32_t obatch; // column searches: not 0: a block's thread rows are outer indices (see arg_cols_kernel)
 };
 
 // Position in a three-digit reduced space that moves by a fixed number of units per step: the element
@@ -1655,37 +1656,39 @@ __global__ __launch_bounds__(1024) void arg_rows_kernel(RedLaunch L, const T *sr
                 const int64_t vend = beg + ((end - beg) / E) * E;
                 const int64_t step = (int64_t)G * E;
                 int64_t pos = beg + (int64_t)lane * E;
+                auto take = [&](const pack<T, E> &v, int64_t at) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        const VT x = to_value(v.v[e]);
+                        if (arg_better<IS_MAX, VT>(x, best)) {
+                            best = x;
+                            bl = (uint32_t)(at + e - beg);
+                        }
+                    }
+                };
                 if (pos < vend) {
-                    best = to_value(load_one(p + pos));
-                    bl = (uint32_t)(pos - beg);
+                    // the lane's first element seeds the running extremum; it comes with the first round of loads
+                    // (read on its own ahead of them it was one more round trip to memory: short rows)
                     have = true;
+                    pack<T, E> v[RED_U];
+#pragma unroll
+                    for (int u = 0; u < RED_U; ++u)
+                        if (pos + u * step < vend) v[u] = load_pack<T, E>(p + pos + u * step);
+                    best = to_value(v[0].v[0]);
+                    bl = (uint32_t)(pos - beg);
+#pragma unroll
+                    for (int u = 0; u < RED_U; ++u)
+                        if (pos + u * step < vend) take(v[u], pos + u * step);
+                    pos += RED_U * step;
                 }
                 for (; pos + (RED_U - 1) * step < vend; pos += RED_U * step) {
                     pack<T, E> v[RED_U];
 #pragma unroll
                     for (int u = 0; u < RED_U; ++u) v[u] = load_pack<T, E>(p + pos + u * step);
 #pragma unroll
-                    for (int u = 0; u < RED_U; ++u)
-#pragma unroll
-                        for (int e = 0; e < E; ++e) {
-                            const VT x = to_value(v[u].v[e]);
-                            if (arg_better<IS_MAX, VT>(x, best)) {
-                                best = x;
-                                bl = (uint32_t)(pos + u * step + e - beg);
-                            }
-                        }
+                    for (int u = 0; u < RED_U; ++u) take(v[u], pos + u * step);
                 }
-                for (; pos < vend; pos += step) {
-                    pack<T, E> v = load_pack<T, E>(p + pos);
-#pragma unroll
-                    for (int e = 0; e < E; ++e) {
-                        const VT x = to_value(v.v[e]);
-                        if (arg_better<IS_MAX, VT>(x, best)) {
-                            best = x;
-                            bl = (uint32_t)(pos + e - beg);
-                        }
-                    }
-                }
+                for (; pos < vend; pos += step) take(load_pack<T, E>(p + pos), pos);
                 if (have) bidx = beg + bl;
                 for (int64_t t = vend + lane; t < end; t += G)
                     arg_merge<IS_MAX, VT>(best, bidx, to_value(load_one(p + t)), t);
@@ -1852,15 +1855,21 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
     extern __shared__ __align__(16) unsigned char smem_raw[];
     int64_t *smi = reinterpret_cast<int64_t *>(smem_raw);
     VT *smv = reinterpret_cast<VT *>(smem_raw + (size_t)blockDim.x * E * sizeof(int64_t));
-    const int TX = 1 << L.g_log2, TY = (int)blockDim.x >> L.g_log2;
-    const int tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> L.g_log2;
+    const int TX = 1 << L.g_log2, TYB = (int)blockDim.x >> L.g_log2;
+    const int tx = threadIdx.x & (TX - 1), tyb = threadIdx.x >> L.g_log2;
+    // obatch != 0 (short columns, many outer indices, one block per column block): the thread rows of a block are
+    // consecutive outer indices and a thread walks its whole column, so nothing is combined in LDS.  Four thread rows
+    // that shared columns of 32 rows spent more time meeting in LDS than reading (65536 x 32 x 128 floats along the
+    // middle axis: 61 % of the HBM rate, 65536 x 64 x 64: 44 %).
+    const bool batch = L.obatch != 0;
+    const int TY = batch ? 1 : TYB, ty = batch ? 0 : tyb; // thread rows that share a column, and this thread's
     int64_t b = blockIdx.x;
     const int64_t cb = b % L.col_blocks;
     b /= L.col_blocks;
     const int split = (int)(b % L.splits);
-    const int64_t outer = b / L.splits;
+    const int64_t outer = batch ? (b / L.splits) * TYB + tyb : b / L.splits;
     const int64_t col_first = (cb * TX + tx) * E;
-    const bool active = col_first < L.inner;
+    const bool active = col_first < L.inner && (!batch || outer < L.m / L.inner);
     // the pack that would cross the end of a row is moved back to end with it; its first `back` places belong
     // to the thread before (see red_cols_kernel)
     const int back = (active && col_first + E > L.inner && L.inner >= E) ? (int)(col_first + E - L.inner) : 0;
@@ -1914,15 +1923,26 @@ __global__ __launch_bounds__(256) void arg_cols_kernel(RedIndex ix, RedLaunch L,
                     }
                 }
             };
-            if (have) { // the first row seeds the running extremum (and is then visited once more)
-                const pack<T, E> v = load(p + r * L.rstride);
+            constexpr int NL = WHOLE ? U : 1; // the element-wise form keeps one pack in flight (registers)
+            if (have) {
+                // The first row seeds the running extremum.  It comes with the first round of loads: read on its
+                // own ahead of them it was one more round trip to memory, half as long again a life for a block
+                // whose threads meet 8 rows (argmax along the middle axis of 65536 x 32 x 128 floats: 55 % of the
+                // HBM rate where max ran at 77 %).
+                pack<T, E> v[NL];
+#pragma unroll
+                for (int u = 0; u < NL; ++u)
+                    if (r + u * TY < end) v[u] = load(p + (r + u * TY) * L.rstride);
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
-                    best[e] = to_value(v.v[e]);
+                    best[e] = to_value(v[0].v[e]);
                     bl[e] = (uint32_t)(r - beg);
                 }
+#pragma unroll
+                for (int u = 1; u < NL; ++u)
+                    if (r + u * TY < end) take(v[u], r + u * TY);
+                r += NL * TY;
             }
-            constexpr int NL = WHOLE ? U : 1; // the element-wise form keeps one pack in flight (registers)
             for (; r + (NL - 1) * TY < end; r += NL * TY) {
                 pack<T, E> v[NL];
 #pragma unroll

@@ -711,6 +711,45 @@ def test_argmax_argmin_down_few_long_columns(dt):
             assert_same(dpnp.asnumpy(dpnp.nanargmax(dpnp.array(a), axis=0)), np.nanargmax(a, axis=0))
 
 
+@pytest.mark.parametrize("dt", ["i1", "u2", "i4", "f2", "f4", "f8", "c8"])
+def test_argmax_argmin_along_a_short_middle_axis(dt):
+    # batch x (8 to 64) x features: a block takes several batch indices, a thread walks its whole column.  Ties
+    # (the first wins), NaNs, batch counts that do not fill the last block, feature counts that end inside a
+    # pack, a sliced and a transposed source, a strided result
+    import dpnp_amd._lib as L
+    rng = np.random.default_rng(45)
+    for shape in ((300, 32, 70), (1000, 8, 128), (77, 64, 33), (4099, 16, 7), (50, 40, 1030)):
+        if np.dtype(dt).kind == "c" and shape[0] > 300:
+            continue  # (the oracle compares complex values one by one in Python)
+        a = random_array(rng, shape, dt, lo=-3, hi=3)
+        da = dev(a)
+        want_max, want_min = orc.argreduce("argmax", np.moveaxis(a, 1, 2), 1), orc.argreduce("argmin", np.moveaxis(a, 1, 2), 1)
+        assert_same(host(dpt.argmax(da, axis=1)), want_max)
+        assert_same(host(dpt.argmin(da, axis=1)), want_min)
+        if np.dtype(dt).kind in "fc":
+            a[rng.random(shape) < 0.01] = np.nan
+            da = dev(a)
+            assert_same(host(dpt.argmax(da, axis=1)), orc.argreduce("argmax", np.moveaxis(a, 1, 2), 1))
+        if np.dtype(dt).kind == "f":
+            a[:, 0, :] = 0
+            assert_same(dpnp.asnumpy(dpnp.nanargmin(dpnp.array(a), axis=1)), np.nanargmin(a, axis=1))
+    a = random_array(rng, (301, 34, 72), dt, lo=-3, hi=3)
+    da = dev(a)
+    if np.dtype(dt).kind != "c":
+        assert_same(host(dpt.argmax(da[1:, 1:-1, 2:], axis=1)), np.argmax(a[1:, 1:-1, 2:], axis=1))
+        out = dpt.zeros((301, 144), dtype="i8")
+        dpt.argmin(da, axis=1, out=out[:, ::2])
+        assert_same(host(out)[:, ::2], np.argmin(a, axis=1))
+        assert (host(out)[:, 1::2] == 0).all()
+        at = np.ascontiguousarray(a.transpose(1, 0, 2))  # the same data with the short axis outermost in memory
+        assert_same(host(dpt.argmax(dpt.permute_dims(dev(at), (1, 0, 2)), axis=1)), np.argmax(a, axis=1))
+    p = L.Plan()
+    res = dpt.empty((300, 70), dtype="i8")
+    v = dpt.permute_dims(dev(random_array(rng, (300, 32, 70), dt, lo=-3, hi=3)), (0, 2, 1))
+    L.check(L.lib.dpx_argreduce_plan(L.SEARCH_ID["argmax"], v._as_view(), 1, res._as_view(), p))
+    assert L.PATH_NAMES[p.path] == "red_cols" and p.block == 256 and p.splits == 1
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 def test_statistics_over_samples_of_few_features(dt):
     # (samples, features) with few features: mean / var / std / logsumexp / hypot / nan forms over axis 0
