@@ -337,6 +337,47 @@ def test_float32_pow_over_the_whole_range():
     assert_ulp(got[ok], exact[ok], 1.0)
 
 
+def test_float16_pow_over_the_whole_range():
+    """float16 pow of contiguous operands: 2^(y log2 x) on the hardware's float log2 / exp2 for a positive finite
+    base and a finite exponent, the general routine otherwise.  Every positive base against a spread of exponents
+    (results that overflow, underflow and land in the subnormal range included), exact cases, the special values."""
+    rng = np.random.default_rng(37)
+    xs = np.arange(1, 0x7c00, dtype="u2").view("f2")              # every positive finite float16
+    x = np.tile(xs, 16)
+    y = np.concatenate([rng.uniform(-4, 4, xs.size), rng.uniform(-40, 40, xs.size), np.round(rng.uniform(-9, 9, xs.size)),
+                        rng.uniform(-1, 1, xs.size) * 24 / np.maximum(np.abs(np.log2(xs.astype("f8"))), 1e-3)]
+                       * 4).astype("f2")
+    got = host(dpt.pow(dev(x), dev(y)))
+    with np.errstate(all="ignore"):
+        exact = np.power(x.astype("f8"), y.astype("f8"))
+        want = exact.astype("f2")
+    fin = np.isfinite(want) & (want != 0)
+    assert fin.sum() > 0.5 * x.size
+    assert_ulp(got[fin], exact[fin], 0.51)
+    # overflow to infinity and underflow to zero happen at the same arguments, up to a result that sits within
+    # 1/100 ULP of the border
+    rest = ~fin
+    near = np.isfinite(exact) & ((np.abs(np.abs(exact) / 65520.0 - 1) < 1e-5) | (np.abs(np.abs(exact) / 2.0 ** -25 - 1) < 1e-5))
+    assert_same(got[rest & ~near], want[rest & ~near])
+    assert_same(host(dpt.pow(dev(np.array([2, 4, 9, 10, 0.5, 7], dtype="f2")), dev(np.array([3, 0.5, 0.5, -2, -3, 0], dtype="f2")))),
+                np.array([8, 2, 3, 0.01, 8, 1], dtype="f2"))
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, 3.0, -3.0, np.inf, -np.inf, np.nan, 6e-8, -6e-8, 65504.0,
+                   6.1e-5, 0.333, 1000.0], dtype="f2")
+    X, Y = [v.ravel() for v in np.meshgrid(sp, sp)]
+    got = host(dpt.pow(dev(X), dev(Y)))
+    with np.errstate(all="ignore"):
+        exact = np.power(X.astype("f8"), Y.astype("f8"))
+        want = exact.astype("f2")
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    np.testing.assert_array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+    assert_ulp(got[ok], exact[ok], 1.0)
+    # the strided kernel evaluates element by element with the general routine: within an ULP of it
+    a, b = rng.uniform(0.1, 8, 4000).astype("f2"), rng.uniform(-4, 4, 4000).astype("f2")
+    with np.errstate(all="ignore"):
+        assert_ulp(host(dpt.pow(dev(a)[::2], dev(b)[::2])), np.power(a[::2].astype("f8"), b[::2].astype("f8")), 1.0)
+
+
 @pytest.mark.parametrize("op", EXACT_UNARY)
 def test_unary_exact(op):
     rng = np.random.default_rng(11)
