@@ -233,6 +233,8 @@ def test_float16_functions_through_their_table(name):
     assert np.array_equal(host(out).view("u2"), small[bits[:-1]])
     got = host(fn(d[::2])).view("u2")  # strided: the plain kernel
     assert np.array_equal(got, small[bits[::2]])
+    fn(d, out=d)  # in place
+    assert np.array_equal(host(d).view("u2"), small[bits])
 
 
 def test_float64_pow_over_the_whole_range():
