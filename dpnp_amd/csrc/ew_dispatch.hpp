@@ -50,7 +50,8 @@ template <class Op, class T> struct UnaryFn {
 template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
 template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct BinaryFn {
-    static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
+    // (pow of floats as well: its table look-up sits in every element's chain like the one of doubles)
+    static constexpr bool two_packs = op_two_packs<Op>::value && (std::is_same_v<T, double> || std::is_same_v<T, float>);
     static constexpr bool two_phase = op_two_phase<Op, T>::value;
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
     DPX_D auto fast(V<T> a, V<T> b) const { return Op::template fast<T>(a, b); }

@@ -9,6 +9,7 @@
 #include "types.hpp"
 #include "erf_table.hpp"
 #include "pow_log_table.hpp"
+#include "powf_log_table.hpp"
 
 namespace dpx {
 
@@ -682,51 +683,63 @@ DPX_FP_FN1(m_sinpi, ::sinpif, ::sinpi)
 #undef DPX_FP_FN1
 // ---- fp32 pow ------------------------------------------------------------------------------------
 // powf of the device library runs at 36 % of the HBM rate (2^27 floats).  For a positive normal base
-// and a finite exponent whose result is a normal number, x^y = 2^(y log2 x) is evaluated here in
-// double precision, where 2^-45 of relative error in log2 x is cheap and leaves the float result
-// within 0.51 ULP: log2 from s = (m - 1)/(m + 1) for the mantissa m in [sqrt(1/2), sqrt(2)) and the
-// odd series 2 s (1 + s^2/3 + ... + s^14/15), 2^t from n = rint(t) and the degree-8 Taylor series of
-// 2^f on |f| <= 1/2.  About 45 vector instructions per element.  Every other argument (zero, negative,
+// and a finite exponent whose result is a normal number, x^y = 2^(y log2 x) is evaluated here in float
+// arithmetic with the logarithm carried as a sum of two floats (float instructions issue at twice the rate of
+// double ones on this GPU; the same scheme in double precision, 45 instructions, ran at 67 %):
+//  * x = 2^k m with m in [sqrt(1/2), sqrt(2)); q = rint(128 / m) from the hardware reciprocal, an integer between
+//    90 and 182, so that r = m q / 128 - 1 comes out of one fma without error and |r| < 0.0056;
+//  * log2 x = (k - log2(q/128)) + log2(1 + r): the first part from powf_log_table.hpp as {hi, lo} with hi a
+//    multiple of 2^-16, so that k + hi is exact; log2(1 + r) = r log2e (1 - r/2 + r^2/3 - r^3/4 + r^4/5) with
+//    r log2e as an exact product in two floats; the sum of the large terms keeps its rounding error.  Relative
+//    error about 2^-33, also next to x = 1 (q = 128, table entry 0);
+//  * t = y log2 x in two floats, n = rint(t), 2^f by the degree-9 Taylor series on |f| <= 1/2, ldexp.
+// Host check against double-precision pow over 2.3e7 arguments (every binade of base and result, bases within
+// 0.001 of 1 with exponents up to 3e4): mean 0.26, worst 0.97 ULP (0.89 away from such bases).  About 50 float
+// instructions, one reciprocal and one 8-byte table look-up per element.  Every other argument (zero, negative,
 // subnormal or infinite base, infinite or NaN exponent, results beyond the normal range) goes to powf.
 // The short routine: NaN where it does not apply.  Straight-line code, so that the chains of a thread's
 // elements interleave when the kernel runs it for all of them before it looks at the NaNs.
 DPX_D float pow_f32_fast(float x, float y)
 {
-    auto K = [](double c) { return scalar_const(c); };
-    double m = __builtin_amdgcn_frexp_mant((double)x); // [0.5, 1)
-    int e = __builtin_amdgcn_frexp_exp((double)x);
-    const bool low = m < 0.70710678118654752440;
-    m = low ? m + m : m;
-    e = low ? e - 1 : e;
-    const double d = m + 1.0;
-    double rc = __builtin_amdgcn_rcp(d);
-    rc = __builtin_fma(__builtin_fma(-d, rc, 1.0), rc, rc);
-    const double sr = (m - 1.0) * rc, z = sr * sr;
-    double p = __builtin_fma(z, K(1.0 / 15.0), K(1.0 / 13.0));
-    p = __builtin_fma(z, p, K(1.0 / 11.0));
-    p = __builtin_fma(z, p, K(1.0 / 9.0));
-    p = __builtin_fma(z, p, K(1.0 / 7.0));
-    p = __builtin_fma(z, p, K(1.0 / 5.0));
-    p = __builtin_fma(z, p, K(1.0 / 3.0));
-    p = __builtin_fma(z, p, 1.0);
-    // log2 x = e + (2 / ln 2) s p
-    const double l2 = __builtin_fma(sr * K(2.88539008177792681472), p, (double)e);
-    const double t = (double)y * l2;
-    const double tc = __builtin_fmin(__builtin_fmax(t, -126.0), 126.0); // keeps the conversion of n in range
-    const double n = __builtin_rint(tc), f = tc - n;
+    constexpr float LOG2E_HI = 0x1.715476p+0f, LOG2E_LO = 0x1.4ae0cp-26f;
+    const uint32_t ix = __float_as_uint(x);
+    const int32_t k = (int32_t)(ix - 0x3f3504f3u) >> 23;               // x = 2^k m
+    const float m = __uint_as_float(ix - ((uint32_t)k << 23));        // [sqrt(1/2), sqrt(2))
+    const float q = __builtin_rintf(128.0f * __builtin_amdgcn_rcpf(m)); // 90 .. 182
+    const float r = __builtin_fmaf(m, q * 0.0078125f, -1.0f);           // exact, |r| < 0.0056
+    int idx = (int)q - POWF_LOG_Q0;
+    idx = idx < 0 ? 0 : (idx > POWF_LOG_N - 1 ? POWF_LOG_N - 1 : idx);  // (arguments the routine is not for)
+    const powf_log_entry ent = powf_log_table[idx];
+    // log2(1 + r) = r log2e (1 + p), p = -r/2 + r^2/3 - r^3/4 + r^4/5
+    float p = __builtin_fmaf(r, 0.2f, -0.25f);
+    p = __builtin_fmaf(r, p, 1.0f / 3);
+    p = __builtin_fmaf(r, p, -0.5f);
+    p = p * r;
+    const float h = r * LOG2E_HI, herr = __builtin_fmaf(r, LOG2E_HI, -h);
+    const float A = (float)k + ent.hi; // exact
+    const float s = A + h;
+    const float e = h - (s - A);       // the sum's rounding error: |A| >= |h| or A == 0
+    float lo = __builtin_fmaf(h, p, __builtin_fmaf(r, LOG2E_LO, herr));
+    lo = (lo + ent.lo) + e;
+    // t = y log2 x
+    const float thi = y * s;
+    const float tlo = __builtin_fmaf(y, lo, __builtin_fmaf(y, s, -thi));
+    const float tc = __builtin_fminf(__builtin_fmaxf(thi, -126.0f), 126.0f); // keeps the conversion of n in range
+    const float n = __builtin_rintf(tc);
+    const float f = (tc - n) + tlo;
     // 2^f = sum (f ln 2)^k / k!
-    double q = __builtin_fma(f, K(1.32154867901443094884e-06), K(1.52527338040598402800e-05));
-    q = __builtin_fma(f, q, K(1.54035303933816099544e-04));
-    q = __builtin_fma(f, q, K(1.33335581464284434234e-03));
-    q = __builtin_fma(f, q, K(9.61812910762847716197e-03));
-    q = __builtin_fma(f, q, K(5.55041086648215799532e-02));
-    q = __builtin_fma(f, q, K(2.40226506959100712334e-01));
-    q = __builtin_fma(f, q, K(6.93147180559945309417e-01));
-    q = __builtin_fma(f, q, 1.0);
-    const float r = (float)__builtin_amdgcn_ldexp(q, (int)n);
-    // +normal base, finite exponent, normal result; NaN in t fails the comparison
-    const bool own = __builtin_amdgcn_classf(x, 0x100) && __builtin_amdgcn_classf(y, 0x1f8) && __builtin_fabs(t) < 126.0;
-    return own ? r : __builtin_nanf("");
+    float g = __builtin_fmaf(f, 0x1.b5253ep-24f, 0x1.62c022p-20f);
+    g = __builtin_fmaf(f, g, 0x1.ffcbfcp-17f);
+    g = __builtin_fmaf(f, g, 0x1.430912p-13f);
+    g = __builtin_fmaf(f, g, 0x1.5d87fep-10f);
+    g = __builtin_fmaf(f, g, 0x1.3b2ab6p-7f);
+    g = __builtin_fmaf(f, g, 0x1.c6b08ep-5f);
+    g = __builtin_fmaf(f, g, 0x1.ebfbep-3f);
+    g = __builtin_fmaf(f, g, 0x1.62e43p-1f);
+    const float res = __builtin_amdgcn_ldexpf(__builtin_fmaf(f, g, 1.0f), (int)n);
+    // +normal base, finite exponent, normal result; NaN in thi fails the comparison
+    const bool own = __builtin_amdgcn_classf(x, 0x100) && __builtin_amdgcn_classf(y, 0x1f8) && __builtin_fabsf(thi) < 125.5f;
+    return own ? res : __builtin_nanf("");
 }
 DPX_D float pow_f32(float x, float y)
 {

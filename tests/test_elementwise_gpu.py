@@ -292,8 +292,8 @@ def test_float64_pow_over_the_whole_range():
 
 
 def test_float32_pow_over_the_whole_range():
-    """pow of floats takes the library's own routine for a positive normal base with a finite exponent and
-    a normal result, the device library's otherwise: every binade of the base, exponents that overflow,
+    """pow of floats takes the library's own routine (float arithmetic, the logarithm in two floats from a small table)
+    for a positive normal base with a finite exponent and a normal result, the device library's otherwise: every binade of the base, exponents that overflow,
     underflow and hit the subnormal range, and the special-value table of C's pow."""
     rng = np.random.default_rng(23)
     n = 200000
@@ -306,9 +306,9 @@ def test_float32_pow_over_the_whole_range():
     got = host(dpt.pow(dev(x), dev(y)))
     with np.errstate(all="ignore"):
         exact = np.power(x.astype("f8"), y.astype("f8"))
-    own = np.abs(y.astype("f8") * np.log2(x.astype("f8"))) < 125.9   # the library's routine: normal results
+    own = np.abs(y.astype("f8") * np.log2(x.astype("f8"))) < 125.4   # the library's routine: normal results
     assert own.sum() > n // 4 and (~own).sum() > n // 10
-    assert_ulp(got[own], exact[own], 0.52)
+    assert_ulp(got[own], exact[own], 1.0)                            # (host check: mean 0.26, worst 0.97 ULP)
     assert_ulp(got[~own], exact[~own], 2.0)                          # the device library's powf
     # the strided and the transposing kernels evaluate element by element: the same values
     assert_same(host(dpt.pow(dev(x)[::2], dev(y)[::2])), got[::2])
