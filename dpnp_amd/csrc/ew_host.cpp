@@ -88,7 +88,8 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     // operands by position modulo / divided by the row length.
     if (pl.nd == 2 && pl.n < ((int64_t)1 << 32) && pl.strides[nops - 1][1] == 1 &&
         pl.strides[nops - 1][0] == pl.shape[1] &&
-        (pl.shape[1] * itemsize_of(dst->dtype) < 512 || pl.shape[1] * itemsize_of(dst->dtype) >= ((int64_t)2 << 20))) {
+        (pl.shape[1] * itemsize_of(dst->dtype) < 512 ||
+         pl.shape[1] * itemsize_of(dst->dtype) >= (int64_t)tune_int("DPX_EW_FLAT_LONG", 2 << 20))) {
         const bool long_rows = pl.shape[1] * itemsize_of(dst->dtype) >= 512;
         bool ok = true, has_row = false;
         for (int k = 0; k + 1 < nops && ok; ++k) {
@@ -149,7 +150,7 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
 {
     if (pl.path == DPX_PATH_NOOP) return;
     const int nops = pl.nops;
-    (void)ptrs, (void)itemsize; // packs need no alignment: any operand whose inner stride is 1 is read in packs
+    // (packs need no alignment: any operand whose inner stride is 1 is read in packs)
     if (pl.path == DPX_PATH_EW_CONTIG) {
         pl.vec = true;
         pl.bcast = 0;
@@ -230,6 +231,28 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     pl.modes |= keep_bits(pl);
     const int64_t per_row = (ncols + E - 1) / E; // threads wanted along a row
     pl.block = env_block("DPX_EW_ROWS_BLOCK", EW_ROWS_BLOCK);
+    {
+        // One full-size input and the output, both in aligned packs, every other input broadcast along some dim
+        // (a matrix plus a row, times a column, minus a per-channel constant): one-wave blocks, like the contiguous
+        // kernel's (fp32 16384 x 16384 plus a row or a column: 74 -> 80 % of the HBM rate).  Calls that only write
+        // (an outer sum) are bound by the rate waves are launched at and keep four waves per block; two full-size
+        // inputs gain nothing, and lose 7 points when their rows do not start on 16-byte boundaries.
+        int streaming = 0;
+        bool aligned = ((pl.modes >> (2 * (nops - 1))) & 3u) == MODE_VEC;
+        for (int k = 0; k < nops; ++k) {
+            const bool out_k = k + 1 == nops;
+            bool bcast = false;
+            for (int d = 0; d < pl.nd && !out_k; ++d) bcast = bcast || (pl.strides[k][d] == 0 && pl.shape[d] > 1);
+            if (bcast) continue;
+            if (!out_k) {
+                ++streaming;
+                aligned = aligned && ((pl.modes >> (2 * k)) & 3u) == MODE_VEC;
+            }
+            aligned = aligned && (uintptr_t)ptrs[k] % 16 == 0;
+            for (int d = 0; d < inner; ++d) aligned = aligned && (pl.strides[k][d] * itemsize[k]) % 16 == 0;
+        }
+        if (streaming == 1 && aligned && per_row >= 64 && tune_int("DPX_EW_ROWS_ONE_WAVE", 1) != 0) pl.block = 64;
+    }
     int lg = 0, lg_max = 0;
     while ((1 << lg_max) < pl.block) ++lg_max;
     while (lg < lg_max && ((int64_t)1 << lg) < per_row) ++lg;

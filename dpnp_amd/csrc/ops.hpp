@@ -1868,7 +1868,8 @@ template <bool LCM> struct GcdOp { // gcd.hpp / lcm.hpp: integers; the result is
 };
 
 // Arithmetic on operands of two different types with the conversion folded into the load:
-// (A, B) -> T where one operand already has the result type T.  The reference has same-type
+// (A, B) -> T where one operand already has the result type T, or (float32 with int32 / int64 -> float64)
+// neither has.  The reference has same-type
 // kernels only and its Python layer casts the other operand into a temporary first
 // (_find_buf_dtype2, dpnp/tensor/_type_utils.py:389-485); converting while reading gives the same
 // values without the extra pass.  f(tag<T>, tag<A>, tag<B>) is called for a supported pair.
@@ -1888,8 +1889,20 @@ template <class F> inline bool for_mixed_pair(int dt1, int dt2, F &&f)
         return true;                                        \
     }
     DPX_MIX(double, float) DPX_MIX(double, int32_t) DPX_MIX(double, int64_t) DPX_MIX(double, bool_t)
-    DPX_MIX(float, bool_t)
+    DPX_MIX(float, bool_t) DPX_MIX(float, int16_t) DPX_MIX(float, int8_t) DPX_MIX(float, uint8_t)
 #undef DPX_MIX
+    // both operands converted: float32 with a 32- or 64-bit integer gives float64
+#define DPX_MIX3(T, X, Y)                                   \
+    if (dt1 == id_of_v<X> && dt2 == id_of_v<Y>) {           \
+        f(tag<T>{}, tag<X>{}, tag<Y>{});                    \
+        return true;                                        \
+    }                                                       \
+    if (dt1 == id_of_v<Y> && dt2 == id_of_v<X>) {           \
+        f(tag<T>{}, tag<Y>{}, tag<X>{});                    \
+        return true;                                        \
+    }
+    DPX_MIX3(double, float, int32_t) DPX_MIX3(double, float, int64_t)
+#undef DPX_MIX3
     return false;
 }
 template <class Op, class T, class A, class B> struct MixedFn {

@@ -477,13 +477,14 @@ class BinaryElementwiseFunc:
                 f"function '{self.name_}' does not support input types ({d1}, {d2}), "
                 "and the inputs could not be safely coerced to any supported types according to "
                 "the casting rule ''safe''.")
-        if (buf1_dt is None) != (buf2_dt is None):
-            # "cast one operand to the result type, then compute": one kernel does both for some pairs
+        if buf1_dt is not None or buf2_dt is not None:
+            # "cast one operand (or both) to the result type, then compute": one kernel does it all for some pairs
             # (a dtype compares equal to None when it is float64, hence the explicit tests)
             fused = self._fused_cast(d1, d2)
             if fused is not None and fused == res_dt and (
-                    (buf1_dt is not None and buf1_dt == res_dt and d2 == res_dt)
-                    or (buf2_dt is not None and buf2_dt == res_dt and d1 == res_dt)):
+                    (buf1_dt is not None and buf1_dt == res_dt and buf2_dt is None and d2 == res_dt)
+                    or (buf2_dt is not None and buf2_dt == res_dt and buf1_dt is None and d1 == res_dt)
+                    or (buf1_dt is not None and buf2_dt is not None and buf1_dt == res_dt and buf2_dt == res_dt)):
                 buf1_dt = buf2_dt = None
         orig_out = out
         if out is not None:

@@ -312,13 +312,14 @@ int dpx_binary_result_type(int op, int dt1, int dt2);
 /* 1 if `lhs op= rhs` has a kernel (py_binary_inplace_ufunc's table,
  * elementwise_functions.hpp:612-650) */
 int dpx_binary_inplace_supported(int op, int lhs_dt, int rhs_dt);
-/* Result dtype of `op` for operands of two different dtypes when the conversion of one of
- * them is folded into the kernel (add, subtract, multiply, divide with one operand already of
- * the result type: float64 with float32/int32/int64/bool, float32 with bool), else -1.
+/* Result dtype of `op` for operands of two different dtypes when the conversion is folded into
+ * the kernel (add, subtract, multiply, divide with one operand already of the result type:
+ * float64 with float32/int32/int64/bool, float32 with bool/int8/uint8/int16; or with both
+ * converted: float32 with int32/int64 gives float64), else -1.
  * No counterpart in the reference, whose kernels take same-dtype pairs and whose Python layer
  * casts the other operand into a temporary first (_find_buf_dtype2,
- * dpnp/tensor/_type_utils.py:389-485): a caller that has settled on "cast operand k to T, then
- * op" may call dpx_binary / dpx_binary_inplace with the original operands instead when this
+ * dpnp/tensor/_type_utils.py:389-485): a caller that has settled on "cast operand k (or both) to
+ * T, then op" may call dpx_binary / dpx_binary_inplace with the original operands instead when this
  * returns T.  dpx_binary_result_type does not report these pairs. */
 int dpx_binary_fused_cast_result_type(int op, int dtype1, int dtype2);
 /* _sum_over_axis_dtype_supported & co., libtensor/source/reductions/sum.cpp:445-456 */

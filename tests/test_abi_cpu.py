@@ -68,7 +68,11 @@ def test_binary_result_types():
     assert lib.dpx_binary_fused_cast_result_type(B["divide"], L.INT32, L.DOUBLE) == L.DOUBLE
     assert lib.dpx_binary_fused_cast_result_type(B["multiply"], L.FLOAT, L.BOOL) == L.FLOAT
     assert lib.dpx_binary_fused_cast_result_type(B["maximum"], L.FLOAT, L.DOUBLE) == -1
-    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.INT32) == -1
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.INT32) == L.DOUBLE  # both operands converted
+    assert lib.dpx_binary_fused_cast_result_type(B["subtract"], L.INT64, L.FLOAT) == L.DOUBLE
+    assert lib.dpx_binary_fused_cast_result_type(B["multiply"], L.INT16, L.FLOAT) == L.FLOAT
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.UINT16) == -1
+    assert lib.dpx_binary_fused_cast_result_type(B["add"], L.INT32, L.INT64) == -1
     assert lib.dpx_binary_fused_cast_result_type(B["add"], L.FLOAT, L.FLOAT) == -1
     assert lib.dpx_binary_result_type(B["less"], L.INT64, L.UINT64) == L.BOOL
     assert lib.dpx_binary_result_type(B["less"], L.UINT64, L.INT64) == L.BOOL
@@ -211,6 +215,19 @@ def test_elementwise_plans():
     assert L.PATH_NAMES[p.path] == "ew_rows"
     p = plan_binary("add", view([5, 100000]), view([5, 100000], [0, 1], ptr=P1), view([5, 100000], ptr=P2))
     assert L.PATH_NAMES[p.path] == "ew_rows"  # 400 KB rows
+    # one full-size input and the output in aligned packs, the other input broadcast: one-wave blocks; an outer
+    # sum (nothing full-size is read), two full-size inputs, rows off the 16-byte grid: four waves per block
+    p = plan_binary("add", view([16384, 16384]), view([16384, 16384], [0, 1], ptr=P1), view([16384, 16384], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 64 and p.grid[0] == 16384 * 64
+    p = plan_binary("multiply", view([16384, 16384]), view([16384, 16384], [1, 0], ptr=P1), view([16384, 16384], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 64
+    p = plan_binary("add", view([16384, 16384], [0, 1]), view([16384, 16384], [1, 0], ptr=P1), view([16384, 16384], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256
+    p = plan_binary("add", view([16384, 8192], [16384, 1]), view([16384, 8192], [16384, 1], ptr=P1),
+                    view([16384, 8192], [16384, 1], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256
+    p = plan_binary("add", view([16384, 16383]), view([16384, 16383], [0, 1], ptr=P1), view([16384, 16383], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256
     # empty
     p = plan_binary("add", view([0, 3]), view([0, 3]), view([0, 3]))
     assert L.PATH_NAMES[p.path] == "noop"

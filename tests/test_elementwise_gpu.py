@@ -1065,7 +1065,8 @@ def test_extension_binary_misc():
 
 # ---- mixed-dtype arithmetic: the cast of one operand is folded into the kernel -------------------
 @pytest.mark.parametrize("op", ["add", "subtract", "multiply", "divide"])
-@pytest.mark.parametrize("pair", [("f8", "f4"), ("f8", "i4"), ("f8", "i8"), ("f8", "?"), ("f4", "?")])
+@pytest.mark.parametrize("pair", [("f8", "f4"), ("f8", "i4"), ("f8", "i8"), ("f8", "?"), ("f4", "?"), ("f4", "i2"),
+                                  ("f4", "i1"), ("f4", "u1")])
 def test_mixed_dtype_arithmetic_equals_cast_then_compute(op, pair):
     import dpnp_amd._lib as L
     from dpnp_amd.tensor._dtypes import dtype_id
@@ -1093,6 +1094,36 @@ def test_mixed_dtype_arithmetic_equals_cast_then_compute(op, pair):
     if op == "add":
         d2 += dev(b)
         assert_same(host(d2), a + b.astype(wide))
+
+
+@pytest.mark.parametrize("op", ["add", "subtract", "multiply", "divide"])
+@pytest.mark.parametrize("idt", ["i4", "i8"])
+def test_float32_with_integer_gives_float64_in_one_kernel(op, idt):
+    # float32 (op) int32 / int64 promotes to float64 (the reference casts both operands into temporaries, then
+    # computes): one kernel converts both while reading; the values are those of cast-then-compute
+    import dpnp_amd._lib as L
+    from dpnp_amd.tensor._dtypes import dtype_id
+
+    rng = np.random.default_rng(152)
+    a = random_array(rng, (37, 130), "f4", -9, 9)
+    b = random_array(rng, (37, 130), idt, -9, 9)
+    b[b == 0] = 3
+    assert L.lib.dpx_binary_fused_cast_result_type(L.BINARY_ID[op], L.FLOAT, dtype_id(np.dtype(idt))) == L.DOUBLE
+    npf = getattr(np, op if op != "divide" else "true_divide")
+    for x, y in ((a, b), (b, a)):
+        want = npf(x.astype("f8"), y.astype("f8"))
+        got = getattr(dpt, op)(dev(x), dev(y))
+        assert got.dtype == np.dtype("f8")
+        assert_same(host(got), want)
+        assert_same(host(getattr(dpt, op)(dev(x)[:, ::2], dev(y)[:, ::2])), want[:, ::2])
+        assert_same(host(getattr(dpt, op)(dev(x.T.copy()).T, dev(y))), want)
+        out = dpt.empty((37, 130), dtype="f8")
+        getattr(dpt, op)(dev(x), dev(y), out=out)
+        assert_same(host(out), want)
+        assert_same(host(getattr(dpt, op)(dev(x), dev(y[:1]))), npf(x.astype("f8"), y[:1].astype("f8")))  # a broadcast row
+    big = random_array(rng, (1 << 16,), "i8", -2 ** 62, 2 ** 62)  # integers float64 cannot hold exactly: rounded once
+    f = random_array(rng, (1 << 16,), "f4", -9, 9)
+    assert_same(host(getattr(dpt, op)(dev(big), dev(f))), npf(big.astype("f8"), f.astype("f8")))
 
 
 @pytest.mark.parametrize("dt", ["i4", "u4"])
