@@ -31,7 +31,7 @@ template <class F> static bool for_nan_pair(int op, int in_dt, int out_dt, F &&f
         DPX_PAIR(float, double)
     }
     else if (op == DPX_R_SQDEV_ONEPASS) { // (no NaN handling: it shares this file's plumbing)
-        DPX_PAIR(float, double) DPX_PAIR(double, double)
+        DPX_PAIR(float, double) DPX_PAIR(double, double) DPX_PAIR(half_t, double)
         // integers: var of an integer array is float64 (the reference casts the array first)
         DPX_PAIR(int8_t, double) DPX_PAIR(uint8_t, double) DPX_PAIR(int16_t, double) DPX_PAIR(uint16_t, double)
         DPX_PAIR(int32_t, double) DPX_PAIR(uint32_t, double) DPX_PAIR(int64_t, double) DPX_PAIR(uint64_t, double)
@@ -55,7 +55,7 @@ template <int KIND> static int nan_run_kind(int op, RedPlan &pl, const dpx_array
         // the pair lists above keep complex inputs away from the ordered and the squared-deviation kinds
         constexpr bool ok = !(is_cplx_v<I> && (kind_is_minmax(KIND) || KIND == K_NANSUMSQDEV || KIND == K_NANVAR)) &&
                             (KIND == K_NANCOUNT) == std::is_same_v<O, int64_t> &&
-                            (KIND == K_SQDEV1 ? (std::is_same_v<O, double> && !is_cplx_v<I> && !std::is_same_v<I, half_t>)
+                            (KIND == K_SQDEV1 ? (std::is_same_v<O, double> && !is_cplx_v<I>)
                                               : !std::is_integral_v<I>);
         if constexpr (ok) {
             if (acc_size) {

@@ -95,9 +95,10 @@ def _var_impl(x, axis, correction, keepdims, dtype=None):
     # float64 accumulation: one pass over the input, whatever its layout, instead of the mean's pass plus the
     # deviations' (the reference, dpnp/tensor/_statistical_functions.py:140-230, reads the
     # input twice and a full-size temporary three times)
-    # A float32 result of float32 input goes the same way: accumulated in float64 (never less accurate than the
-    # float32 accumulation of the reference), then rounded; the result arrays are small.
-    acc_dt = float64 if (x.dtype == _as_dtype("f4") and res_dt == _as_dtype("f4")) else res_dt
+    # A float32 result of float32 input (a float16 one of float16 input) goes the same way: accumulated in float64
+    # (never less accurate than the float32 / float16 accumulation of the reference, whose float16 sums overflow
+    # beyond 65504), then rounded; the result arrays are small.
+    acc_dt = float64 if (x.dtype in (_as_dtype("f4"), _as_dtype("f2")) and res_dt == x.dtype) else res_dt
     if nelems > 0 and x.size and tri._sqdev_onepass_dtype_supported(x.dtype, acc_dt):
         arr = permute_dims(x, perm)
         res_shape = arr.shape[: nd - red_nd]

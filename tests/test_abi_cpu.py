@@ -328,8 +328,8 @@ def test_reduction_plans():
                                 view([128, 128], dt=L.DOUBLE, ptr=P1), p))
     assert L.PATH_NAMES[p.path] in ("red_cols", "red_cols_split") and p.red_nd == 2
     assert [(s, d) for s in range(14) for d in range(14) if lib.dpx_reduce_dtype_supported(op, s, d)] \
-        == [(s, L.DOUBLE) for s in (L.INT8, L.UINT8, L.INT16, L.UINT16, L.INT32, L.UINT32, L.INT64, L.UINT64, L.FLOAT,
-                                    L.DOUBLE)]
+        == [(s, L.DOUBLE) for s in (L.INT8, L.UINT8, L.INT16, L.UINT16, L.INT32, L.UINT32, L.INT64, L.UINT64, L.HALF,
+                                    L.FLOAT, L.DOUBLE)]
     # searches walk the reduced space too (its dims keep their order)
     L.check(lib.dpx_argreduce_plan(0, view([16384, 16382], [16384, 1]), 2, view([], dt=L.INT64, ptr=P1), pa))
     assert L.PATH_NAMES[pa.path] == "red_generic" and pa.red_nd == 2 and pa.vec == 1

@@ -1074,6 +1074,16 @@ def test_variance_in_one_pass_over_contiguous_runs(dt):
     assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
     a[123] = np.inf
     assert np.isnan(host(dpt.var(dev(a), dtype="f8")))
+    # float16 input with a float16 result: accumulated in float64, rounded once (runs whose float16 sum would overflow)
+    if dt == "f4":
+        h = (rng.standard_normal((300, 70000)) * 3 + 40).astype("f2")
+        for ax in (None, 0, 1):
+            got = host(dpt.var(dev(h), axis=ax))
+            assert got.dtype == np.float16
+            np.testing.assert_array_equal(got, _exact_var(h, ax).astype("f2"))
+        # (std is the square root of the rounded variance, taken in float16: within an ULP of the exact one)
+        np.testing.assert_allclose(host(dpt.std(dev(h), axis=1, correction=1)).astype("f8"), np.sqrt(_exact_var(h, 1, 1)),
+                                   rtol=1e-3)
     # integer input: float64 result straight from the integers
     for idt in ("i1", "u2", "i4", "u8"):
         a = rng.integers(0, 100, (300, 700)).astype(idt)
