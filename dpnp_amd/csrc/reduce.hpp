@@ -311,12 +311,23 @@ template <int KIND, class T> DPX_D T red_identity()
 template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy {
     using In = In_;
     using Out = Out_;
+    // Sums of bools and of 1- and 2-byte integers into a float32 or float64 result (mean of an image stack,
+    // sum(mask, dtype=float)) are added up in 64-bit integers, exactly, and converted once: the reference converts
+    // every element first (reductions.hpp:482-491) and rounds along the way, so this is never less accurate, and
+    // the integer kernels' word arithmetic and narrow column sums apply (uint8 16384 x 65536 averaged down the
+    // columns: 41 % of the HBM rate with a conversion and a double addition per element).
+    static constexpr bool int_sum = KIND == K_SUM && !FINAL && sizeof(In_) <= 2 &&
+                                    (std::is_integral_v<In_> || is_bool_v<In_>) &&
+                                    (std::is_same_v<Out_, float> || std::is_same_v<Out_, double>);
+    using IntSumAcc = std::conditional_t<std::is_signed_v<In_> && !is_bool_v<In_>, int64_t, uint64_t>;
     using Acc = std::conditional_t<
+        int_sum, IntSumAcc,
+        std::conditional_t<
         KIND == K_SQDEV1, sqdev_acc<acc_of_t<Out_>>,
         std::conditional_t<KIND == K_LOGSUMEXP, lse_acc<acc_of_t<Out_>>,
         std::conditional_t<
             kind_has_count(KIND), mean_acc<acc_of_t<Out_>>,
-            std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>>;
+            std::conditional_t<kind_is_minmax(KIND), std::conditional_t<is_bool_v<Out_>, int32_t, Out_>, acc_of_t<Out_>>>>>>;
     // sum(|z - mean|^2) of complex input into a real result (variance of complex data,
     // dpnp/dpnp_iface_statistics.py:1849-1851: x * conj(x), real part): the mean is a complex number of the
     // result's precision, the deviation's two parts are squared and added in the real accumulator
@@ -348,6 +359,10 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     DPX_D static Acc pre(In x, AuxAcc aux)
     {
         if constexpr (FINAL) return x; // In == Acc
+        else if constexpr (int_sum) {
+            if constexpr (is_bool_v<In>) return (Acc)(x.v != 0);
+            else return (Acc)x;
+        }
         else if constexpr (cplx_dev) {
             const Acc dr = (Acc)x.re - aux.re, di = (Acc)x.im - aux.im;
             return dr * dr + di * di;
@@ -406,7 +421,7 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     static constexpr bool has_pack_fold =
         !FINAL && sizeof(In) == 1 &&
         (KIND == K_ANY || KIND == K_ALL || KIND == K_COUNT_NONZERO ||
-         (KIND == K_SUM && (is_int_v<In> || is_bool_v<In>) && is_int_v<Out>));
+         (KIND == K_SUM && (is_int_v<In> || is_bool_v<In>) && (is_int_v<Out> || int_sum)));
     DPX_D static Acc fold_pack(Acc acc, const u32x4 &words)
     {
         // (the kernel loads the words as such: a pack of bytes viewed as words makes the compiler

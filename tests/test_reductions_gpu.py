@@ -750,6 +750,31 @@ def test_argmax_argmin_along_a_short_middle_axis(dt):
     assert L.PATH_NAMES[p.path] == "red_cols" and p.block == 256 and p.splits == 1
 
 
+@pytest.mark.parametrize("dt", ["?", "i1", "u1", "i2", "u2"])
+@pytest.mark.parametrize("odt", ["f4", "f8"])
+def test_sums_of_narrow_integers_into_floats_are_exact(dt, odt):
+    # added up in 64-bit integers and converted once: the exact sum, correctly rounded, in every kernel family
+    # (rows, columns, flat short rows, staged short rows, walked views, split runs), and mean through them
+    rng = np.random.default_rng(46)
+    def exact(a, axis):
+        return np.sum(a.astype("i8"), axis=axis).astype(odt)
+    for shape, axis in (((1 << 22,), None), ((3000, 4097), 1), ((3000, 4097), 0), ((100003, 7), 0), ((100003, 7), 1),
+                        ((64, 7, 4096), (0, 2)), ((300, 1100), None), ((5, 1 << 20), 1), ((1 << 18, 40), 0)):
+        a = random_array(rng, shape, dt, -300, 300)
+        assert_same(host(dpt.sum(dev(a), axis=axis, dtype=odt)), exact(a, axis))
+    a = random_array(rng, (700, 900), dt, -300, 300)
+    assert_same(host(dpt.sum(dev(a)[1:-1, ::2], dtype=odt)), exact(a[1:-1, ::2], None))
+    assert_same(host(dpt.sum(dev(a)[:, ::2], axis=0, dtype=odt)), exact(a[:, ::2], 0))
+    out = dpt.zeros(1800, dtype=odt)
+    dpt.sum(dev(a), axis=0, dtype=odt, out=out[::2])
+    assert_same(host(out)[::2], exact(a, 0))
+    if dt != "?":  # the mean of integers is their float64 sum over the count
+        img = random_array(rng, (50, 64, 300), dt, -300, 300)
+        np.testing.assert_allclose(host(dpt.mean(dev(img), axis=0)), img.astype("f8").mean(axis=0), rtol=1e-15)
+        np.testing.assert_allclose(dpnp.asnumpy(dpnp.mean(dpnp.array(img), axis=(1, 2))), img.astype("f8").mean(axis=(1, 2)),
+                                   rtol=1e-15)
+
+
 @pytest.mark.parametrize("dt", ["f4", "f8"])
 def test_statistics_over_samples_of_few_features(dt):
     # (samples, features) with few features: mean / var / std / logsumexp / hypot / nan forms over axis 0
