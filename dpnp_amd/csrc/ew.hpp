@@ -124,15 +124,17 @@ DPX_D void ew_contig_pack(const Fn &fn, Out *out, int64_t base,
     (keep_whole(std::get<I>(v)), ...);
     pack<Out, E> r;
     if constexpr (fn_two_phase<Fn>::value) {
-        // a whole wave of arguments the functor has a cheap form for (x ** 2) takes only that
-        bool cheap = true;
+        if constexpr (Fn::has_cheap) {
+            // a whole wave of arguments the functor has a cheap form for (x ** 2) takes only that
+            bool cheap = true;
 #pragma unroll
-        for (int e = 0; e < E; ++e) cheap = cheap && fn.cheap_applies(to_value(std::get<I>(v).v[e])...);
-        if (__builtin_amdgcn_ballot_w64(!cheap) == 0) {
+            for (int e = 0; e < E; ++e) cheap = cheap && fn.cheap_applies(to_value(std::get<I>(v).v[e])...);
+            if (__builtin_amdgcn_ballot_w64(!cheap) == 0) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn.cheap(to_value(std::get<I>(v).v[e])...));
-            store_pack<Out, E>(out + base, r);
-            return;
+                for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn.cheap(to_value(std::get<I>(v).v[e])...));
+                store_pack<Out, E>(out + base, r);
+                return;
+            }
         }
         // the straight-line part for every element first, then the rare branches
         decltype(fn.fast(to_value(std::get<I>(v).v[0])...)) t[E];

@@ -30,16 +30,23 @@ template <class Op> struct op_two_packs : std::false_type {};
 #define DPX_TWO_PACKS(OP) \
     template <> struct op_two_packs<OP> : std::true_type {};
 DPX_TWO_PACKS(Expm1Op) DPX_TWO_PACKS(Log2Op) DPX_TWO_PACKS(SinhOp) DPX_TWO_PACKS(TanhOp)
-// (log1p and the inverse hyperbolic functions through it: a table look-up that waits for the argument sits in
-// the element's chain, a wave with one pack spends most of its life waiting)
+// (log1p and the inverse hyperbolic functions: 60 to 90 instructions in one dependent chain per element)
 DPX_TWO_PACKS(Log1pOp) DPX_TWO_PACKS(AsinhOp) DPX_TWO_PACKS(AcoshOp) DPX_TWO_PACKS(AtanhOp)
 // (pow of doubles: a table look-up that waits for the base sits in every element's chain; a second pack per
 // thread keeps the memory system busy meanwhile)
 DPX_TWO_PACKS(PowOp)
+// (tan of doubles: 60 instructions in one chain; 65 -> 69 % of the HBM rate with the second pack)
+DPX_TWO_PACKS(TanOp)
 #undef DPX_TWO_PACKS
+template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
+template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct UnaryFn {
     static constexpr bool two_packs = op_two_packs<Op>::value && std::is_same_v<T, double>;
+    static constexpr bool two_phase = op_two_phase<Op, T>::value; // (see BinaryFn)
+    static constexpr bool has_cheap = false;
     DPX_D auto operator()(V<T> x) const { return Op::template apply<T>(x); }
+    DPX_D auto fast(V<T> x) const { return Op::template fast<T>(x); }
+    DPX_D auto fixup(V<T> r, V<T> x) const { return Op::template fixup<T>(r, x); }
 };
 // An op may split its work in two phases for element type T (Op::two_phase<T>): fast(a, b) is
 // straight-line code that gives the result or NaN where it does not apply, fixup(r, a, b) branches to the
@@ -47,12 +54,11 @@ template <class Op, class T> struct UnaryFn {
 // before the second, so that the chains of the elements interleave (see ew_contig_pack).  Such an op
 // also names arguments with a cheap exact form (cheap_applies / cheap), which a wave takes alone when
 // all its lanes have them.
-template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
-template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct BinaryFn {
     // (pow of floats as well: its table look-up sits in every element's chain like the one of doubles)
     static constexpr bool two_packs = op_two_packs<Op>::value && (std::is_same_v<T, double> || std::is_same_v<T, float>);
     static constexpr bool two_phase = op_two_phase<Op, T>::value;
+    static constexpr bool has_cheap = true;
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
     DPX_D auto fast(V<T> a, V<T> b) const { return Op::template fast<T>(a, b); }
     DPX_D auto fixup(V<T> r, V<T> a, V<T> b) const { return Op::template fixup<T>(r, a, b); }

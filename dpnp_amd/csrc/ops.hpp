@@ -96,19 +96,13 @@ template <class T> DPX_HD T min_nan(T x, T y)
 // over 4 M arguments (all binades, dense around 1): error below 0.82 ULP (the device
 // library's: 0.63 ULP); 2^27 elements take 0.37 ms instead of 0.57 ms.
 // k and log(m) = hi + lo for x = 2^k m, sqrt(1/2) <= m < sqrt(2) (x > 0 and finite)
-DPX_D void log_f64_parts(double x, double &dk, double &f, double &hfsq, double &tail)
+// log(1 + f) = f - hfsq + tail for 1 + f in [sqrt(1/2), sqrt(2))
+DPX_D void log_f64_series(double f, double &hfsq, double &tail)
 {
     constexpr double Lg1 = 6.666666666666735130e-01, Lg2 = 3.999999999940941908e-01,
                      Lg3 = 2.857142874366239149e-01, Lg4 = 2.222219843214978396e-01,
                      Lg5 = 1.818357216161805012e-01, Lg6 = 1.531383769920937332e-01,
                      Lg7 = 1.479819860511658591e-01;
-    double m = __builtin_amdgcn_frexp_mant(x); // [0.5, 1), subnormals included
-    int e = __builtin_amdgcn_frexp_exp(x);
-    const bool low = m < 0.70710678118654752440;
-    m = low ? m * 2.0 : m;
-    e = low ? e - 1 : e;
-    f = m - 1.0;
-    dk = (double)e;
     const double d = 2.0 + f;
     double rc = __builtin_amdgcn_rcp(d);
     rc = __builtin_fma(__builtin_fma(-d, rc, 1.0), rc, rc);
@@ -118,7 +112,23 @@ DPX_D void log_f64_parts(double x, double &dk, double &f, double &hfsq, double &
     const double p2 = __builtin_fma(w, __builtin_fma(w, __builtin_fma(w, Lg7, Lg5), Lg3), Lg1);
     const double R = __builtin_fma(z, p2, t1);
     hfsq = (0.5 * f) * f;
-    tail = s * (hfsq + R); // log(m) = f - hfsq + tail
+    tail = s * (hfsq + R);
+}
+// k and m - 1 for x = 2^k m, sqrt(1/2) <= m < sqrt(2) (x > 0 and finite)
+DPX_D void log_f64_split(double x, double &dk, double &f)
+{
+    double m = __builtin_amdgcn_frexp_mant(x); // [0.5, 1), subnormals included
+    int e = __builtin_amdgcn_frexp_exp(x);
+    const bool low = m < 0.70710678118654752440;
+    m = low ? m * 2.0 : m;
+    e = low ? e - 1 : e;
+    f = m - 1.0;
+    dk = (double)e;
+}
+DPX_D void log_f64_parts(double x, double &dk, double &f, double &hfsq, double &tail)
+{
+    log_f64_split(x, dk, f);
+    log_f64_series(f, hfsq, tail); // log(m) = f - hfsq + tail
 }
 DPX_D double log_special(double x, double r)
 {
@@ -159,13 +169,13 @@ DPX_D double log10_f64(double x)
     return log_scaled_f64(x, 4.34294481903251816668e-01, 1.09831965021676510e-17, 3.01029995663611771306e-01,
                           3.69423907715893078616e-13);
 }
-// n / d for doubles of moderate size through the hardware reciprocal: two Newton steps on it and one
-// correction of the quotient (8 instructions, about 1 ULP; the IEEE division sequence takes 25).
+// n / d for doubles of moderate size through the hardware reciprocal: one Newton step on it (a relative error e of
+// the reciprocal leaves e^2 in the corrected quotient, so 2^-40 after the step is plenty) and one correction of
+// the quotient by its exact remainder (6 instructions, within 0.51 ULP; the IEEE division sequence takes 25).
 // Not for results or divisors near the ends of the exponent range.
 DPX_D double div_f64_fast(double n, double d)
 {
     double r = __builtin_amdgcn_rcp(d);
-    r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
     r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
     const double q = n * r;
     return __builtin_fma(__builtin_fma(-d, q, n), r, q);
@@ -176,69 +186,39 @@ template <class R> DPX_D R div_moderate(R n, R d)
     else return n / d;
 }
 
-// log1p: log(u) for u = 1 + x rounded, plus the rounding error of that sum over u
-// (log(1 + x) = log(u) + log(1 + c/u), c = (1 + x) - u).
-template <class R, class LOG> DPX_D R log1p_via(R x, LOG log_fn)
+// log(y + e) for a positive normal y and |e| far below an ULP of y (the low part of a two-double argument):
+// the series of log_f64 with e / y among its low-order terms.  `extra` = e / y, to the accuracy the result needs.
+DPX_D double log_f64_two(double y, double extra)
 {
-    const R u = R(1) + x;
-    const R c = (x < R(1) && x > R(-1)) ? x - (u - R(1)) : R(1) - (u - x);
-    // c / u through the hardware reciprocal (about 25 bits for a double: two Newton steps; for tiny x
-    // the quotient is the whole result)
-    R rcp;
-    if constexpr (std::is_same_v<R, double>) {
-        rcp = __builtin_amdgcn_rcp(u);
-        rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
-        rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
-    }
-    else rcp = __builtin_amdgcn_rcpf(u);
-    R r = log_fn(u) + c * rcp;
-    r = (u == R(0)) ? -(R)__builtin_inff() : r; // x = -1
-    r = (x == (R)__builtin_inff()) ? x : r;
-    const R ax = x < R(0) ? -x : x;
-    return (ax < (std::is_same_v<R, double> ? R(1e-17) : R(1e-8))) ? x : r; // also keeps -0.0
+    constexpr double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
+    double dk, f, hfsq, tail;
+    log_f64_parts(y, dk, f, hfsq, tail);
+    const double in = __builtin_fma(dk, ln2_lo, extra) + tail;
+    return __builtin_fma(dk, ln2_hi, -((hfsq - in) - f));
 }
-// log(u) + extra for a positive normal u, from the table of pow_f64_fast (pow_log_table.hpp): u = 2^k z,
-// z / c - 1 = r formed without error, log u = (k LN2_HI + log c) + r + [k LN2_LO + rest of log c + the rounding
-// error of r - r^2/2 + ... - r^8/8 + extra]; the first sum is exact, the second keeps its rounding error (next
-// to u = 1 the two terms cancel), so the result is good to 0.8 ULP over the whole range.  `extra`: a small
-// addend that joins the low-order terms (the correction c/u of log1p).  About 35 vector instructions and one
-// 16-byte look-up (log_f64 above: 48, and log1p through it 82).
-DPX_D double log_tab_f64(double u, double extra)
-{
-    auto K = [](double v) { return scalar_const(v); };
-    constexpr double LN2_HI = 0x1.62e42fefa3800p-1, LN2_LO = 0x1.ef35793c76730p-45;
-    const uint64_t ix = (uint64_t)__double_as_longlong(u), tmp = ix - POW_LOG_OFF;
-    const pow_log_entry ent = pow_log_table[(tmp >> 45) & 127];
-    const double kd = (double)(int)((int64_t)tmp >> 52);
-    const double z = __longlong_as_double((long long)(ix - (tmp & (0xfffull << 52))));
-    const double invc = (double)ent.invc;
-    const double ph = z * invc, r_lo = __builtin_fma(z, invc, -ph), r = ph - 1.0;
-    const double t1 = __builtin_fma(kd, K(LN2_HI), ent.logc); // exact
-    double q = __builtin_fma(r, K(-1.0 / 8), K(1.0 / 7));
-    q = __builtin_fma(r, q, K(-1.0 / 6));
-    q = __builtin_fma(r, q, K(1.0 / 5));
-    q = __builtin_fma(r, q, K(-1.0 / 4));
-    q = __builtin_fma(r, q, K(1.0 / 3));
-    q = __builtin_fma(r, q, -0.5);
-    const double small = __builtin_fma(r * r, q, __builtin_fma(kd, K(LN2_LO), (double)ent.logctail) + (r_lo + extra));
-    const double t2 = t1 + r, e2 = (t1 - t2) + r; // |t1| >= |r| or t1 == 0: the sum's rounding error
-    return t2 + (e2 + small);
-}
-// log1p(x) = log(u) + c/u, u = 1 + x rounded and c the rounding error of that sum.  Host check against long
-// double over 3e7 arguments (|x| < 1, tiny x, x up to 1e304, x next to -1): mean 0.20, worst 1.05 ULP.
+// log1p after fdlibm's s_log1p.c, without its branches: between sqrt(1/2) - 1 and sqrt(2) - 1 the series of log
+// takes x itself (k = 0, nothing is rounded); elsewhere it takes u = 1 + x rounded, and the rounding error c of that
+// sum over u joins the low-order terms (there the result is at least 0.29 in magnitude and c/u at most 2^-53, so
+// the float reciprocal is more than enough).  60 vector instructions and no look-up: a form through a table
+// logarithm (pow's table: 35 and a 16-byte gather per element, plus the correction's full-precision reciprocal) was
+// 5 to 12 % slower.  Host check against long double over 3.6e7 arguments (|x| < 1, tiny and subnormal x, x up to
+// 2^1023, x next to -1 and around both switches, the float reciprocal off by an ULP either way): mean 0.22,
+// worst 0.89 ULP.
 DPX_D double log1p_f64(double x)
 {
+    constexpr double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
     const double u = 1.0 + x;
-    if (!__builtin_amdgcn_class(u, 0x100)) { // x <= -1, x = inf, NaN: the general routine's cases
-        asm volatile("" ::: "memory");        // (not to be executed speculatively)
-        return log1p_via<double>(x, [](double v) { return log_f64(v); });
-    }
-    const double c = (x < 1.0 && x > -1.0) ? x - (u - 1.0) : 1.0 - (u - x);
-    double rcp = __builtin_amdgcn_rcp(u);
-    rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
-    rcp = __builtin_fma(__builtin_fma(-u, rcp, 1.0), rcp, rcp);
-    const double r = log_tab_f64(u, c * rcp);
-    return (__builtin_fabs(x) < 1e-17) ? x : r; // also keeps -0.0
+    const bool mid = x > -0.2928932188134525 && x < 0.4142135623730950;
+    double dk, f, hfsq, tail;
+    log_f64_split(u, dk, f);
+    f = mid ? x : f;
+    dk = mid ? 0.0 : dk;
+    double c = (x < 1.0) ? x - (u - 1.0) : 1.0 - (u - x);
+    c = mid ? 0.0 : c * (double)__builtin_amdgcn_rcpf((float)u);
+    log_f64_series(f, hfsq, tail);
+    const double in = __builtin_fma(dk, ln2_lo, c) + tail;
+    const double r = __builtin_fma(dk, ln2_hi, -((hfsq - in) - f));
+    return (x == 0.0) ? x : log_special(u, r); // (-0.0 stays; u = 0, u < 0, +inf, NaN as for log)
 }
 // ---- fp32 log1p and inverse hyperbolic functions through double arithmetic ------------------------
 // The argument y of the logarithm (1 + x; a + sqrt(a^2 + 1); (1 + a)/(1 - a)) is formed in double, where
@@ -278,11 +258,12 @@ DPX_D float log1p_f32(float x)
 //   asinh a = log(a + sqrt(a^2 + 1)),  acosh x = log(x + sqrt(x^2 - 1)),  atanh a = log((1 + a)/(1 - a))/2
 // with the argument y carried as yhi + ylo (the square with the error of its product, the sum with 1 as an exact
 // two-sum, the square root from the hardware estimate with one coupled step and its residual, the quotient with
-// its remainder) straight into the table logarithm: log y = log_tab_f64(yhi, ylo / yhi).  No division, no IEEE
+// its remainder) straight into the logarithm's series: log y = log_f64_two(yhi, ylo / yhi).  No division, no IEEE
 // square root (17 fp64-FMA equivalents on this GPU; the estimate and its steps: 10), no log1p wrapper around the
-// logarithm: about 70 equivalents where the fdlibm forms through log1p took 98.  Host check against long double
-// (4e6 arguments per range: ordinary, 2^-60 .. 2^709, next to 0, next to 1, around the switch to the series):
-// asinh 0.98, acosh 1.01, atanh 0.90 ULP at worst (the forms through log1p: 1.69, 1.97, 1.79).
+// logarithm, no look-up (the same functions through pow's logarithm table were 5 to 8 % slower).  Host check
+// against long double (4e6 arguments per range: ordinary, 2^-60 .. 2^709, next to 0, next to 1, around the switch
+// to the series, hardware estimates off by an ULP either way): asinh 0.84, acosh 0.82, atanh 0.90 ULP at worst
+// (the fdlibm forms through log1p: 1.69, 1.97, 1.79).
 DPX_D void sqrt_f64_two(double thi, double tlo, double &g, double &slo) // sqrt(thi + tlo) = g + slo
 {
     const double r0 = __builtin_amdgcn_rsq(thi);
@@ -308,7 +289,7 @@ DPX_D double asinh_f64(double x)
     sqrt_f64_two(thi, te + pe, g, slo);
     const double yhi = g + a, ylo = (a - (yhi - g)) + slo; // g >= a
     const bool big = a > 0x1p500;                           // a^2 + 1 = a^2 long before: log(2a)
-    double r = log_tab_f64(big ? a : yhi, big ? 0.0 : ylo * rcp_f64_seed_f32(yhi));
+    double r = log_f64_two(big ? a : yhi, big ? 0.0 : ylo * (double)__builtin_amdgcn_rcpf((float)yhi));
     r = big ? r + 0.69314718055994530942 : r;
     r = (a < 0x1p-13) ? __builtin_fma(a * p, -1.0 / 6, a) : r; // also keeps zeros and subnormals
     r = (a == (double)__builtin_inff()) ? a : r;
@@ -326,7 +307,8 @@ DPX_D double acosh_f64(double x)
     slo = one ? 0.0 : slo;
     const double yhi = x + g, ylo = (g - (yhi - x)) + slo; // x >= g
     const bool big = x > 0x1p500;
-    double r = log_tab_f64(big ? x : yhi, big ? 0.0 : ylo * rcp_f64_seed_f32(yhi));
+    // (next to x = 1 the result is of the order of ylo / yhi's 2^25-fold: the float reciprocal alone is too coarse)
+    double r = log_f64_two(big ? x : yhi, big ? 0.0 : ylo * rcp_f64_seed_f32(yhi));
     r = big ? r + 0.69314718055994530942 : r;
     r = (x == (double)__builtin_inff()) ? x : r;
     r = (x < 1.0) ? (double)__builtin_nanf("") : r;
@@ -341,7 +323,7 @@ DPX_D double atanh_f64(double x)
     rc = __builtin_fma(__builtin_fma(-dhi, rc, 1.0), rc, rc);
     const double qhi = nhi * rc;
     const double qlo = (__builtin_fma(-qhi, dhi, nhi) + __builtin_fma(-qhi, dlo, nlo)) * rc; // the remainder over 1 - a
-    double r = 0.5 * log_tab_f64(qhi, qlo * (double)__builtin_amdgcn_rcpf((float)qhi));
+    double r = 0.5 * log_f64_two(qhi, qlo * (double)__builtin_amdgcn_rcpf((float)qhi));
     r = (a < 0x1p-13) ? __builtin_fma(a * a * a, 1.0 / 3, a) : r; // also keeps zeros and subnormals
     r = (a == 1.0) ? (double)__builtin_inff() : r;
     r = (a > 1.0) ? (double)__builtin_nanf("") : r;
@@ -544,23 +526,31 @@ DPX_D int sincos_f64(double x, double &s, double &c)
     return (int)n;
 }
 constexpr double TRIG_FAST_LIMIT = 1e6; // n stays below 2^20
-DPX_D double sin_f64(double x)
+// (the *_below_limit forms: straight-line code, valid for |x| < TRIG_FAST_LIMIT, anything elsewhere)
+DPX_D double sin_f64_below_limit(double x)
 {
-    const double a = __builtin_fabs(x);
-    if (!(a < TRIG_FAST_LIMIT)) return ::sin(x);
     double s, c;
     const int q = sincos_f64(x, s, c);
     double v = (q & 1) ? c : s;
     v = (q & 2) ? -v : v;
-    return a < 0x1p-27 ? x : v; // sin x = x to the last bit, and -0 stays -0
+    return __builtin_fabs(x) < 0x1p-27 ? x : v; // sin x = x to the last bit, and -0 stays -0
 }
-DPX_D double cos_f64(double x)
+DPX_D double cos_f64_below_limit(double x)
 {
-    if (!(__builtin_fabs(x) < TRIG_FAST_LIMIT)) return ::cos(x);
     double s, c;
     const int q = sincos_f64(x, s, c);
     const double v = (q & 1) ? s : c;
     return ((q + 1) & 2) ? -v : v;
+}
+DPX_D double sin_f64(double x)
+{
+    if (!(__builtin_fabs(x) < TRIG_FAST_LIMIT)) return ::sin(x);
+    return sin_f64_below_limit(x);
+}
+DPX_D double cos_f64(double x)
+{
+    if (!(__builtin_fabs(x) < TRIG_FAST_LIMIT)) return ::cos(x);
+    return cos_f64_below_limit(x);
 }
 
 // sin and cos of one argument from one reduction (the complex functions need both)
@@ -582,6 +572,72 @@ DPX_D void sincos_both_f64(double x, double &sn, double &cs)
     sn = a < 0x1p-27 ? x : vs;
     const double vc = (q & 1) ? s : c;
     cs = ((q + 1) & 2) ? -vc : vc;
+}
+
+// ---- fp64 tan ----------------------------------------------------------------------------------------
+// For |x| < 1e6: x = n pi/2 + r as for sin and cos, with r carried as a sum of two doubles (the product n P2 with the
+// error of its rounding, the difference as an exact two-term sum: next to a multiple of pi/2 the result is r or
+// -1/r, so r's relative error is the result's); t = tan(r/2) from the fdlibm kernel (k_tan.c: T0..T12, good
+// for arguments up to 0.67, here at most pi/8), again as two doubles; then tan r = 2t / (1 - t^2) in even
+// quadrants and -(1 - t^2) / 2t in odd ones: one quotient of two-double operands through the hardware reciprocal,
+// a Newton step and the exact remainder.  About 60 vector instructions and no branch where the device library's
+// routine executes 185 (65 % of the HBM rate on 2^26 doubles).  Host check against an 80-bit evaluation over 4e7
+// arguments (dense below 50 and up to 1e6, every small binade, neighbourhoods of multiples of pi/4 down to the
+// neighbouring doubles, the reciprocal estimate off by 2^-22): mean 0.19, worst 0.66 ULP.
+DPX_D double tan_f64_below_limit(double x)
+{
+    auto K = [](double v) { return scalar_const(v); };
+    constexpr double P1 = 0x1.921fb54442d18p+0, P2 = 0x1.1a62633145c07p-54, P3 = -0x1.f1976b7ed8fbcp-110,
+                     TWO_OVER_PI = 0x1.45f306dc9c883p-1;
+    constexpr double T0 = 3.33333333333334091986e-01, T1 = 1.33333333333201242699e-01,
+                     T2 = 5.39682539762260521377e-02, T3 = 2.18694882948595424599e-02,
+                     T4 = 8.86323982359930005737e-03, T5 = 3.59207910759131235356e-03,
+                     T6 = 1.45620945432529025516e-03, T7 = 5.88041240820264096874e-04,
+                     T8 = 2.46463134818469906812e-04, T9 = 7.81794442939557092300e-05,
+                     T10 = 7.14072491382608190305e-05, T11 = -1.85586374855275456654e-05,
+                     T12 = 2.59073051863633712884e-05;
+    const double n = __builtin_rint(x * K(TWO_OVER_PI));
+    const double r1 = __builtin_fma(-n, K(P1), x); // exact
+    const double p2 = n * K(P2), p2e = __builtin_fma(n, K(P2), -p2);
+    const double r0 = r1 - p2;
+    double tail = ((r1 - r0) - p2) - p2e;
+    tail = 0.5 * __builtin_fma(-n, K(P3), tail);
+    const double r = 0.5 * r0;
+    const double z = r * r, w = z * z;
+    double pr = __builtin_fma(w, K(T11), K(T9));
+    pr = __builtin_fma(w, pr, K(T7));
+    pr = __builtin_fma(w, pr, K(T5));
+    pr = __builtin_fma(w, pr, K(T3));
+    pr = __builtin_fma(w, pr, K(T1));
+    double pv = __builtin_fma(w, K(T12), K(T10));
+    pv = __builtin_fma(w, pv, K(T8));
+    pv = __builtin_fma(w, pv, K(T6));
+    pv = __builtin_fma(w, pv, K(T4));
+    pv = __builtin_fma(w, pv, K(T2));
+    pv = z * pv;
+    const double s = z * r;
+    double rr = __builtin_fma(z, __builtin_fma(s, pr + pv, tail), tail);
+    rr = __builtin_fma(K(T0), s, rr);             // tan(r + tail) = r + rr
+    const double th = r + rr, tl = (r - th) + rr; // = th + tl, |tl| below half an ULP of th
+    const double p = th * th, pe = __builtin_fma(th, th, -p);
+    const double uh = 0.5 - 0.5 * p;              // (1 - t^2) / 2 = uh + ul
+    const double ul = ((0.5 - uh) - 0.5 * p) - __builtin_fma(th, tl, 0.5 * pe);
+    const bool odd = ((int)n & 1) != 0;
+    const double nh = odd ? -uh : th, nl = odd ? -ul : tl, dh = odd ? th : uh, dl = odd ? tl : ul;
+    double rc = __builtin_amdgcn_rcp(dh);
+    rc = __builtin_fma(__builtin_fma(-dh, rc, 1.0), rc, rc);
+    const double q = nh * rc;
+    const double rem = __builtin_fma(-q, dh, nh) + __builtin_fma(-q, dl, nl);
+    const double res = __builtin_fma(rem, rc, q);
+    return __builtin_fabs(x) < 0x1p-27 ? x : res; // tan x = x to the last bit, and -0 stays -0
+}
+DPX_D double tan_f64(double x)
+{
+    if (!(__builtin_fabs(x) < TRIG_FAST_LIMIT)) {
+        asm volatile("" ::: "memory"); // (not to be executed speculatively, see sincos_both_f64)
+        return ::tan(x);
+    }
+    return tan_f64_below_limit(x);
 }
 
 // ---- fp64 asin, acos -----------------------------------------------------------------------------
@@ -672,7 +728,7 @@ DPX_FP_FN1(m_log, ::logf, log_f64)
 DPX_FP_FN1(m_erf, ::erff, erf_f64)
 DPX_FP_FN1(m_sin, ::sinf, sin_f64)
 DPX_FP_FN1(m_cos, ::cosf, cos_f64)
-DPX_FP_FN1(m_tan, ::tanf, ::tan)
+DPX_FP_FN1(m_tan, ::tanf, tan_f64)
 DPX_FP_FN1(m_tanh, ::tanhf, tanh_f64)
 DPX_FP_FN1(m_exp2, ::exp2f, ::exp2)
 DPX_FP_FN1(m_expm1, ::expm1f, ::expm1)
@@ -1041,15 +1097,7 @@ template <class R> DPX_D cplx<R> c_tanh(cplx<R> z)
     const R x = z.re, y = z.im;
     // Kahan's formulation: no cancellation near the poles at x = 0, y = pi/2 + k pi.  rho = sqrt(1 + sinh^2 x) is
     // cosh x; the sign of sin y cos y and of sin 2y, which the large and infinite cases ask for, is that of tan y
-    R t;
-    if constexpr (std::is_same_v<R, double>) {
-        // the quotient of this library's sin and cos (about 65 vector instructions; the device library's tan takes 185
-        // inside this kernel); cos y is accurate to 1.5 ULP also next to its zeros, where tan y has its poles
-        R sn, cs;
-        sincos_both_f64(y, sn, cs);
-        t = (sn == R(0)) ? sn * cs : div_moderate<R>(sn, cs); // (the short division would turn -0 into +0)
-    }
-    else t = m_tan(y);
+    const R t = m_tan(y);
     R sh, rho;
     m_sinhcosh(x, sh, rho);
     const R q_nan = (R)__builtin_nanf("");
@@ -1526,9 +1574,33 @@ struct SquareOp { // square.hpp:64-90; bool -> int8
 DPX_FPC_UNARY(SqrtOp, m_sqrt(x), c_sqrt(x))
 DPX_FPC_UNARY(ExpOp, m_exp(x), c_exp(x))
 DPX_FPC_UNARY(LogOp, m_log(x), c_log(x))
-DPX_FPC_UNARY(SinOp, (x == T(0)) ? x : m_sin(x), c_sin(x)) // sin.hpp:186-194: a zero comes back as it is
-DPX_FPC_UNARY(CosOp, m_cos(x), c_cos(x))
-DPX_FPC_UNARY(TanOp, m_tan(x), c_tan(x))
+// sin, cos, tan: for doubles the contiguous kernel runs the straight-line routine for the arguments below 1e6 over
+// a whole pack first, so that the elements' chains interleave, and then the device library's for what is left
+// (with the hand-over test in front of each element's routine the elements ran one after the other: tan 5 % slower)
+#define DPX_TRIG_UNARY(NAME, EXPR, CEXPR, BELOW, LIBM)                            \
+    struct NAME {                                                               \
+        template <class T> static constexpr bool ok = is_fp_v<T> || is_cplx_v<T>; \
+        template <class T> using out = T;                                       \
+        template <class T> DPX_D static T apply(T x)                            \
+        {                                                                       \
+            if constexpr (is_cplx_v<T>) return CEXPR;                           \
+            else return EXPR;                                                   \
+        }                                                                       \
+        template <class T> static constexpr bool two_phase = std::is_same_v<T, double>; \
+        template <class T> DPX_D static double fast(double x) { return BELOW(x); } \
+        template <class T> DPX_D static double fixup(double r, double x)        \
+        {                                                                       \
+            if (!(__builtin_fabs(x) < TRIG_FAST_LIMIT)) {                       \
+                asm volatile("" ::: "memory"); /* (not to be executed speculatively) */ \
+                r = LIBM(x);                                                    \
+            }                                                                   \
+            return r;                                                           \
+        }                                                                       \
+    };
+DPX_TRIG_UNARY(SinOp, (x == T(0)) ? x : m_sin(x), c_sin(x), sin_f64_below_limit, ::sin) // sin.hpp:186-194: a zero comes back as it is
+DPX_TRIG_UNARY(CosOp, m_cos(x), c_cos(x), cos_f64_below_limit, ::cos)
+DPX_TRIG_UNARY(TanOp, m_tan(x), c_tan(x), tan_f64_below_limit, ::tan)
+#undef DPX_TRIG_UNARY
 DPX_FPC_UNARY(TanhOp, m_tanh(x), c_tanh(x))
 DPX_FPC_UNARY(Exp2Op, m_exp2(x), c_exp2(x))
 DPX_FPC_UNARY(Expm1Op, (x == T(0)) ? x : m_expm1(x), c_expm1(x)) // expm1.hpp:139-146

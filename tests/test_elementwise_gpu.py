@@ -497,9 +497,10 @@ def test_unary_transcendentals_within_4_ulp(op):
 
 
 def test_float64_trigonometric_functions_on_hard_arguments():
-    """asin, acos and, below 1e6 in magnitude, sin and cos of doubles are the library's own routines, tan
-    and the rest the device library's: against an 80-bit evaluation on every binade, next to multiples of
-    pi/2 (where the reduced argument cancels), across the hand-over at 1e6, next to +-1 and +-1/2."""
+    """asin, acos and, below 1e6 in magnitude, sin, cos and tan of doubles are the library's own routines, the
+    rest the device library's: against an 80-bit evaluation on every binade, next to multiples of pi/2 and
+    pi/4 (where the reduced argument cancels, and where tan's half-angle form has its quotient's extremes),
+    across the hand-over at 1e6, next to +-1 and +-1/2."""
     if np.finfo(np.longdouble).nmant < 63:
         pytest.skip("needs an extended-precision long double")
     rng = np.random.default_rng(31)
@@ -513,6 +514,13 @@ def test_float64_trigonometric_functions_on_hard_arguments():
     for op, bound in (("sin", 2.0), ("cos", 2.0), ("tan", 2.0)):
         got = host(getattr(dpt, op)(dev(a)))
         assert_ulp(got, orc.hi_precision(op, a), bound)
+    # tan below the hand-over: the own routine stays within an ULP, also on the doubles next to multiples of pi/4
+    k4 = rng.integers(1, 1272000, 60000).astype("f8")
+    m4 = k4 * (np.pi / 4)
+    near4 = np.concatenate([m4, np.nextafter(m4, 0), np.nextafter(m4, 2e6), m4 + rng.choice([1e-9, -1e-9, 3e-13, -1e-5], m4.size)])
+    t = np.concatenate([a[np.abs(a) < 999900.0], near4[near4 < 999900.0], -near4[:20000][near4[:20000] < 999900.0],
+                        rng.uniform(-1.6, 1.6, 40000)])
+    assert_ulp(host(dpt.tan(dev(t))), orc.hi_precision("tan", t), 1.0)
     m1 = np.exp(rng.uniform(np.log(tiny * 4), 0.0, 40000))
     b = np.concatenate([m1, 1.0 - m1[m1 < 0.5], 0.5 + rng.uniform(-1e-3, 1e-3, 5000), rng.uniform(0, 1, 40000),
                         np.array([0.0, 0.5, 1.0, np.nextafter(1.0, 0), np.nextafter(0.5, 0), np.nextafter(0.5, 1)])])
