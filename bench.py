@@ -81,7 +81,7 @@ WORKLOADS = {
               "without a cross-block step, every-other-column reads, 512-byte runs on both sides of a transposition",
     "survey": "functions outside the named configurations that run furthest below the HBM rate: fp64 pow / asinh / atanh / "
               "log1p / tan over 2^26 elements, complex128 exp / sin / cos / sinh / tanh / expm1 over 2^25, float16 sin / sinh "
-              "over 2^27, column sums of a 16384x16384 int8 matrix",
+              "over 2^27, column sums of a 32768x32768 int8 matrix",
     "colsearch": "argmax and max down the columns of fp32 matrices of 2^28 elements with 128 to 4096 columns, and argmax "
                  "along the middle axis of 65536x32x128",
     "layouts": "fp32 2^28 elements reduced over dims that do not collapse into one run: a sliced matrix summed whole, "
@@ -96,7 +96,7 @@ def _device_array(dpnp, torch, t):
     library's stream, before anything is timed."""
     from dpnp_amd.tensor._usmarray import usm_ndarray
 
-    names = {torch.float32: "f4", torch.float64: "f8", torch.int32: "i4", torch.bool: "?"}
+    names = {torch.float32: "f4", torch.float64: "f8", torch.int32: "i4", torch.int8: "i1", torch.bool: "?"}
     t = t.contiguous()
     arr = dpnp.empty(tuple(t.shape), dtype=names[t.dtype])
     torch.cuda.synchronize()  # t is complete (torch's stream) before the library's stream reads it
@@ -280,9 +280,9 @@ def build_workload(name, dpnp, torch):
         oz = dpnp.empty(n2, dtype="c16")
         xh = dpnp.astype(uniform(n3), "f2")
         oh = dpnp.empty(n3, dtype="f2")
-        B8 = _device_array(dpnp, torch, torch.randint(0, 100, (1 << 14, 1 << 14), device="cuda", generator=g,
-                                                      dtype=torch.int32)).astype("i1")
-        o8 = dpnp.empty(1 << 14, dtype="i8")
+        B8 = _device_array(dpnp, torch, torch.randint(-100, 100, (1 << 15, 1 << 15), device="cuda", generator=g,
+                                                      dtype=torch.int8))
+        o8 = dpnp.empty(1 << 15, dtype="i8")
         ops = [("pow_f64", lambda: dpnp.power(x, y, out=o), 24 * n, n)]
         for fn in ("arcsinh", "arctanh", "log1p", "tan"):
             ops.append((f"{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))
@@ -290,7 +290,7 @@ def build_workload(name, dpnp, torch):
             ops.append((f"{fn}_c128", lambda f=getattr(dpnp, fn): f(z, out=oz), 32 * n2, n2))
         for fn in ("sin", "sinh"):
             ops.append((f"{fn}_f16", lambda f=getattr(dpnp, fn): f(xh, out=oh), 4 * n3, n3))
-        ops.append(("sum_axis0_int8_16384sq", lambda: dpnp.sum(B8, axis=0, out=o8), 1 << 28, 1 << 28))
+        ops.append(("sum_axis0_int8_32768sq", lambda: dpnp.sum(B8, axis=0, out=o8), 1 << 30, 1 << 30))
         # the real functions the complex ones are built from (only with --ops: for instruction counts)
         for fn in ("exp", "sin", "cos", "sinh", "cosh", "expm1", "log"):
             ops.append((f"ref:{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))

@@ -1162,43 +1162,147 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                     }
                     return;
                 }
-                // sums and counts of 1- and 2-byte integers into 64-bit accumulators: 16384 rows of a thread at a
-                // time are added up in 32 bits (a sign extension and an add per element instead of four
-                // instructions, half the registers), then moved on to the wide accumulators
-                constexpr bool NARROW = WHOLE && sizeof(In) <= 2 && sizeof(Acc) == 8 && std::is_integral_v<Acc> &&
-                                        !P::has_aux && (P::kind == K_SUM || P::kind == K_COUNT_NONZERO);
-                if constexpr (NARROW) {
+                // 1- and 2-byte inputs, whose packs hold 16 or 8 columns: two packs are sent for before the two in
+                // hand are taken apart and added up.  A block of these kernels has a CU to itself, its waves in step,
+                // and the 30 to 130 vector instructions a pair of packs costs otherwise pass with nothing in flight;
+                // more than two pairs in flight are slower again (int8 summed down the columns of 2^30 bytes, 8 packs
+                // loaded and then added up: 65 - 72 % of the HBM rate over the shapes; 8 + 8 in flight 69 - 81;
+                // 2 + 2: 73 - 83).
+                // Sums and counts of integers into wider integers (NARROW) add up 16384 rows of a thread at a time
+                // in 32 bits, an element by one dot-product instruction, before they move on to the wide accumulators.
+                constexpr bool PIPE = WHOLE && sizeof(In) <= 2;
+                constexpr bool NARROW = PIPE && sizeof(Acc) >= 4 && std::is_integral_v<Acc> && !P::has_aux &&
+                                        (P::kind == K_SUM || P::kind == K_COUNT_NONZERO);
+                if constexpr (PIPE) {
                     using A32 = std::conditional_t<std::is_signed_v<Acc>, int32_t, uint32_t>;
-                    constexpr int ROUNDS = 16384 / NL;
-                    while (r + (NL - 1) * TY < end) {
-                        A32 n32[U][E];
+                    constexpr int H = 2, ROUNDS = 16384 / H;
+                    [[maybe_unused]] A32 n32[NARROW ? U : 1][NARROW ? E : 1];
+                    if constexpr (NARROW) {
 #pragma unroll
                         for (int u = 0; u < U; ++u)
 #pragma unroll
                             for (int e = 0; e < E; ++e) n32[u][e] = 0;
-                        for (int round = 0; round < ROUNDS && r + (NL - 1) * TY < end; ++round, r += NL * TY) {
-                            pack<In, E> v[NL];
+                    }
+                    // (the packs cross the loop's back edge as the words that were loaded: carried as elements, each
+                    // in a register of its own, they are taken apart where they are loaded, which waits for them there)
+                    static_assert(sizeof(In) * E == 16);
+                    u32x4 va[H], vb[H];
+                    int round = 0;
+                    auto send_for = [&](u32x4(&d)[H], int64_t row) {
 #pragma unroll
-                            for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
+                        for (int u = 0; u < H; ++u) d[u] = load_words16(p + next_row(row + u * TY));
+                        asm volatile("" ::: "memory"); // (the loads stay in front of the arithmetic that follows)
+                    };
+                    auto add_up = [&](u32x4(&d)[H]) {
 #pragma unroll
-                            for (int u = 0; u < NL; ++u)
+                        for (int u = 0; u < H; ++u) {
+                            union {
+                                u32x4 r;
+                                pack<In, E> p;
+                            } c;
+                            c.r = d[u];
+                            asm volatile("" : "+v"(c.r)); // (taken apart here, not where it is loaded)
+                            if constexpr (!NARROW) {
 #pragma unroll
-                                for (int e = 0; e < E; ++e) n32[u % U][e] += int_cast<A32>(P::pre(v[u].v[e], a[e]));
+                                for (int e = 0; e < E; ++e)
+                                    acc[u % U][e] = P::combine(acc[u % U][e], P::pre(c.p.v[e], a[e]));
+                                continue;
+                            }
+                            // an element into its sum by one dot-product instruction (the word times a word with a one
+                            // in the element's place); counts and bools first turn each element into 0 or 1
+                            constexpr bool ZERO_ONE = P::kind == K_COUNT_NONZERO || is_bool_v<In>;
+                            constexpr bool SIGNED = std::is_signed_v<In> && !ZERO_ONE;
+#pragma unroll
+                            for (int i = 0; i < (NARROW ? 4 : 0); ++i) {
+                                uint32_t w = c.r[i];
+                                if constexpr (sizeof(In) == 1) {
+                                    if constexpr (ZERO_ONE) w = ((((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) >> 7) & 0x01010101u;
+#pragma unroll
+                                    for (int b = 0; b < 4; ++b) {
+                                        A32 &t = n32[u % U][4 * i + b];
+                                        if constexpr (SIGNED) t = (A32)__builtin_amdgcn_sdot4((int)w, 1 << (8 * b), (int)t, false);
+                                        else t = (A32)__builtin_amdgcn_udot4(w, 1u << (8 * b), (uint32_t)t, false);
+                                    }
+                                }
+                                else {
+                                    typedef short s16x2 __attribute__((ext_vector_type(2)));
+                                    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+                                    if constexpr (ZERO_ONE) w = ((((w & 0x7fff7fffu) + 0x7fff7fffu) | w) >> 15) & 0x00010001u;
+#pragma unroll
+                                    for (int b = 0; b < 2; ++b) {
+                                        A32 &t = n32[u % U][2 * i + b];
+                                        union {
+                                            uint32_t w;
+                                            s16x2 s;
+                                            u16x2 u;
+                                        } x, m;
+                                        x.w = w;
+                                        m.w = 1u << (16 * b);
+                                        if constexpr (SIGNED) t = (A32)__builtin_amdgcn_sdot2(x.s, m.s, (int)t, false);
+                                        else t = (A32)__builtin_amdgcn_udot2(x.u, m.u, (uint32_t)t, false);
+                                    }
+                                }
+                            }
                         }
+                    };
+                    auto move_on = [&](bool last) {
+                        if constexpr (!NARROW) return;
+                        if (++round >= ROUNDS || last) {
 #pragma unroll
-                        for (int u = 0; u < U; ++u)
+                            for (int u = 0; u < U; ++u)
 #pragma unroll
-                            for (int e = 0; e < E; ++e) acc[u][e] = P::combine(acc[u][e], int_cast<Acc>(n32[u][e]));
+                                for (int e = 0; e < E; ++e) {
+                                    acc[u][e] = P::combine(acc[u][e], int_cast<Acc>(n32[u][e]));
+                                    n32[u][e] = 0;
+                                }
+                            round = 0;
+                        }
+                    };
+                    // Two halves change places, so that no register is moved (a move waits for its load), and the
+                    // loop holds no load under a condition and no exit between its halves (either makes the compiler
+                    // wait for loads in flight that it cannot tell apart): it runs while three more halves exist.
+                    if (r + (H - 1) * TY < end) {
+                        send_for(va, r);
+                        while (r + (3 * H - 1) * TY < end) {
+                            send_for(vb, r + H * TY);
+                            add_up(va);
+                            move_on(false);
+                            send_for(va, r + 2 * H * TY);
+                            add_up(vb);
+                            move_on(false);
+                            r += 2 * H * TY;
+                        }
+                        add_up(va);
+                        move_on(false);
+                        r += H * TY;
+                    }
+                    // what is left, fewer than 2 H rows: the sums send for them together, as zeros where there is no
+                    // row (the others leave them to the loop at the end, one round trip each)
+                    if constexpr (NARROW) {
+                        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                            for (int u = 0; u < H; ++u) {
+                                va[u] = u32x4{0, 0, 0, 0};
+                                if (r + u * TY < end) va[u] = load_words16(p + next_row(r + u * TY));
+                            }
+                            add_up(va);
+                            r += H * TY;
+                        }
+                        move_on(true);
                     }
                 }
-                for (; r + (NL - 1) * TY < end; r += NL * TY) {
-                    pack<In, E> v[NL];
+                // (not after the loop above, which leaves fewer than a round's rows: this one's element-wise
+                // temporaries would set the kernel's register count)
+                if constexpr (!PIPE) {
+                    for (; r + (NL - 1) * TY < end; r += NL * TY) {
+                        pack<In, E> v[NL];
 #pragma unroll
-                    for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
+                        for (int u = 0; u < NL; ++u) v[u] = load(p + next_row(r + u * TY));
 #pragma unroll
-                    for (int u = 0; u < NL; ++u)
+                        for (int u = 0; u < NL; ++u)
 #pragma unroll
-                        for (int e = 0; e < E; ++e) acc[u % U][e] = P::combine(acc[u % U][e], P::pre(v[u].v[e], a[e]));
+                            for (int e = 0; e < E; ++e) acc[u % U][e] = P::combine(acc[u % U][e], P::pre(v[u].v[e], a[e]));
+                    }
                 }
                 for (; r < end; r += TY) {
                     pack<In, E> v = load(p + next_row(r));

@@ -806,6 +806,43 @@ def test_statistics_over_samples_of_few_features(dt):
     assert_same(r1, r2)
 
 
+@pytest.mark.parametrize("dt", ["?", "i1", "u1", "i2", "u2", "f2"])
+def test_column_reductions_of_narrow_types_every_row_count(dt):
+    # 1- and 2-byte inputs go down the columns two packs at a time with the next two in flight, the integer sums
+    # through dot-product instructions: every count of rows per thread around the loop's steps, the extreme values
+    # of the type, whole packs and a row length that ends inside one, one block and several
+    rng = np.random.default_rng(53)
+    lo, hi = (0, 2) if dt == "?" else ((-4, 5) if dt == "f2" else (np.iinfo(dt).min, np.iinfo(dt).max + 1))
+    for rows in list(range(1, 40)) + [63, 64, 65, 97, 130, 257, 1000, 4099, 70001]:
+        for cols in (1024, 1000 + 7):
+            if rows > 5000 and cols != 1024:
+                continue
+            a = rng.integers(lo, hi, (rows, cols)).astype(dt)
+            if dt not in ("?", "f2"):
+                a[rng.random(a.shape) < 0.2] = np.iinfo(dt).min
+                a[rng.random(a.shape) < 0.2] = np.iinfo(dt).max
+            da = dev(a)
+            if dt == "f2":
+                np.testing.assert_allclose(host(dpt.sum(da, axis=0)).astype("f8"), a.astype("f8").sum(axis=0), rtol=2e-3, atol=0.5)
+            else:
+                wide = "u8" if dt in ("u1", "u2") else "i8"
+                assert_same(host(dpt.sum(da, axis=0)), a.astype(wide).sum(axis=0))
+                assert_same(host(dpt.sum(da, axis=0, dtype="i4")), a.astype("i8").sum(axis=0).astype("i4"))
+            assert_same(host(dpt.count_nonzero(da, axis=0)), np.count_nonzero(a, axis=0).astype("i8"))
+            assert_same(host(dpt.max(da, axis=0)), a.max(axis=0))
+            assert_same(host(dpt.min(da, axis=0)), a.min(axis=0))
+            assert_same(host(dpt.any(da, axis=0)), a.astype(bool).any(axis=0))
+    # rows that are slices of wider rows, and every other row (a walked view)
+    a = rng.integers(lo, hi, (3001, 2100)).astype(dt)
+    da = dev(a)
+    if dt != "f2":
+        wide = "u8" if dt in ("u1", "u2") else "i8"
+        assert_same(host(dpt.sum(da[:, 16:1040], axis=0)), a[:, 16:1040].astype(wide).sum(axis=0))
+        assert_same(host(dpt.sum(da[::2, 16:1040], axis=0)), a[::2, 16:1040].astype(wide).sum(axis=0))
+        assert_same(host(dpt.count_nonzero(da[1::3, :1024], axis=0)), np.count_nonzero(a[1::3, :1024], axis=0).astype("i8"))
+    assert_same(host(dpt.max(da[::2, 16:1040], axis=0)), a[::2, 16:1040].max(axis=0))
+
+
 @pytest.mark.parametrize("dt", ["?", "i1", "u1"])
 def test_one_byte_counting_reductions_word_arithmetic(dt):
     # sum / any / all / count_nonzero of one-byte types fold 16 elements at a time with word arithmetic:
