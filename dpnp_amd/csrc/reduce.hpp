@@ -1279,7 +1279,7 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                     // what is left, fewer than 2 H rows: the sums send for them together, as zeros where there is no
                     // row (the others leave them to the loop at the end, one round trip each)
                     if constexpr (NARROW) {
-                        for (int half = 0; half < 2; ++half) {
+                        for (int part = 0; part < 2; ++part) {
 #pragma unroll
                             for (int u = 0; u < H; ++u) {
                                 va[u] = u32x4{0, 0, 0, 0};
