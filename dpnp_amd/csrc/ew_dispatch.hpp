@@ -35,9 +35,15 @@ DPX_TWO_PACKS(Log1pOp) DPX_TWO_PACKS(AsinhOp) DPX_TWO_PACKS(AcoshOp) DPX_TWO_PAC
 // (pow of doubles: a table look-up that waits for the base sits in every element's chain; a second pack per
 // thread keeps the memory system busy meanwhile)
 DPX_TWO_PACKS(PowOp)
-// (tan of doubles: 60 instructions in one chain; 65 -> 69 % of the HBM rate with the second pack)
-DPX_TWO_PACKS(TanOp)
+// (sin, cos, tan of doubles: 45 to 60 instructions in one chain; sin 70-78 -> 82 %, cos 75-78 -> 82 %, tan 65 -> 69 % of
+// the HBM rate with the second pack; log, log10, exp, erf, acos, atan gain nothing or lose a point)
+DPX_TWO_PACKS(SinOp) DPX_TWO_PACKS(CosOp) DPX_TWO_PACKS(TanOp)
+// (logaddexp and logaddexp2 of doubles, an exp and a log1p per element: 63-68 -> 70-75 %)
+DPX_TWO_PACKS(LogaddexpOp) DPX_TWO_PACKS(Logaddexp2Op)
 #undef DPX_TWO_PACKS
+// ... and of floats (pow: its table look-up sits in every element's chain like the one of doubles)
+template <class Op> struct op_two_packs_float : std::false_type {};
+template <> struct op_two_packs_float<PowOp> : std::true_type {};
 template <class Op, class T, class = void> struct op_two_phase : std::false_type {};
 template <class Op, class T> struct op_two_phase<Op, T, std::enable_if_t<Op::template two_phase<T>>> : std::true_type {};
 template <class Op, class T> struct UnaryFn {
@@ -55,8 +61,8 @@ template <class Op, class T> struct UnaryFn {
 // also names arguments with a cheap exact form (cheap_applies / cheap), which a wave takes alone when
 // all its lanes have them.
 template <class Op, class T> struct BinaryFn {
-    // (pow of floats as well: its table look-up sits in every element's chain like the one of doubles)
-    static constexpr bool two_packs = op_two_packs<Op>::value && (std::is_same_v<T, double> || std::is_same_v<T, float>);
+    static constexpr bool two_packs = (op_two_packs<Op>::value && std::is_same_v<T, double>) ||
+                                      (op_two_packs_float<Op>::value && std::is_same_v<T, float>);
     static constexpr bool two_phase = op_two_phase<Op, T>::value;
     static constexpr bool has_cheap = true;
     DPX_D auto operator()(V<T> a, V<T> b) const { return Op::template apply<T>(a, b); }
