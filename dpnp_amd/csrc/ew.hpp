@@ -18,6 +18,7 @@
 //   * strided kernels keep threads adjacent along the innermost output
 //     dimension and pay one div/mod chain per thread, not per element.
 #pragma once
+#include <array>
 #include <atomic>
 #include <tuple>
 #include <utility>
@@ -374,6 +375,122 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_rows_kernel(Fn fn,
     ew_rows_body<Fn, Out, Ins...>(fn, ix, out, in, modes, tx_log2, nrows, col_blocks,
                                   std::index_sequence_for<Ins...>{});
 }
+
+// ---- calls that only write: an outer sum, a row plus a column --------------------------------
+// Every input is either a row vector (contiguous along the inner dim, the same for all rows of dim inner - 1) or
+// one value per row (it does not move along the inner dim; `per_row` has its bit).  A block owns up to
+// EW_OUTER_ROWS consecutive rows of dim inner - 1 under one index of the dims before it and blockDim.x * E columns:
+// a thread loads its pack of every row vector once, lane l of each wave the per-row values of row l, and then a
+// row is a lane read (v_readlane), the arithmetic and one 16-byte store.  The rows kernel above spends its index
+// arithmetic and a load of every operand on each pack of output (fp32 row + column into 16384 x 16384: 63 % of
+// the HBM rate where a fill of the same matrix writes at 84 %).  Few rows per block: a thread that stores one
+// row after the other writes slower the longer it goes on (a stand-alone kernel of 256 threads storing 4 KiB runs
+// of 2 / 4 / 8 / 16 / 64 rows: 84 / 82 / 82 / 78 / 55 % of the HBM rate).
+constexpr int EW_OUTER_ROWS = 8;
+template <class T> DPX_D T lane_value(T v, int lane) // v of lane `lane` (uniform), for every lane
+{
+    constexpr int W = (sizeof(T) + 3) / 4;
+    union {
+        T t;
+        uint32_t w[W];
+    } a, b;
+#pragma unroll
+    for (int i = 0; i < W; ++i) a.w[i] = 0;
+    a.t = v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) b.w[i] = (uint32_t)__builtin_amdgcn_readlane((int)a.w[i], lane);
+    return b.t;
+}
+template <class Fn, class Out, class... Ins, size_t... I>
+DPX_D void ew_outer_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out *out,
+                         const InPtrs<sizeof...(Ins)> &in, uint32_t per_row, uint32_t mid_blocks, uint32_t col_blocks,
+                         std::index_sequence<I...>)
+{
+    constexpr int N = sizeof...(Ins);
+    constexpr int E = ew_traits<Out, Ins...>::E;
+    const int inner = ix.nd - 1, mid = inner - 1;
+    const int64_t ncols = ix.shape[inner];
+    uint32_t b = blockIdx.x;
+    const uint32_t cb = b % col_blocks;
+    b /= col_blocks;
+    const uint32_t mb = b % mid_blocks;
+    uint32_t o = b / mid_blocks; // index over the dims before `mid`
+    const int64_t row0 = (int64_t)mb * EW_OUTER_ROWS;
+    const int nr = (ix.shape[mid] - row0 < EW_OUTER_ROWS) ? (int)(ix.shape[mid] - row0) : EW_OUTER_ROWS;
+    int64_t base[N + 1];
+#pragma unroll
+    for (int k = 0; k <= N; ++k) base[k] = 0;
+    for (int d = mid - 1; d >= 0; --d) {
+        const uint32_t q = (d == 0) ? 0u : o / (uint32_t)ix.shape[d];
+        const int64_t i = o - q * (uint32_t)ix.shape[d];
+#pragma unroll
+        for (int k = 0; k <= N; ++k) base[k] += i * ix.strides[k][d];
+        o = q;
+    }
+    const int lane = threadIdx.x & 63;
+    const int64_t col0 = ((int64_t)cb * blockDim.x + threadIdx.x) * E;
+    const bool active = col0 < ncols;
+    const int cnt = (ncols - col0 < E) ? (int)(ncols - col0) : E;
+    // the per-row values of row `lane` (every lane of the wave takes part, also those past the row's end) ...
+    std::tuple<Ins...> mine;
+    auto load_row_value = [&](auto *p, int64_t bk, int64_t sm, bool is_per_row) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+        T v{};
+        if (is_per_row && lane < nr) v = load_one(p + bk + (row0 + lane) * sm);
+        return v;
+    };
+    ((std::get<I>(mine) = load_row_value((const Ins *)in.p[I], base[I], ix.strides[I][mid], (per_row >> I) & 1u)), ...);
+    // ... and this thread's pack of the row vectors: one for all rows, or one per row where the vector moves along
+    // dim inner - 1 (it is then the same for every index of an earlier dim: X[:, None, :] - Y[None, :, :])
+    constexpr int R = EW_OUTER_ROWS;
+    std::tuple<std::array<pack<Ins, E>, R>...> vec;
+    auto load_vectors = [&](auto &dstv, auto *p, int64_t bk, int64_t sm, bool is_per_row) {
+        using T = std::remove_cv_t<std::remove_pointer_t<decltype(p)>>;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            dstv[j] = pack<T, E>{};
+            if (is_per_row || !active || j >= nr || (j > 0 && sm == 0)) continue;
+            const T *src = p + bk + (row0 + j) * sm + col0;
+            if (cnt == E) dstv[j] = load_pack<T, E, false>(src);
+            else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dstv[j].v[e] = load_one(src + (e < cnt ? e : 0));
+            }
+        }
+    };
+    (load_vectors(std::get<I>(vec), (const Ins *)in.p[I], base[I], ix.strides[I][mid], (per_row >> I) & 1u), ...);
+    Out *q = out + base[N] + row0 * ix.strides[N][mid] + col0;
+    const int64_t ostep = ix.strides[N][mid];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        if (j >= nr) break;
+        std::tuple<pack<Ins, E>...> x;
+        ((std::get<I>(x) = ((per_row >> I) & 1u) ? splat<Ins, E>(lane_value(std::get<I>(mine), j))
+                                                 : std::get<I>(vec)[ix.strides[I][mid] == 0 ? 0 : j]),
+         ...);
+        pack<Out, E> r;
+#pragma unroll
+        for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(x).v[e])...));
+        if (active) {
+            if (cnt == E) store_pack<Out, E>(q + j * ostep, r);
+            else {
+                // (places by constant index: indexed by a running one the pack is kept in LDS, full packs included)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if (e < cnt) q[j * ostep + e] = r.v[e];
+            }
+        }
+    }
+}
+template <class Fn, class Out, class... Ins>
+__global__ __launch_bounds__(EW_BLOCK) void ew_outer_kernel(Fn fn, NdIndex<sizeof...(Ins) + 1> ix, Out *out,
+                                                           InPtrs<sizeof...(Ins)> in, uint32_t per_row,
+                                                           uint32_t mid_blocks, uint32_t col_blocks)
+{
+    ew_outer_body<Fn, Out, Ins...>(fn, ix, out, in, per_row, mid_blocks, col_blocks, std::index_sequence_for<Ins...>{});
+}
+// functors whose calls may take it (two-operand functions: one more kernel per functor and element type)
+template <class Fn> struct outer_enabled : std::false_type {};
 
 // ---- two rows per thread, the way each input is read fixed at compile time --------------------
 // The kernel for calls with a stride-2 input (x[:, ::2], the real or imaginary parts of a complex
@@ -754,6 +871,11 @@ struct EwPlan {
     uint32_t rows2_scalar, rows2_waves;
     int rows2_wpb; // waves per block
     int64_t rows2_pairs;
+    // ew_outer_kernel (outer != 0): inputs that are one value per row, blocks along dim inner - 1
+    // (outer_fit: the call fits it, with the launch shape below; outer: the functor has it and it is taken)
+    int outer, outer_fit, outer_block;
+    uint32_t outer_per_row, outer_mid_blocks;
+    int64_t outer_col_blocks, outer_grid;
     // tile path
     uint32_t tmask; // inputs staged through LDS
     int dT;         // the dim those inputs are contiguous along
@@ -795,6 +917,15 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
                     if (pl.rows2_pat == decltype(pat_c)::value) pl.path = DPX_PATH_EW_ROWS2;
                 },
                 typename rows2_patterns<N>::seq{});
+    }
+    pl.outer = 0;
+    if constexpr (outer_enabled<Fn>::value) {
+        if (pl.path == DPX_PATH_EW_ROWS && pl.outer_fit) {
+            pl.outer = 1;
+            pl.block = pl.outer_block;
+            pl.col_blocks = pl.outer_col_blocks;
+            pl.grid = pl.outer_grid;
+        }
     }
     if (pl.path == DPX_PATH_NOOP || dry) return hipSuccess;
     InPtrs<N> in;
@@ -849,6 +980,13 @@ inline hipError_t ew_launch(const Fn &fn, EwPlan &pl, const dpx_array_view *cons
                                                stream, fn, ix, out, in, pl.rows2_scalar, pl.rows2_waves, pl.rows2_pairs);
                     },
                     typename rows2_patterns<N>::seq{});
+                return hipGetLastError();
+            }
+        }
+        if constexpr (outer_enabled<Fn>::value) {
+            if (pl.outer) {
+                hipLaunchKernelGGL((ew_outer_kernel<Fn, Out, Ins...>), dim3((unsigned)pl.grid), dim3(pl.block), 0, stream,
+                                   fn, ix, out, in, pl.outer_per_row, pl.outer_mid_blocks, (uint32_t)pl.col_blocks);
                 return hipGetLastError();
             }
         }

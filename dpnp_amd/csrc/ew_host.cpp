@@ -52,6 +52,7 @@ void ew_make_plan(EwPlan &pl, int nops, const dpx_array_view *const *views)
     pl.bcast = pl.modes = 0;
     pl.tx_log2 = 0;
     pl.rows2_pat = -1;
+    pl.outer = pl.outer_fit = 0;
     pl.rows2_scalar = pl.rows2_waves = 0;
     pl.rows2_pairs = 0;
     pl.rows2_wpb = 1;
@@ -235,7 +236,7 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
         // One full-size input and the output, both in aligned packs, every other input broadcast along some dim
         // (a matrix plus a row, times a column, minus a per-channel constant): one-wave blocks, like the contiguous
         // kernel's (fp32 16384 x 16384 plus a row or a column: 74 -> 80 % of the HBM rate).  Calls that only write
-        // (an outer sum) are bound by the rate waves are launched at and keep four waves per block; two full-size
+        // (an outer sum) keep four waves per block (and, for two-operand functions, take ew_outer_kernel); two full-size
         // inputs gain nothing, and lose 7 points when their rows do not start on 16-byte boundaries.
         int streaming = 0;
         bool aligned = ((pl.modes >> (2 * (nops - 1))) & 3u) == MODE_VEC;
@@ -260,6 +261,38 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
     const int64_t tx = (int64_t)1 << lg, ty = pl.block / tx;
     pl.col_blocks = (per_row + tx - 1) / tx;
     pl.grid = pl.col_blocks * ((pl.nrows + ty - 1) / ty);
+    // Does the call fit ew_outer_kernel?  Two inputs, a contiguous output, and every input one value per row, or a
+    // row vector (contiguous along the inner dim) that is the same for all rows of dim inner - 1 or for all indices
+    // of an earlier dim: nothing of the output's size is read.  Enough rows and columns for its blocks.
+    pl.outer_fit = 0;
+    if (pl.nd >= 2 && nops == 3 && pl.strides[nops - 1][inner] == 1 && pl.shape[inner - 1] >= 16 && per_row >= 16 &&
+        tune_int("DPX_EW_OUTER", 1) != 0) {
+        bool ok = true;
+        uint32_t mask = 0;
+        for (int k = 0; k + 1 < nops; ++k) {
+            const int64_t si = pl.strides[k][inner], sm = pl.strides[k][inner - 1];
+            if (si == 0) mask |= 1u << k;
+            else if (si != 1) ok = false;
+            else if (sm != 0) {
+                // a vector per row: only one that is the same for every index of some earlier dim (a small operand)
+                bool repeats = false;
+                for (int d = 0; d < inner - 1; ++d) repeats = repeats || (pl.strides[k][d] == 0 && pl.shape[d] > 1);
+                ok = ok && repeats;
+            }
+        }
+        int64_t before = 1;
+        for (int d = 0; d < inner - 1; ++d) before *= pl.shape[d];
+        const int block = (int)std::min<int64_t>(256, (per_row + 63) / 64 * 64);
+        const int64_t cbs = (per_row + block - 1) / block, mbs = (pl.shape[inner - 1] + EW_OUTER_ROWS - 1) / EW_OUTER_ROWS;
+        if (ok && before <= 0x7fffffff && cbs * mbs <= 0x7fffffff / std::max<int64_t>(before, 1)) {
+            pl.outer_fit = 1;
+            pl.outer_per_row = mask;
+            pl.outer_mid_blocks = (uint32_t)mbs;
+            pl.outer_block = block;
+            pl.outer_col_blocks = cbs;
+            pl.outer_grid = cbs * mbs * before;
+        }
+    }
     // Does the call fit ew_rows2_kernel?  Rows of whole waves of packs, an even number of them along
     // dim inner - 1, a contiguous output, and every input one of: stride 2 along the inner dim
     // (elements as wide as a pack allows), contiguous and moving with the rows, or the same for

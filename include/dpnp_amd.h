@@ -264,7 +264,8 @@ typedef enum dpx_search_op {
 typedef enum dpx_path {
     DPX_PATH_NOOP = 0,          /* zero-size: nothing launched */
     DPX_PATH_EW_CONTIG = 1,     /* 1-D unit-stride, 128-bit accesses */
-    DPX_PATH_EW_ROWS = 2,       /* N-D, threads vectorised along the inner dim */
+    DPX_PATH_EW_ROWS = 2,       /* N-D, threads vectorised along the inner dim (calls of two-operand functions that
+                                   read nothing of the output's size, an outer sum, take blocks of 8 rows) */
     DPX_PATH_EW_ROWS2 = 3,      /* a stride-2 input, rows of whole waves: two rows per thread, reads fixed at compile time */
     DPX_PATH_EW_TILE = 4,       /* inputs contiguous along another dim than the output: LDS tile */
     DPX_PATH_RED_ROWS = 10,     /* reduced run contiguous: block or wave per output */

@@ -228,6 +228,15 @@ def test_elementwise_plans():
     assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256
     p = plan_binary("add", view([16384, 16383]), view([16384, 16383], [0, 1], ptr=P1), view([16384, 16383], ptr=P2))
     assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256
+    # a row plus a column (nothing of the output's size is read): blocks of 8 rows x 256 packs
+    p = plan_binary("add", view([16384, 16384], [0, 1]), view([16384, 16384], [1, 0], ptr=P1), view([16384, 16384], ptr=P2))
+    assert L.PATH_NAMES[p.path] == "ew_rows" and p.block == 256 and p.grid[0] == (16384 // 8) * (16384 // 1024)
+    # ... X[:, None, :] - Y[None, :, :] as well; a full-size operand keeps the general kernel's one row per thread
+    p = plan_binary("subtract", view([64, 512, 1024], [1024, 0, 1]), view([64, 512, 1024], [0, 1024, 1], ptr=P1),
+                    view([64, 512, 1024], ptr=P2))
+    assert p.block == 256 and p.grid[0] == 64 * (512 // 8)
+    p = plan_binary("add", view([16384, 16384]), view([16384, 16384], [1, 0], ptr=P1), view([16384, 16384], ptr=P2))
+    assert p.grid[0] == 16384 * 16384 // 4 // p.block
     # empty
     p = plan_binary("add", view([0, 3]), view([0, 3]), view([0, 3]))
     assert L.PATH_NAMES[p.path] == "noop"

@@ -1104,6 +1104,59 @@ def test_mixed_dtype_arithmetic_equals_cast_then_compute(op, pair):
         assert_same(host(d2), a + b.astype(wide))
 
 
+@pytest.mark.parametrize("dt", ["?", "i1", "u2", "i4", "i8", "f2", "f4", "f8", "c8", "c16"])
+def test_calls_that_only_write_outer_forms(dt):
+    # a row vector with one value per row (an outer sum, a row minus a column, 3-d forms of the same): blocks of 64
+    # rows, the per-row values handed from lane to lane.  Every row and column count around the block's edges, both
+    # operand orders, results of another type (comparisons), rows of a wider matrix as output, a column read
+    # backwards, and the same calls through dpnp's `outer`
+    import dpnp_amd as dpnp
+
+    rng = np.random.default_rng(61)
+    ops = ["add", "subtract", "multiply", "less", "maximum"] if dt not in ("c8", "c16") else ["add", "subtract", "multiply", "equal"]
+    if dt == "?":
+        ops = ["logical_and", "logical_xor", "add", "not_equal"]
+    for rows, cols in ((16, 64), (17, 67), (63, 256), (64, 1024), (65, 1031), (130, 4100), (1000, 259), (20, 20000)):
+        r = random_array(rng, (1, cols), dt, -50, 50)
+        c = random_array(rng, (rows, 1), dt, -50, 50)
+        for op in ops:
+            f = getattr(np, op)
+            with np.errstate(all="ignore"):
+                if op == "multiply" and dt in ("c8", "c16"):  # (the last bit of a complex product depends on fusion)
+                    tol = 1e-6 if dt == "c8" else 1e-14
+                    np.testing.assert_allclose(host(dpt.multiply(dev(r), dev(c))), f(r, c), rtol=tol, atol=tol * 2500)
+                    np.testing.assert_allclose(host(dpt.multiply(dev(c), dev(r))), f(c, r), rtol=tol, atol=tol * 2500)
+                    continue
+                assert_same(host(getattr(dpt, op)(dev(r), dev(c))), f(r, c))
+                assert_same(host(getattr(dpt, op)(dev(c), dev(r))), f(c, r))
+    r = random_array(rng, (1, 777), dt, -50, 50)
+    c = random_array(rng, (300, 1), dt, -50, 50)
+    op = ops[1]
+    with np.errstate(all="ignore"):
+        want = getattr(np, op)(r, c[::-1])
+    assert_same(host(getattr(dpt, op)(dev(r), dev(c)[::-1])), want)                    # the column read backwards
+    big = dpt.zeros((300, 1000), dtype=want.dtype)
+    getattr(dpt, op)(dev(r), dev(c)[::-1], out=big[:, 100:877])                         # rows of a wider matrix
+    assert_same(host(big)[:, 100:877], want)
+    assert not host(big)[:, :100].any() and not host(big)[:, 877:].any()
+    # three dims: (B, 1, C) with (1, M, 1), and (B, M, 1) with (1, 1, C)
+    p3, q3 = random_array(rng, (5, 1, 300), dt, -50, 50), random_array(rng, (1, 70, 1), dt, -50, 50)
+    u3, v3 = random_array(rng, (5, 70, 1), dt, -50, 50), random_array(rng, (1, 1, 300), dt, -50, 50)
+    with np.errstate(all="ignore"):
+        assert_same(host(getattr(dpt, op)(dev(p3), dev(q3))), getattr(np, op)(p3, q3))
+        assert_same(host(getattr(dpt, op)(dev(u3), dev(v3))), getattr(np, op)(u3, v3))
+    # pairwise forms, X[:, None, :] with Y[None, :, :]: one operand's vector moves with the rows, the other's stays
+    for n, m, d in ((7, 40, 64), (3, 17, 257), (20, 9, 1000)):
+        xa, ya = random_array(rng, (n, 1, d), dt, -50, 50), random_array(rng, (1, m, d), dt, -50, 50)
+        with np.errstate(all="ignore"):
+            assert_same(host(getattr(dpt, op)(dev(xa), dev(ya))), getattr(np, op)(xa, ya))
+            assert_same(host(getattr(dpt, op)(dev(ya), dev(xa))), getattr(np, op)(ya, xa))
+    if dt in ("f4", "f8", "i4"):
+        x, y = random_array(rng, (500,), dt, -50, 50), random_array(rng, (333,), dt, -50, 50)
+        assert_same(dpnp.asnumpy(dpnp.multiply.outer(dpnp.array(x), dpnp.array(y))), np.multiply.outer(x, y))
+        assert_same(dpnp.asnumpy(dpnp.subtract.outer(dpnp.array(x), dpnp.array(y))), np.subtract.outer(x, y))
+
+
 @pytest.mark.parametrize("op", ["add", "subtract", "multiply", "divide"])
 @pytest.mark.parametrize("idt", ["i4", "i8"])
 def test_float32_with_integer_gives_float64_in_one_kernel(op, idt):
