@@ -385,7 +385,10 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_rows_kernel(Fn fn,
 // arithmetic and a load of every operand on each pack of output (fp32 row + column into 16384 x 16384: 63 % of
 // the HBM rate where a fill of the same matrix writes at 84 %).  Few rows per block: a thread that stores one
 // row after the other writes slower the longer it goes on (a stand-alone kernel of 256 threads storing 4 KiB runs
-// of 2 / 4 / 8 / 16 / 64 rows: 84 / 82 / 82 / 78 / 55 % of the HBM rate).
+// of 2 / 4 / 8 / 16 / 64 rows of 64 KiB: 84 / 82 / 82 / 78 / 55 % of the HBM rate; where the rows are no longer than
+// the runs, so that a block's rows lie end to end, 2 / 8 rows: 75 / 67 %; rows dealt to the blocks in turn instead
+// of in runs: 60 %).  Two rows per block for such short rows help where the row vector is one for the whole call
+// (67 -> 74 %) and cost more than that where every block has to fetch its own (68 -> 49 %), so 8 it is.
 constexpr int EW_OUTER_ROWS = 8;
 template <class T> DPX_D T lane_value(T v, int lane) // v of lane `lane` (uniform), for every lane
 {
