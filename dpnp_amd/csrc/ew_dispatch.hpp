@@ -75,5 +75,6 @@ template <class Op, class T> struct BinaryFn {
 template <class Op, class T> struct rows2_enabled<UnaryFn<Op, T>> : std::true_type {};
 template <class Op, class T> struct rows2_enabled<BinaryFn<Op, T>> : std::true_type {};
 template <class Op, class T> struct outer_enabled<BinaryFn<Op, T>> : std::true_type {};
+template <class Op, class T> struct straight_rows_enabled<BinaryFn<Op, T>> : std::true_type {};
 
 } // namespace dpx
