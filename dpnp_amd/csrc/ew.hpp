@@ -286,7 +286,8 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     const int inner = ix.nd - 1;
     const int64_t ncols = ix.shape[inner];
     const int64_t col0 = (((int64_t)cb << tx_log2) + tx) * E;
-    if (row >= nrows || col0 >= ncols) return;
+    // (STRAIGHT: the packs are moved back by up to E - 1 columns, below, and the host counts a thread more per row)
+    if (row >= nrows || col0 >= ncols + (STRAIGHT ? E - 1 : 0)) return;
 
     int64_t off[N + 1];
 #pragma unroll
@@ -317,17 +318,25 @@ DPX_D void ew_rows_body(const Fn &fn, const NdIndex<sizeof...(Ins) + 1> &ix, Out
     const bool wave_full = tx_log2 >= 6 && col0 - (int64_t)(threadIdx.x & 63) * E + 64 * E < ncols;
     if constexpr (STRAIGHT) {
         // (fp32 A[:, :h] + A[:, h:] and A[::2] + B[::2] over 16384 x 16384: 73 -> 77-79 % of the HBM rate)
-        if (cnt == E) {
+        // The packs of a row are laid so that the stores are aligned: a row of the output that starts m elements
+        // past a pack boundary (rows of A[1:-1, 1:-1], rows of odd length) has its packs moved back by m columns;
+        // the first thread of the row then holds E - m elements, the last what is left.
+        const int m = (int)(((uintptr_t)(out + off[N] - col0) / sizeof(Out)) & (uintptr_t)(E - 1));
+        const int64_t c = col0 - m;
+        const int64_t first = c < 0 ? 0 : c, last = (c + E < ncols) ? c + E : ncols;
+        if (last <= first) return;
+        const int64_t shift = first - col0;
+        if (last - first == E) {
             std::tuple<pack<Ins, E>...> x;
-            ((std::get<I>(x) = load_pack<Ins, E>((const Ins *)in.p[I] + off[I])), ...);
+            ((std::get<I>(x) = load_pack<Ins, E>((const Ins *)in.p[I] + off[I] + shift)), ...);
             (keep_whole(std::get<I>(x)), ...);
             pack<Out, E> r;
 #pragma unroll
             for (int e = 0; e < E; ++e) r.v[e] = to_storage<Out>(fn(to_value(std::get<I>(x).v[e])...));
-            store_pack<Out, E>(out + off[N], r);
+            store_pack<Out, E>(out + off[N] + shift, r);
         }
         else {
-            for (int e = 0; e < cnt; ++e)
+            for (int64_t e = shift; e < last - col0; ++e)
                 out[off[N] + e] = to_storage<Out>(fn(to_value(load_one((const Ins *)in.p[I] + off[I] + e))...));
         }
         return;

@@ -230,7 +230,19 @@ void ew_finish_plan(EwPlan &pl, int E, int U, const int *itemsize, const void *c
         pl.modes |= mode << (2 * k);
     }
     pl.modes |= keep_bits(pl);
-    const int64_t per_row = (ncols + E - 1) / E; // threads wanted along a row
+    // threads wanted along a row (every operand contiguous along the inner dim and read once: the straight-line
+    // form of the rows kernel may move a row's packs back by up to E - 1 columns, which takes one thread more)
+    bool all_vec = !(pl.modes >> MODE_KEEP_SHIFT);
+    for (int k = 0; k < nops; ++k) all_vec = all_vec && ((pl.modes >> (2 * k)) & 3u) == MODE_VEC;
+    {
+        // (... unless every row of the output starts on a pack boundary)
+        const int64_t pack_bytes = (int64_t)E * itemsize[nops - 1];
+        bool rows_aligned = (uintptr_t)ptrs[nops - 1] % (uintptr_t)pack_bytes == 0;
+        for (int d = 0; d < inner; ++d)
+            rows_aligned = rows_aligned && (pl.shape[d] == 1 || (pl.strides[nops - 1][d] * itemsize[nops - 1]) % pack_bytes == 0);
+        all_vec = all_vec && !rows_aligned;
+    }
+    const int64_t per_row = (ncols + (all_vec ? E - 1 : 0) + E - 1) / E;
     pl.block = env_block("DPX_EW_ROWS_BLOCK", EW_ROWS_BLOCK);
     {
         // One full-size input and the output, both in aligned packs, every other input broadcast along some dim

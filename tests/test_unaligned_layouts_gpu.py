@@ -160,3 +160,37 @@ def test_matrix_with_rows_of_megabytes_plus_a_row(dt):
     np.testing.assert_array_equal(host(dpt.multiply(da, dcol)), a * col)
     np.testing.assert_array_equal(host(dpt.where(dpt.greater(dpt.real(da) if dt == "c8" else da, 0), da, drow)),
                                   np.where(a.real > 0, a, row))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", ["i1", "f2", "f4", "f8", "c16"])
+def test_two_sliced_operands_every_alignment_of_the_output_rows(dt):
+    # a + b over column slices of wider matrices: the rows kernel's straight-line form lays a row's packs so that the
+    # stores are aligned, whatever the first column of the output slice; every offset of the three operands up to
+    # two packs, row lengths around whole packs, result rows as rows of a wider matrix, every other row, reversed
+    # rows, and a result type narrower than the operands (a comparison).  Guard columns stay untouched.
+    rng = np.random.default_rng(67)
+    per_pack = 16 // np.dtype(dt).itemsize
+    wide = 4 * per_pack + 300
+    a = random_array(rng, (37, wide), dt, -60, 60)
+    b = random_array(rng, (37, wide), dt, -60, 60)
+    da, db = dev(a), dev(b)
+    for length in (1, per_pack - 1, per_pack, per_pack + 1, 5 * per_pack + 3, 256, 257):
+        for oa, ob, oo in ((0, 0, 0), (1, 1, 1), (1, 2, 3), (per_pack - 1, 0, per_pack + 1), (3, per_pack, 2 * per_pack - 1),
+                           (2, 2, 0), (0, 1, per_pack)):
+            if max(oa, ob, oo) + length > wide:
+                continue
+            want = a[:, oa:oa + length] + b[:, ob:ob + length]
+            out = dpt.full((37, wide), 7, dtype=dt)
+            dpt.add(da[:, oa:oa + length], db[:, ob:ob + length], out=out[:, oo:oo + length])
+            got = host(out)
+            assert_same(got[:, oo:oo + length], want)
+            assert (got[:, :oo] == 7).all() and (got[:, oo + length:] == 7).all()
+    assert_same(host(dpt.subtract(da[:36:2, 1:-1], db[1::2, 2:])), a[:36:2, 1:-1] - b[1::2, 2:])
+    assert_same(host(dpt.add(da[::-1, 3:-2], db[:, 1:-4])), a[::-1, 3:-2] + b[:, 1:-4])
+    if dt != "c16":
+        assert_same(host(dpt.less(da[:, 1:-1], db[:, 2:])), a[:, 1:-1] < b[:, 2:])
+    # three dims, interior of a volume
+    v = random_array(rng, (6, 9, 70), dt, -60, 60)
+    dv = dev(v)
+    assert_same(host(dpt.add(dv[1:-1, 1:-1, 1:-1], dv[:-2, 2:, 2:])), v[1:-1, 1:-1, 1:-1] + v[:-2, 2:, 2:])
