@@ -84,6 +84,9 @@ WORKLOADS = {
               "over 2^27, column sums of a 32768x32768 int8 matrix",
     "colsearch": "argmax and max down the columns of fp32 matrices of 2^28 elements with 128 to 4096 columns, and argmax "
                  "along the middle axis of 65536x32x128",
+    "ewlayouts": "fp32 elementwise calls over 16384x16384 outside the named configurations: a matrix with a row / a "
+                 "column, calls that only write (an outer sum, pairwise differences, a fill), two operands over slices "
+                 "of wider matrices (halves, every other row, the interior), a transposed operand",
     "layouts": "fp32 2^28 elements reduced over dims that do not collapse into one run: a sliced matrix summed whole, "
                "axes (0, 2) of 3-d and 4-d arrays, every other column (sum, max, mean, argmax)",
 }
@@ -267,6 +270,28 @@ def build_workload(name, dpnp, torch):
                # the 8192 results to float32, two small launches)
                ("var_every_other_column_axis0", lambda: dpnp.var(A[:, ::2], axis=0, out=rh), 4 * n, n // 2),
                ("var_axes02_256x1024x1024", lambda: dpnp.var(X3s, axis=(0, 2), out=r1024), 4 * n, n)]
+        return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
+    if name == "ewlayouts":
+        side = 1 << 14
+        n, h = side * side, side // 2
+        A, B = normal((side, side)), normal((side, side))
+        C = dpnp.empty((side, side), dtype="f4")
+        row, col = normal((1, side)), normal((side, 1))
+        X, Y = normal((1024, 1, 1024)), normal((1, 256, 1024))
+        P = dpnp.empty((1024, 256, 1024), dtype="f4")
+        inner = (side - 2) * (side - 2)
+        ops = [("add_A_B", lambda: dpnp.add(A, B, out=C), 12 * n, n),
+               ("add_A_row", lambda: dpnp.add(A, row, out=C), 8 * n, n),
+               ("multiply_A_col", lambda: dpnp.multiply(A, col, out=C), 8 * n, n),
+               ("fill", lambda: C.fill(1.5), 4 * n, n),
+               ("outer_add_row_col", lambda: dpnp.add(row, col, out=C), 4 * n, n),
+               ("pairwise_subtract_1024x256x1024", lambda: dpnp.subtract(X, Y, out=P), 4 * n, n),
+               ("add_halves_of_the_columns", lambda: dpnp.add(A[:, :h], A[:, h:], out=C[:, :h]), 6 * n, n // 2),
+               ("add_every_other_row", lambda: dpnp.add(A[::2], B[::2], out=C[::2]), 6 * n, n // 2),
+               ("add_interior", lambda: dpnp.add(A[1:-1, 1:-1], B[1:-1, 1:-1], out=C[1:-1, 1:-1]), 12 * inner, inner),
+               ("sqrt_interior", lambda: dpnp.sqrt(A[1:-1, 1:-1], out=C[1:-1, 1:-1]), 8 * inner, inner),
+               ("add_A_BT", lambda: dpnp.add(A, B.T, out=C), 12 * n, n),
+               ("copy_AT", lambda: dpnp.copyto(C, A.T), 8 * n, n)]
         return ops, "f32", "synthetic (seeded normal(0,1), resident in HBM)"
     if name == "floors":
         return build_floors(dpnp, torch, uniform, normal)
@@ -539,7 +564,7 @@ def main():
                     help="metric workload only: leave out the short runs of cfg1..cfg5 that fill `configs`")
     ap.add_argument("--dump-steps", action="store_true", help="print every step's per-op times to stderr")
     ap.add_argument("--workload", default="metric",
-                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5, layouts "
+                    help="metric (default, the headline step) or one of the parity configurations cfg1..cfg5, layouts, ewlayouts "
                          "or floors, measured the same way")
     ap.add_argument("--ops", default=None,
                     help="comma-separated subset of the workload's ops (profiling runs); 'copy' in the metric "
