@@ -80,8 +80,9 @@ WORKLOADS = {
               "call it bounds: Black-Scholes split into its memory streams and its arithmetic, the 2^24 read with and "
               "without a cross-block step, every-other-column reads, 512-byte runs on both sides of a transposition",
     "survey": "functions outside the named configurations that run furthest below the HBM rate: fp64 pow / asinh / atanh / "
-              "log1p / tan over 2^26 elements, complex128 exp / sin / cos / sinh / tanh / expm1 over 2^25, float16 sin / sinh "
-              "over 2^27, column sums of a 32768x32768 int8 matrix",
+              "log1p / tan / sin / cos / logaddexp over 2^26 elements, complex128 exp / sin / cos / sinh / tanh / expm1 over "
+              "2^25, float16 sin / sinh over 2^27, column sums of a 32768x32768 int8 matrix, the variance of a 16384x32768 "
+              "float16 matrix down its columns",
     "colsearch": "argmax and max down the columns of fp32 matrices of 2^28 elements with 128 to 4096 columns, and argmax "
                  "along the middle axis of 65536x32x128",
     "ewlayouts": "fp32 elementwise calls over 16384x16384 outside the named configurations: a matrix with a row / a "
@@ -311,11 +312,18 @@ def build_workload(name, dpnp, torch):
         ops = [("pow_f64", lambda: dpnp.power(x, y, out=o), 24 * n, n)]
         for fn in ("arcsinh", "arctanh", "log1p", "tan"):
             ops.append((f"{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))
+        for fn in ("sin", "cos"):
+            ops.append((f"{fn}_f64", lambda f=getattr(dpnp, fn): f(y, out=o), 16 * n, n))
+        ops.append(("logaddexp_f64", lambda: dpnp.logaddexp(x, y, out=o), 24 * n, n))
         for fn in ("exp", "sin", "cos", "sinh", "tanh", "expm1"):
             ops.append((f"{fn}_c128", lambda f=getattr(dpnp, fn): f(z, out=oz), 32 * n2, n2))
         for fn in ("sin", "sinh"):
             ops.append((f"{fn}_f16", lambda f=getattr(dpnp, fn): f(xh, out=oh), 4 * n3, n3))
         ops.append(("sum_axis0_int8_32768sq", lambda: dpnp.sum(B8, axis=0, out=o8), 1 << 30, 1 << 30))
+        H16 = dpnp.astype(uniform((1 << 14, 1 << 15)), "f2")
+        ov = dpnp.empty(1 << 15, dtype="f2")
+        # (variance in one pass, float64 accumulation; the time includes two small launches that finish the result)
+        ops.append(("var_axis0_f16_16384x32768", lambda: dpnp.var(H16, axis=0, out=ov), 1 << 30, 1 << 29))
         # the real functions the complex ones are built from (only with --ops: for instruction counts)
         for fn in ("exp", "sin", "cos", "sinh", "cosh", "expm1", "log"):
             ops.append((f"ref:{fn}_f64", lambda f=getattr(dpnp, fn): f(xs, out=o), 16 * n, n))
