@@ -1142,11 +1142,13 @@ __global__ __launch_bounds__(COLS_MAX_BLOCK) void red_cols_kernel(RedIndex ix, R
                             }
                         };
                         if constexpr (WHOLE && sizeof(In) <= 2) {
-                            // 1- and 2-byte inputs: two packs sent for before the two in hand are taken (the loop of the
-                            // sums below, see there: 64 to 128 elements a round at five double-precision instructions
-                            // each otherwise pass with nothing in flight; float16 16384 x 32768: 38 % of the HBM rate)
+                            // 1- and 2-byte inputs: a round's packs are sent for before the round in hand is taken (the
+                            // loop of the sums below, see there: 64 to 128 elements a round at five double-precision
+                            // instructions each otherwise pass with nothing in flight).  Unlike the sums, whose arithmetic
+                            // is next to nothing, this loop wants whole rounds in flight: float16 16384 x 32768 with 8
+                            // packs loaded and then taken 38 % of the HBM rate, 2 + 2 in flight 57 %, 4 + 4: 72 %, 8 + 8: 74 %.
                             static_assert(sizeof(In) * E == 16);
-                            constexpr int H = 2;
+                            constexpr int H = E >= 16 ? 4 : 8;
                             u32x4 va[H], vb[H];
                             auto send_for = [&](u32x4(&d)[H], int64_t row) {
 #pragma unroll
