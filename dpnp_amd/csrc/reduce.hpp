@@ -421,7 +421,8 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
     static constexpr bool has_pack_fold =
         !FINAL && sizeof(In) == 1 &&
         (KIND == K_ANY || KIND == K_ALL || KIND == K_COUNT_NONZERO ||
-         (KIND == K_SUM && (is_int_v<In> || is_bool_v<In>) && (is_int_v<Out> || int_sum)));
+         (KIND == K_SUM && (is_int_v<In> || is_bool_v<In>) && (is_int_v<Out> || int_sum)) ||
+         ((KIND == K_MAX || KIND == K_MIN) && is_int_v<In> && std::is_same_v<In, Out>));
     DPX_D static Acc fold_pack(Acc acc, const u32x4 &words)
     {
         // (the kernel loads the words as such: a pack of bytes viewed as words makes the compiler
@@ -429,7 +430,30 @@ template <int KIND, class In_, class Out_, bool FINAL = false> struct RedPolicy 
         struct {
             uint32_t w[4];
         } u = {{words[0], words[1], words[2], words[3]}};
-        if constexpr (KIND == K_ANY) return acc | (Acc)((u.w[0] | u.w[1] | u.w[2] | u.w[3]) != 0);
+        if constexpr (KIND == K_MAX || KIND == K_MIN) {
+            // the bytes of even and of odd places as pairs of 16-bit numbers, eight pairs folded by the packed
+            // maximum: 23 instructions for 16 elements where taking them one by one costs about 40
+            using S = std::conditional_t<std::is_signed_v<In>, short, unsigned short>;
+            typedef S s2 __attribute__((ext_vector_type(2)));
+            auto even = [](uint32_t w) {
+                if constexpr (std::is_signed_v<In>) return (__builtin_bit_cast(s2, w) << 8) >> 8;
+                else return __builtin_bit_cast(s2, w & 0x00ff00ffu);
+            };
+            auto odd = [](uint32_t w) {
+                if constexpr (std::is_signed_v<In>) return __builtin_bit_cast(s2, w) >> 8;
+                else return __builtin_bit_cast(s2, (w >> 8) & 0x00ff00ffu);
+            };
+            auto op = [](s2 a, s2 b) {
+                if constexpr (KIND == K_MAX) return __builtin_elementwise_max(a, b);
+                else return __builtin_elementwise_min(a, b);
+            };
+            s2 m = op(even(u.w[0]), odd(u.w[0]));
+#pragma unroll
+            for (int i = 1; i < 4; ++i) m = op(m, op(even(u.w[i]), odd(u.w[i])));
+            const S r = (KIND == K_MAX) ? (m.x > m.y ? m.x : m.y) : (m.x < m.y ? m.x : m.y);
+            return combine(acc, (Acc)(In)r);
+        }
+        else if constexpr (KIND == K_ANY) return acc | (Acc)((u.w[0] | u.w[1] | u.w[2] | u.w[3]) != 0);
         else if constexpr (KIND == K_ALL) {
             uint32_t z = 0; // bit 7 of a byte set: that byte is zero
 #pragma unroll

@@ -857,6 +857,9 @@ def test_one_byte_counting_reductions_word_arithmetic(dt):
             assert_same(host(dpt.sum(dv)), orc.reduce("sum", v, 1))
             assert_same(host(dpt.count_nonzero(dv)), np.array(np.count_nonzero(v), "i8"))
             assert bool(dpt.any(dv)) == bool(v.any()) and bool(dpt.all(dv)) == bool(v.all())
+            if dt != "?" and v.size:  # max and min fold a pack with packed 16-bit instructions
+                assert_same(host(dpt.max(dv)), np.array(v.max(), dt))
+                assert_same(host(dpt.min(dv)), np.array(v.min(), dt))
     z = np.zeros(100003, dtype=dt)
     assert not bool(dpt.any(dev(z))) and int(dpt.count_nonzero(dev(z))) == 0
     z[77777] = True if dt == "?" else (-128 if dt == "i1" else 128)
@@ -870,6 +873,18 @@ def test_one_byte_counting_reductions_word_arithmetic(dt):
     assert_same(host(dpt.sum(dm, axis=1)), orc.reduce("sum", m, 1))
     assert_same(host(dpt.count_nonzero(dm, axis=1)), np.count_nonzero(m, axis=1).astype("i8"))
     assert_same(host(dpt.all(dm, axis=1)), m.astype(bool).all(axis=1))
+    if dt != "?":
+        # the extreme of each row planted at every place of a pack, among values next to it
+        lo, hi = (np.iinfo(dt).min, np.iinfo(dt).max)
+        e = rng.integers(lo + 2, hi - 1, (64, 4099)).astype(dt)
+        for r in range(64):
+            e[r, 2048 + r] = hi if r % 2 else hi - 1
+            e[r, 1000 + 3 * r] = lo if r % 3 else lo + 1
+        de = dev(e)
+        assert_same(host(dpt.max(de, axis=1)), e.max(axis=1))
+        assert_same(host(dpt.min(de, axis=1)), e.min(axis=1))
+        assert_same(host(dpt.max(de[:, 1:])), np.array(e[:, 1:].max(), dt))
+        assert_same(host(dpt.min(de[3:, 5:4000], axis=1)), e[3:, 5:4000].min(axis=1))
     assert_same(host(dpt.any(dm[:, :5], axis=1)), m[:, :5].astype(bool).any(axis=1))
     assert_same(host(dpt.sum(dm, axis=1, dtype="i4")), orc.reduce("sum", m, 1, out_dtype="i4"))
 
